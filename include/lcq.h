@@ -1,0 +1,122 @@
+/* lcq.h — C ABI of liblcq.so: gfx950 (MI355X) kernels for the layer-wise
+ * quantization hot path of ModelTC/LightCompress (`llmc`).
+ *
+ * The reference has no FFI: its boundary for this path is a Python class API
+ * (IntegerQuantizer / FloatQuantizer, GPTQ, Awq, *RealQuantLinear.pack).  The
+ * Python layer in `lightcompress_amd/` keeps those classes and calls the
+ * entry points below through ctypes.  Each entry point cites the reference
+ * function it replaces as file:line under llmc/compression/quantization/.
+ *
+ * Conventions
+ *  - every pointer is a DEVICE pointer owned by the caller (a torch tensor's
+ *    data_ptr()); `stream` is a hipStream_t passed as void* (NULL = default
+ *    stream); calls only enqueue work and return immediately;
+ *  - no entry point allocates: scratch memory is a caller-provided workspace
+ *    whose size the matching *_workspace_bytes() call returns;
+ *  - return value: 0 ok, <0 rejected before any launch (LCQ_E*);
+ *  - matrices are dense row-major;
+ *  - stateless and re-entrant; calls on one stream execute in order.
+ */
+#ifndef LCQ_H
+#define LCQ_H
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types */
+#define LCQ_F32 0
+#define LCQ_BF16 1
+#define LCQ_F16 2
+
+/* storage of integer / float codes */
+#define LCQ_CODE_NONE 0
+#define LCQ_CODE_U8 1
+#define LCQ_CODE_I8 2
+#define LCQ_CODE_I32 3
+#define LCQ_CODE_SAME 4      /* codes stored as floats of the input type (what .quant() returns) */
+#define LCQ_CODE_F32 5       /* FloatQuantizer.quant(): fp32 values on the minifloat grid */
+#define LCQ_CODE_FP8 6       /* float8_e4m3fn / float8_e5m2 bytes */
+
+/* flags */
+#define LCQ_FLAG_SYM 1            /* symmetric: zero point is 0 */
+#define LCQ_FLAG_NO_ROUND_ZP 2    /* round_zp=False, quant.py:556-557,702-706 */
+#define LCQ_FLAG_STATIC 4         /* scales/zeros are INPUTS (…_static methods) */
+#define LCQ_FLAG_SCALAR_QP 8      /* one (scale, zero) for the whole tensor (per_tensor) */
+#define LCQ_FLAG_TIE_EVEN 16      /* minifloat rounding: ties to even instead of away from zero */
+#define LCQ_FLAG_NO_SUBNORMALS 32 /* minifloat rounding: flush below the minimum normal */
+#define LCQ_FLAG_DQ_F32 64        /* lcq_quant_fp: write dq as fp32 instead of the input type */
+
+/* errors */
+#define LCQ_OK 0
+#define LCQ_EINVAL (-1)
+#define LCQ_EALIGN (-2)
+#define LCQ_EDTYPE (-3)
+#define LCQ_ELAUNCH (-4)
+
+/* ---- integer quantizer -------------------------------------------------- */
+
+/* Fused get_tensor_qparams + quant (+ dequant) over `rows` rows of `cols`
+ * elements (the reshaped tensor of quant.py:611-641).
+ * Replaces quant.py:134-145 (min/max), :544-558 (get_qparams), :698-716
+ * (quant / dequant / quant_dequant) and so the bodies of
+ * fake_quant_{weight,act}_{dynamic,static} (:718-868) and
+ * real_quant_weight_{dynamic,static} (:870-952).
+ *  x       [rows, cols] of `dtype` (LCQ_F32 | LCQ_BF16)
+ *  dq      same shape/type or NULL        -> (q - z) * (s * out_scale_factor)
+ *  codes   [rows, cols] of code_dtype or NULL
+ *  scales  [rows] (or [1] with SCALAR_QP) of `dtype`: output, input if STATIC
+ *  zeros   likewise; may be NULL (zero point 0; never written when SYM)
+ * bf16 rows round to bf16 after every arithmetic step like torch does. */
+int lcq_quant_int(const void* x, int dtype, int64_t rows, int64_t cols, float qmin, float qmax, int flags,
+                  float out_scale_factor, void* dq, void* codes, int code_dtype, void* scales, void* zeros,
+                  void* stream);
+
+/* get_minmax_range, quant.py:141-143: per-row amin / amax, outputs [rows] of `dtype`. */
+int lcq_minmax_rows(const void* x, int dtype, int64_t rows, int64_t cols, void* min_out, void* max_out, void* stream);
+
+/* get_minmax_range per_tensor, quant.py:135-137: outputs [1] of `dtype`. */
+int64_t lcq_minmax_all_workspace_bytes(void);
+int lcq_minmax_all(const void* x, int dtype, int64_t n, void* min_out, void* max_out, void* workspace, void* stream);
+
+/* get_qparams, quant.py:544-558, on n explicit (min, max) pairs. */
+int lcq_qparams_int(const void* min_in, const void* max_in, int dtype, int64_t n, float qmin, float qmax, int flags,
+                    void* scales, void* zeros, void* stream);
+
+/* dequant, quant.py:709-711: out = (q - z) * (s * out_scale_factor). */
+int lcq_dequant_int(const void* q, int dtype, int64_t rows, int64_t cols, const void* scales, const void* zeros,
+                    int flags, float out_scale_factor, void* out, void* stream);
+
+/* ---- minifloat quantizer (FloatQuantizer, use_qtorch=True) -------------- */
+
+/* Fused get_tensor_qparams + quant (+ dequant), quant.py:1042-1080 and the
+ * bodies of fake_quant_* (:1082-1158) and real_quant_weight_* (:1160-1220):
+ *   s = clamp(absmax, 1e-5) / qmax;  t = x / s + 0;  q = float_quantize(float(t));
+ *   dq = (q - 0) * s  (fp32), cast to the row type unless LCQ_FLAG_DQ_F32.
+ *  codes: LCQ_CODE_F32 (what .quant() returns) or LCQ_CODE_FP8 (e4m3fn / e5m2 bytes)
+ * float_quantize's tie rule / subnormal handling are third-party semantics
+ * (QPyTorch) selectable with LCQ_FLAG_TIE_EVEN / LCQ_FLAG_NO_SUBNORMALS. */
+int lcq_quant_fp(const void* x, int dtype, int64_t rows, int64_t cols, int e_bits, int m_bits, float qmax, int flags,
+                 void* dq, void* codes, int code_dtype, void* scales, void* stream);
+
+/* FloatQuantizer.dequant, quant.py:1073-1075, on fp32 codes: out = (q - 0) * s in fp32. */
+int lcq_dequant_fp(const float* q, int64_t rows, int64_t cols, const void* scales, int scale_dtype, int flags,
+                   float* out, void* stream);
+
+/* ---- packing ------------------------------------------------------------ */
+
+/* VllmRealQuantLinear.pack, module_utils.py:929-955 (compressed-tensors order).
+ *  codes [R, K] of LCQ_CODE_I32 | LCQ_CODE_I8 | LCQ_CODE_U8 ; packed [R, ceil(K / (32/bits))] int32 */
+int lcq_pack_ct(const void* codes, int code_dtype, int64_t R, int64_t K, int bits, int32_t* packed, void* stream);
+
+/* AutoawqRealQuantLinear.gemm_pack, module_utils.py:1097-1158 (4-bit, order 0,2,4,6,1,3,5,7).
+ *  w [R, K] of `dtype` (F32 | BF16 | F16); scales [R, K/g] of `dtype`; zeros [R, K/g] int32
+ *  qweight [K, R/8] int32 ; scales_f16_out [K/g, R] fp16 ; qzeros [K/g, R/8] int32 ; R % 32 == 0 */
+int lcq_pack_awq(const void* w, int dtype, const void* scales, const int32_t* zeros, int64_t R, int64_t K, int group_size,
+                 int32_t* qweight, void* scales_f16_out, int32_t* qzeros, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LCQ_H */

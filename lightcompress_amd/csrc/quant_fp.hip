@@ -1,0 +1,212 @@
+// Minifloat ("FPx": e4m3, e5m2, e2m1, e3m2, e4m7) quantizer for gfx950,
+// the qtorch branch of FloatQuantizer:
+//   get_tensor_qparams / quant / dequant / quant_dequant, fake_quant_*_dynamic|
+//   static, real_quant_weight_dynamic|static
+// (llmc/compression/quantization/quant.py:962-1002, 1042-1080, 1099-1220).
+//
+// Per row:  s = clamp(absmax, 1e-5) / qmax ;  per element:
+//   t = x / s + 0.0            (in the row dtype: bf16 rows round to bf16)
+//   q = float_quantize(float(t), e_bits, m_bits, 'nearest')   (fp32, on the grid)
+//   dq = (q - 0.0) * s         (fp32 arithmetic, then cast to the output type)
+//
+// float_quantize is third-party (QPyTorch); its algorithm on the fp32 bit
+// pattern is restated here: add half of the dropped-mantissa ulp and truncate
+// (ties away from zero; LCQ_FLAG_TIE_EVEN switches to round-half-even, which
+// is what a native float8 cast does), fixed-step rounding below the minimum
+// normal (LCQ_FLAG_NO_SUBNORMALS flushes instead), exponent clipped at
+// 2^(e_bits-1).
+#include "rowquant.h"
+
+namespace {
+using namespace lcq;
+
+struct FpRow {
+  float s, r;
+  int fast;
+};
+
+template <bool BF_>
+struct FpOp {
+  static constexpr bool BF = BF_;
+  using Row = FpRow;
+  float qmax;
+  int e_bits, m_bits, tie_even, subnormals;
+  int is_static, scalar_qp, dq_f32, code_dtype;
+  // derived
+  uint32_t half, keep, max_mag;
+  int drop, min_exp, max_exp;
+  float min_normal;
+
+  __device__ __forceinline__ Row finish(float s) const {
+    Row p;
+    if (s == 0.0f) s = 1.0f;                               // scales[scales == 0] = 1, quant.py:1061
+    p.s = s;
+    p.r = 1.0f / s;
+    const float a = fabsf(s);
+    p.fast = (a > 8.6736174e-19f) && (a < 1.1529215e18f);
+    return p;
+  }
+  // get_qparams symmetric branch, quant.py:548-552 (qmax is a float tensor here)
+  __device__ __forceinline__ Row make(float mn, float mx) const {
+    const float cmin = BF ? 1.0013580322265625e-05f : 1e-5f;
+    float a = nan_max(fabsf(mx), fabsf(mn));
+    a = clamp_min_nan(a, cmin);
+    return finish(rnd<BF>(a / qmax));
+  }
+  __device__ __forceinline__ Row load(const void* scales, const void*, int64_t row) const {
+    return finish(load_scalar<BF>(scales, scalar_qp ? 0 : row));
+  }
+  __device__ __forceinline__ void store_qp(void* scales, void*, int64_t row, const Row& p) const {
+    store_scalar<BF>(scales, row, p.s);
+  }
+
+  __device__ __forceinline__ uint32_t round_mag(uint32_t m) const {
+    if (tie_even) return (m + half - 1u + ((m >> drop) & 1u)) & keep;
+    return (m + half) & keep;
+  }
+
+  // rounding of an fp32 value to the (e_bits, m_bits) grid
+  __device__ __forceinline__ float grid_round(float t) const {
+    const uint32_t bits = f2u(t);
+    const uint32_t sign = bits & 0x80000000u;
+    const uint32_t mag = bits & 0x7fffffffu;
+    const int ex = (int)(mag >> 23) - 127;
+    uint32_t out;
+    if (ex == 128) {
+      out = mag;                                           // inf / nan pass through
+    } else if (ex < min_exp) {
+      float v;
+      if (subnormals) {
+        const float sh = u2f(mag) + min_normal;
+        v = u2f(round_mag(f2u(sh))) - min_normal;
+      } else {
+        v = (u2f(mag) > 0.5f * min_normal) ? min_normal : 0.0f;
+      }
+      out = f2u(v);
+    } else {
+      out = round_mag(mag);
+      if ((int)(out >> 23) - 127 > max_exp) out = max_mag;
+    }
+    return u2f(out | sign);
+  }
+
+  __device__ __forceinline__ float code(float x, const Row& p) const {
+    float t = x * p.r;
+    bool ok;
+    if constexpr (BF) {
+      const uint32_t low = f2u(t) & 0xffffu;               // bf16 rounding midpoint nearby?
+      ok = (low - 0x7ff8u) > 0x10u;
+    } else {
+      // grid midpoints sit at mantissa pattern 1000.. below the kept bits; the
+      // sub-minimum-normal range uses absolute steps, so it always divides.
+      const uint32_t lowm = f2u(t) & ((1u << drop) - 1u);
+      ok = ((lowm - (half - 8u)) > 16u) && (fabsf(t) >= 1.0001f * min_normal);
+    }
+    ok = ok && p.fast;
+    if (__builtin_expect(!ok, 0)) t = x / p.s;
+    t = rnd_e<BF>(t);
+    t = t + 0.0f;                                          // "+ zeros": turns -0 into +0
+    return grid_round(t);
+  }
+
+  // (q - 0.0) * s in fp32, then the cast of fake_quant_* (quant.py:1107,1153)
+  __device__ __forceinline__ float deq(float q, const Row& p) const {
+    const float d = (q - 0.0f) * p.s;
+    return dq_f32 ? d : rnd_e<BF>(d);
+  }
+
+  // float8 storage of an on-grid value
+  __device__ __forceinline__ uint32_t byte(float q) const {
+    const uint32_t bits = f2u(q);
+    const uint32_t sign = (bits >> 24) & 0x80u;
+    const uint32_t mag = bits & 0x7fffffffu;
+    if (e_bits == 4) {                                     // float8_e4m3fn: bias 7, no inf, 0x7f = nan
+      if (mag > 0x43e00000u) return sign | 0x7fu;          // > 448 (or nan/inf)
+      const int ex = (int)(mag >> 23) - 127;
+      if (ex < -6) return sign | (uint32_t)(u2f(mag) * 512.0f);   // multiples of 2^-9
+      return sign | ((uint32_t)(ex + 7) << 3) | ((mag >> 20) & 7u);
+    }
+    // float8_e5m2: the top byte of the fp16 encoding
+    if (mag > 0x7f800000u) return sign | 0x7fu;
+    if (mag > 0x47600000u) return sign | 0x7cu;            // > 57344 -> inf
+    const int ex = (int)(mag >> 23) - 127;
+    if (ex < -14) return sign | (uint32_t)(u2f(mag) * 65536.0f);  // multiples of 2^-16
+    return sign | ((uint32_t)(ex + 15) << 2) | ((mag >> 21) & 3u);
+  }
+};
+
+template <bool BF>
+FpOp<BF> make_op(int e_bits, int m_bits, float qmax, int flags, int code_dtype) {
+  FpOp<BF> c;
+  c.qmax = qmax; c.e_bits = e_bits; c.m_bits = m_bits;
+  c.tie_even = (flags & LCQ_FLAG_TIE_EVEN) != 0;
+  c.subnormals = (flags & LCQ_FLAG_NO_SUBNORMALS) == 0;
+  c.is_static = (flags & LCQ_FLAG_STATIC) != 0;
+  c.scalar_qp = (flags & LCQ_FLAG_SCALAR_QP) != 0;
+  c.dq_f32 = (flags & LCQ_FLAG_DQ_F32) != 0;
+  c.code_dtype = code_dtype;
+  c.drop = 23 - m_bits;
+  c.half = 1u << (c.drop - 1);
+  c.keep = ~((1u << c.drop) - 1u);
+  c.min_exp = -((1 << (e_bits - 1)) - 2);
+  c.max_exp = 1 << (e_bits - 1);
+  c.max_mag = ((uint32_t)(c.max_exp + 127) << 23) | (((1u << m_bits) - 1u) << c.drop);
+  c.min_normal = __builtin_ldexpf(1.0f, c.min_exp);
+  return c;
+}
+
+// FloatQuantizer.dequant on stored fp32 codes: out = (q - 0) * s in fp32
+template <bool BF>
+__global__ __launch_bounds__(256) void dequant_fp_kernel(const float* __restrict__ q, int64_t rows, int64_t cols,
+                                                         const void* __restrict__ scales, float* __restrict__ out,
+                                                         int scalar_qp) {
+  const int64_t n = rows * cols;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n; e += (int64_t)gridDim.x * 256) {
+    const float s = load_scalar<BF>(scales, scalar_qp ? 0 : e / cols);
+    out[e] = (q[e] - 0.0f) * s;
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int lcq_quant_fp(const void* x, int dtype, int64_t rows, int64_t cols, int e_bits, int m_bits, float qmax, int flags,
+                 void* dq, void* codes, int code_dtype, void* scales, void* stream) {
+  if (!x || rows < 0 || cols <= 0 || !scales) return LCQ_EINVAL;
+  if (rows == 0) return LCQ_OK;
+  if (e_bits < 2 || e_bits > 5 || m_bits < 1 || m_bits > 10 || !(qmax > 0.0f)) return LCQ_EINVAL;
+  if (codes) {
+    if (code_dtype == LCQ_CODE_FP8) {
+      if (!((e_bits == 4 && m_bits == 3) || (e_bits == 5 && m_bits == 2))) return LCQ_EDTYPE;
+    } else if (code_dtype != LCQ_CODE_F32) return LCQ_EDTYPE;
+  } else code_dtype = LCQ_CODE_NONE;
+  if ((flags & LCQ_FLAG_SCALAR_QP) && !(flags & LCQ_FLAG_STATIC)) return LCQ_EINVAL;
+  hipStream_t st = (hipStream_t)stream;
+  int rc;
+  if (dtype == LCQ_F32)
+    rc = dispatch_rows(x, rows, cols, dq, codes, scales, (void*)nullptr, make_op<false>(e_bits, m_bits, qmax, flags, code_dtype), false, st);
+  else if (dtype == LCQ_BF16)
+    rc = dispatch_rows(x, rows, cols, dq, codes, scales, (void*)nullptr, make_op<true>(e_bits, m_bits, qmax, flags, code_dtype), false, st);
+  else return LCQ_EDTYPE;
+  if (rc != LCQ_OK) return rc;
+  LCQ_CHECK_LAUNCH();
+  return LCQ_OK;
+}
+
+int lcq_dequant_fp(const float* q, int64_t rows, int64_t cols, const void* scales, int scale_dtype, int flags,
+                   float* out, void* stream) {
+  if (!q || !scales || !out || rows < 0 || cols <= 0) return LCQ_EINVAL;
+  if (rows == 0) return LCQ_OK;
+  const int scalar_qp = (flags & LCQ_FLAG_SCALAR_QP) != 0;
+  int64_t grid = (rows * cols + 255) / 256;
+  if (grid > 65536) grid = 65536;
+  hipStream_t st = (hipStream_t)stream;
+  if (scale_dtype == LCQ_F32) dequant_fp_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>(q, rows, cols, scales, out, scalar_qp);
+  else if (scale_dtype == LCQ_BF16) dequant_fp_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>(q, rows, cols, scales, out, scalar_qp);
+  else return LCQ_EDTYPE;
+  LCQ_CHECK_LAUNCH();
+  return LCQ_OK;
+}
+
+}  // extern "C"

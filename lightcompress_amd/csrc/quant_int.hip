@@ -1,0 +1,302 @@
+// Integer quantizer for gfx950: row-wise min/max -> scale/zero -> quantize ->
+// dequantize / integer codes in ONE pass over HBM (skeleton in rowquant.h).
+//
+// Replaces the ~9 eager torch kernels behind
+//   IntegerQuantizer.get_tensor_qparams / quant / dequant / quant_dequant /
+//   fake_quant_*_dynamic|static / real_quant_weight_dynamic|static
+// (llmc/compression/quantization/quant.py:134-145, 544-558, 689-716, 753-952).
+//
+// A "row" is one row of the reshaped tensor (quant.py:611-641): a group of
+// `group_size` weights (per_group), a whole weight row (per_channel), a token
+// (per_token) or a head (per_head).
+//
+// Arithmetic contract (bit-exact with the reference's torch op sequence):
+//   fp32 rows : every step is one IEEE fp32 op (true division, rintf).
+//   bf16 rows : every step is computed in fp32 and rounded to bf16 (RNE)
+//               before the next step, as torch does for bf16 tensors.
+// The per-element division x/s is evaluated as x*(1/s) with an exactness
+// guard: whenever the approximate quotient is close enough to a rounding
+// boundary that the IEEE quotient could round differently, the lane falls
+// back to the true division.  Both paths give the same bits by construction.
+#include "rowquant.h"
+
+namespace {
+using namespace lcq;
+
+struct IntRow {
+  float s, z, r, sdq;
+  int fast;
+};
+
+// FAST: round_zp and |qmin|,qmax <= 256 (every stock configuration).
+template <bool BF_, bool FAST>
+struct IntOp {
+  static constexpr bool BF = BF_;
+  using Row = IntRow;
+  float qmin, qmax, qrange, osf;
+  int sym, round_zp, is_static, scalar_qp, dq_f32, code_dtype;
+
+  __device__ __forceinline__ Row finish(float s, float z) const {
+    Row p;
+    p.s = s; p.z = z;
+    p.r = 1.0f / s;
+    const float a = fabsf(s);
+    p.fast = (a > 8.6736174e-19f) && (a < 1.1529215e18f);   // 2^-60 .. 2^60
+    p.sdq = rnd<BF>(s * osf);
+    return p;
+  }
+
+  // get_qparams, quant.py:544-558
+  __device__ __forceinline__ Row make(float mn, float mx) const {
+    const float cmin = BF ? 1.0013580322265625e-05f : 1e-5f;     // clamp(min=1e-5) in the tensor dtype
+    float s, z;
+    if (sym) {
+      float a = nan_max(fabsf(mx), fabsf(mn));
+      a = clamp_min_nan(a, cmin);
+      s = rnd<BF>(a / qmax);
+      z = 0.0f;
+    } else {
+      float d = rnd<BF>(mx - mn);
+      d = clamp_min_nan(d, cmin);
+      s = rnd<BF>(d / qrange);
+      const float t = rnd<BF>(mn / s);
+      if (round_zp) {
+        z = rnd<BF>(qmin - rintf(t));
+        z = fminf(fmaxf(z, qmin), qmax);
+      } else {
+        z = rnd<BF>(qmin - t);
+      }
+    }
+    return finish(s, z);
+  }
+
+  __device__ __forceinline__ Row load(const void* scales, const void* zeros, int64_t row) const {
+    const int64_t i = scalar_qp ? 0 : row;
+    const float s = load_scalar<BF>(scales, i);
+    const float z = zeros ? load_scalar<BF>(zeros, i) : 0.0f;
+    return finish(s, z);
+  }
+
+  __device__ __forceinline__ void store_qp(void* scales, void* zeros, int64_t row, const Row& p) const {
+    store_scalar<BF>(scales, row, p.s);
+    if (zeros && !sym) store_scalar<BF>(zeros, row, p.z);
+  }
+
+  // quant, quant.py:698-707: the integer code as a float
+  __device__ __forceinline__ float code(float x, const Row& p) const {
+    float q;
+    if constexpr (FAST) {
+      float t = x * p.r;
+      bool ok;
+      if constexpr (BF) {
+        const uint32_t low = f2u(t) & 0xffffu;              // distance to a bf16 rounding midpoint
+        ok = (low - 0x7ff8u) > 0x10u;
+      } else {
+        // |t - x/s| <= 2^-22 |t| <= 2^-12 for |t| <= 1024: safe unless within 2^-11 of a half integer
+        const float d = t - rintf(t);
+        ok = (fabsf(fabsf(d) - 0.5f) > 4.8828125e-04f) && (fabsf(t) <= 1024.0f);
+      }
+      ok = ok && p.fast;
+      if (__builtin_expect(!ok, 0)) t = x / p.s;             // IEEE quotient near a boundary
+      t = rnd_e<BF>(t);
+      q = rintf(t) + p.z;
+    } else if (round_zp) {
+      const float t = rnd<BF>(x / p.s);
+      q = rnd<BF>(rintf(t) + p.z);
+    } else {
+      const float lo = BF ? 1.00044417e-09f : 1e-9f;         // scales.clamp_min(1e-9)
+      const float t = rnd<BF>(x / clamp_min_nan(p.s, lo));
+      q = rintf(rnd<BF>(t + p.z));
+    }
+    return __builtin_amdgcn_fmed3f(q, qmin, qmax);
+  }
+
+  // dequant, quant.py:709-711 (scale already multiplied by output_scale_factor)
+  __device__ __forceinline__ float deq(float q, const Row& p) const {
+    float d = q - p.z;                                       // exact for small integer codes
+    if constexpr (BF && !FAST) d = bf16_round(d);
+    return rnd_e<BF>(d * p.sdq);
+  }
+
+  __device__ __forceinline__ uint32_t byte(float q) const { return (uint32_t)(int32_t)q & 0xffu; }
+};
+
+template <class Op>
+Op make_op(float qmin, float qmax, int flags, float osf, int code_dtype) {
+  Op c;
+  c.qmin = qmin; c.qmax = qmax; c.qrange = qmax - qmin; c.osf = osf;
+  c.sym = (flags & LCQ_FLAG_SYM) != 0;
+  c.round_zp = (flags & LCQ_FLAG_NO_ROUND_ZP) == 0;
+  c.is_static = (flags & LCQ_FLAG_STATIC) != 0;
+  c.scalar_qp = (flags & LCQ_FLAG_SCALAR_QP) != 0;
+  c.dq_f32 = 0;
+  c.code_dtype = code_dtype;
+  return c;
+}
+
+template <bool BF>
+int run(const void* x, int64_t rows, int64_t cols, float qmin, float qmax, int flags, float osf, void* dq,
+        void* codes, int code_dtype, void* scales, void* zeros, hipStream_t st) {
+  const bool big = (qmax > 256.0f) || (qmin < -256.0f);
+  const bool general = big || (flags & LCQ_FLAG_NO_ROUND_ZP);
+  if (general)
+    return dispatch_rows(x, rows, cols, dq, codes, scales, zeros,
+                         make_op<IntOp<BF, false>>(qmin, qmax, flags, osf, code_dtype), true, st);
+  return dispatch_rows(x, rows, cols, dq, codes, scales, zeros,
+                       make_op<IntOp<BF, true>>(qmin, qmax, flags, osf, code_dtype), false, st);
+}
+
+// get_minmax_range (row-wise), quant.py:141-143
+template <bool BF>
+__global__ __launch_bounds__(256) void minmax_rows_kernel(const void* __restrict__ x, int64_t rows, int64_t cols,
+                                                          void* __restrict__ mn_out, void* __restrict__ mx_out) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  float mn = __builtin_inff(), mx = -__builtin_inff();
+  for (int64_t j = lane; j < cols; j += 64) {
+    const float v = load_scalar<BF>(x, row * cols + j);
+    mn = nan_min(mn, v); mx = nan_max(mx, v);
+  }
+  mn = team_reduce<64, false>(mn);
+  mx = team_reduce<64, true>(mx);
+  if (lane == 0) { store_scalar<BF>(mn_out, row, mn); store_scalar<BF>(mx_out, row, mx); }
+}
+
+// per_tensor range, quant.py:135-137: stage 1 writes one (min,max) per workgroup
+template <bool BF>
+__global__ __launch_bounds__(256) void minmax_all_stage1(const void* __restrict__ x, int64_t n, float* __restrict__ part) {
+  __shared__ float sm[8];
+  float mn = __builtin_inff(), mx = -__builtin_inff();
+  for (int64_t j = (int64_t)blockIdx.x * 256 + threadIdx.x; j < n; j += (int64_t)gridDim.x * 256) {
+    const float v = load_scalar<BF>(x, j);
+    mn = nan_min(mn, v); mx = nan_max(mx, v);
+  }
+  mn = block_reduce<false>(mn, sm);
+  mx = block_reduce<true>(mx, sm);
+  if (threadIdx.x == 0) { part[2 * blockIdx.x] = mn; part[2 * blockIdx.x + 1] = mx; }
+}
+template <bool BF>
+__global__ __launch_bounds__(256) void minmax_all_stage2(const float* __restrict__ part, int nparts,
+                                                         void* __restrict__ mn_out, void* __restrict__ mx_out) {
+  __shared__ float sm[8];
+  float mn = __builtin_inff(), mx = -__builtin_inff();
+  for (int j = threadIdx.x; j < nparts; j += 256) { mn = nan_min(mn, part[2 * j]); mx = nan_max(mx, part[2 * j + 1]); }
+  mn = block_reduce<false>(mn, sm);
+  mx = block_reduce<true>(mx, sm);
+  if (threadIdx.x == 0) { store_scalar<BF>(mn_out, 0, mn); store_scalar<BF>(mx_out, 0, mx); }
+}
+
+// get_qparams on explicit ranges, quant.py:544-558
+template <bool BF>
+__global__ void qparams_kernel(const void* __restrict__ mn, const void* __restrict__ mx, int64_t n,
+                               void* __restrict__ scales, void* __restrict__ zeros, IntOp<BF, false> op) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const IntRow p = op.make(load_scalar<BF>(mn, i), load_scalar<BF>(mx, i));
+  op.store_qp(scales, zeros, i, p);
+}
+
+// dequant, quant.py:709-711, on stored float codes
+template <bool BF>
+__global__ __launch_bounds__(256) void dequant_kernel(const void* __restrict__ q, int64_t rows, int64_t cols,
+                                                      const void* __restrict__ scales, const void* __restrict__ zeros,
+                                                      void* __restrict__ out, int scalar_qp, float osf) {
+  const int64_t n = rows * cols;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n; e += (int64_t)gridDim.x * 256) {
+    const int64_t row = scalar_qp ? 0 : e / cols;
+    const float s = load_scalar<BF>(scales, row);
+    const float z = zeros ? load_scalar<BF>(zeros, row) : 0.0f;
+    const float d = rnd<BF>(load_scalar<BF>(q, e) - z);
+    store_scalar<BF>(out, e, rnd<BF>(d * rnd<BF>(s * osf)));
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int lcq_quant_int(const void* x, int dtype, int64_t rows, int64_t cols, float qmin, float qmax, int flags,
+                  float out_scale_factor, void* dq, void* codes, int code_dtype, void* scales, void* zeros,
+                  void* stream) {
+  if (!x || rows < 0 || cols <= 0 || !scales) return LCQ_EINVAL;
+  if (rows == 0) return LCQ_OK;
+  if (codes && !(code_dtype == LCQ_CODE_U8 || code_dtype == LCQ_CODE_I8 || code_dtype == LCQ_CODE_I32 ||
+                 code_dtype == LCQ_CODE_SAME)) return LCQ_EDTYPE;
+  if (!(qmax > qmin)) return LCQ_EINVAL;
+  if ((flags & LCQ_FLAG_SCALAR_QP) && !(flags & LCQ_FLAG_STATIC)) return LCQ_EINVAL;
+  if (!codes) code_dtype = LCQ_CODE_NONE;
+  hipStream_t st = (hipStream_t)stream;
+  int rc;
+  if (dtype == LCQ_F32) rc = run<false>(x, rows, cols, qmin, qmax, flags, out_scale_factor, dq, codes, code_dtype, scales, zeros, st);
+  else if (dtype == LCQ_BF16) rc = run<true>(x, rows, cols, qmin, qmax, flags, out_scale_factor, dq, codes, code_dtype, scales, zeros, st);
+  else return LCQ_EDTYPE;
+  if (rc != LCQ_OK) return rc;
+  LCQ_CHECK_LAUNCH();
+  return LCQ_OK;
+}
+
+int lcq_minmax_rows(const void* x, int dtype, int64_t rows, int64_t cols, void* min_out, void* max_out, void* stream) {
+  if (!x || !min_out || !max_out || rows < 0 || cols <= 0) return LCQ_EINVAL;
+  if (rows == 0) return LCQ_OK;
+  const int64_t grid = (rows + 3) / 4;
+  if (grid > 0x7fffffff) return LCQ_EINVAL;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == LCQ_F32) minmax_rows_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>(x, rows, cols, min_out, max_out);
+  else if (dtype == LCQ_BF16) minmax_rows_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>(x, rows, cols, min_out, max_out);
+  else return LCQ_EDTYPE;
+  LCQ_CHECK_LAUNCH();
+  return LCQ_OK;
+}
+
+int64_t lcq_minmax_all_workspace_bytes(void) { return 2 * 2048 * sizeof(float); }
+
+int lcq_minmax_all(const void* x, int dtype, int64_t n, void* min_out, void* max_out, void* workspace, void* stream) {
+  if (!x || !min_out || !max_out || !workspace || n <= 0) return LCQ_EINVAL;
+  int64_t blocks = (n + 256 * 16 - 1) / (256 * 16);
+  if (blocks > 2048) blocks = 2048;
+  hipStream_t st = (hipStream_t)stream;
+  float* part = (float*)workspace;
+  if (dtype == LCQ_F32) {
+    minmax_all_stage1<false><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(x, n, part);
+    minmax_all_stage2<false><<<dim3(1), dim3(256), 0, st>>>(part, (int)blocks, min_out, max_out);
+  } else if (dtype == LCQ_BF16) {
+    minmax_all_stage1<true><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(x, n, part);
+    minmax_all_stage2<true><<<dim3(1), dim3(256), 0, st>>>(part, (int)blocks, min_out, max_out);
+  } else return LCQ_EDTYPE;
+  LCQ_CHECK_LAUNCH();
+  return LCQ_OK;
+}
+
+int lcq_qparams_int(const void* min_in, const void* max_in, int dtype, int64_t n, float qmin, float qmax, int flags,
+                    void* scales, void* zeros, void* stream) {
+  if (!min_in || !max_in || !scales || n <= 0) return LCQ_EINVAL;
+  const int64_t grid = (n + 255) / 256;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == LCQ_F32)
+    qparams_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>(
+        min_in, max_in, n, scales, zeros, make_op<IntOp<false, false>>(qmin, qmax, flags, 1.0f, LCQ_CODE_NONE));
+  else if (dtype == LCQ_BF16)
+    qparams_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>(
+        min_in, max_in, n, scales, zeros, make_op<IntOp<true, false>>(qmin, qmax, flags, 1.0f, LCQ_CODE_NONE));
+  else return LCQ_EDTYPE;
+  LCQ_CHECK_LAUNCH();
+  return LCQ_OK;
+}
+
+int lcq_dequant_int(const void* q, int dtype, int64_t rows, int64_t cols, const void* scales, const void* zeros,
+                    int flags, float out_scale_factor, void* out, void* stream) {
+  if (!q || !scales || !out || rows < 0 || cols <= 0) return LCQ_EINVAL;
+  if (rows == 0) return LCQ_OK;
+  const int scalar_qp = (flags & LCQ_FLAG_SCALAR_QP) != 0;
+  int64_t grid = (rows * cols + 255) / 256;
+  if (grid > 65536) grid = 65536;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == LCQ_F32) dequant_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>(q, rows, cols, scales, zeros, out, scalar_qp, out_scale_factor);
+  else if (dtype == LCQ_BF16) dequant_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>(q, rows, cols, scales, zeros, out, scalar_qp, out_scale_factor);
+  else return LCQ_EDTYPE;
+  LCQ_CHECK_LAUNCH();
+  return LCQ_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,335 @@
+// Row-wise fused quantizer skeleton for gfx950, shared by the integer and the
+// minifloat quantizers.  One pass over HBM: load a row (16-byte chunks per
+// lane), reduce min/max across the lanes that share the row (DPP /
+// ds_swizzle butterflies), derive the row's parameters, emit codes and/or
+// dequantized values.
+//
+// An Op policy supplies the arithmetic:
+//   static constexpr bool BF            rows are bf16 (else fp32)
+//   struct Row                          per-row parameters
+//   Row  make(mn, mx)                   dynamic parameters from the row range
+//   Row  load(scales, zeros, row)       static parameters
+//   void store_qp(scales, zeros, row, Row)
+//   float code(x, Row)                  quantized value as a float
+//   float deq(q, Row)                   dequantized value (already rounded to the output type)
+//   uint32_t byte(q)                    1-byte storage of a code (U8 / I8 / FP8)
+//   bool is_static, dq_f32; int code_dtype
+#pragma once
+#include "common.h"
+#include "lcq_internal.h"
+
+namespace lcq {
+
+template <bool BF> struct Vec { static constexpr int N = BF ? 8 : 4; };
+
+template <bool BF> __device__ __forceinline__ float rnd(float v) {
+  if constexpr (BF) return bf16_round(v); else return v;
+}
+// per-element rounding: hardware RNE convert (v_cvt_pk_bf16_f32)
+template <bool BF> __device__ __forceinline__ float rnd_e(float v) {
+  if constexpr (BF) return (float)(__bf16)v; else return v;
+}
+__device__ __forceinline__ float clamp_min_nan(float v, float lo) { return (v != v) ? v : fmaxf(v, lo); }
+
+template <bool BF>
+__device__ __forceinline__ void unpack(const u32x4& raw, float* v) {
+  if constexpr (BF) {
+    #pragma unroll
+    for (int i = 0; i < 4; ++i) { v[2 * i] = bf16_lo(raw[i]); v[2 * i + 1] = bf16_hi(raw[i]); }
+  } else {
+    #pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = u2f(raw[i]);
+  }
+}
+template <bool BF>
+__device__ __forceinline__ u32x4 pack(const float* v) {
+  u32x4 raw;
+  if constexpr (BF) {
+    #pragma unroll
+    for (int i = 0; i < 4; ++i) raw[i] = bf16_pack(v[2 * i], v[2 * i + 1]);
+  } else {
+    #pragma unroll
+    for (int i = 0; i < 4; ++i) raw[i] = f2u(v[i]);
+  }
+  return raw;
+}
+
+template <bool BF>
+__device__ __forceinline__ float load_scalar(const void* p, int64_t i) {
+  if constexpr (BF) return u2f((uint32_t)((const uint16_t*)p)[i] << 16);
+  else return ((const float*)p)[i];
+}
+template <bool BF>
+__device__ __forceinline__ void store_scalar(void* p, int64_t i, float v) {
+  if constexpr (BF) ((uint16_t*)p)[i] = (uint16_t)(f2u(v) >> 16);
+  else ((float*)p)[i] = v;
+}
+
+// N codes of one 16-byte input chunk -> storage
+template <class Op>
+__device__ __forceinline__ void store_codes(const Op& op, void* codes, int64_t elem0, const float* q) {
+  constexpr bool BF = Op::BF;
+  constexpr int N = Vec<BF>::N;
+  const int cd = op.code_dtype;
+  if (cd == LCQ_CODE_I32) {
+    int32_t* p = (int32_t*)codes + elem0;
+    #pragma unroll
+    for (int i = 0; i < N; i += 4) {
+      u32x4 w;
+      #pragma unroll
+      for (int j = 0; j < 4; ++j) w[j] = (uint32_t)(int32_t)q[i + j];
+      *(u32x4*)(p + i) = w;
+    }
+  } else if (cd == LCQ_CODE_F32) {
+    float* p = (float*)codes + elem0;
+    #pragma unroll
+    for (int i = 0; i < N; i += 4) {
+      u32x4 w;
+      #pragma unroll
+      for (int j = 0; j < 4; ++j) w[j] = f2u(q[i + j]);
+      *(u32x4*)(p + i) = w;
+    }
+  } else if (cd == LCQ_CODE_U8 || cd == LCQ_CODE_I8 || cd == LCQ_CODE_FP8) {
+    uint8_t* p = (uint8_t*)codes + elem0;
+    #pragma unroll
+    for (int i = 0; i < N; i += 4) {
+      uint32_t w = 0;
+      #pragma unroll
+      for (int j = 0; j < 4; ++j) w |= op.byte(q[i + j]) << (8 * j);
+      *(uint32_t*)(p + i) = w;
+    }
+  } else if (cd == LCQ_CODE_SAME) {
+    *((u32x4*)codes + elem0 / N) = pack<BF>(q);
+  }
+}
+template <class Op>
+__device__ __forceinline__ void store_code1(const Op& op, void* codes, int64_t e, float q) {
+  const int cd = op.code_dtype;
+  if (cd == LCQ_CODE_I32) ((int32_t*)codes)[e] = (int32_t)q;
+  else if (cd == LCQ_CODE_F32) ((float*)codes)[e] = q;
+  else if (cd == LCQ_CODE_U8 || cd == LCQ_CODE_I8 || cd == LCQ_CODE_FP8) ((uint8_t*)codes)[e] = (uint8_t)op.byte(q);
+  else if (cd == LCQ_CODE_SAME) store_scalar<Op::BF>(codes, e, q);
+}
+
+// codes + dq of one chunk
+template <class Op>
+__device__ __forceinline__ void emit_chunk(const Op& op, const typename Op::Row& p, const u32x4& r, int64_t cidx,
+                                           void* dq, void* codes) {
+  constexpr bool BF = Op::BF;
+  constexpr int N = Vec<BF>::N;
+  float v[N], q[N];
+  unpack<BF>(r, v);
+  #pragma unroll
+  for (int i = 0; i < N; ++i) q[i] = op.code(v[i], p);
+  if (codes) store_codes(op, codes, cidx * N, q);
+  if (dq) {
+    #pragma unroll
+    for (int i = 0; i < N; ++i) v[i] = op.deq(q[i], p);
+    if (op.dq_f32) {
+      #pragma unroll
+      for (int i = 0; i < N; i += 4) {
+        u32x4 w;
+        #pragma unroll
+        for (int j = 0; j < 4; ++j) w[j] = f2u(v[i + j]);
+        __builtin_nontemporal_store(w, (u32x4*)dq + (cidx * N + i) / 4);
+      }
+    } else {
+      __builtin_nontemporal_store(pack<BF>(v), (u32x4*)dq + cidx);
+    }
+  }
+}
+
+template <class Op>
+__device__ __forceinline__ void chunk_minmax(const u32x4& r, float& mn, float& mx) {
+  constexpr int N = Vec<Op::BF>::N;
+  float v[N];
+  unpack<Op::BF>(r, v);
+  #pragma unroll
+  for (int i = 0; i < N; ++i) { mn = nan_min(mn, v[i]); mx = nan_max(mx, v[i]); }
+}
+
+// ---------------------------------------------------------------------------
+// short rows: TEAM lanes per row, ITERS chunks per lane, UNR row batches per wave
+// ---------------------------------------------------------------------------
+template <class Op, int TEAM, int ITERS, int UNR>
+__global__ __launch_bounds__(256) void row_team_kernel(
+    const u32x4* __restrict__ x, void* __restrict__ dq, void* __restrict__ codes,
+    void* __restrict__ scales, void* __restrict__ zeros, int64_t rows, int nchunks, Op op) {
+  constexpr int RPW = LCQ_WAVE / TEAM;                      // rows per wave per batch
+  const int lane = threadIdx.x & 63;
+  const int t = lane & (TEAM - 1);
+  const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int64_t row0 = wave * (RPW * UNR) + (lane / TEAM);
+
+  u32x4 raw[UNR][ITERS];
+  #pragma unroll
+  for (int u = 0; u < UNR; ++u) {
+    const int64_t row = row0 + (int64_t)u * RPW;
+    #pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int ch = t + it * TEAM;
+      if (row < rows && ch < nchunks) raw[u][it] = __builtin_nontemporal_load(x + row * nchunks + ch);
+      else raw[u][it] = u32x4{0, 0, 0, 0};
+    }
+  }
+
+  #pragma unroll
+  for (int u = 0; u < UNR; ++u) {
+    const int64_t row = row0 + (int64_t)u * RPW;
+    const bool row_ok = row < rows;
+    typename Op::Row p;
+    if (!op.is_static) {
+      float mn = __builtin_inff(), mx = -__builtin_inff();
+      #pragma unroll
+      for (int it = 0; it < ITERS; ++it)
+        if (t + it * TEAM < nchunks) chunk_minmax<Op>(raw[u][it], mn, mx);
+      mn = team_reduce<TEAM, false>(mn);
+      mx = team_reduce<TEAM, true>(mx);
+      p = op.make(mn, mx);
+      if (row_ok && t == 0) op.store_qp(scales, zeros, row, p);
+    } else {
+      p = op.load(scales, zeros, row_ok ? row : 0);
+    }
+    #pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int ch = t + it * TEAM;
+      if (row_ok && ch < nchunks) emit_chunk(op, p, raw[u][it], row * nchunks + ch, dq, codes);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// long rows: one 256-thread workgroup per row, first CACHE chunks per thread
+// stay in registers, the rest is re-read (L2 resident: a row is a few 10 KB)
+// ---------------------------------------------------------------------------
+template <bool IS_MAX>
+__device__ __forceinline__ float block_reduce(float v, float* sm) {
+  v = team_reduce<64, IS_MAX>(v);
+  const int w = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) sm[w] = v;
+  __syncthreads();
+  float r = sm[0];
+  for (int i = 1; i < nw; ++i) r = IS_MAX ? nan_max(r, sm[i]) : nan_min(r, sm[i]);
+  return r;
+}
+
+template <class Op, int CACHE>
+__global__ __launch_bounds__(256) void row_block_kernel(
+    const u32x4* __restrict__ x, void* __restrict__ dq, void* __restrict__ codes,
+    void* __restrict__ scales, void* __restrict__ zeros, int64_t rows, int nchunks, Op op) {
+  __shared__ float sm[8];
+  const int64_t row = blockIdx.x;
+  const u32x4* xr = x + row * nchunks;
+  u32x4 raw[CACHE];
+  #pragma unroll
+  for (int k = 0; k < CACHE; ++k) {
+    const int ch = threadIdx.x + k * 256;
+    raw[k] = (ch < nchunks) ? __builtin_nontemporal_load(xr + ch) : u32x4{0, 0, 0, 0};
+  }
+  typename Op::Row p;
+  if (!op.is_static) {
+    float mn = __builtin_inff(), mx = -__builtin_inff();
+    #pragma unroll
+    for (int k = 0; k < CACHE; ++k)
+      if ((int)threadIdx.x + k * 256 < nchunks) chunk_minmax<Op>(raw[k], mn, mx);
+    for (int ch = threadIdx.x + CACHE * 256; ch < nchunks; ch += 256) chunk_minmax<Op>(xr[ch], mn, mx);
+    mn = block_reduce<false>(mn, sm);
+    mx = block_reduce<true>(mx, sm);
+    p = op.make(mn, mx);
+    if (threadIdx.x == 0) op.store_qp(scales, zeros, row, p);
+  } else {
+    p = op.load(scales, zeros, row);
+  }
+  #pragma unroll
+  for (int k = 0; k < CACHE; ++k) {
+    const int ch = threadIdx.x + k * 256;
+    if (ch < nchunks) emit_chunk(op, p, raw[k], row * nchunks + ch, dq, codes);
+  }
+  for (int ch = threadIdx.x + CACHE * 256; ch < nchunks; ch += 256) emit_chunk(op, p, xr[ch], row * nchunks + ch, dq, codes);
+}
+
+// ---------------------------------------------------------------------------
+// any row length / alignment: one wave per row, one element per lane-step
+// ---------------------------------------------------------------------------
+template <class Op>
+__global__ __launch_bounds__(256) void row_scalar_kernel(
+    const void* __restrict__ x, void* __restrict__ dq, void* __restrict__ codes,
+    void* __restrict__ scales, void* __restrict__ zeros, int64_t rows, int64_t cols, Op op) {
+  constexpr bool BF = Op::BF;
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= rows) return;                                   // whole wave leaves together
+  typename Op::Row p;
+  if (!op.is_static) {
+    float mn = __builtin_inff(), mx = -__builtin_inff();
+    for (int64_t j = lane; j < cols; j += 64) {
+      const float v = load_scalar<BF>(x, row * cols + j);
+      mn = nan_min(mn, v); mx = nan_max(mx, v);
+    }
+    mn = team_reduce<64, false>(mn);
+    mx = team_reduce<64, true>(mx);
+    p = op.make(mn, mx);
+    if (lane == 0) op.store_qp(scales, zeros, row, p);
+  } else {
+    p = op.load(scales, zeros, row);
+  }
+  for (int64_t j = lane; j < cols; j += 64) {
+    const int64_t e = row * cols + j;
+    const float q = op.code(load_scalar<BF>(x, e), p);
+    if (codes) store_code1(op, codes, e, q);
+    if (dq) {
+      const float d = op.deq(q, p);
+      if (op.dq_f32) ((float*)dq)[e] = d; else store_scalar<BF>(dq, e, d);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host-side dispatch.  Each lane takes up to four 16-byte chunks of its row
+// so the per-row parameter arithmetic (IEEE divisions) is amortised over
+// 16..32 elements.
+// ---------------------------------------------------------------------------
+template <class Op, int TEAM, int ITERS, int UNR>
+void launch_team(const void* x, void* dq, void* codes, void* scales, void* zeros, int64_t rows, int nchunks,
+                 const Op& op, hipStream_t st) {
+  constexpr int RPW = LCQ_WAVE / TEAM;
+  const int64_t rows_per_block = (int64_t)RPW * UNR * 4;
+  const int64_t grid = (rows + rows_per_block - 1) / rows_per_block;
+  row_team_kernel<Op, TEAM, ITERS, UNR><<<dim3((unsigned)grid), dim3(256), 0, st>>>(
+      (const u32x4*)x, dq, codes, scales, zeros, rows, nchunks, op);
+}
+
+template <class Op>
+int dispatch_rows(const void* x, int64_t rows, int64_t cols, void* dq, void* codes, void* scales, void* zeros,
+                  const Op& op, bool force_scalar, hipStream_t st) {
+  constexpr int N = Vec<Op::BF>::N;
+  if (rows > 0x7fffffff) return LCQ_EINVAL;
+  const bool aligned = (cols % N == 0) && (((uintptr_t)x | (uintptr_t)dq | (uintptr_t)codes) % 16 == 0);
+  if (!aligned || force_scalar) {
+    const int64_t grid = (rows + 3) / 4;
+    row_scalar_kernel<Op><<<dim3((unsigned)grid), dim3(256), 0, st>>>(x, dq, codes, scales, zeros, rows, cols, op);
+    return LCQ_OK;
+  }
+  const int64_t nch64 = cols / N;
+  if (nch64 > 0x7fffffff) return LCQ_EINVAL;
+  const int nchunks = (int)nch64;
+  #define LCQ_TEAM(T, I, U) launch_team<Op, T, I, U>(x, dq, codes, scales, zeros, rows, nchunks, op, st)
+  if (nchunks <= 1) LCQ_TEAM(1, 1, 4);
+  else if (nchunks <= 2) LCQ_TEAM(1, 2, 2);
+  else if (nchunks <= 4) LCQ_TEAM(1, 4, 1);
+  else if (nchunks <= 8) LCQ_TEAM(2, 4, 1);
+  else if (nchunks <= 16) LCQ_TEAM(4, 4, 1);
+  else if (nchunks <= 32) LCQ_TEAM(8, 4, 1);
+  else if (nchunks <= 64) LCQ_TEAM(16, 4, 1);
+  else if (nchunks <= 128) LCQ_TEAM(32, 4, 1);
+  else if (nchunks <= 256) LCQ_TEAM(64, 4, 1);
+  else {
+    row_block_kernel<Op, 8><<<dim3((unsigned)rows), dim3(256), 0, st>>>(
+        (const u32x4*)x, dq, codes, scales, zeros, rows, nchunks, op);
+  }
+  #undef LCQ_TEAM
+  return LCQ_OK;
+}
+
+}  // namespace lcq

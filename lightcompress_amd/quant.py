@@ -1,0 +1,581 @@
+"""Quantizer primitives with the reference's class API, running on liblcq.
+
+Mirrors ``llmc/compression/quantization/quant.py`` of ModelTC/LightCompress:
+``IntegerQuantizer`` (quant.py:660-959) and ``FloatQuantizer`` (quant.py:962-1228)
+with the same constructor kwargs, method names, argument order and return
+tuples, so algorithm code written against the reference runs unchanged.
+
+Every arithmetic method launches hand-written gfx950 kernels through the C
+ABI in ``include/lcq.h``.  There is no CPU path: CPU tensors raise
+``LcqError``.  Reshapes/views, index mixing and dtype casts stay in torch.
+
+Not carried over (they raise ``NotImplementedError``): the ``mse`` /
+``learnable`` / ``hqq`` / ``static_hist`` calibrators, STE rounding (training
+only), the ``rounding`` override of ``fake_quant_weight_static``, ``per_block``
+granularity and ``FloatQuantizer(use_qtorch=False)``.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib as L
+
+
+def ceil_div(x, y):
+    return (x + y - 1) // y
+
+
+class BaseQuantizer(object):
+    """Constructor surface of quant.py:48-103."""
+
+    def __init__(self, bit, symmetric, granularity, **kwargs):
+        self.bit = bit
+        self.sym = symmetric
+        self.granularity = granularity
+        self.kwargs = kwargs
+
+        self.calib_algo = self.kwargs.get('calib_algo', 'minmax')
+        if self.granularity == 'per_group':
+            self.group_size = self.kwargs['group_size']
+        elif self.granularity == 'per_head':
+            self.head_num = self.kwargs['head_num']
+        elif self.granularity == 'per_block':
+            raise NotImplementedError('per_block (FP8 block-wise checkpoints) is not part of this path')
+
+        if self.kwargs.get('ste', False) or self.kwargs.get('ste_all', False):
+            raise NotImplementedError('straight-through rounding is a training feature; not on this path')
+        self.round_func = torch.round
+        self.ste_all = False
+        self.round_zp = self.kwargs.get('round_zp', True)
+
+    # -- calibration -------------------------------------------------------
+    def get_tensor_range(self, tensor, args={}):
+        if self.calib_algo != 'minmax':
+            raise NotImplementedError(f'calib_algo={self.calib_algo!r}: only minmax runs on liblcq')
+        return self.get_minmax_range(tensor)
+
+    def get_minmax_range(self, tensor):
+        """quant.py:134-145 -> (min_val, max_val)."""
+        dt = L.dtype_code(tensor.dtype)
+        t = tensor.contiguous()
+        if self.granularity == 'per_tensor':
+            mn = torch.empty((), dtype=t.dtype, device=t.device)
+            mx = torch.empty((), dtype=t.dtype, device=t.device)
+            ws = torch.empty(L.lib().lcq_minmax_all_workspace_bytes(), dtype=torch.uint8, device=t.device)
+            L.check(L.lib().lcq_minmax_all(L.ptr(t), dt, L.i64(t.numel()), L.ptr(mn), L.ptr(mx), L.ptr(ws),
+                                           L.stream()), 'lcq_minmax_all')
+            return (mn, mx)
+        cols = t.shape[-1]
+        rows = t.numel() // cols
+        shape = (*t.shape[:-1], 1)
+        mn = torch.empty(shape, dtype=t.dtype, device=t.device)
+        mx = torch.empty(shape, dtype=t.dtype, device=t.device)
+        L.check(L.lib().lcq_minmax_rows(L.ptr(t), dt, L.i64(rows), L.i64(cols), L.ptr(mn), L.ptr(mx), L.stream()),
+                'lcq_minmax_rows')
+        return (mn, mx)
+
+    def _int_flags(self):
+        return (L.FLAG_SYM if self.sym else 0) | (0 if self.round_zp else L.FLAG_NO_ROUND_ZP)
+
+    def get_qparams(self, tensor_range, device):
+        """quant.py:544-558 -> (scales, zeros, qmax, qmin)."""
+        min_val, max_val = tensor_range[0].contiguous(), tensor_range[1].contiguous()
+        qmin = self.qmin.to(device)
+        qmax = self.qmax.to(device)
+        scales = torch.empty_like(max_val)
+        zeros = torch.tensor(0.0) if self.sym else torch.empty_like(max_val)
+        L.check(L.lib().lcq_qparams_int(L.ptr(min_val), L.ptr(max_val), L.dtype_code(max_val.dtype),
+                                        L.i64(max_val.numel()), L.f32(self.qmin), L.f32(self.qmax),
+                                        L.i32(self._int_flags()), L.ptr(scales),
+                                        L.ptr(None if self.sym else zeros), L.stream()), 'lcq_qparams_int')
+        return scales, zeros, qmax, qmin
+
+    # -- views (quant.py:611-657); torch view ops only ----------------------
+    def reshape_tensor(self, tensor, allow_padding=False):
+        if self.granularity == 'per_group':
+            if tensor.shape[-1] >= self.group_size:
+                if tensor.shape[-1] % self.group_size == 0:
+                    t = tensor.reshape(-1, self.group_size)
+                elif allow_padding:
+                    deficiency = self.group_size - tensor.shape[1] % self.group_size
+                    pad = torch.zeros((*tensor.shape[:-1], deficiency), device=tensor.device, dtype=tensor.dtype)
+                    t = torch.cat((tensor, pad), dim=-1).reshape(-1, self.group_size)
+                else:
+                    raise ValueError(
+                        f'Dimension {tensor.shape[-1]} '
+                        f'not divisible by group size {self.group_size}'
+                    )
+            else:
+                t = tensor
+        elif self.granularity == 'per_head':
+            t = tensor.reshape(self.head_num, -1)
+        else:
+            t = tensor
+        return t
+
+    def restore_tensor(self, tensor, shape):
+        if tensor.shape == shape:
+            return tensor
+        try:
+            return tensor.reshape(shape)
+        except RuntimeError:
+            deficiency = self.group_size - shape[1] % self.group_size
+            return tensor.reshape(*shape[:-1], -1)[..., :-deficiency]
+
+
+def _rows_cols(t):
+    """A reshaped tensor as (rows, cols) for the row kernels."""
+    if t.dim() == 0:
+        return 1, 1
+    cols = t.shape[-1]
+    return (t.numel() // cols if cols else 0), cols
+
+
+def _static_layout(t, scales):
+    """How static qparams map onto rows of `t`: one per row, or one scalar."""
+    rows, cols = _rows_cols(t)
+    n = scales.numel()
+    if n == 1:
+        return rows, cols, True
+    if n == rows:
+        return rows, cols, False
+    raise L.LcqError(f'qparams of shape {tuple(scales.shape)} do not match rows of tensor {tuple(t.shape)}')
+
+
+def _is_cpu_zero(z):
+    return z.device.type == 'cpu' and z.numel() == 1 and float(z) == 0.0
+
+
+class IntegerQuantizer(BaseQuantizer):
+    """quant.py:660-959."""
+
+    def __init__(self, bit, symmetric, granularity, **kwargs):
+        super().__init__(bit, symmetric, granularity, **kwargs)
+        self.quant_type = 'int-quant'
+        if 'int_range' in self.kwargs:
+            self.qmin = self.kwargs['int_range'][0]
+            self.qmax = self.kwargs['int_range'][1]
+        else:
+            if self.sym:
+                self.qmin = -(2 ** (self.bit - 1))
+                self.qmax = 2 ** (self.bit - 1) - 1
+            else:
+                self.qmin = 0.0
+                self.qmax = 2 ** self.bit - 1
+        self.qmin = torch.tensor(self.qmin)
+        self.qmax = torch.tensor(self.qmax)
+        self.dst_nbins = 2 ** bit
+        self._bounds_dev = {}
+
+    def _dev_bounds(self, device):
+        """qmax / qmin as 0-dim tensors on `device` (what the reference hands out), cached."""
+        key = str(device)
+        if key not in self._bounds_dev:
+            self._bounds_dev[key] = (self.qmax.to(device), self.qmin.to(device))
+        return self._bounds_dev[key]
+
+    def _bound(self, v):
+        """Python float of a qmin/qmax argument without a device sync for our own tensors."""
+        if not torch.is_tensor(v):
+            return float(v)
+        for qmax_d, qmin_d in self._bounds_dev.values():
+            if v is qmax_d:
+                return float(self.qmax)
+            if v is qmin_d:
+                return float(self.qmin)
+        return float(v)
+
+    # -- one fused launch -----------------------------------------------------
+    def _launch(self, rows_t, *, static, scales=None, zeros=None, want_dq=False, want_codes=None,
+                osf=1.0, qmin=None, qmax=None):
+        """Run lcq_quant_int over a reshaped tensor.
+
+        Returns (dq | None, codes | None, scales, zeros).  Dynamic mode creates
+        scales / zeros of shape [rows, 1] (0-dim for per_tensor).
+        """
+        t = rows_t.contiguous()
+        flags = self._int_flags()
+        qmin = self._bound(self.qmin if qmin is None else qmin)
+        qmax = self._bound(self.qmax if qmax is None else qmax)
+        if static:
+            # dimensioned qparams of another float type promote the computation like torch would
+            if scales.dim() > 0 and scales.dtype != t.dtype:
+                common = torch.promote_types(t.dtype, scales.dtype)
+                t = t.to(common)
+            scales = scales.to(t.dtype).contiguous()
+            rows, cols, scalar = _static_layout(t, scales)
+            flags |= L.FLAG_STATIC | (L.FLAG_SCALAR_QP if scalar else 0)
+            z = None
+            if zeros is not None and not _is_cpu_zero(zeros):
+                z = zeros.to(device=t.device, dtype=t.dtype).contiguous()
+                if z.numel() != scales.numel():
+                    z = z.expand_as(scales).contiguous()
+        else:
+            if self.granularity == 'per_tensor':
+                lo, hi = self.get_minmax_range(t)
+                scales, zeros, _, _ = self.get_qparams((lo, hi), t.device)
+                return self._launch(t, static=True, scales=scales, zeros=zeros, want_dq=want_dq,
+                                    want_codes=want_codes, osf=osf)
+            rows, cols = _rows_cols(t)
+            scales = torch.empty((rows, 1), dtype=t.dtype, device=t.device)
+            z = None if self.sym else torch.empty((rows, 1), dtype=t.dtype, device=t.device)
+        dq = torch.empty_like(t) if want_dq else None
+        codes, cd = None, L.CODE_NONE
+        if want_codes is not None:
+            if want_codes == 'same':
+                codes, cd = torch.empty_like(t), L.CODE_SAME
+            else:
+                codes = torch.empty(t.shape, dtype=want_codes, device=t.device)
+                cd = {torch.int32: L.CODE_I32, torch.int8: L.CODE_I8, torch.uint8: L.CODE_U8}[want_codes]
+        L.check(L.lib().lcq_quant_int(L.ptr(t), L.dtype_code(t.dtype), L.i64(rows), L.i64(cols), L.f32(qmin),
+                                      L.f32(qmax), L.i32(flags), L.f32(osf), L.ptr(dq), L.ptr(codes), L.i32(cd),
+                                      L.ptr(scales), L.ptr(z), L.stream()), 'lcq_quant_int')
+        if not static:
+            zeros = torch.tensor(0.0) if self.sym else z
+        return dq, codes, scales, zeros
+
+    # -- reference API ----------------------------------------------------------
+    def get_tensor_qparams(self, tensor, args={}):
+        """quant.py:689-696 -> (tensor_reshaped, scales, zeros, qmax, qmin)."""
+        if self.calib_algo != 'minmax':
+            raise NotImplementedError(f'calib_algo={self.calib_algo!r}: only minmax runs on liblcq')
+        tensor = self.reshape_tensor(tensor)
+        if self.granularity == 'per_tensor':
+            scales, zeros, qmax, qmin = self.get_qparams(self.get_minmax_range(tensor), tensor.device)
+            return tensor, scales, zeros, qmax, qmin
+        _, _, scales, zeros = self._launch(tensor, static=False)
+        if tensor.dim() != 2:
+            scales = scales.view(*tensor.shape[:-1], 1)
+            if not self.sym:
+                zeros = zeros.view(*tensor.shape[:-1], 1)
+        qmax, qmin = self._dev_bounds(tensor.device)
+        return tensor, scales, zeros, qmax, qmin
+
+    def quant(self, tensor, scales, zeros, qmax, qmin):
+        """quant.py:698-707: integer codes stored as floats."""
+        _, codes, _, _ = self._launch(tensor, static=True, scales=scales, zeros=zeros, want_codes='same',
+                                      qmin=qmin, qmax=qmax)
+        return codes.view(tensor.shape)
+
+    def dequant(self, tensor, scales, zeros):
+        """quant.py:709-711."""
+        t = tensor.contiguous()
+        if scales.dim() > 0 and scales.dtype != t.dtype:
+            t = t.to(torch.promote_types(t.dtype, scales.dtype))
+        s = scales.to(t.dtype).contiguous()
+        rows, cols, scalar = _static_layout(t, s)
+        z = None
+        if zeros is not None and not _is_cpu_zero(zeros):
+            z = zeros.to(device=t.device, dtype=t.dtype).contiguous()
+        out = torch.empty_like(t)
+        L.check(L.lib().lcq_dequant_int(L.ptr(t), L.dtype_code(t.dtype), L.i64(rows), L.i64(cols), L.ptr(s), L.ptr(z),
+                                        L.i32(L.FLAG_SCALAR_QP if scalar else 0), L.f32(1.0), L.ptr(out),
+                                        L.stream()), 'lcq_dequant_int')
+        return out
+
+    def quant_dequant(self, tensor, scales, zeros, qmax, qmin, output_scale_factor=1):
+        """quant.py:713-716."""
+        dq, _, _, _ = self._launch(tensor, static=True, scales=scales, zeros=zeros, want_dq=True,
+                                   osf=output_scale_factor, qmin=qmin, qmax=qmax)
+        return dq.view(tensor.shape)
+
+    def _fake_dynamic(self, t):
+        shape, dtype = t.shape, t.dtype
+        rows_t = self.reshape_tensor(t)
+        dq, _, _, _ = self._launch(rows_t, static=False, want_dq=True)
+        return self.restore_tensor(dq.view(rows_t.shape), shape).to(dtype)
+
+    def _fake_static(self, t, args):
+        shape, dtype = t.shape, t.dtype
+        rows_t = self.reshape_tensor(t)
+        dq, _, _, _ = self._launch(rows_t, static=True, scales=args['scales'], zeros=args['zeros'], want_dq=True,
+                                   osf=args.get('output_scale_factor', 1), qmin=args['qmin'], qmax=args['qmax'])
+        return self.restore_tensor(dq.view(rows_t.shape), shape).to(dtype)
+
+    def fake_quant_act_static(self, act, args={}):
+        """quant.py:718-751."""
+        if 'int_indices' in args:
+            q_act = act[:, :, args['int_indices']]
+            fp_act = act[:, :, args['fp_indices']]
+        else:
+            q_act = act
+        q_act = self._fake_static(q_act, args)
+        if 'int_indices' in args:
+            mix_act = torch.zeros_like(act)
+            mix_act[:, :, args['int_indices']] = q_act
+            mix_act[:, :, args['fp_indices']] = fp_act
+            return mix_act
+        return q_act
+
+    def fake_quant_act_dynamic(self, act, args={}):
+        """quant.py:753-782."""
+        if 'int_indices' in args:
+            q_act = act[:, :, args['int_indices']]
+            fp_act = act[:, :, args['fp_indices']]
+        else:
+            q_act = act
+        q_act = self._fake_dynamic(q_act)
+        if 'int_indices' in args:
+            mix_act = torch.zeros_like(act)
+            mix_act[:, :, args['int_indices']] = q_act
+            mix_act[:, :, args['fp_indices']] = fp_act
+            return mix_act
+        return q_act
+
+    def _weight_view(self, weight, args):
+        if 'int_indices' in args:
+            if self.granularity == 'per_group':
+                assert len(args['int_indices']) % self.group_size == 0
+            return weight[:, args['int_indices']], weight[:, args['fp_indices']]
+        if 'dim' in args and 'ic' in args['dim']:
+            return weight.T, None
+        return weight, None
+
+    def _weight_merge(self, weight, q_weight, fp_weight, args):
+        if 'int_indices' in args:
+            mix_weight = torch.zeros_like(weight)
+            mix_weight[:, args['int_indices']] = q_weight
+            mix_weight[:, args['fp_indices']] = fp_weight
+            return mix_weight
+        if 'dim' in args and 'ic' in args['dim']:
+            return q_weight.T
+        return q_weight
+
+    def fake_quant_weight_static(self, weight, args):
+        """quant.py:784-830."""
+        if 'rounding' in args:
+            raise NotImplementedError("the 'rounding' override is not on this path")
+        q_weight, fp_weight = self._weight_view(weight, args)
+        q_weight = self._fake_static(q_weight, args)
+        return self._weight_merge(weight, q_weight, fp_weight, args)
+
+    def fake_quant_weight_dynamic(self, weight, args={}):
+        """quant.py:832-868."""
+        q_weight, fp_weight = self._weight_view(weight, args)
+        q_weight = self._fake_dynamic(q_weight)
+        return self._weight_merge(weight, q_weight, fp_weight, args)
+
+    def _code_dtype(self):
+        if self.bit == 8:
+            return torch.int8 if self.qmin != 0 else torch.uint8
+        return torch.int32
+
+    def _finish_real(self, codes, scales, zeros, output_scale_factor):
+        scales = scales * output_scale_factor
+        dtype = self._code_dtype()
+        if not self.sym and self.round_zp:
+            zeros = zeros.to(dtype)
+        elif self.sym:
+            zeros = None
+        qparams_shape = 1 if self.granularity == 'per_tensor' else (codes.shape[0], -1)
+        if zeros is not None:
+            zeros = zeros.view(qparams_shape)
+        scales = scales.view(qparams_shape)
+        return codes, scales, zeros
+
+    def real_quant_weight_static(self, weight, args):
+        """quant.py:870-913 -> (codes, scales, zeros|None)."""
+        org_w_shape = weight.shape
+        output_scale_factor = args.pop('output_scale_factor', 1)
+        rows_t = self.reshape_tensor(weight)
+        _, codes, _, _ = self._launch(rows_t, static=True, scales=args['scales'], zeros=args['zeros'],
+                                      want_codes=self._code_dtype(), qmin=args['qmin'], qmax=args['qmax'])
+        codes = self.restore_tensor(codes.view(rows_t.shape), org_w_shape)
+        return self._finish_real(codes, args['scales'], args['zeros'], output_scale_factor)
+
+    def real_quant_weight_dynamic(self, weight, args={}):
+        """quant.py:915-952 -> (codes, scales, zeros|None)."""
+        org_w_shape = weight.shape
+        output_scale_factor = args.pop('output_scale_factor', 1) if 'output_scale_factor' in args else 1
+        rows_t = self.reshape_tensor(weight)
+        _, codes, scales, zeros = self._launch(rows_t, static=False, want_codes=self._code_dtype())
+        codes = self.restore_tensor(codes.view(rows_t.shape), org_w_shape)
+        return self._finish_real(codes, scales, zeros, output_scale_factor)
+
+    def __repr__(self):
+        return (
+            f'IntegerQuantizer(bit={self.bit}, sym={self.sym},'
+            f'granularity={self.granularity},'
+            f'kwargs={self.kwargs}, qmin={self.qmin}, qmax={self.qmax})'
+        )
+
+
+class FloatQuantizer(BaseQuantizer):
+    """quant.py:962-1228, qtorch branch.
+
+    The minifloat rounding the reference delegates to QPyTorch's
+    ``float_quantize(x, e, m, rounding='nearest')`` runs inside the kernel.  Two
+    extra kwargs select its unpinned details: ``fp_tie`` ('away' default |
+    'even') and ``fp_subnormals`` (True default).
+    """
+
+    _RANGES = {('e4m3', 8): torch.float8_e4m3fn, ('e5m2', 8): torch.float8_e5m2,
+               ('e3m2', 6): (-28, 28), ('e4m7', 12): (-510, 510), ('e2m1', 4): (-6, 6)}
+
+    def __init__(self, bit, symmetric, granularity, **kwargs):
+        super().__init__(bit, symmetric, granularity, **kwargs)
+        self.sym = True
+        self.quant_type = 'float-quant'
+        self.e_bits = int(self.bit[1])
+        self.m_bits = int(self.bit[-1])
+        self.sign_bits = 1
+        self.num_bits = self.e_bits + self.m_bits + self.sign_bits
+        self.default_bias = 2 ** (self.e_bits - 1)
+        self.dst_nbins = 2 ** self.num_bits
+        self.use_qtorch = self.kwargs.get('use_qtorch')
+        if not self.use_qtorch:
+            raise NotImplementedError('FloatQuantizer(use_qtorch=False) is not on this path')
+        if 'float_range' in self.kwargs:
+            self.qmin, self.qmax = self.kwargs['float_range']
+        else:
+            key = (self.bit, self.num_bits)
+            if key not in self._RANGES:
+                raise NotImplementedError('Only 4, 6, 8, and 12-bit quantization is supported.')
+            if isinstance(self._RANGES[key], tuple):
+                self.qmin, self.qmax = self._RANGES[key]
+            else:
+                finfo = torch.finfo(self._RANGES[key])
+                self.qmin, self.qmax = finfo.min, finfo.max
+        self.qmax = torch.tensor(self.qmax)
+        self.qmin = torch.tensor(self.qmin)
+        self.fp_tie = self.kwargs.get('fp_tie', 'away')
+        self.fp_subnormals = self.kwargs.get('fp_subnormals', True)
+
+    def _fp_flags(self):
+        return ((L.FLAG_TIE_EVEN if self.fp_tie == 'even' else 0)
+                | (0 if self.fp_subnormals else L.FLAG_NO_SUBNORMALS))
+
+    def get_qparams(self, tensor_range, device):
+        """Symmetric branch of quant.py:544-552 with the float qmax."""
+        min_val, max_val = tensor_range[0].contiguous(), tensor_range[1].contiguous()
+        scales = torch.empty_like(max_val)
+        L.check(L.lib().lcq_qparams_int(L.ptr(min_val), L.ptr(max_val), L.dtype_code(max_val.dtype),
+                                        L.i64(max_val.numel()), L.f32(-float(self.qmax)), L.f32(self.qmax),
+                                        L.i32(L.FLAG_SYM), L.ptr(scales), L.ptr(None), L.stream()),
+                'lcq_qparams_int')
+        return scales, torch.tensor(0.0), self.qmax.to(device), self.qmin.to(device)
+
+    def _launch(self, rows_t, *, static, scales=None, want_dq=None, want_codes=None):
+        t = rows_t.contiguous()
+        flags = self._fp_flags()
+        if static:
+            scales[scales == 0] = 1                      # quant.py:1061 mutates the caller's tensor
+            if scales.dim() > 0 and scales.dtype != t.dtype:
+                t = t.to(torch.promote_types(t.dtype, scales.dtype))
+            s = scales.to(t.dtype).contiguous()
+            rows, cols, scalar = _static_layout(t, s)
+            flags |= L.FLAG_STATIC | (L.FLAG_SCALAR_QP if scalar else 0)
+        else:
+            if self.granularity == 'per_tensor':
+                s, _, _, _ = self.get_qparams(self.get_minmax_range(t), t.device)
+                return self._launch(t, static=True, scales=s, want_dq=want_dq, want_codes=want_codes)
+            rows, cols = _rows_cols(t)
+            s = torch.empty((rows, 1), dtype=t.dtype, device=t.device)
+        dq = None
+        if want_dq == 'f32':
+            dq = torch.empty(t.shape, dtype=torch.float32, device=t.device)
+            flags |= L.FLAG_DQ_F32
+        elif want_dq:
+            dq = torch.empty_like(t)
+        codes, cd = None, L.CODE_NONE
+        if want_codes == 'f32':
+            codes, cd = torch.empty(t.shape, dtype=torch.float32, device=t.device), L.CODE_F32
+        elif want_codes is not None:
+            codes, cd = torch.empty(t.shape, dtype=want_codes, device=t.device), L.CODE_FP8
+        L.check(L.lib().lcq_quant_fp(L.ptr(t), L.dtype_code(t.dtype), L.i64(rows), L.i64(cols), L.i32(self.e_bits),
+                                     L.i32(self.m_bits), L.f32(self.qmax), L.i32(flags), L.ptr(dq), L.ptr(codes),
+                                     L.i32(cd), L.ptr(s), L.stream()), 'lcq_quant_fp')
+        return dq, codes, s
+
+    def get_tensor_qparams(self, tensor, args={}):
+        """quant.py:1042-1058 -> (tensor_reshaped, scales, zeros, qmax, qmin)."""
+        if self.calib_algo != 'minmax':
+            raise NotImplementedError(f'calib_algo={self.calib_algo!r}: only minmax runs on liblcq')
+        tensor = self.reshape_tensor(tensor)
+        if self.granularity == 'per_tensor':
+            s, z, qmax, qmin = self.get_qparams(self.get_minmax_range(tensor), tensor.device)
+            return tensor, s, z, qmax, qmin
+        _, _, s = self._launch(tensor, static=False)
+        if tensor.dim() != 2:
+            s = s.view(*tensor.shape[:-1], 1)
+        return tensor, s, torch.tensor(0.0), self.qmax.to(tensor.device), self.qmin.to(tensor.device)
+
+    def quant(self, tensor, scales, zeros, qmax, qmin):
+        """quant.py:1060-1071: fp32 values on the minifloat grid."""
+        _, codes, _ = self._launch(tensor, static=True, scales=scales, want_codes='f32')
+        return codes.view(tensor.shape)
+
+    def dequant(self, tensor, scales, zeros):
+        """quant.py:1073-1075 on fp32 codes."""
+        t = tensor.float().contiguous()
+        s = scales.contiguous()
+        rows, cols, scalar = _static_layout(t, s)
+        out = torch.empty_like(t)
+        L.check(L.lib().lcq_dequant_fp(L.ptr(t), L.i64(rows), L.i64(cols), L.ptr(s), L.dtype_code(s.dtype),
+                                       L.i32(L.FLAG_SCALAR_QP if scalar else 0), L.ptr(out), L.stream()),
+                'lcq_dequant_fp')
+        return out
+
+    def quant_dequant(self, tensor, scales, zeros, qmax, qmin):
+        """quant.py:1077-1080: fp32 result (the float codes promote it)."""
+        dq, _, _ = self._launch(tensor, static=True, scales=scales, want_dq='f32')
+        return dq.view(tensor.shape)
+
+    def _fake(self, t, static_scales=None):
+        shape, dtype = t.shape, t.dtype
+        rows_t = self.reshape_tensor(t)
+        if static_scales is None:
+            dq, _, _ = self._launch(rows_t, static=False, want_dq=True)
+        else:
+            dq, _, _ = self._launch(rows_t, static=True, scales=static_scales, want_dq=True)
+        return self.restore_tensor(dq.view(rows_t.shape), shape).to(dtype)
+
+    def fake_quant_act_static(self, act, args={}):
+        return self._fake(act, args['scales'])
+
+    def fake_quant_act_dynamic(self, act, args={}):
+        return self._fake(act)
+
+    def fake_quant_weight_static(self, weight, args):
+        if 'rounding' in args:
+            raise NotImplementedError("the 'rounding' override is not on this path")
+        ic = 'dim' in args and 'ic' in args['dim']
+        q = self._fake(weight.T if ic else weight, args['scales'])
+        return q.T if ic else q
+
+    def fake_quant_weight_dynamic(self, weight, args={}):
+        ic = 'dim' in args and 'ic' in args['dim']
+        q = self._fake(weight.T if ic else weight)
+        return q.T if ic else q
+
+    def _real(self, weight, static_scales, output_scale_factor):
+        assert self.bit in ['e4m3', 'e5m2'], 'Only FP8 E4M3 and E5M2 support real quant'
+        dtype = torch.float8_e4m3fn if self.e_bits == 4 else torch.float8_e5m2
+        org_w_shape = weight.shape
+        rows_t = self.reshape_tensor(weight)
+        if static_scales is None:
+            _, codes, scales = self._launch(rows_t, static=False, want_codes=dtype)
+        else:
+            _, codes, _ = self._launch(rows_t, static=True, scales=static_scales, want_codes=dtype)
+            scales = static_scales
+        codes = self.restore_tensor(codes.view(rows_t.shape), org_w_shape)
+        scales = scales * output_scale_factor
+        qparams_shape = 1 if self.granularity == 'per_tensor' else (codes.shape[0], -1)
+        return codes, scales.view(qparams_shape), None
+
+    def real_quant_weight_static(self, weight, args):
+        """quant.py:1160-1192."""
+        return self._real(weight, args['scales'], args.pop('output_scale_factor', 1))
+
+    def real_quant_weight_dynamic(self, weight, args={}):
+        """quant.py:1194-1220."""
+        osf = args.pop('output_scale_factor', 1) if 'output_scale_factor' in args else 1
+        return self._real(weight, None, osf)
+
+    def __repr__(self):
+        return (
+            f'FloatQuantizer(bit={self.bit},'
+            f'e_bits={self.e_bits}, m_bits={self.m_bits},'
+            f'granularity={self.granularity},'
+            f'kwargs={self.kwargs}, qmin={self.qmin}, qmax={self.qmax})'
+        )

@@ -1,0 +1,326 @@
+"""Oracle: integer / minifloat quantizer arithmetic (test infrastructure only).
+
+Restates quant.py of the reference as free functions over CPU torch tensors.
+The op ORDER and the dtype each op runs in are what make results bit-exact,
+so every line keeps the reference's op sequence (one torch op per arithmetic
+step, no fusing) while the structure (functions + a small spec object instead
+of a class hierarchy) is this repo's own.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+
+# ----------------------------------------------------------------------------
+# spec
+# ----------------------------------------------------------------------------
+@dataclass
+class IntSpec:
+    """Mirror of the ctor surface, quant.py:49-103 and 660-677."""
+    bit: int
+    symmetric: bool
+    granularity: str                      # per_tensor|per_channel|per_group|per_head|per_token
+    group_size: int = 0
+    head_num: int = 0
+    round_zp: bool = True
+    int_range: tuple | None = None
+    qmin: torch.Tensor = field(init=False)
+    qmax: torch.Tensor = field(init=False)
+
+    def __post_init__(self):
+        if self.int_range is not None:
+            lo, hi = self.int_range
+        elif self.symmetric:
+            lo, hi = -(2 ** (self.bit - 1)), 2 ** (self.bit - 1) - 1
+        else:
+            lo, hi = 0.0, 2 ** self.bit - 1          # qmin is a python float there (quant.py:672)
+        self.qmin = torch.tensor(lo)
+        self.qmax = torch.tensor(hi)
+
+
+# ----------------------------------------------------------------------------
+# reshape / restore   (quant.py:611-657)
+# ----------------------------------------------------------------------------
+def reshape_rows(spec, t: torch.Tensor, allow_padding=False) -> torch.Tensor:
+    if spec.granularity == 'per_group':
+        g = spec.group_size
+        if t.shape[-1] < g:
+            return t
+        if t.shape[-1] % g == 0:
+            return t.reshape(-1, g)
+        if not allow_padding:
+            raise ValueError(f'Dimension {t.shape[-1]} not divisible by group size {g}')
+        lack = g - t.shape[1] % g
+        pad = torch.zeros((*t.shape[:-1], lack), dtype=t.dtype)
+        return torch.cat((t, pad), dim=-1).reshape(-1, g)
+    if spec.granularity == 'per_head':
+        return t.reshape(spec.head_num, -1)
+    return t
+
+
+def restore_rows(spec, t: torch.Tensor, shape) -> torch.Tensor:
+    if t.shape == shape:
+        return t
+    try:
+        return t.reshape(shape)
+    except RuntimeError:
+        lack = spec.group_size - shape[1] % spec.group_size
+        return t.reshape(*shape[:-1], -1)[..., :-lack]
+
+
+# ----------------------------------------------------------------------------
+# range -> qparams   (quant.py:134-145, 544-558)
+# ----------------------------------------------------------------------------
+def minmax_range(spec, t: torch.Tensor):
+    if spec.granularity == 'per_tensor':
+        return torch.min(t), torch.max(t)
+    return t.amin(dim=-1, keepdim=True), t.amax(dim=-1, keepdim=True)
+
+
+def int_qparams(spec, lo: torch.Tensor, hi: torch.Tensor):
+    qmin, qmax = spec.qmin, spec.qmax
+    if spec.symmetric:
+        span = torch.max(hi.abs(), lo.abs())
+        span = span.clamp(min=1e-5)
+        scales = span / qmax
+        zeros = torch.tensor(0.0)
+    else:
+        scales = (hi - lo).clamp(min=1e-5) / (qmax - qmin)
+        zeros = (qmin - torch.round(lo / scales)).clamp(qmin, qmax)
+        if not spec.round_zp:
+            zeros = qmin - (lo / scales)
+    return scales, zeros, qmax, qmin
+
+
+def int_tensor_qparams(spec, t: torch.Tensor):
+    """quant.py:689-696 (minmax calibration)."""
+    rows = reshape_rows(spec, t)
+    lo, hi = minmax_range(spec, rows)
+    s, z, qmax, qmin = int_qparams(spec, lo, hi)
+    return rows, s, z, qmax, qmin
+
+
+# ----------------------------------------------------------------------------
+# quant / dequant   (quant.py:698-716)
+# ----------------------------------------------------------------------------
+def int_quant(spec, t, scales, zeros, qmax, qmin):
+    if spec.round_zp:
+        return torch.clamp(torch.round(t / scales) + zeros, qmin, qmax)
+    return torch.clamp(torch.round(t / scales.clamp_min(1e-9) + zeros), qmin, qmax)
+
+
+def int_dequant(t, scales, zeros):
+    return (t - zeros) * scales
+
+
+def int_quant_dequant(spec, t, scales, zeros, qmax, qmin, output_scale_factor=1):
+    q = int_quant(spec, t, scales, zeros, qmax, qmin)
+    return int_dequant(q, scales * output_scale_factor, zeros)
+
+
+def int_fake_quant_dynamic(spec, w: torch.Tensor) -> torch.Tensor:
+    """fake_quant_weight_dynamic / fake_quant_act_dynamic, quant.py:753-782, 832-868."""
+    shape, dtype = w.shape, w.dtype
+    rows, s, z, qmax, qmin = int_tensor_qparams(spec, w)
+    out = int_quant_dequant(spec, rows, s, z, qmax, qmin)
+    return restore_rows(spec, out, shape).to(dtype)
+
+
+def int_fake_quant_static(spec, w, scales, zeros, qmax, qmin, output_scale_factor=1):
+    """fake_quant_weight_static, quant.py:784-830 (no index mixing)."""
+    shape, dtype = w.shape, w.dtype
+    rows = reshape_rows(spec, w)
+    out = int_quant_dequant(spec, rows, scales, zeros, qmax, qmin, output_scale_factor)
+    return restore_rows(spec, out, shape).to(dtype)
+
+
+def _code_dtype(spec):
+    if spec.bit == 8:
+        return torch.int8 if spec.qmin != 0 else torch.uint8
+    return torch.int32
+
+
+def _qparam_shape(spec, codes):
+    return 1 if spec.granularity == 'per_tensor' else (codes.shape[0], -1)
+
+
+def int_real_quant_dynamic(spec, w, output_scale_factor=1):
+    """real_quant_weight_dynamic, quant.py:915-952."""
+    shape = w.shape
+    rows, s, z, qmax, qmin = int_tensor_qparams(spec, w)
+    codes = restore_rows(spec, int_quant(spec, rows, s, z, qmax, qmin), shape)
+    s = s * output_scale_factor
+    dt = _code_dtype(spec)
+    codes = codes.to(dt)
+    if not spec.symmetric and spec.round_zp:
+        z = z.to(dt)
+    elif spec.symmetric:
+        z = None
+    shp = _qparam_shape(spec, codes)
+    if z is not None:
+        z = z.view(shp)
+    return codes, s.view(shp), z
+
+
+def int_real_quant_static(spec, w, scales, zeros, qmax, qmin, output_scale_factor=1):
+    """real_quant_weight_static, quant.py:870-913."""
+    shape = w.shape
+    rows = reshape_rows(spec, w)
+    codes = restore_rows(spec, int_quant(spec, rows, scales, zeros, qmax, qmin), shape)
+    s = scales * output_scale_factor
+    dt = _code_dtype(spec)
+    codes = codes.to(dt)
+    z = zeros
+    if not spec.symmetric and spec.round_zp:
+        z = z.to(dt)
+    elif spec.symmetric:
+        z = None
+    shp = _qparam_shape(spec, codes)
+    if z is not None:
+        z = z.view(shp)
+    return codes, s.view(shp), z
+
+
+# ----------------------------------------------------------------------------
+# minifloat ("FPx") quantizer, qtorch mode   (quant.py:962-1002, 1042-1080)
+# ----------------------------------------------------------------------------
+_FLOAT_RANGE = {'e4m3': 448.0, 'e5m2': 57344.0, 'e3m2': 28.0, 'e4m7': 510.0, 'e2m1': 6.0}
+
+
+@dataclass
+class FloatSpec:
+    bit: str                       # 'e4m3' ...
+    granularity: str
+    group_size: int = 0
+    head_num: int = 0
+    float_range: tuple | None = None
+    # rounding model of the third-party float_quantize (parity unpinned)
+    tie: str = 'away'              # 'away' (add-half-then-truncate) | 'even'
+    subnormals: bool = True
+    symmetric: bool = True         # forced, quant.py:965
+    round_zp: bool = True
+
+    def __post_init__(self):
+        self.e_bits = int(self.bit[1])
+        self.m_bits = int(self.bit[-1])
+        if self.float_range is not None:
+            lo, hi = self.float_range
+        else:
+            hi = _FLOAT_RANGE[self.bit]
+            lo = -hi
+        self.qmin = torch.tensor(float(lo))
+        self.qmax = torch.tensor(float(hi))
+
+
+def float_quantize_nearest(x: torch.Tensor, e_bits: int, m_bits: int,
+                           tie: str = 'away', subnormals: bool = True) -> torch.Tensor:
+    """Round fp32 ``x`` to a (1, e_bits, m_bits) minifloat grid, result in fp32.
+
+    Restates the *published* algorithm of QPyTorch's ``float_quantize(...,
+    rounding='nearest')`` (third-party, absent from the reference tree;
+    call site quant.py:1065-1067), working on the fp32 bit pattern:
+
+    * normal range: add half of the dropped-mantissa ulp to the raw bits and
+      truncate (``tie='away'``: ties go away from zero) — or RNE for
+      ``tie='even'`` (what a native float8 cast does);
+    * below the minimum normal 2**(2 - 2**(e_bits-1)): with ``subnormals`` the
+      value is rounded on the fixed step  min_normal * 2**-m_bits  (by adding
+      +-min_normal, rounding the mantissa, subtracting again); without, it is
+      flushed to 0 or +-min_normal whichever is nearer;
+    * the exponent is clipped at 2**(e_bits-1): the largest magnitude is
+      2**(2**(e_bits-1)) * (2 - 2**-m_bits)  (480 for e4m3, above the 448 the
+      reference scales to, so saturation never fires on in-range inputs).
+    """
+    assert x.dtype == torch.float32
+    a = np.ascontiguousarray(x.detach().numpy())
+    bits = a.view(np.uint32).astype(np.uint64)
+    sign = bits & 0x80000000
+    mag = bits & 0x7FFFFFFF
+    drop = 23 - m_bits
+    half = np.uint64(1 << (drop - 1))
+    keep = np.uint64(~((1 << drop) - 1) & 0xFFFFFFFF)
+
+    def round_mag(m):
+        if tie == 'away':
+            return (m + half) & keep
+        lsb = (m >> np.uint64(drop)) & np.uint64(1)
+        return (m + half - np.uint64(1) + lsb) & keep
+
+    min_exp = -((1 << (e_bits - 1)) - 2)              # exponent of the minimum normal
+    max_exp = 1 << (e_bits - 1)
+    exp_field = (mag >> np.uint64(23)).astype(np.int64) - 127
+    is_sub = exp_field < min_exp
+    finite = (mag >> np.uint64(23)) != 0xFF
+
+    out_norm = round_mag(mag)
+    # exponent clipping (saturate to the largest representable magnitude)
+    max_mag = np.uint64(((max_exp + 127) << 23) | (((1 << m_bits) - 1) << drop))
+    out_norm = np.where((out_norm >> np.uint64(23)).astype(np.int64) - 127 > max_exp, max_mag, out_norm)
+
+    mn = np.float32(2.0 ** min_exp)
+    absx = np.abs(a)
+    if subnormals:
+        shifted = (absx.astype(np.float32) + mn).astype(np.float32)
+        sb = round_mag(shifted.view(np.uint32).astype(np.uint64))
+        sub_val = (sb.astype(np.uint32).view(np.float32) - mn).astype(np.float32)
+    else:
+        sub_val = np.where(absx > mn / 2, mn, np.float32(0)).astype(np.float32)
+    sub_bits = sub_val.view(np.uint32).astype(np.uint64)
+
+    out = np.where(is_sub, sub_bits, out_norm)
+    out = np.where(finite, out, mag)                   # inf / nan pass through
+    res = (out | sign).astype(np.uint32).view(np.float32)
+    return torch.from_numpy(res.copy()).reshape(x.shape)
+
+
+def float_qparams(spec, lo, hi):
+    """get_qparams (symmetric branch) as used by FloatQuantizer, quant.py:544-552, 1048-1051."""
+    span = torch.max(hi.abs(), lo.abs())
+    span = span.clamp(min=1e-5)
+    scales = span / spec.qmax
+    zeros = torch.tensor(0.0)
+    return scales, zeros, spec.qmax, spec.qmin
+
+
+def float_tensor_qparams(spec, t):
+    rows = reshape_rows(spec, t)
+    lo, hi = minmax_range(spec, rows)
+    s, z, qmax, qmin = float_qparams(spec, lo, hi)
+    return rows, s, z, qmax, qmin
+
+
+def float_quant(spec, t, scales, zeros):
+    """quant.py:1060-1071 (qtorch branch): result is fp32 whatever the input dtype."""
+    scales[scales == 0] = 1
+    scaled = t / scales + zeros
+    return float_quantize_nearest(scaled.float(), spec.e_bits, spec.m_bits, spec.tie, spec.subnormals)
+
+
+def float_dequant(t, scales, zeros):
+    return (t - zeros) * scales
+
+
+def float_fake_quant_dynamic(spec, w):
+    """quant.py:1099-1108, 1141-1158."""
+    shape, dtype = w.shape, w.dtype
+    rows, s, z, _, _ = float_tensor_qparams(spec, w)
+    q = float_quant(spec, rows, s, z)
+    out = float_dequant(q, s, z)
+    return restore_rows(spec, out, shape).to(dtype)
+
+
+def float_real_quant_dynamic(spec, w, output_scale_factor=1):
+    """quant.py:1194-1220."""
+    assert spec.bit in ('e4m3', 'e5m2')
+    dt = torch.float8_e4m3fn if spec.e_bits == 4 else torch.float8_e5m2
+    shape = w.shape
+    rows, s, z, _, _ = float_tensor_qparams(spec, w)
+    q = restore_rows(spec, float_quant(spec, rows, s, z), shape)
+    s = s * output_scale_factor
+    q = q.to(dt)
+    shp = 1 if spec.granularity == 'per_tensor' else (q.shape[0], -1)
+    return q, s.view(shp), None

@@ -1,0 +1,276 @@
+"""Pins the CPU oracle of the quantizer arithmetic (no GPU needed).
+
+The reference ships no golden vectors for this path, so the oracle is pinned
+against what the mathematics fixes: exact rational arithmetic on small inputs,
+an independent bit-level bf16 model, invariants of min/max quantization, the
+float8 casts torch itself provides, and pack/unpack round trips.
+"""
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import pack_ref, quant_ref as Q
+from tests.helpers import assert_bit_equal, gen, weight_like
+
+
+# --------------------------------------------------------------------------
+# integer quantizer, fp32: exact rational arithmetic
+# --------------------------------------------------------------------------
+def _rne_int(fr: Fraction) -> int:
+    fl = fr.numerator // fr.denominator
+    rem = fr - fl
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1):
+        return fl + 1
+    return fl
+
+
+def _near_tie(fr: Fraction, tol=Fraction(1, 1 << 18)) -> bool:
+    frac = fr - (fr.numerator // fr.denominator)
+    return abs(frac - Fraction(1, 2)) < tol
+
+
+@pytest.mark.parametrize('bit,sym', [(4, False), (4, True), (8, False), (8, True), (3, False)])
+def test_int_fp32_codes_match_exact_rationals(bit, sym):
+    spec = Q.IntSpec(bit, sym, 'per_group', group_size=32)
+    w = weight_like(6, 64, seed=bit + 10 * sym, outlier_frac=0.02)
+    rows, s, z, qmax, qmin = Q.int_tensor_qparams(spec, w)
+    q = Q.int_quant(spec, rows, s, z, qmax, qmin)
+    lo, hi = float(qmin), float(qmax)
+    checked = 0
+    for r in range(rows.shape[0]):
+        # the scale itself: one fp32 rounding of the exact quotient
+        vals = [Fraction(float(v)) for v in rows[r]]
+        span = (max(vals) - min(vals)) if not sym else max(abs(max(vals)), abs(min(vals)))
+        span = max(span, Fraction(float(np.float32(1e-5))))
+        if not sym:
+            span32 = Fraction(float(np.float32(float(max(vals))) - np.float32(float(min(vals)))))   # fp32 subtract
+            span32 = max(span32, Fraction(float(np.float32(1e-5))))
+            exact_scale = span32 / Fraction(int(hi - lo))
+        else:
+            exact_scale = span / Fraction(int(hi))
+        assert float(s[r]) == float(np.float32(float(exact_scale))) or abs(Fraction(float(s[r])) - exact_scale) <= Fraction(float(s[r])) / (1 << 23)
+        S = Fraction(float(s[r]))
+        if sym:
+            Z = 0
+        else:
+            zq = Fraction(float(min(vals))) / S
+            if _near_tie(zq):
+                continue
+            Z = int(min(max(lo - _rne_int(zq), lo), hi))
+            assert Z == int(z[r]), (r, Z, z[r])
+        for c in range(rows.shape[1]):
+            fr = vals[c] / S
+            if _near_tie(fr):
+                continue                                  # an fp32 rounding of x/s may legally cross the tie
+            want = min(max(_rne_int(fr) + Z, lo), hi)
+            assert float(q[r, c]) == want, (r, c, float(q[r, c]), want)
+            checked += 1
+    assert checked > 300
+
+
+def test_int_invariants_and_idempotence():
+    spec = Q.IntSpec(4, False, 'per_group', group_size=128)
+    w = weight_like(64, 512, seed=3)
+    rows, s, z, qmax, qmin = Q.int_tensor_qparams(spec, w)
+    q = Q.int_quant(spec, rows, s, z, qmax, qmin)
+    assert q.min() >= 0 and q.max() <= 15 and torch.equal(q, q.round())
+    # the group maximum lands on the top code, the minimum on the zero point (clamped)
+    assert torch.all(q.gather(1, rows.argmax(1, keepdim=True)) >= 14)
+    assert torch.equal(q.gather(1, rows.argmin(1, keepdim=True)), torch.clamp(torch.round(rows.amin(1, keepdim=True) / s) + z, 0, 15))
+    dq = Q.int_dequant(q, s, z)
+    assert torch.all((dq - rows).abs() <= s * 0.5001 + 1e-12)
+    # closed form of the asymmetric 4-bit scale
+    assert_bit_equal(s, (rows.amax(1, keepdim=True) - rows.amin(1, keepdim=True)).clamp(min=1e-5) / 15.0, 'scale')
+    # quantizing an already quantized tensor with the same qparams changes nothing
+    again = Q.int_quant_dequant(spec, dq, s, z, qmax, qmin)
+    assert_bit_equal(again, dq, 'idempotence')
+    # fake quant == restore(dequant(quant))
+    fq = Q.int_fake_quant_dynamic(spec, w)
+    assert_bit_equal(fq, dq.reshape(w.shape), 'fake quant')
+
+
+def test_int_real_quant_layout():
+    w = weight_like(16, 256, seed=5)
+    for bit, sym, dt in [(4, False, torch.int32), (8, False, torch.uint8), (8, True, torch.int8), (4, True, torch.int32)]:
+        spec = Q.IntSpec(bit, sym, 'per_group', group_size=128)
+        codes, s, z = Q.int_real_quant_dynamic(spec, w)
+        assert codes.dtype == dt and codes.shape == w.shape and s.shape == (16, 2)
+        assert (z is None) == sym
+        if z is not None:
+            assert z.dtype == dt and z.shape == (16, 2)
+    spec = Q.IntSpec(8, True, 'per_tensor')
+    codes, s, z = Q.int_real_quant_dynamic(spec, w)
+    assert s.shape == (1,) and z is None
+    spec = Q.IntSpec(8, True, 'per_channel')
+    codes, s, z = Q.int_real_quant_dynamic(spec, w)
+    assert s.shape == (16, 1)
+
+
+# --------------------------------------------------------------------------
+# integer quantizer, bf16: independent numpy model that rounds after each op
+# --------------------------------------------------------------------------
+def _bf16r(a):
+    """fp32 ndarray -> nearest-even bf16 -> fp32 (bit twiddling, no torch)."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+    return u.astype(np.uint32).view(np.float32)
+
+
+def _np_int_fake_quant_bf16(w_bf16: torch.Tensor, bit, sym, g):
+    x = w_bf16.float().numpy().reshape(-1, g)
+    one = np.float32
+    mx, mn = x.max(1, keepdims=True), x.min(1, keepdims=True)
+    cmin = _bf16r(np.array([1e-5], dtype=np.float32))[0]
+    if sym:
+        qmin, qmax = one(-(2 ** (bit - 1))), one(2 ** (bit - 1) - 1)
+        a = np.maximum(np.maximum(np.abs(mx), np.abs(mn)), cmin)
+        s = _bf16r(a / qmax)
+        z = np.zeros_like(s)
+    else:
+        qmin, qmax = one(0), one(2 ** bit - 1)
+        d = np.maximum(_bf16r(mx - mn), cmin)
+        s = _bf16r(d / (qmax - qmin))
+        z = np.clip(_bf16r(qmin - np.rint(_bf16r(mn / s))), qmin, qmax)
+    q = np.clip(_bf16r(np.rint(_bf16r(x / s)) + z), qmin, qmax)
+    dq = _bf16r(_bf16r(q - z) * s)
+    return dq.reshape(w_bf16.shape), s, z, q
+
+
+@pytest.mark.parametrize('bit,sym', [(4, False), (4, True), (8, False), (8, True)])
+def test_int_bf16_matches_bitlevel_model(bit, sym):
+    w = weight_like(96, 512, seed=7 + bit, dtype=torch.bfloat16)
+    spec = Q.IntSpec(bit, sym, 'per_group', group_size=128)
+    fq = Q.int_fake_quant_dynamic(spec, w)
+    assert fq.dtype == torch.bfloat16
+    dq, s, z, q = _np_int_fake_quant_bf16(w, bit, sym, 128)
+    assert_bit_equal(fq.float(), torch.from_numpy(dq.copy()), 'bf16 fake quant')
+    rows, so, zo, qmax, qmin = Q.int_tensor_qparams(spec, w)
+    assert so.dtype == torch.bfloat16
+    assert_bit_equal(so.float(), torch.from_numpy(s.copy()), 'bf16 scales')
+    if not sym:
+        assert_bit_equal(zo.float(), torch.from_numpy(z.copy()), 'bf16 zeros')
+    # the double rounding (x/s -> bf16 -> round) really happens: it changes some codes
+    exact = torch.clamp(torch.round(rows.float() / so.float()) + (zo.float() if not sym else 0), float(qmin), float(qmax))
+    assert (exact != torch.from_numpy(q.copy())).any()
+
+
+# --------------------------------------------------------------------------
+# minifloat rounding
+# --------------------------------------------------------------------------
+def _grid(e_bits, m_bits):
+    """All non-negative values of the (e,m) minifloat with exponent range [2-2^(e-1), 2^(e-1)]."""
+    min_exp = -((1 << (e_bits - 1)) - 2)
+    max_exp = 1 << (e_bits - 1)
+    vals = {Fraction(0)}
+    for k in range(1, 1 << m_bits):                       # subnormals
+        vals.add(Fraction(k, 1 << m_bits) * Fraction(2) ** min_exp)
+    for e in range(min_exp, max_exp + 1):
+        for k in range(1 << m_bits):
+            vals.add((1 + Fraction(k, 1 << m_bits)) * Fraction(2) ** e)
+    return sorted(vals)
+
+
+@pytest.mark.parametrize('fmt', ['e4m3', 'e5m2', 'e2m1', 'e3m2'])
+@pytest.mark.parametrize('tie', ['away', 'even'])
+def test_float_quantize_is_nearest_grid_point(fmt, tie):
+    e, m = int(fmt[1]), int(fmt[3])
+    grid = _grid(e, m)
+    top = float(grid[-1])
+    g = gen(11)
+    x = torch.cat([
+        (torch.rand(400, generator=g) * 2 - 1) * top * 0.99,
+        (torch.rand(200, generator=g) * 2 - 1) * float(grid[1 << m]) * 2,        # around the subnormal range
+        torch.tensor([float(a + b) / 2 for a, b in zip(grid[:-1], grid[1:])]),     # every exact tie
+        -torch.tensor([float(a + b) / 2 for a, b in zip(grid[:-1], grid[1:])]),
+        torch.tensor([float(v) for v in grid]), torch.tensor([0.0, -0.0]),
+    ]).float()
+    got = Q.float_quantize_nearest(x, e, m, tie=tie)
+    for xv, gv in zip(x.tolist(), got.tolist()):
+        a = abs(Fraction(xv))
+        best = min(grid, key=lambda v: abs(v - a))
+        cands = [v for v in grid if abs(v - a) == abs(best - a)]
+        if len(cands) == 2:
+            if tie == 'away':
+                best = max(cands)
+            else:                                          # even mantissa: the one whose last kept bit is 0
+                best = [v for v in cands if (v / (Fraction(2) ** (max(_exp(v), -((1 << (e - 1)) - 2)) - m))) % 2 == 0][0]
+        want = float(best) * (-1 if (xv < 0 or str(xv) == '-0.0') else 1)
+        assert gv == want, (fmt, tie, xv, gv, want)
+    # saturation at the largest magnitude
+    big = torch.tensor([top * 4, -top * 4])
+    assert Q.float_quantize_nearest(big, e, m, tie=tie).tolist() == [top, -top]
+
+
+def _exp(v: Fraction) -> int:
+    if v == 0:
+        return -(1 << 20)
+    e = 0
+    while v >= 2:
+        v /= 2; e += 1
+    while v < 1:
+        v *= 2; e -= 1
+    return e
+
+
+def test_float_quantize_even_equals_torch_float8_casts():
+    g = gen(12)
+    x = torch.cat([torch.randn(20000, generator=g) * 50, torch.randn(20000, generator=g) * 0.01,
+                   (torch.randn(20000, generator=g) * 30).bfloat16().float()])
+    x = x.clamp(-448, 448)
+    assert_bit_equal(Q.float_quantize_nearest(x, 4, 3, tie='even'), x.to(torch.float8_e4m3fn).float(), 'e4m3')
+    y = (x * 100).clamp(-57344, 57344)
+    assert_bit_equal(Q.float_quantize_nearest(y, 5, 2, tie='even'), y.to(torch.float8_e5m2).float(), 'e5m2')
+
+
+def test_float_real_quant_is_on_grid_and_scaled_to_448():
+    w = weight_like(32, 512, seed=13, dtype=torch.bfloat16, std=0.006, outlier_frac=0.0005, outlier_mul=30)
+    spec = Q.FloatSpec('e4m3', 'per_channel')
+    codes, s, z = Q.float_real_quant_dynamic(spec, w)
+    assert codes.dtype == torch.float8_e4m3fn and s.shape == (32, 1) and z is None and s.dtype == torch.bfloat16
+    assert_bit_equal(s, (w.abs().amax(1, keepdim=True).clamp(min=1e-5) / 448.0), 'fp8 scale')
+    assert codes.float().abs().max() <= 448
+    fq = Q.float_fake_quant_dynamic(spec, w)
+    assert_bit_equal(fq, (codes.float() * s).to(torch.bfloat16), 'fake == real dequantized')
+    # a sixteenth of bf16 inputs are exact e4m3 ties: the tie rule is visible
+    ev = Q.float_fake_quant_dynamic(Q.FloatSpec('e4m3', 'per_channel', tie='even'), w)
+    assert (ev != fq).float().mean() > 0.005
+
+
+# --------------------------------------------------------------------------
+# packing
+# --------------------------------------------------------------------------
+def test_pack_ct_roundtrip_and_padding():
+    g = gen(14)
+    codes = torch.randint(-8, 8, (5, 37), generator=g, dtype=torch.int32)
+    packed, s16 = pack_ref.pack_ct(codes, torch.ones(5, 1), 4)
+    assert packed.shape == (5, 5) and packed.dtype == torch.int32 and s16.dtype == torch.float16
+    assert torch.equal(pack_ref.unpack_ct(packed, 4, 37), codes)
+    # brute force one word, and the zero padding of the tail word
+    r, j = 2, 1
+    word = 0
+    for i in range(8):
+        word |= (int(codes[r, 8 * j + i]) + 8) << (4 * i)
+    assert int(packed[r, j]) & 0xFFFFFFFF == word
+    assert (int(packed[0, 4]) & 0xFFFFFFFF) >> 20 == 0
+    codes8 = torch.randint(-128, 128, (3, 10), generator=g, dtype=torch.int8)
+    p8, _ = pack_ref.pack_ct(codes8, torch.ones(3, 1), 8)
+    assert torch.equal(pack_ref.unpack_ct(p8, 8, 10), codes8.to(torch.int32))
+
+
+def test_gemm_pack_order_bruteforce():
+    w = weight_like(32, 256, seed=15, dtype=torch.bfloat16)
+    spec = Q.IntSpec(4, False, 'per_group', group_size=128)
+    codes, s, z = Q.int_real_quant_dynamic(spec, w)
+    qweight, s16, qzeros = pack_ref.gemm_pack(w, s, z, 128)
+    assert qweight.shape == (256, 4) and s16.shape == (2, 32) and qzeros.shape == (2, 4)
+    iw = pack_ref.gemm_unpack(qweight)
+    # nibble i of word c holds output channel 8c + order[i]: spot check by hand
+    k, c = 17, 2
+    word = int(qweight[k, c]) & 0xFFFFFFFF
+    for i, o in enumerate((0, 2, 4, 6, 1, 3, 5, 7)):
+        assert (word >> (4 * i)) & 15 == int(iw[k, 8 * c + o])
+    # with fp16 scales the re-derived integers equal the quantizer's codes almost everywhere
+    assert (iw.t() == codes).float().mean() > 0.99
+    assert torch.equal(pack_ref.gemm_unpack(qzeros).t().contiguous(), z)

@@ -1,0 +1,222 @@
+"""GPU parity: lightcompress_amd quantizers / packers vs the CPU oracle, bit-exact."""
+import pytest
+import torch
+
+from oracle import pack_ref, quant_ref as Q
+from tests.helpers import assert_bit_equal, gen, weight_like
+
+pytestmark = pytest.mark.gpu
+
+
+def _iq(bit, sym, gran, **kw):
+    from lightcompress_amd import IntegerQuantizer
+    return IntegerQuantizer(bit, sym, gran, **kw)
+
+
+INT_CASES = [
+    # bit, sym, granularity, kwargs, shape
+    (4, False, 'per_group', dict(group_size=128), (256, 1024)),
+    (4, True, 'per_group', dict(group_size=128), (256, 1024)),
+    (4, False, 'per_group', dict(group_size=64), (128, 512)),
+    (4, False, 'per_group', dict(group_size=32), (128, 256)),
+    (3, False, 'per_group', dict(group_size=256), (64, 1024)),
+    (8, True, 'per_channel', {}, (300, 4096)),
+    (8, False, 'per_channel', {}, (64, 11008)),
+    (4, False, 'per_channel', {}, (33, 1000)),       # 1000 % 8 == 0, % 16 != 0
+    (8, True, 'per_channel', {}, (17, 1001)),        # odd length -> element-wise kernel
+    (8, True, 'per_tensor', {}, (128, 512)),
+    (8, False, 'per_tensor', {}, (128, 512)),
+    (4, False, 'per_group', dict(group_size=128, round_zp=False), (64, 512)),
+    (6, True, 'per_head', dict(head_num=8), (64, 512)),
+]
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('bit,sym,gran,kw,shape', INT_CASES)
+def test_int_fake_and_real_quant_bit_exact(dev, dtype, bit, sym, gran, kw, shape):
+    w = weight_like(*shape, seed=bit + shape[0], dtype=dtype, outlier_frac=0.002)
+    spec = Q.IntSpec(bit, sym, gran, group_size=kw.get('group_size', 0), head_num=kw.get('head_num', 0),
+                     round_zp=kw.get('round_zp', True))
+    q = _iq(bit, sym, gran, **kw)
+    wd = w.to(dev)
+
+    assert_bit_equal(q.fake_quant_weight_dynamic(wd), Q.int_fake_quant_dynamic(spec, w), 'fake_quant_weight_dynamic')
+
+    rows, s, z, qmax, qmin = q.get_tensor_qparams(wd)
+    orows, os_, oz, _, _ = Q.int_tensor_qparams(spec, w)
+    assert tuple(rows.shape) == tuple(orows.shape)
+    assert_bit_equal(s, os_, 'scales')
+    if not sym:
+        assert_bit_equal(z, oz, 'zeros')
+
+    assert_bit_equal(q.quant(rows, s, z, qmax, qmin), Q.int_quant(spec, orows, os_, oz, spec.qmax, spec.qmin), 'quant')
+    assert_bit_equal(q.quant_dequant(rows, s, z, qmax, qmin),
+                     Q.int_quant_dequant(spec, orows, os_, oz, spec.qmax, spec.qmin), 'quant_dequant')
+
+    if kw.get('round_zp', True):
+        codes, rs, rz = q.real_quant_weight_dynamic(wd)
+        ocodes, ors, orz = Q.int_real_quant_dynamic(spec, w)
+        assert_bit_equal(codes, ocodes, 'codes')
+        assert_bit_equal(rs, ors, 'real scales')
+        assert (rz is None) == (orz is None)
+        if rz is not None:
+            assert_bit_equal(rz, orz, 'real zeros')
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+def test_int_static_paths_and_minmax(dev, dtype):
+    w = weight_like(128, 1024, seed=21, dtype=dtype)
+    spec = Q.IntSpec(4, False, 'per_group', group_size=128)
+    q = _iq(4, False, 'per_group', group_size=128)
+    orows, os_, oz, oqmax, oqmin = Q.int_tensor_qparams(spec, w)
+    # qparams from one tensor applied to another (static), with an output scale factor
+    w2 = weight_like(128, 1024, seed=22, dtype=dtype)
+    args = dict(scales=os_.to(dev), zeros=oz.to(dev), qmax=oqmax, qmin=oqmin, output_scale_factor=0.5)
+    got = q.fake_quant_weight_static(w2.to(dev), dict(args))
+    want = Q.int_fake_quant_static(spec, w2, os_, oz, oqmax, oqmin, output_scale_factor=0.5)
+    assert_bit_equal(got, want, 'fake_quant_weight_static')
+    codes, s, z = q.real_quant_weight_static(w2.to(dev), dict(args))
+    ocodes, os2, oz2 = Q.int_real_quant_static(spec, w2, os_, oz, oqmax, oqmin, output_scale_factor=0.5)
+    assert_bit_equal(codes, ocodes, 'static codes')
+    assert_bit_equal(s, os2, 'static scales')
+    assert_bit_equal(z, oz2, 'static zeros')
+    mn, mx = q.get_minmax_range(q.reshape_tensor(w.to(dev)))
+    omn, omx = Q.minmax_range(spec, orows)
+    assert_bit_equal(mn, omn, 'min'); assert_bit_equal(mx, omx, 'max')
+    s3, z3, _, _ = q.get_qparams((mn, mx), dev)
+    assert_bit_equal(s3, os_, 'get_qparams scales'); assert_bit_equal(z3, oz, 'get_qparams zeros')
+    dq = q.dequant(q.quant(q.reshape_tensor(w.to(dev)), s3, z3, oqmax, oqmin), s3, z3)
+    assert_bit_equal(dq, Q.int_dequant(Q.int_quant(spec, orows, os_, oz, oqmax, oqmin), os_, oz), 'dequant')
+    # activations: per-token rows of a 3-D tensor
+    act = (torch.randn(4, 64, 512, generator=gen(23)) * 3).to(dtype)
+    aq = _iq(8, True, 'per_token')
+    assert_bit_equal(aq.fake_quant_act_dynamic(act.to(dev)), Q.int_fake_quant_dynamic(Q.IntSpec(8, True, 'per_token'), act), 'act')
+
+
+def test_int_boundary_cases_hit_the_exact_division_path(dev):
+    """Inputs built to sit on and next to rounding ties (k + 0.5) * s."""
+    g = gen(31)
+    s = (torch.rand(512, 1, generator=g) * 0.01 + 1e-3)
+    k = torch.randint(0, 15, (512, 128), generator=g).float()
+    ulp = torch.randint(-2, 3, (512, 128), generator=g)
+    x = ((k + 0.5) * s)
+    x = (x.view(torch.int32) + ulp).view(torch.float32)
+    x[:, 0] = 0.0
+    x[:, 1] = s[:, 0] * 15                                   # pins min = 0 and max = 15 * s
+    for dtype in (torch.float32, torch.bfloat16):
+        xd = x.to(dtype)
+        spec = Q.IntSpec(4, False, 'per_group', group_size=128)
+        got = _iq(4, False, 'per_group', group_size=128).real_quant_weight_dynamic(xd.to(dev))
+        want = Q.int_real_quant_dynamic(spec, xd)
+        assert_bit_equal(got[0], want[0], f'tie codes {dtype}')
+        assert_bit_equal(got[1], want[1], f'tie scales {dtype}')
+
+
+def test_int_edge_shapes(dev):
+    q = _iq(4, False, 'per_group', group_size=128)
+    spec = Q.IntSpec(4, False, 'per_group', group_size=128)
+    # fewer columns than a group: one row-wise range (quant.py:613-631)
+    w = weight_like(8, 96, seed=41)
+    assert_bit_equal(q.fake_quant_weight_dynamic(w.to(dev)), Q.int_fake_quant_dynamic(spec, w), 'short rows')
+    # constant rows: the 1e-5 clamp decides the scale
+    w = torch.full((4, 128), 0.25)
+    assert_bit_equal(q.fake_quant_weight_dynamic(w.to(dev)), Q.int_fake_quant_dynamic(spec, w), 'constant rows')
+    w = torch.zeros(4, 128, dtype=torch.bfloat16)
+    assert_bit_equal(q.fake_quant_weight_dynamic(w.to(dev)), Q.int_fake_quant_dynamic(spec, w), 'zero rows')
+    # a single group, and a row count that does not fill a wave
+    w = weight_like(1, 128, seed=42)
+    assert_bit_equal(q.fake_quant_weight_dynamic(w.to(dev)), Q.int_fake_quant_dynamic(spec, w), 'one group')
+    w = weight_like(3, 640, seed=43, dtype=torch.bfloat16)
+    assert_bit_equal(q.fake_quant_weight_dynamic(w.to(dev)), Q.int_fake_quant_dynamic(spec, w), 'ragged')
+    # transposed view ('dim': 'ic')
+    w = weight_like(256, 64, seed=44)
+    got = q.fake_quant_weight_dynamic(w.to(dev), {'dim': 'ic'})
+    want = Q.int_fake_quant_dynamic(spec, w.T).T
+    assert_bit_equal(got.contiguous(), want.contiguous(), 'dim=ic')
+
+
+FP_CASES = [('e4m3', 'per_channel', (64, 7168)), ('e4m3', 'per_channel', (128, 2048)), ('e4m3', 'per_token', (96, 7168)),
+            ('e5m2', 'per_channel', (64, 1024)), ('e4m3', 'per_group', (64, 1024)), ('e4m3', 'per_tensor', (64, 512)),
+            ('e2m1', 'per_group', (64, 512)), ('e3m2', 'per_channel', (32, 520)), ('e4m3', 'per_channel', (9, 1003))]
+
+
+@pytest.mark.parametrize('tie', ['away', 'even'])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('fmt,gran,shape', FP_CASES)
+def test_float_quant_bit_exact(dev, tie, dtype, fmt, gran, shape):
+    from lightcompress_amd import FloatQuantizer
+    w = weight_like(*shape, seed=shape[1], dtype=dtype, std=0.006, outlier_frac=0.0005, outlier_mul=30)
+    w[0, :4] = torch.tensor([0.0, -0.0, 1e-9, -1e-9], dtype=dtype)      # zeros and deep subnormal-range values
+    kw = dict(group_size=128) if gran == 'per_group' else {}
+    spec = Q.FloatSpec(fmt, gran, group_size=kw.get('group_size', 0), tie=tie)
+    q = FloatQuantizer(fmt, True, gran, use_qtorch=True, fp_tie=tie, **kw)
+    wd = w.to(dev)
+    assert_bit_equal(q.fake_quant_weight_dynamic(wd), Q.float_fake_quant_dynamic(spec, w), 'float fake quant')
+    rows, s, z, qmax, qmin = q.get_tensor_qparams(wd)
+    orows, os_, oz, _, _ = Q.float_tensor_qparams(spec, w)
+    assert_bit_equal(s, os_, 'float scales')
+    assert_bit_equal(q.quant(rows, s.clone(), z, qmax, qmin), Q.float_quant(spec, orows, os_.clone(), oz), 'float quant')
+    want_dq = Q.float_dequant(Q.float_quant(spec, orows, os_.clone(), oz), os_, oz)
+    assert_bit_equal(q.quant_dequant(rows, s.clone(), z, qmax, qmin), want_dq, 'float quant_dequant')
+    if fmt in ('e4m3', 'e5m2'):
+        codes, rs, rz = q.real_quant_weight_dynamic(wd)
+        ocodes, ors, _ = Q.float_real_quant_dynamic(spec, w)
+        assert rz is None
+        assert_bit_equal(codes, ocodes, 'fp8 codes')
+        assert_bit_equal(rs, ors, 'fp8 scales')
+
+
+def test_float_act_fake_quant_3d(dev):
+    from lightcompress_amd import FloatQuantizer
+    act = (torch.randn(2, 48, 7168, generator=gen(51)) * torch.exp(torch.randn(7168, generator=gen(52)))).bfloat16()
+    q = FloatQuantizer('e4m3', True, 'per_token', use_qtorch=True)
+    assert_bit_equal(q.fake_quant_act_dynamic(act.to(dev)), Q.float_fake_quant_dynamic(Q.FloatSpec('e4m3', 'per_token'), act), 'fp8 act')
+
+
+@pytest.mark.parametrize('bits,dt', [(4, torch.int32), (8, torch.int8)])
+@pytest.mark.parametrize('shape', [(64, 4096), (7, 37), (128, 7168), (3, 8)])
+def test_pack_ct_bit_exact(dev, bits, dt, shape):
+    from lightcompress_amd.module_utils import VllmRealQuantLinear
+    lo = -(1 << (bits - 1))
+    codes = torch.randint(lo, -lo, shape, generator=gen(61), dtype=dt)
+    scales = torch.rand(shape[0], 1, generator=gen(62))
+    got, gs = VllmRealQuantLinear.pack(codes.to(dev), scales.to(dev), {'weight': {'bit': bits}})
+    want, ws = pack_ref.pack_ct(codes, scales, bits)
+    assert_bit_equal(got, want, 'packed'); assert_bit_equal(gs, ws, 'fp16 scales')
+    assert torch.equal(pack_ref.unpack_ct(got.cpu(), bits, shape[1]), codes.to(torch.int32))
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize('shape', [(64, 256), (320, 1024), (2048, 512)])
+def test_gemm_pack_bit_exact(dev, dtype, shape):
+    from lightcompress_amd.module_utils import AutoawqRealQuantLinear
+    w = weight_like(*shape, seed=71, dtype=dtype)
+    spec = Q.IntSpec(4, False, 'per_group', group_size=128)
+    _, s, z = Q.int_real_quant_dynamic(spec, w.float() if dtype == torch.float16 else w)
+    s = s.to(dtype)
+    cfg = {'weight': {'bit': 4, 'group_size': 128}}
+    got = AutoawqRealQuantLinear.gemm_pack(None, w.to(dev), s.to(dev), z.to(dev), cfg)
+    want = pack_ref.gemm_pack(w, s, z, 128)
+    for a, b, n in zip(got, want, ('qweight', 'scales', 'qzeros')):
+        assert_bit_equal(a, b, n)
+
+
+def test_full_size_rtn_properties(dev):
+    """BASELINE config 1 at full size, through size-independent properties."""
+    w = weight_like(4096, 4096, seed=0)
+    q = _iq(4, False, 'per_group', group_size=128)
+    wd = w.to(dev)
+    codes, s, z = q.real_quant_weight_dynamic(wd)
+    fq = q.fake_quant_weight_dynamic(wd)
+    assert codes.dtype == torch.int32 and int(codes.min()) == 0 and int(codes.max()) == 15
+    # dequantising the codes reproduces the fake-quantised weights exactly
+    dq = ((codes.view(-1, 128).float() - z.view(-1, 1).float()) * s.view(-1, 1)).view(4096, 4096)
+    assert torch.equal(dq, fq)
+    assert float((fq - wd).abs().max()) <= float(s.max()) * 0.5001
+    # idempotence: fake-quantising the result again is a fixed point of the codes
+    codes2, _, _ = q.real_quant_weight_static(fq, {'scales': s.view(-1, 1), 'zeros': z.view(-1, 1).float(), 'qmax': q.qmax, 'qmin': q.qmin})
+    assert torch.equal(codes2, codes)
+    # a 256-row slice against the oracle, bit for bit
+    spec = Q.IntSpec(4, False, 'per_group', group_size=128)
+    oc, os_, oz = Q.int_real_quant_dynamic(spec, w[1000:1256])
+    assert_bit_equal(codes[1000:1256], oc, 'slice codes'); assert_bit_equal(s[1000:1256], os_, 'slice scales')
