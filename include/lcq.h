@@ -47,6 +47,12 @@ extern "C" {
 #define LCQ_FLAG_TIE_EVEN 16      /* minifloat rounding: ties to even instead of away from zero */
 #define LCQ_FLAG_NO_SUBNORMALS 32 /* minifloat rounding: flush below the minimum normal */
 #define LCQ_FLAG_DQ_F32 64        /* lcq_quant_fp: write dq as fp32 instead of the input type */
+#define LCQ_FLAG_RANGE_BF16 128   /* lcq_qparams_int on fp32 I/O: (max-min) and the 1e-5 clamp act in bf16,
+                                     the rest in fp32 — torch's promotion when 0-dim bf16 ranges meet the
+                                     0-dim fp32 (qmax-qmin) of a per_tensor quantizer */
+#define LCQ_FLAG_SCALE_F32 256    /* STATIC only: `scales` / `zeros` hold fp32 even for bf16 rows and enter the
+                                     arithmetic unrounded (a 0-dim fp32 qparam next to a bf16 tensor); results
+                                     still round to the row type */
 
 /* errors */
 #define LCQ_OK 0
@@ -54,6 +60,7 @@ extern "C" {
 #define LCQ_EALIGN (-2)
 #define LCQ_EDTYPE (-3)
 #define LCQ_ELAUNCH (-4)
+#define LCQ_EWORKSPACE (-5)
 
 /* ---- integer quantizer -------------------------------------------------- */
 
@@ -115,6 +122,44 @@ int lcq_pack_ct(const void* codes, int code_dtype, int64_t R, int64_t K, int bit
  *  qweight [K, R/8] int32 ; scales_f16_out [K/g, R] fp16 ; qzeros [K/g, R/8] int32 ; R % 32 == 0 */
 int lcq_pack_awq(const void* w, int dtype, const void* scales, const int32_t* zeros, int64_t R, int64_t K, int group_size,
                  int32_t* qweight, void* scales_f16_out, int32_t* qzeros, void* stream);
+
+/* ---- GPTQ --------------------------------------------------------------- */
+
+/* GPTQ.add_batch, gptq.py:253-295:  H <- alpha*H + beta * X^T X  with
+ * alpha = n/(n+b), beta = 2/(n+b) (n = batches seen so far, b = batches in this call).
+ *  H [K, K] fp32; X [T, K] tokens x in_features of LCQ_BF16 | LCQ_F16, 16-byte aligned; K % 8 == 0.
+ * Only the 256x256 tiles on or above the diagonal are updated: call
+ * lcq_symmetrize before reading the lower triangle. alpha == 0 does not read H. */
+int lcq_hessian_accum(float* H, int64_t K, const void* X, int dtype, int64_t T, float alpha, float beta, void* stream);
+
+/* H[j][i] = H[i][j] for i < j. */
+int lcq_symmetrize(float* H, int64_t K, void* stream);
+
+/* Dead columns, act-order permutation, damping and the Cholesky chain of
+ * GPTQ.process_hessian_and_weights, gptq.py:139-141, 150-153, 169-174:
+ *   dead = diag(H)==0; H[dead,dead] = 1; W[:,dead] = 0; H = H[perm][:,perm];
+ *   H += percdamp*mean(diag H)*I; U = chol(cholesky_inverse(chol(H)), upper)
+ *  H [K,K] fp32, valid on and above the diagonal (its diagonal is rewritten for dead columns)
+ *  perm [K] int64 or NULL (identity); W [R,K] fp32 in ORIGINAL column order or NULL
+ *  U [K,K] fp32 out: upper triangular, zeros below the diagonal; U may alias H
+ *  status [1] int32 device word or NULL: 1 if a non-positive pivot was met (H not positive definite) */
+int64_t lcq_chol_inv_upper_workspace_bytes(int64_t K);
+int lcq_chol_inv_upper(float* H, int64_t K, const int64_t* perm, float percdamp, float* W, int64_t R, float* U,
+                       void* workspace, int64_t workspace_bytes, int* status, void* stream);
+
+/* One lazy-batch block of GPTQ.weight_transform, gptq.py:203-243 (columns i1 .. i1+count, count <= 128):
+ * per-group scale/zero refresh (search_column_qparams, :358-366), quantize-dequantize,
+ * tmp[:, i] = w, Losses[:, i], in-block error feedback; Err [R,128] receives Err1.
+ *  W, tmp, Losses [R,K] fp32; U [K,K] upper factor; scales / zeros [R,G] fp32
+ *  dynamic groups (default): group_size > 0, G >= ceil(K/group_size), qparams are written
+ *  LCQ_FLAG_STATIC: qparams are inputs; group of column c is gidx[c] (or c/group_size, or 0 if group_size == 0) */
+int lcq_gptq_block(float* W, float* tmp, float* Losses, float* Err, const float* U, int64_t R, int64_t K, int64_t i1,
+                   int count, int group_size, float qmin, float qmax, int flags, float* scales, float* zeros,
+                   const int32_t* gidx, int64_t G, void* stream);
+
+/* Deferred update of gptq.py:244:  W[:, i2:] -= Err[:, :i2-i1] @ U[i1:i2, i2:]  (fp32 MFMA). */
+int lcq_gptq_trailing(float* W, const float* Err, const float* U, int64_t R, int64_t K, int64_t i1, int64_t i2,
+                      void* stream);
 
 #ifdef __cplusplus
 }

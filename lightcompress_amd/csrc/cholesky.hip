@@ -1,0 +1,245 @@
+// Damped Cholesky chain of GPTQ for gfx950.
+//
+// Replaces, in GPTQ.process_hessian_and_weights (gptq.py:139-141, 150-153, 169-174):
+//   dead = diag(H) == 0; H[dead, dead] = 1; W[:, dead] = 0
+//   H = H[perm][:, perm]
+//   H += percdamp * mean(diag(H)) * I
+//   H = cholesky(H); H = cholesky_inverse(H); H = cholesky(H, upper=True)
+// The result U is upper triangular with U^T U = (H + damp I)^-1.
+//
+// Instead of three factorizations (4/3 K^3 flop) the chain is computed as
+//   J H J = L L^T  (J = index reversal, L lower)   ->   U = J L^-1 J,
+// one Cholesky plus one triangular inverse (2/3 K^3 flop): L^-1 lower with a
+// positive diagonal, reversed on both axes, is upper triangular and
+// (J L^-1 J)^T (J L^-1 J) = J (L L^T)^-1 J = H^-1, so it IS the unique upper
+// Cholesky factor of H^-1.
+//
+// Kernels
+//   diag_prep      diagonal scan: dead columns, mean(diag) -> damp
+//   build          gather  A[a][b] = H[p(K-1-a)][p(K-1-b)] (+damp on the diagonal), a >= b
+//   potrf_diag     128x128 diagonal block in LDS: L11 and L11^-1 (one workgroup)
+//   gemm_f32       fp32 MFMA: panel solve  A21 <- A21 L11^-T  and trailing  A22 -= A21 A21^T
+//   (batched)      triangular inverse by pairwise merging of inverted diagonal
+//                  blocks: [[A,0],[B,C]]^-1 = [[A^-1,0],[-C^-1 B A^-1, C^-1]]
+//   scatter        U[i][j] = Linv[K-1-i][K-1-j], j >= i; zeros below the diagonal
+#include "gemm_f32.h"
+#include "lcq_internal.h"
+
+namespace {
+using namespace lcq;
+
+constexpr int NB = 128;
+
+struct PrepScalars {
+  float damp;
+  int status;      // 0 ok, 1 non-positive pivot met
+};
+
+// one workgroup: dead-column fix on the diagonal, damp = percdamp * mean(diag)
+__global__ __launch_bounds__(1024) void diag_prep_kernel(float* __restrict__ H, int K, float percdamp,
+                                                         uint8_t* __restrict__ dead, PrepScalars* sc) {
+  __shared__ float part[16];
+  float s = 0.0f;
+  for (int j = threadIdx.x; j < K; j += 1024) {
+    float d = H[(long long)j * K + j];
+    const bool is_dead = (d == 0.0f);
+    if (is_dead) { d = 1.0f; H[(long long)j * K + j] = 1.0f; }
+    dead[j] = is_dead;
+    s += d;
+  }
+  s = team_sum<64>(s);
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float t = 0.0f;
+    for (int i = 0; i < 16; ++i) t += part[i];
+    sc->damp = percdamp * (t / (float)K);
+    sc->status = 0;
+  }
+}
+
+// W[:, dead] = 0
+__global__ __launch_bounds__(256) void apply_dead_kernel(float* __restrict__ W, long long R, int K,
+                                                         const uint8_t* __restrict__ dead) {
+  const long long n = R * K;
+  for (long long e = (long long)blockIdx.x * 256 + threadIdx.x; e < n; e += (long long)gridDim.x * 256)
+    if (dead[e % K]) W[e] = 0.0f;
+}
+
+// A (lower triangle, reversed + permuted + damped); strict upper triangle zeroed
+__global__ __launch_bounds__(256) void build_kernel(const float* __restrict__ H, int K, const long long* __restrict__ perm,
+                                                    const PrepScalars* __restrict__ sc, float* __restrict__ A) {
+  const int a = blockIdx.y;
+  const int b = blockIdx.x * 256 + threadIdx.x;
+  if (b >= K) return;
+  float v = 0.0f;
+  if (b <= a) {
+    long long i = K - 1 - a, j = K - 1 - b;
+    if (perm) { i = perm[i]; j = perm[j]; }
+    const long long lo = i < j ? i : j, hi = i < j ? j : i;     // H is valid on and above the diagonal
+    v = H[lo * K + hi];
+    if (a == b) v += sc->damp;
+  }
+  A[(long long)a * K + b] = v;
+}
+
+// diagonal block: Cholesky (left-looking) and inverse of the factor, all in LDS
+__global__ __launch_bounds__(256) void potrf_diag_kernel(float* __restrict__ Ablk, int lda, int nb,
+                                                         float* __restrict__ Dinv, PrepScalars* sc) {
+  __shared__ float Ls[NB * (NB + 1)];
+  __shared__ float Xs[NB * NB];
+  __shared__ float piv;
+  constexpr int P = NB + 1;
+  const int tid = threadIdx.x;
+  for (int e = tid; e < NB * NB; e += 256) {
+    const int r = e / NB, c = e % NB;
+    Ls[r * P + c] = (r < nb && c <= r) ? Ablk[(long long)r * lda + c] : 0.0f;
+    Xs[e] = 0.0f;
+  }
+  __syncthreads();
+  const int i = tid >> 1, half = tid & 1;
+  for (int j = 0; j < nb; ++j) {
+    float dot = 0.0f;
+    if (i >= j && i < nb)
+      for (int k = half; k < j; k += 2) dot += Ls[i * P + k] * Ls[j * P + k];
+    dot += lane_xor<1>(dot);
+    const float v = Ls[i * P + j] - dot;
+    if (i == j && half == 0) {
+      if (!(v > 0.0f)) sc->status = 1;
+      piv = sqrtf(v);
+    }
+    __syncthreads();
+    if (half == 0 && i < nb) {
+      if (i == j) Ls[i * P + j] = piv;
+      else if (i > j) Ls[i * P + j] = v / piv;
+    }
+    __syncthreads();
+  }
+  // X = L^-1, row by row: X[r][c] = (delta_rc - sum_{k<r} L[r][k] X[k][c]) / L[r][r]
+  const int c = tid >> 1;
+  for (int r = 0; r < nb; ++r) {
+    float dot = 0.0f;
+    if (c <= r)
+      for (int k = c + half; k < r; k += 2) dot += Ls[r * P + k] * Xs[k * NB + c];
+    dot += lane_xor<1>(dot);
+    if (half == 0 && c <= r) Xs[r * NB + c] = ((r == c ? 1.0f : 0.0f) - dot) / Ls[r * P + r];
+    __syncthreads();
+  }
+  for (int e = tid; e < NB * NB; e += 256) {
+    const int r = e / NB, cc = e % NB;
+    if (r < nb && cc < nb) Ablk[(long long)r * lda + cc] = (cc <= r) ? Ls[r * P + cc] : 0.0f;
+    Dinv[e] = Xs[e];
+  }
+}
+
+// copy the inverted diagonal blocks into place
+__global__ __launch_bounds__(256) void place_diag_kernel(float* __restrict__ A, int K, const float* __restrict__ Dinv) {
+  const int blk = blockIdx.x, k0 = blk * NB;
+  const int nb = min(NB, K - k0);
+  const float* D = Dinv + (long long)blk * NB * NB;
+  for (int e = threadIdx.x; e < NB * NB; e += 256) {
+    const int r = e / NB, c = e % NB;
+    if (r < nb && c < nb) A[(long long)(k0 + r) * K + k0 + c] = D[e];
+  }
+}
+
+__global__ __launch_bounds__(256) void scatter_kernel(const float* __restrict__ Linv, int K, float* __restrict__ U) {
+  const int i = blockIdx.y;
+  const int j = blockIdx.x * 256 + threadIdx.x;
+  if (j >= K) return;
+  U[(long long)i * K + j] = (j >= i) ? Linv[(long long)(K - 1 - i) * K + (K - 1 - j)] : 0.0f;
+}
+
+}  // namespace
+
+extern "C" {
+
+int64_t lcq_chol_inv_upper_workspace_bytes(int64_t K) {
+  const int64_t nblk = (K + NB - 1) / NB;
+  return K * K * 4 + nblk * NB * NB * 4 + ((K + 255) / 256) * 256 + 256;
+}
+
+int lcq_chol_inv_upper(float* H, int64_t K64, const int64_t* perm, float percdamp, float* W, int64_t R, float* U,
+                       void* workspace, int64_t workspace_bytes, int* status, void* stream) {
+  if (!H || !U || !workspace || K64 <= 0 || K64 > 65536 || R < 0) return LCQ_EINVAL;
+  if (workspace_bytes < lcq_chol_inv_upper_workspace_bytes(K64)) return LCQ_EWORKSPACE;
+  if (((uintptr_t)workspace % 16) != 0) return LCQ_EALIGN;
+  const int K = (int)K64;
+  const int nblk = (K + NB - 1) / NB;
+  hipStream_t st = (hipStream_t)stream;
+  float* A = (float*)workspace;
+  float* Dinv = A + (long long)K * K;
+  uint8_t* dead = (uint8_t*)(Dinv + (long long)nblk * NB * NB);
+  PrepScalars* sc = (PrepScalars*)(dead + ((K + 255) / 256) * 256);
+
+  diag_prep_kernel<<<dim3(1), dim3(1024), 0, st>>>(H, K, percdamp, dead, sc);
+  if (W && R > 0) {
+    long long g = ((long long)R * K + 255) / 256;
+    if (g > 65536) g = 65536;
+    apply_dead_kernel<<<dim3((unsigned)g), dim3(256), 0, st>>>(W, R, K, dead);
+  }
+  build_kernel<<<dim3((unsigned)((K + 255) / 256), (unsigned)K), dim3(256), 0, st>>>(H, K, (const long long*)perm, sc, A);
+
+  // blocked right-looking Cholesky
+  for (int b = 0; b < nblk; ++b) {
+    const int k0 = b * NB, nb = (K - k0 < NB) ? (K - k0) : NB;
+    float* Akk = A + (long long)k0 * K + k0;
+    float* Db = Dinv + (long long)b * NB * NB;
+    potrf_diag_kernel<<<dim3(1), dim3(256), 0, st>>>(Akk, K, nb, Db, sc);
+    const int M = K - k0 - nb;
+    if (M > 0) {
+      float* A21 = A + (long long)(k0 + nb) * K + k0;
+      float* A22 = A + (long long)(k0 + nb) * K + (k0 + nb);
+      launch_gemm<true>(GemmProblem{A21, Db, A21, M, nb, nb, K, NB, K}, 1.0f, 0.0f, 0, st);       // A21 L11^-T
+      launch_gemm<true>(GemmProblem{A21, A21, A22, M, M, nb, K, K, K}, -1.0f, 1.0f, GEMM_LOWER_TILES, st);
+    }
+  }
+
+  // triangular inverse: inverted diagonal blocks, then pairwise merges
+  place_diag_kernel<<<dim3((unsigned)nblk), dim3(256), 0, st>>>(A, K, Dinv);
+  int nseg = nblk;
+  int seg_start[512], seg_size[512];
+  if (nblk > 512) return LCQ_EINVAL;
+  for (int b = 0; b < nblk; ++b) { seg_start[b] = b * NB; seg_size[b] = (K - b * NB < NB) ? (K - b * NB) : NB; }
+  float* T = U;                                  // scratch until the final scatter
+  while (nseg > 1) {
+    const int npairs = nseg / 2;
+    for (int p0 = 0; p0 < npairs; p0 += GEMM_MAX_BATCH) {
+      const int np = (npairs - p0 < GEMM_MAX_BATCH) ? (npairs - p0) : GEMM_MAX_BATCH;
+      GemmBatch b1, b2;
+      int maxM = 0, maxN = 0;
+      for (int q = 0; q < np; ++q) {
+        const int sa = seg_start[2 * (p0 + q)], na = seg_size[2 * (p0 + q)];
+        const int sc_ = seg_start[2 * (p0 + q) + 1], nc = seg_size[2 * (p0 + q) + 1];
+        const long long offBlk = (long long)sc_ * K + sa;          // B block (rows of C-part, cols of A-part)
+        // T1 = B * Ainv
+        b1.offA[q] = offBlk; b1.offB[q] = (long long)sa * K + sa; b1.offC[q] = offBlk;
+        b1.M[q] = nc; b1.N[q] = na; b1.Kc[q] = na;
+        // X = -Cinv * T1
+        b2.offA[q] = (long long)sc_ * K + sc_; b2.offB[q] = offBlk; b2.offC[q] = offBlk;
+        b2.M[q] = nc; b2.N[q] = na; b2.Kc[q] = nc;
+        if (nc > maxM) maxM = nc;
+        if (na > maxN) maxN = na;
+      }
+      const dim3 grid((unsigned)((maxN + GT - 1) / GT), (unsigned)((maxM + GT - 1) / GT), (unsigned)np);
+      gemm_f32_batched_kernel<false><<<grid, dim3(256), 0, st>>>(A, K, A, K, T, K, b1, 1.0f, 0.0f, GEMM_K_FROM_N);
+      gemm_f32_batched_kernel<false><<<grid, dim3(256), 0, st>>>(A, K, T, K, A, K, b2, -1.0f, 0.0f, GEMM_K_TO_M);
+    }
+    int w = 0;
+    for (int p = 0; p < npairs; ++p) {
+      seg_start[w] = seg_start[2 * p];
+      seg_size[w] = seg_size[2 * p] + seg_size[2 * p + 1];
+      ++w;
+    }
+    if (nseg & 1) { seg_start[w] = seg_start[nseg - 1]; seg_size[w] = seg_size[nseg - 1]; ++w; }
+    nseg = w;
+  }
+
+  scatter_kernel<<<dim3((unsigned)((K + 255) / 256), (unsigned)K), dim3(256), 0, st>>>(A, K, U);
+  if (status)
+    (void)hipMemcpyAsync(status, &sc->status, sizeof(int), hipMemcpyDeviceToDevice, st);
+  LCQ_CHECK_LAUNCH();
+  return LCQ_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,208 @@
+// fp32 MFMA GEMM building block for gfx950 (v_mfma_f32_32x32x2f32), used by the
+// blocked Cholesky / triangular-inverse chain and by GPTQ's deferred rank-128
+// update.  Plain fp32 in, fp32 accumulate: no reduced-precision tricks, the
+// GPTQ code agreement depends on it.
+//
+//   C[M x N] = alpha * A[M x Kc] * op(B) + beta * C
+//     A is row-major with the contraction index contiguous;
+//     B_T  : B is [N x Kc] row-major (contraction contiguous)   -> A * B^T
+//     !B_T : B is [Kc x N] row-major (output column contiguous) -> A * B
+//
+// One 256-thread workgroup per 128x128 tile of C, four waves of 64x64 (2x2 MFMA
+// blocks each), contraction staged 32 at a time through LDS.  LDS pitches are
+// chosen so that the 32 lanes that read one operand column hit 32 banks.
+//
+// Triangular structure is exploited by clipping the contraction range per
+// tile (GEMM_K_FROM_N / GEMM_K_TO_M) and by skipping tiles above the diagonal
+// (GEMM_LOWER_TILES).  Batched launches take per-problem offsets from
+// GemmBatch (blockIdx.z).
+#pragma once
+#include "common.h"
+
+namespace lcq {
+
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+constexpr int GT = 128;            // C tile edge
+constexpr int GK = 32;             // contraction slab
+constexpr int GPA = GK + 1;        // pitch of a [rows][k] operand tile (floats)
+constexpr int GPB = GT + 32;       // pitch of a [k][cols] operand tile (floats)
+
+enum : int {
+  GEMM_LOWER_TILES = 1,   // only tiles with n0 <= m0 (C symmetric / lower triangular)
+  GEMM_K_FROM_N = 2,      // B is lower triangular [k][n]: terms with k < n0 vanish
+  GEMM_K_TO_M = 4,        // A is lower triangular [m][k]: terms with k >= m0 + GT vanish
+};
+
+struct GemmProblem {
+  const float* A; const float* B; float* C;
+  int M, N, Kc;
+  int lda, ldb, ldc;
+};
+
+constexpr int GEMM_MAX_BATCH = 64;
+struct GemmBatch {
+  // element offsets added to the base pointers, and per-problem sizes
+  long long offA[GEMM_MAX_BATCH], offB[GEMM_MAX_BATCH], offC[GEMM_MAX_BATCH];
+  int M[GEMM_MAX_BATCH], N[GEMM_MAX_BATCH], Kc[GEMM_MAX_BATCH];
+};
+
+template <bool B_T>
+__device__ __forceinline__ void gemm_tile(const float* A, int lda, const float* B, int ldb,
+                                          float* C, int ldc, int M, int N, int Kc, float alpha, float beta,
+                                          int flags, int m0, int n0, float* sA, float* sB) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wr = wave >> 1, wc = wave & 1;
+
+  int kb = 0, ke = Kc;
+  if (flags & GEMM_K_FROM_N) kb = (n0 / GK) * GK;
+  if (flags & GEMM_K_TO_M) ke = min(Kc, m0 + GT);
+
+  f32x16 acc[2][2];
+  #pragma unroll
+  for (int i = 0; i < 2; ++i)
+    #pragma unroll
+    for (int j = 0; j < 2; ++j)
+      #pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  // staging registers: A tile 128 x 32 floats = 1024 float4 -> 4 per thread; B likewise
+  f32x4 ra[4], rb[4];
+  auto gload = [&](int k0) {
+    #pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int idx = p * 256 + tid;
+      {   // A: row = idx / 8, k4 = idx % 8
+        const int r = idx >> 3, k = k0 + (idx & 7) * 4;
+        const int gm = m0 + r;
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+        if (gm < M) {
+          const float* p0 = A + (long long)gm * lda + k;
+          if (k + 3 < ke && ((((uintptr_t)p0) & 15) == 0)) v = *(const f32x4*)p0;
+          else {
+            #pragma unroll
+            for (int e = 0; e < 4; ++e) if (k + e < ke) v[e] = p0[e];
+          }
+        }
+        ra[p] = v;
+      }
+      if constexpr (B_T) {   // B[n][k]: same shape as A
+        const int r = idx >> 3, k = k0 + (idx & 7) * 4;
+        const int gn = n0 + r;
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+        if (gn < N) {
+          const float* p0 = B + (long long)gn * ldb + k;
+          if (k + 3 < ke && ((((uintptr_t)p0) & 15) == 0)) v = *(const f32x4*)p0;
+          else {
+            #pragma unroll
+            for (int e = 0; e < 4; ++e) if (k + e < ke) v[e] = p0[e];
+          }
+        }
+        rb[p] = v;
+      } else {               // B[k][n]: k = idx / 32, n4 = idx % 32
+        const int k = k0 + (idx >> 5), n = n0 + (idx & 31) * 4;
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+        if (k < ke) {
+          const float* p0 = B + (long long)k * ldb + n;
+          if (n + 3 < N && ((((uintptr_t)p0) & 15) == 0)) v = *(const f32x4*)p0;
+          else {
+            #pragma unroll
+            for (int e = 0; e < 4; ++e) if (n + e < N) v[e] = p0[e];
+          }
+        }
+        rb[p] = v;
+      }
+    }
+  };
+  auto lstore = [&]() {
+    #pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int idx = p * 256 + tid;
+      {
+        const int r = idx >> 3, k = (idx & 7) * 4;
+        #pragma unroll
+        for (int e = 0; e < 4; ++e) sA[r * GPA + k + e] = ra[p][e];
+      }
+      if constexpr (B_T) {
+        const int r = idx >> 3, k = (idx & 7) * 4;
+        #pragma unroll
+        for (int e = 0; e < 4; ++e) sB[r * GPA + k + e] = rb[p][e];
+      } else {
+        const int k = idx >> 5, n = (idx & 31) * 4;
+        *(f32x4*)(sB + k * GPB + n) = rb[p];
+      }
+    }
+  };
+
+  const int lm = lane & 31, lk = lane >> 5;
+  if (kb < ke) gload(kb);
+  for (int k0 = kb; k0 < ke; k0 += GK) {
+    __syncthreads();                       // previous slab fully consumed
+    lstore();
+    __syncthreads();
+    if (k0 + GK < ke) gload(k0 + GK);      // next slab in flight while this one is multiplied
+    #pragma unroll
+    for (int kk = 0; kk < GK; kk += 2) {
+      float a[2], b[2];
+      #pragma unroll
+      for (int i = 0; i < 2; ++i) a[i] = sA[(wr * 64 + i * 32 + lm) * GPA + kk + lk];
+      #pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if constexpr (B_T) b[j] = sB[(wc * 64 + j * 32 + lm) * GPA + kk + lk];
+        else b[j] = sB[(kk + lk) * GPB + wc * 64 + j * 32 + lm];
+      }
+      #pragma unroll
+      for (int i = 0; i < 2; ++i)
+        #pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+  }
+
+  // accumulator register r of lane l: row 8*(r/4) + 4*(l/32) + r%4, column l%32
+  #pragma unroll
+  for (int i = 0; i < 2; ++i)
+    #pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int gn = n0 + wc * 64 + j * 32 + lm;
+      #pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int gm = m0 + wr * 64 + i * 32 + 8 * (r >> 2) + 4 * lk + (r & 3);
+        if (gm < M && gn < N) {
+          float* p = C + (long long)gm * ldc + gn;
+          const float v = alpha * acc[i][j][r];
+          *p = (beta != 0.0f) ? (beta * *p + v) : v;
+        }
+      }
+    }
+}
+
+template <bool B_T>
+__global__ __launch_bounds__(256) void gemm_f32_kernel(GemmProblem g, float alpha, float beta, int flags) {
+  __shared__ float sA[GT * GPA];
+  __shared__ float sB[B_T ? GT * GPA : GK * GPB];
+  const int m0 = blockIdx.y * GT, n0 = blockIdx.x * GT;
+  if ((flags & GEMM_LOWER_TILES) && n0 > m0) return;
+  gemm_tile<B_T>(g.A, g.lda, g.B, g.ldb, g.C, g.ldc, g.M, g.N, g.Kc, alpha, beta, flags, m0, n0, sA, sB);
+}
+
+template <bool B_T>
+__global__ __launch_bounds__(256) void gemm_f32_batched_kernel(const float* A, int lda, const float* B, int ldb, float* C,
+                                                               int ldc, GemmBatch bt, float alpha, float beta, int flags) {
+  __shared__ float sA[GT * GPA];
+  __shared__ float sB[B_T ? GT * GPA : GK * GPB];
+  const int z = blockIdx.z;
+  const int m0 = blockIdx.y * GT, n0 = blockIdx.x * GT;
+  if (m0 >= bt.M[z] || n0 >= bt.N[z]) return;
+  gemm_tile<B_T>(A + bt.offA[z], lda, B + bt.offB[z], ldb, C + bt.offC[z], ldc, bt.M[z], bt.N[z], bt.Kc[z], alpha, beta,
+                 flags, m0, n0, sA, sB);
+}
+
+template <bool B_T>
+inline void launch_gemm(const GemmProblem& g, float alpha, float beta, int flags, hipStream_t st) {
+  if (g.M <= 0 || g.N <= 0) return;
+  const dim3 grid((unsigned)((g.N + GT - 1) / GT), (unsigned)((g.M + GT - 1) / GT));
+  gemm_f32_kernel<B_T><<<grid, dim3(256), 0, st>>>(g, alpha, beta, flags);
+}
+
+}  // namespace lcq

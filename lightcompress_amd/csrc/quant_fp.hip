@@ -21,7 +21,7 @@ namespace {
 using namespace lcq;
 
 struct FpRow {
-  float s, r;
+  float s, r, sm;   // divisor, its reciprocal, multiplier of the dequantization
   int fast;
 };
 
@@ -31,7 +31,7 @@ struct FpOp {
   using Row = FpRow;
   float qmax;
   int e_bits, m_bits, tie_even, subnormals;
-  int is_static, scalar_qp, dq_f32, code_dtype;
+  int is_static, scalar_qp, dq_f32, code_dtype, scale_f32;
   // derived
   uint32_t half, keep, max_mag;
   int drop, min_exp, max_exp;
@@ -40,6 +40,7 @@ struct FpOp {
   __device__ __forceinline__ Row finish(float s) const {
     Row p;
     if (s == 0.0f) s = 1.0f;                               // scales[scales == 0] = 1, quant.py:1061
+    p.sm = s;
     p.s = s;
     p.r = 1.0f / s;
     const float a = fabsf(s);
@@ -54,7 +55,8 @@ struct FpOp {
     return finish(rnd<BF>(a / qmax));
   }
   __device__ __forceinline__ Row load(const void* scales, const void*, int64_t row) const {
-    return finish(load_scalar<BF>(scales, scalar_qp ? 0 : row));
+    const int64_t i = scalar_qp ? 0 : row;
+    return finish(scale_f32 ? ((const float*)scales)[i] : load_scalar<BF>(scales, i));
   }
   __device__ __forceinline__ void store_qp(void* scales, void*, int64_t row, const Row& p) const {
     store_scalar<BF>(scales, row, p.s);
@@ -111,7 +113,7 @@ struct FpOp {
 
   // (q - 0.0) * s in fp32, then the cast of fake_quant_* (quant.py:1107,1153)
   __device__ __forceinline__ float deq(float q, const Row& p) const {
-    const float d = (q - 0.0f) * p.s;
+    const float d = (q - 0.0f) * p.sm;
     return dq_f32 ? d : rnd_e<BF>(d);
   }
 
@@ -144,6 +146,7 @@ FpOp<BF> make_op(int e_bits, int m_bits, float qmax, int flags, int code_dtype) 
   c.is_static = (flags & LCQ_FLAG_STATIC) != 0;
   c.scalar_qp = (flags & LCQ_FLAG_SCALAR_QP) != 0;
   c.dq_f32 = (flags & LCQ_FLAG_DQ_F32) != 0;
+  c.scale_f32 = (flags & LCQ_FLAG_SCALE_F32) != 0;
   c.code_dtype = code_dtype;
   c.drop = 23 - m_bits;
   c.half = 1u << (c.drop - 1);
@@ -182,6 +185,7 @@ int lcq_quant_fp(const void* x, int dtype, int64_t rows, int64_t cols, int e_bit
     } else if (code_dtype != LCQ_CODE_F32) return LCQ_EDTYPE;
   } else code_dtype = LCQ_CODE_NONE;
   if ((flags & LCQ_FLAG_SCALAR_QP) && !(flags & LCQ_FLAG_STATIC)) return LCQ_EINVAL;
+  if ((flags & LCQ_FLAG_SCALE_F32) && !(flags & LCQ_FLAG_STATIC)) return LCQ_EINVAL;
   hipStream_t st = (hipStream_t)stream;
   int rc;
   if (dtype == LCQ_F32)

@@ -34,7 +34,7 @@ struct IntOp {
   static constexpr bool BF = BF_;
   using Row = IntRow;
   float qmin, qmax, qrange, osf;
-  int sym, round_zp, is_static, scalar_qp, dq_f32, code_dtype;
+  int sym, round_zp, is_static, scalar_qp, dq_f32, code_dtype, range_bf16, scale_f32;
 
   __device__ __forceinline__ Row finish(float s, float z) const {
     Row p;
@@ -42,13 +42,13 @@ struct IntOp {
     p.r = 1.0f / s;
     const float a = fabsf(s);
     p.fast = (a > 8.6736174e-19f) && (a < 1.1529215e18f);   // 2^-60 .. 2^60
-    p.sdq = rnd<BF>(s * osf);
+    p.sdq = scale_f32 ? s * osf : rnd<BF>(s * osf);
     return p;
   }
 
   // get_qparams, quant.py:544-558
   __device__ __forceinline__ Row make(float mn, float mx) const {
-    const float cmin = BF ? 1.0013580322265625e-05f : 1e-5f;     // clamp(min=1e-5) in the tensor dtype
+    const float cmin = (BF || range_bf16) ? 1.0013580322265625e-05f : 1e-5f;   // clamp(min=1e-5) in the range dtype
     float s, z;
     if (sym) {
       float a = nan_max(fabsf(mx), fabsf(mn));
@@ -57,6 +57,7 @@ struct IntOp {
       z = 0.0f;
     } else {
       float d = rnd<BF>(mx - mn);
+      if (range_bf16) d = bf16_round(d);
       d = clamp_min_nan(d, cmin);
       s = rnd<BF>(d / qrange);
       const float t = rnd<BF>(mn / s);
@@ -72,6 +73,7 @@ struct IntOp {
 
   __device__ __forceinline__ Row load(const void* scales, const void* zeros, int64_t row) const {
     const int64_t i = scalar_qp ? 0 : row;
+    if (scale_f32) return finish(((const float*)scales)[i], zeros ? ((const float*)zeros)[i] : 0.0f);
     const float s = load_scalar<BF>(scales, i);
     const float z = zeros ? load_scalar<BF>(zeros, i) : 0.0f;
     return finish(s, z);
@@ -130,6 +132,8 @@ Op make_op(float qmin, float qmax, int flags, float osf, int code_dtype) {
   c.is_static = (flags & LCQ_FLAG_STATIC) != 0;
   c.scalar_qp = (flags & LCQ_FLAG_SCALAR_QP) != 0;
   c.dq_f32 = 0;
+  c.range_bf16 = (flags & LCQ_FLAG_RANGE_BF16) != 0;
+  c.scale_f32 = (flags & LCQ_FLAG_SCALE_F32) != 0;
   c.code_dtype = code_dtype;
   return c;
 }
@@ -201,14 +205,14 @@ __global__ void qparams_kernel(const void* __restrict__ mn, const void* __restri
 template <bool BF>
 __global__ __launch_bounds__(256) void dequant_kernel(const void* __restrict__ q, int64_t rows, int64_t cols,
                                                       const void* __restrict__ scales, const void* __restrict__ zeros,
-                                                      void* __restrict__ out, int scalar_qp, float osf) {
+                                                      void* __restrict__ out, int scalar_qp, int scale_f32, float osf) {
   const int64_t n = rows * cols;
   for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n; e += (int64_t)gridDim.x * 256) {
     const int64_t row = scalar_qp ? 0 : e / cols;
-    const float s = load_scalar<BF>(scales, row);
-    const float z = zeros ? load_scalar<BF>(zeros, row) : 0.0f;
+    const float s = scale_f32 ? ((const float*)scales)[row] : load_scalar<BF>(scales, row);
+    const float z = !zeros ? 0.0f : (scale_f32 ? ((const float*)zeros)[row] : load_scalar<BF>(zeros, row));
     const float d = rnd<BF>(load_scalar<BF>(q, e) - z);
-    store_scalar<BF>(out, e, rnd<BF>(d * rnd<BF>(s * osf)));
+    store_scalar<BF>(out, e, rnd<BF>(d * (scale_f32 ? s * osf : rnd<BF>(s * osf))));
   }
 }
 
@@ -225,6 +229,7 @@ int lcq_quant_int(const void* x, int dtype, int64_t rows, int64_t cols, float qm
                  code_dtype == LCQ_CODE_SAME)) return LCQ_EDTYPE;
   if (!(qmax > qmin)) return LCQ_EINVAL;
   if ((flags & LCQ_FLAG_SCALAR_QP) && !(flags & LCQ_FLAG_STATIC)) return LCQ_EINVAL;
+  if ((flags & LCQ_FLAG_SCALE_F32) && !(flags & LCQ_FLAG_STATIC)) return LCQ_EINVAL;
   if (!codes) code_dtype = LCQ_CODE_NONE;
   hipStream_t st = (hipStream_t)stream;
   int rc;
@@ -289,11 +294,12 @@ int lcq_dequant_int(const void* q, int dtype, int64_t rows, int64_t cols, const 
   if (!q || !scales || !out || rows < 0 || cols <= 0) return LCQ_EINVAL;
   if (rows == 0) return LCQ_OK;
   const int scalar_qp = (flags & LCQ_FLAG_SCALAR_QP) != 0;
+  const int scale_f32 = (flags & LCQ_FLAG_SCALE_F32) != 0;
   int64_t grid = (rows * cols + 255) / 256;
   if (grid > 65536) grid = 65536;
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == LCQ_F32) dequant_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>(q, rows, cols, scales, zeros, out, scalar_qp, out_scale_factor);
-  else if (dtype == LCQ_BF16) dequant_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>(q, rows, cols, scales, zeros, out, scalar_qp, out_scale_factor);
+  if (dtype == LCQ_F32) dequant_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>(q, rows, cols, scales, zeros, out, scalar_qp, scale_f32, out_scale_factor);
+  else if (dtype == LCQ_BF16) dequant_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>(q, rows, cols, scales, zeros, out, scalar_qp, scale_f32, out_scale_factor);
   else return LCQ_EDTYPE;
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;

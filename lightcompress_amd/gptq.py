@@ -1,0 +1,328 @@
+"""GPTQ with the reference's method surface, running on liblcq.
+
+Mirrors ``llmc/compression/quantization/gptq.py`` of ModelTC/LightCompress
+(class ``GPTQ``): ``layer_init`` / ``add_batch`` (Hessian accumulation,
+gptq.py:253-308), ``hessian_sorting`` (:58-64), ``process_hessian_and_weights``
+(:128-176), ``weight_transform`` (:198-244, upstream GPTQ's "fasterquant"),
+``update_layer_with_transformed_weights`` (:178-196), ``layer_transform``,
+``subset_transform``, ``w_q`` / ``w_qdq`` (:411-452) and the qparam bookkeeping
+(:332-409).  The model walk (blocks, hooks, deploy) of the reference's base
+class is not part of this path: a "layer" here is any object with a
+``weight`` tensor (an ``nn.Linear``).
+
+Differences a caller can observe
+  * one process / one GPU: the per-call all-reduce of add_batch is not issued;
+  * H is kept valid on and above the diagonal only while it accumulates
+    (``hessian(name)`` returns the full symmetric matrix);
+  * per-group qparams of the loop live in two [R, G] tensors instead of a
+    Python list of dicts; ``layer.buf_scales`` / ``buf_zeros`` get the same
+    [R*G, 1] layout the reference writes;
+  * OWQ (outlier columns kept in fp16) is not carried over.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import _lib as L
+from .quant import IntegerQuantizer
+
+
+class GPTQ:
+    def __init__(self, quant_config, model_dtype=torch.bfloat16, wquantizer=None):
+        self.quant_config = quant_config
+        self.dev = torch.device('cuda')
+        self.model_dtype = model_dtype
+        wcfg = dict(quant_config['weight'])
+        self.wquantizer = wquantizer or IntegerQuantizer(**wcfg)
+        self.add_quant_config()
+        self.layers_cache = {}
+        self.qparams = {}
+        self._shared = {}          # leader name -> dict(U=..., perm=..., invperm=..., status=...)
+
+    # -- configuration (gptq.py:33-56) ---------------------------------------
+    def add_quant_config(self):
+        special_config = self.quant_config['special']
+        self.true_sequential = special_config.get('true_sequential', True)
+        self.static_groups = special_config['static_groups']
+        self.actorder = special_config['actorder']
+        self.percdamp = special_config['percdamp']
+        self.blocksize = special_config['blocksize']
+        self.owq = special_config.get('owq', False)
+        self.chunk_num = special_config.get('chunk_num', 1)
+        self.check_positive_definite = special_config.get('check_positive_definite', True)
+        if self.owq:
+            raise NotImplementedError('OWQ is not on this path')
+        if self.blocksize > 128:
+            raise NotImplementedError('blocksize above 128 is not supported by the column-loop kernel')
+        self.need_perm = (
+            self.wquantizer.granularity == 'per_group'
+            and not self.static_groups
+            and self.actorder
+        )
+
+    # -- Hessian (gptq.py:253-308) ---------------------------------------------
+    @torch.no_grad()
+    def layer_init(self, layer, name):
+        W = layer.weight.data
+        K = W.shape[1] if W.dim() == 2 else W.flatten(1).shape[1]
+        self.layers_cache.setdefault(name, {})
+        self.layers_cache[name]['H'] = torch.zeros((K, K), device=self.dev)
+        self.layers_cache[name]['nsamples'] = 0
+        self.layers_cache[name]['columns'] = K
+        self.layers_cache[name].pop('leader', None)
+
+    @torch.no_grad()
+    def subset_init(self, subset):
+        self.named_layers = subset['layers']
+        for name in self.named_layers:
+            self.layers_cache[name] = {}
+            self.layer_init(self.named_layers[name], name)
+
+    def share_input(self, names):
+        """Layers that see the same input (q/k/v, gate/up) may share one Hessian and one
+        Cholesky chain: the first name accumulates, the others alias it."""
+        leader = names[0]
+        for n in names[1:]:
+            self.layers_cache[n]['H'] = self.layers_cache[leader]['H']
+            self.layers_cache[n]['leader'] = leader
+        self.layers_cache[leader]['leader'] = leader
+
+    @torch.no_grad()
+    def add_batch(self, layer, name, inp, out=None):
+        cache = self.layers_cache[name]
+        if cache.get('leader', name) != name:
+            return                                      # aliased: the leader accumulates
+        if len(inp.shape) == 2:
+            inp = inp.unsqueeze(0)
+        tmp = inp.shape[0]
+        if len(inp.shape) == 3:
+            inp = inp.reshape((-1, inp.shape[-1]))
+        if inp.dtype not in (torch.bfloat16, torch.float16):
+            raise NotImplementedError(f'add_batch streams bf16/fp16 activations through MFMA; got {inp.dtype}')
+        assert inp.shape[0] % self.chunk_num == 0, \
+            f'Error: inp.shape[1] ({inp.shape[0]}) cannot be evenly divided by chunk_num.'
+        x = inp.contiguous()
+        n = cache['nsamples']
+        alpha = n / (n + tmp)
+        cache['nsamples'] = n + tmp
+        beta = 2.0 / cache['nsamples']
+        H = cache['H']
+        L.check(L.lib().lcq_hessian_accum(L.ptr(H), L.i64(H.shape[0]), L.ptr(x), L.i32(L.dtype_code(x.dtype)),
+                                          L.i64(x.shape[0]), L.f32(alpha), L.f32(beta), L.stream()),
+                'lcq_hessian_accum')
+        cache['upper_only'] = True
+
+    def hessian(self, name):
+        """The full symmetric H of a layer (fills the lower triangle on demand)."""
+        cache = self.layers_cache[name]
+        H = cache['H']
+        if cache.get('upper_only', False) or self.layers_cache.get(cache.get('leader', name), {}).get('upper_only'):
+            L.check(L.lib().lcq_symmetrize(L.ptr(H), L.i64(H.shape[0]), L.stream()), 'lcq_symmetrize')
+            cache['upper_only'] = False
+        return H
+
+    def hessian_sorting(self, name):
+        """gptq.py:58-64: act-order permutation from the raw diagonal."""
+        H = self.layers_cache[name]['H']
+        if self.actorder:
+            self.perm = torch.argsort(torch.diag(H), descending=True)
+
+    # -- per-layer driver (gptq.py:96-196) -----------------------------------------
+    @torch.no_grad()
+    def subset_transform(self, subset, input_feat=None, subset_kwargs=None):
+        layers_dict = subset['layers']
+        for name in layers_dict:
+            self.layer_transform(layers_dict[name], name)
+            self.free(name)
+
+    @torch.no_grad()
+    def layer_transform(self, layer, name):
+        self.initialize_qparams_and_prepare_weights(layer, name)
+        W, H = self.process_hessian_and_weights(layer, name)
+        self.update_layer_with_transformed_weights(layer, W, H, name)
+
+    def initialize_qparams_and_prepare_weights(self, layer, name):
+        self.qparams = {}
+        self.columns = self.layers_cache[name]['columns']
+        self.n_out = 0
+        self.n_nonout = self.columns
+        cache = self.layers_cache[name]
+        leader = cache.get('leader', name)
+        if leader in self._shared:
+            self.perm = self._shared[leader].get('perm')
+        elif self.actorder:
+            self.hessian_sorting(name)
+
+    def process_hessian_and_weights(self, layer, name):
+        """-> (W [R,K] fp32 in processing order, Hinv: upper factor of the damped inverse)."""
+        W = layer.weight.data.clone()
+        if W.dim() > 2:
+            W = W.flatten(1)
+        W = W.float().contiguous()
+        R, K = W.shape
+        cache = self.layers_cache[name]
+        leader = cache.get('leader', name)
+        H = cache['H']
+        del cache['H']
+
+        self._setup_groups(layer, R, K)
+
+        is_shared = any(c.get('leader') == leader for n, c in self.layers_cache.items() if n != name) \
+            or leader != name
+        shared = self._shared.get(leader)
+        if shared is None:
+            perm = self.perm if self.actorder else None
+            # followers of a shared chain need the dead-column mask after H is gone
+            dead = (torch.diag(H) == 0) if is_shared else None
+            ws_bytes = L.lib().lcq_chol_inv_upper_workspace_bytes(L.i64(K))
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=self.dev)
+            status = torch.zeros(1, dtype=torch.int32, device=self.dev)
+            L.check(L.lib().lcq_chol_inv_upper(L.ptr(H), L.i64(K), L.ptr(perm), L.f32(self.percdamp), L.ptr(W),
+                                               L.i64(R), L.ptr(H), L.ptr(ws), L.i64(ws_bytes), L.ptr(status),
+                                               L.stream()), 'lcq_chol_inv_upper')
+            del ws
+            shared = dict(U=H, perm=perm, status=status, dead=dead)
+            if is_shared:
+                self._shared[leader] = shared
+        else:
+            W.masked_fill_(shared['dead'].unsqueeze(0), 0.0)
+        U = shared['U']
+        self._status = shared['status']
+
+        if self.actorder:
+            W = W[:, self.perm].contiguous()
+            self.invperm = torch.argsort(self.perm)
+            layer.buf_perm = self.perm
+            layer.buf_invperm = self.invperm
+        return W, U
+
+    def _setup_groups(self, layer, R, K):
+        """Storage of the loop's qparams: [R, G] scales / zeros (+ column -> group map when static)."""
+        wq = self.wquantizer
+        self._gidx = None
+        if wq.granularity == 'per_group':
+            g = wq.group_size
+            G = math.ceil(K / g)
+            self._g, self._G = g, G
+            if self.static_groups:
+                self._scales = layer.buf_scales.reshape(R, G).float().contiguous()
+                self._zeros = None if wq.sym else layer.buf_zeros.reshape(R, G).float().contiguous()
+                cols = torch.arange(K, device=self.dev)
+                if self.actorder:
+                    cols = self.perm
+                self._gidx = (cols // g).to(torch.int32).contiguous()
+                self._static = True
+            else:
+                self._scales = torch.empty((R, G), device=self.dev)
+                self._zeros = None if wq.sym else torch.empty((R, G), device=self.dev)
+                self._static = False
+        else:
+            self._g, self._G = 0, 1
+            self._scales = layer.buf_scales.reshape(R, 1).float().contiguous()
+            self._zeros = None if wq.sym else layer.buf_zeros.reshape(R, 1).float().contiguous()
+            self._static = True
+
+    def update_layer_with_transformed_weights(self, layer, W, H, name):
+        Losses = torch.zeros_like(W)
+        tmp = torch.zeros_like(W)
+        self.weight_transform(W, H, Losses, tmp)
+        self.last_error = torch.sum(Losses)              # device scalar; .item() it to log like the reference
+        if self.check_positive_definite and int(self._status.item()) != 0:
+            raise torch.linalg.LinAlgError('GPTQ: the damped Hessian is not positive-definite')
+        if self.actorder:
+            tmp = tmp[:, self.invperm]
+        layer.weight.data = tmp.reshape(layer.weight.shape)
+        if self.wquantizer.granularity == 'per_group' and not self.static_groups:
+            self.update_model_qparams(layer)
+
+    @torch.no_grad()
+    def weight_transform(self, W, Hinv, Losses, tmp):
+        """gptq.py:198-244, in place on W, Losses, tmp."""
+        R, K = W.shape
+        wq = self.wquantizer
+        if not hasattr(self, '_scales') or self._scales.shape[0] != R:
+            raise L.LcqError('weight_transform needs process_hessian_and_weights (or _setup_groups) first')
+        flags = (L.FLAG_SYM if wq.sym else 0) | (L.FLAG_STATIC if self._static else 0)
+        Err = torch.empty((R, 128), device=W.device)
+        lib = L.lib()
+        st = L.stream()
+        qmin, qmax = L.f32(wq.qmin), L.f32(wq.qmax)
+        for i1 in range(0, self.n_nonout, self.blocksize):
+            i2 = min(i1 + self.blocksize, self.n_nonout)
+            L.check(lib.lcq_gptq_block(L.ptr(W), L.ptr(tmp), L.ptr(Losses), L.ptr(Err), L.ptr(Hinv), L.i64(R), L.i64(K),
+                                       L.i64(i1), L.i32(i2 - i1), L.i32(self._g), qmin, qmax, L.i32(flags),
+                                       L.ptr(self._scales), L.ptr(self._zeros), L.ptr(self._gidx), L.i64(self._G), st),
+                    'lcq_gptq_block')
+            L.check(lib.lcq_gptq_trailing(L.ptr(W), L.ptr(Err), L.ptr(Hinv), L.i64(R), L.i64(K), L.i64(i1), L.i64(i2),
+                                          st), 'lcq_gptq_trailing')
+
+    # -- qparam bookkeeping (gptq.py:332-409) ---------------------------------------
+    @torch.no_grad()
+    def collect_layer_qparams(self, layer):
+        """What collect_block_qparams (base_blockwise_quantization.py:348-376) registers per Linear."""
+        _, scales, zeros, max_int, min_int = self.wquantizer.get_tensor_qparams(layer.weight.data)
+        layer.buf_scales = scales.detach()
+        layer.buf_zeros = zeros.detach()
+        layer.buf_qmax = max_int.clone().to(self.dev)
+        layer.buf_qmin = min_int.clone().to(self.dev)
+
+    @torch.no_grad()
+    def update_model_qparams(self, layer):
+        layer.buf_scales = self._scales.reshape(-1, 1).clone()
+        if not self.wquantizer.sym:
+            layer.buf_zeros = self._zeros.reshape(-1, 1).clone()
+
+    @property
+    def groups(self):
+        """The reference's list of per-group dicts, materialised from the [R, G] tensors."""
+        out = []
+        for gi in range(self._G):
+            out.append({'scale': self._scales[:, gi:gi + 1],
+                        'zero': torch.tensor(0.0) if self.wquantizer.sym else self._zeros[:, gi:gi + 1],
+                        'qmax': self.wquantizer.qmax, 'qmin': self.wquantizer.qmin})
+        return out
+
+    # -- deploy-time partials (gptq.py:411-452) -----------------------------------------
+    @torch.no_grad()
+    def w_q(self, module, wquantizer):
+        weight = module.weight.data
+        args = {}
+        args['scales'] = module.buf_scales
+        args['zeros'] = module.buf_zeros if hasattr(module, 'buf_zeros') else None
+        args['qmax'] = module.buf_qmax
+        args['qmin'] = module.buf_qmin
+        args['scales'] = args['scales'].to(self.model_dtype)
+        return wquantizer.real_quant_weight_static(weight, args)
+
+    @torch.no_grad()
+    def w_qdq(self, module, wquantizer):
+        weight = module.weight
+        if self.need_perm:
+            weight = module.weight[:, module.buf_perm]
+        args = {}
+        args['scales'] = module.buf_scales
+        args['zeros'] = module.buf_zeros if hasattr(module, 'buf_zeros') else None
+        args['qmax'] = module.buf_qmax
+        args['qmin'] = module.buf_qmin
+        weight = wquantizer.fake_quant_weight_static(weight, args).to(self.model_dtype)
+        if self.need_perm:
+            weight = weight[:, module.buf_invperm]
+        return weight
+
+    @torch.no_grad()
+    def free(self, name):
+        self.H = None
+        self.Losses = None
+        self.Trace = None
+        leader = self.layers_cache.get(name, {}).get('leader', name)
+        self.layers_cache.pop(name, None)
+        if leader in self._shared and not any(c.get('leader') == leader for c in self.layers_cache.values()):
+            del self._shared[leader]
+
+    @torch.no_grad()
+    def ready(self):
+        if 'scale' not in self.qparams:
+            return False
+        return torch.all(self.qparams['scale'] != 0)

@@ -82,11 +82,16 @@ class BaseQuantizer(object):
         min_val, max_val = tensor_range[0].contiguous(), tensor_range[1].contiguous()
         qmin = self.qmin.to(device)
         qmax = self.qmax.to(device)
+        flags = self._int_flags()
+        # 0-dim ranges (per_tensor) meet the 0-dim fp32 (qmax - qmin): torch promotes the result to fp32
+        if max_val.dim() == 0 and not self.sym and max_val.dtype != torch.float32:
+            flags |= L.FLAG_RANGE_BF16
+            min_val, max_val = min_val.float(), max_val.float()
         scales = torch.empty_like(max_val)
         zeros = torch.tensor(0.0) if self.sym else torch.empty_like(max_val)
         L.check(L.lib().lcq_qparams_int(L.ptr(min_val), L.ptr(max_val), L.dtype_code(max_val.dtype),
                                         L.i64(max_val.numel()), L.f32(self.qmin), L.f32(self.qmax),
-                                        L.i32(self._int_flags()), L.ptr(scales),
+                                        L.i32(flags), L.ptr(scales),
                                         L.ptr(None if self.sym else zeros), L.stream()), 'lcq_qparams_int')
         return scales, zeros, qmax, qmin
 
@@ -202,12 +207,17 @@ class IntegerQuantizer(BaseQuantizer):
             if scales.dim() > 0 and scales.dtype != t.dtype:
                 common = torch.promote_types(t.dtype, scales.dtype)
                 t = t.to(common)
-            scales = scales.to(t.dtype).contiguous()
+            # a 0-dim fp32 qparam next to a bf16 tensor enters the arithmetic unrounded
+            qp_dtype = t.dtype
+            if scales.dim() == 0 and scales.dtype == torch.float32 and t.dtype != torch.float32:
+                flags |= L.FLAG_SCALE_F32
+                qp_dtype = torch.float32
+            scales = scales.to(device=t.device, dtype=qp_dtype).contiguous()
             rows, cols, scalar = _static_layout(t, scales)
             flags |= L.FLAG_STATIC | (L.FLAG_SCALAR_QP if scalar else 0)
             z = None
             if zeros is not None and not _is_cpu_zero(zeros):
-                z = zeros.to(device=t.device, dtype=t.dtype).contiguous()
+                z = zeros.to(device=t.device, dtype=qp_dtype).contiguous()
                 if z.numel() != scales.numel():
                     z = z.expand_as(scales).contiguous()
         else:
@@ -262,14 +272,17 @@ class IntegerQuantizer(BaseQuantizer):
         t = tensor.contiguous()
         if scales.dim() > 0 and scales.dtype != t.dtype:
             t = t.to(torch.promote_types(t.dtype, scales.dtype))
-        s = scales.to(t.dtype).contiguous()
+        qp_dtype, flags = t.dtype, 0
+        if scales.dim() == 0 and scales.dtype == torch.float32 and t.dtype != torch.float32:
+            qp_dtype, flags = torch.float32, L.FLAG_SCALE_F32
+        s = scales.to(device=t.device, dtype=qp_dtype).contiguous()
         rows, cols, scalar = _static_layout(t, s)
         z = None
         if zeros is not None and not _is_cpu_zero(zeros):
-            z = zeros.to(device=t.device, dtype=t.dtype).contiguous()
+            z = zeros.to(device=t.device, dtype=qp_dtype).contiguous()
         out = torch.empty_like(t)
         L.check(L.lib().lcq_dequant_int(L.ptr(t), L.dtype_code(t.dtype), L.i64(rows), L.i64(cols), L.ptr(s), L.ptr(z),
-                                        L.i32(L.FLAG_SCALAR_QP if scalar else 0), L.f32(1.0), L.ptr(out),
+                                        L.i32(flags | (L.FLAG_SCALAR_QP if scalar else 0)), L.f32(1.0), L.ptr(out),
                                         L.stream()), 'lcq_dequant_int')
         return out
 
@@ -448,10 +461,15 @@ class FloatQuantizer(BaseQuantizer):
     def get_qparams(self, tensor_range, device):
         """Symmetric branch of quant.py:544-552 with the float qmax."""
         min_val, max_val = tensor_range[0].contiguous(), tensor_range[1].contiguous()
+        flags = L.FLAG_SYM
+        # 0-dim ranges (per_tensor) divided by the 0-dim fp32 qmax promote to fp32
+        if max_val.dim() == 0 and max_val.dtype != torch.float32:
+            flags |= L.FLAG_RANGE_BF16
+            min_val, max_val = min_val.float(), max_val.float()
         scales = torch.empty_like(max_val)
         L.check(L.lib().lcq_qparams_int(L.ptr(min_val), L.ptr(max_val), L.dtype_code(max_val.dtype),
                                         L.i64(max_val.numel()), L.f32(-float(self.qmax)), L.f32(self.qmax),
-                                        L.i32(L.FLAG_SYM), L.ptr(scales), L.ptr(None), L.stream()),
+                                        L.i32(flags), L.ptr(scales), L.ptr(None), L.stream()),
                 'lcq_qparams_int')
         return scales, torch.tensor(0.0), self.qmax.to(device), self.qmin.to(device)
 
@@ -462,7 +480,11 @@ class FloatQuantizer(BaseQuantizer):
             scales[scales == 0] = 1                      # quant.py:1061 mutates the caller's tensor
             if scales.dim() > 0 and scales.dtype != t.dtype:
                 t = t.to(torch.promote_types(t.dtype, scales.dtype))
-            s = scales.to(t.dtype).contiguous()
+            if scales.dim() == 0 and scales.dtype == torch.float32 and t.dtype != torch.float32:
+                s = scales.contiguous()                  # x / s rounds s to the row type, dq keeps fp32
+                flags |= L.FLAG_SCALE_F32
+            else:
+                s = scales.to(t.dtype).contiguous()
             rows, cols, scalar = _static_layout(t, s)
             flags |= L.FLAG_STATIC | (L.FLAG_SCALAR_QP if scalar else 0)
         else:

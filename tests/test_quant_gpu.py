@@ -53,7 +53,7 @@ def test_int_fake_and_real_quant_bit_exact(dev, dtype, bit, sym, gran, kw, shape
     assert_bit_equal(q.quant_dequant(rows, s, z, qmax, qmin),
                      Q.int_quant_dequant(spec, orows, os_, oz, spec.qmax, spec.qmin), 'quant_dequant')
 
-    if kw.get('round_zp', True):
+    if kw.get('round_zp', True) and gran != 'per_head':      # per_head real quant raises in the reference too
         codes, rs, rz = q.real_quant_weight_dynamic(wd)
         ocodes, ors, orz = Q.int_real_quant_dynamic(spec, w)
         assert_bit_equal(codes, ocodes, 'codes')
