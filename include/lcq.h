@@ -161,6 +161,30 @@ int lcq_gptq_block(float* W, float* tmp, float* Losses, float* Err, const float*
 int lcq_gptq_trailing(float* W, const float* Err, const float* U, int64_t R, int64_t K, int64_t i1, int64_t i2,
                       void* stream);
 
+/* ---- AWQ scale search ------------------------------------------------------- */
+
+/* Awq.fake_quantize_weight, awq.py:147-164 with scaling_weight :39-46 fused in:
+ *   out = fake_quant_weight_dynamic(W * s[None, :])   (W*s rounds to the tensor type first)
+ *  W, out [R, K] of `dtype`; colscale [K] of `dtype`, 16-byte aligned; group_size 0 = per_channel.
+ * W is not modified (the reference multiplies in place and restores the weights afterwards). */
+int lcq_awq_scale_quant(const void* w, int dtype, int64_t R, int64_t K, const void* colscale, int group_size,
+                        float qmin, float qmax, int flags, void* out, void* stream);
+
+int64_t lcq_awq_workspace_bytes(int64_t K);
+
+/* Awq.get_act_scale, awq.py:74-85: out[k] = mean_t |x[t, k]| (fp32 accumulation, result in `dtype`). */
+int lcq_absmean_cols(const void* x, int dtype, int64_t T, int64_t K, void* out, void* workspace, void* stream);
+
+/* Awq.get_weight_scale (one layer), awq.py:58-66: out[k] = mean_r ( |W[r,k]| / max|W[r, group(k)]| ). */
+int lcq_awq_weight_scale(const void* w, int dtype, int64_t R, int64_t K, int group_size, void* out, void* workspace,
+                         void* stream);
+
+/* scaling_input, base_blockwise_quantization.py:899-912: out = x / s[None, :]. */
+int lcq_div_cols(const void* x, int dtype, int64_t T, int64_t K, const void* s, void* out, void* stream);
+
+/* Awq.calculate_loss, awq.py:134-145: out[0] = mean( float((a - b) in `dtype`)^2 ), kept on the device. */
+int lcq_sq_err_mean(const void* a, const void* b, int dtype, int64_t n, float* out, void* workspace, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

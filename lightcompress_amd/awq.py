@@ -1,0 +1,241 @@
+"""AWQ scale search with the reference's method surface, running on liblcq.
+
+Mirrors ``llmc/compression/quantization/awq.py`` of ModelTC/LightCompress
+(class ``Awq``): ``get_weight_scale`` (:48-72), ``get_act_scale`` (:74-85),
+``get_scales`` (:87-108), ``fake_quantize_weight`` (:147-164),
+``calculate_loss`` (:134-145), ``search_scale_subset`` (:178-278) and
+``scaling_input`` (base_blockwise_quantization.py:899-912).
+
+What changes under the API
+  * W*s and the fake quantization are one kernel writing a scratch tensor, so
+    the layer weights are never modified and never restored from a host copy
+    (the reference multiplies in place and reloads the state dict from CPU at
+    every grid point);
+  * mean|x| is computed once per input instead of once per grid point;
+  * the 20 losses stay on the device and are compared once (first minimum
+    wins, as ``loss < best`` does), instead of one ``.item()`` per point;
+  * the inspect-module forward itself (library GEMMs) is whatever the caller
+    passes; the O(K) scale arithmetic (pow / clamp / normalise) uses torch ops
+    on the [K] vector like the reference;
+  * one process / one GPU: no all_reduce / broadcast of the winner; GQA
+    (prev_op = v_proj feeding o_proj with repeated heads) is not carried over.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib as L
+from .quant import IntegerQuantizer
+
+
+class Awq:
+    def __init__(self, quant_config, wquantizer=None, aquantizer=None):
+        self.quant_config = quant_config
+        special_config = quant_config.get('special', {})
+        self.trans = special_config.get('trans', True)
+        self.trans_version = special_config.get('trans_version', 'v2')
+        self.awq_bs = special_config.get('awq_bs', None)
+        self.save_mem = special_config.get('save_mem', True)
+        self.wquantizer = wquantizer or IntegerQuantizer(**quant_config['weight'])
+        self.aquantizer = aquantizer
+        self.w_only = aquantizer is None
+        self.padding_mask = None
+        self._ws = {}
+
+    def _workspace(self, K, device):
+        key = (int(K), str(device))
+        if key not in self._ws:
+            n = L.lib().lcq_awq_workspace_bytes(L.i64(K))
+            self._ws[key] = torch.empty(n, dtype=torch.uint8, device=device)
+        return self._ws[key]
+
+    # -- awq.py:39-46 -----------------------------------------------------------
+    @torch.no_grad()
+    def scaling_weight(self, w, scales, is_gqa):
+        if is_gqa:
+            raise NotImplementedError('GQA scale repetition is not on this path')
+        w.mul_(scales.view(1, -1))
+        return w
+
+    # -- awq.py:48-72 -------------------------------------------------------------
+    def get_weight_scale(self, layers_dict):
+        layers = list(layers_dict.values())
+        total_scale = None
+        wq = self.wquantizer
+        for _m in layers:
+            w = _m.weight.data.contiguous()
+            R, K = w.shape
+            g = wq.group_size if wq.granularity == 'per_group' else K
+            out = torch.empty(K, dtype=w.dtype, device=w.device)
+            L.check(L.lib().lcq_awq_weight_scale(L.ptr(w), L.i32(L.dtype_code(w.dtype)), L.i64(R), L.i64(K), L.i32(g),
+                                                 L.ptr(out), L.ptr(self._workspace(K, w.device)), L.stream()),
+                    'lcq_awq_weight_scale')
+            if total_scale is None:
+                total_scale = out
+            else:
+                total_scale.add_(out)
+        return total_scale.div_(len(layers))
+
+    # -- awq.py:74-85 ---------------------------------------------------------------
+    def _absmean(self, x):
+        K = x.shape[-1]
+        x2 = x.reshape(-1, K).contiguous()
+        out = torch.empty(K, dtype=x.dtype, device=x.device)
+        L.check(L.lib().lcq_absmean_cols(L.ptr(x2), L.i32(L.dtype_code(x.dtype)), L.i64(x2.shape[0]), L.i64(K),
+                                         L.ptr(out), L.ptr(self._workspace(K, x.device)), L.stream()),
+                'lcq_absmean_cols')
+        return out
+
+    def get_act_scale(self, x):
+        if x.shape[0] == self._bs:
+            return self._absmean(x)
+        batch_means = []
+        b_num = x.shape[0] // self._bs
+        for num in range(b_num):
+            batch_means.append(self._absmean(x[num * self._bs:(num + 1) * self._bs]))
+        return sum(batch_means) / len(batch_means)
+
+    # -- awq.py:87-108 -----------------------------------------------------------------
+    @torch.no_grad()
+    def get_scales(self, prev_op, x, w_max, is_gqa, ratio, x_mean=None):
+        if is_gqa:
+            raise NotImplementedError('GQA scale search is not on this path')
+        x_tmp = self.get_act_scale(x) if x_mean is None else x_mean
+        if self.trans_version == 'v1':
+            scales = (x_tmp.pow(ratio) / w_max.pow(1 - ratio)).clamp(min=1e-4).view(-1)
+        else:
+            scales = x_tmp.pow(ratio).clamp(min=1e-4).view(-1)
+        scales = scales / (scales.max() * scales.min()).sqrt()
+        return scales
+
+    # -- awq.py:110-145 ------------------------------------------------------------------
+    def inspect_module_forward(self, x, inspect_module, kwargs):
+        if self._bs == x.shape[0]:
+            with torch.no_grad():
+                out = inspect_module(x, **kwargs)
+                if isinstance(out, tuple):
+                    out = out[0]
+            return out
+        outs = []
+        b_num = x.shape[0] // self._bs
+        for num in range(b_num):
+            _x = x[num * self._bs:(num + 1) * self._bs]
+            out = inspect_module(_x, **kwargs)
+            if isinstance(out, tuple):
+                out = out[0]
+            outs.append(out)
+        return torch.cat(outs, dim=0)
+
+    @torch.no_grad()
+    def get_original_out(self, x, inspect_module, subset_kwargs):
+        return self.inspect_module_forward(x, inspect_module, subset_kwargs)
+
+    def _loss_device(self, org_out, out):
+        """mean squared difference as a 1-element device tensor (no host sync)."""
+        def one(a, b):
+            a, b = a.contiguous(), b.contiguous()
+            res = torch.empty(1, dtype=torch.float32, device=a.device)
+            L.check(L.lib().lcq_sq_err_mean(L.ptr(a), L.ptr(b), L.i32(L.dtype_code(a.dtype)), L.i64(a.numel()),
+                                            L.ptr(res), L.ptr(self._workspace(a.shape[-1], a.device)), L.stream()),
+                    'lcq_sq_err_mean')
+            return res
+        if out.shape[0] == self._bs:
+            return one(org_out, out)
+        b_num = org_out.shape[0] // self._bs
+        total = None
+        for num in range(b_num):
+            l = one(org_out[num * self._bs:(num + 1) * self._bs], out[num * self._bs:(num + 1) * self._bs])
+            total = l if total is None else total + l
+        return total / b_num
+
+    def calculate_loss(self, org_out, out):
+        return self._loss_device(org_out, out).item()
+
+    # -- awq.py:147-176 ----------------------------------------------------------------------
+    def _scale_quant(self, weight, scales):
+        wq = self.wquantizer
+        w = weight.contiguous()
+        R, K = w.shape
+        g = wq.group_size if wq.granularity == 'per_group' else 0
+        if wq.granularity not in ('per_group', 'per_channel'):
+            raise NotImplementedError(f'AWQ weight granularity {wq.granularity}')
+        out = torch.empty_like(w)
+        s = scales.to(w.dtype).contiguous()
+        L.check(L.lib().lcq_awq_scale_quant(L.ptr(w), L.i32(L.dtype_code(w.dtype)), L.i64(R), L.i64(K), L.ptr(s), L.i32(g),
+                                            L.f32(wq.qmin), L.f32(wq.qmax), L.i32(L.FLAG_SYM if wq.sym else 0),
+                                            L.ptr(out), L.stream()), 'lcq_awq_scale_quant')
+        return out
+
+    def fake_quantize_weight(self, fc, scales, is_gqa, layer_name):
+        if is_gqa:
+            raise NotImplementedError('GQA scale search is not on this path')
+        fc.weight.data = self._scale_quant(fc.weight.data, scales)
+        return fc.weight
+
+    def fake_quantize_input(self, x_tmp, layers_dict):
+        if self._bs == x_tmp.shape[0]:
+            return self.aquantizer.fake_quant_act_dynamic(x_tmp)
+        return torch.stack([self.aquantizer.fake_quant_act_dynamic(x_tmp[i]) for i in range(x_tmp.shape[0])])
+
+    # -- base_blockwise_quantization.py:899-912 --------------------------------------------------
+    @torch.no_grad()
+    def scaling_input(self, x, scales, is_gqa):
+        if is_gqa:
+            raise NotImplementedError('GQA scale search is not on this path')
+        K = x.shape[-1]
+        x2 = x.contiguous()
+        s = scales.to(x.dtype).contiguous()
+        out = torch.empty_like(x2)
+        L.check(L.lib().lcq_div_cols(L.ptr(x2), L.i32(L.dtype_code(x.dtype)), L.i64(x2.numel() // K), L.i64(K), L.ptr(s),
+                                     L.ptr(out), L.stream()), 'lcq_div_cols')
+        return out
+
+    # -- awq.py:178-278 ------------------------------------------------------------------------------
+    @torch.no_grad()
+    def search_scale_subset(self, prev_op, layers_dict, input, inspect_module, is_gqa, subset_kwargs):
+        if self.awq_bs is None:
+            self._bs = input[0].shape[0]
+        else:
+            self._bs = self.awq_bs
+        w_max = self.get_weight_scale(layers_dict) if self.trans_version == 'v1' else None
+        n_grid = 20
+        originals = {name: fc.weight.data for name, fc in layers_dict.items()}
+        device = next(iter(originals.values())).device
+        n_samples = input[0].shape[0] if len(input) == 1 else sum(x.shape[0] for x in input)
+
+        org_out_dict, x_mean_dict = {}, {}
+        loss_rows, scale_rows = [], []
+        for n in range(n_grid):
+            loss_mean = 0
+            scales_mean = 0
+            for i in range(len(input)):
+                input[i] = input[i].to(device)
+                x = input[i]
+                kwargs = subset_kwargs[i] if isinstance(subset_kwargs, list) else (subset_kwargs or {})
+                if i not in org_out_dict:
+                    org_out_dict[i] = self.get_original_out(x, inspect_module, kwargs)
+                    x_mean_dict[i] = self.get_act_scale(x)
+                org_out = org_out_dict[i]
+                ratio = n * 1 / n_grid
+                scales = self.get_scales(prev_op, x, w_max, is_gqa, ratio, x_mean=x_mean_dict[i])
+                for layer_name, fc in layers_dict.items():
+                    fc.weight.data = self._scale_quant(originals[layer_name], scales)
+                x_tmp = self.scaling_input(x, scales, is_gqa)
+                if not self.w_only:
+                    x_tmp = self.fake_quantize_input(x_tmp, layers_dict)
+                out = self.inspect_module_forward(x_tmp, inspect_module, kwargs)
+                if self.padding_mask and org_out.shape[1] == self.padding_mask[i].shape[-1]:
+                    m = self.padding_mask[i].unsqueeze(dim=-1).to(org_out.device)
+                    org_out, out = org_out * m, out * m
+                loss = self._loss_device(org_out, out)
+                loss_mean = loss_mean + x.shape[0] * 1.0 / n_samples * loss
+                scales_mean = scales_mean + x.shape[0] * 1.0 / n_samples * scales
+                for layer_name, fc in layers_dict.items():      # the originals were never touched
+                    fc.weight.data = originals[layer_name]
+            loss_rows.append(loss_mean.reshape(1))
+            scale_rows.append(scales_mean)
+        losses = torch.cat(loss_rows)
+        best = torch.argmin(losses)                              # first minimum, like `loss < best_error`
+        self.search_losses = losses
+        best_scales = torch.stack(scale_rows)[best]
+        return best_scales

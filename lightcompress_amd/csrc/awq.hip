@@ -1,0 +1,228 @@
+// AWQ scale-search helpers for gfx950 (the weight side, W*s -> fake quant, is
+// lcq_awq_scale_quant in quant_int.hip).
+//
+//   lcq_absmean_cols   Awq.get_act_scale            awq.py:74-85     mean_t |x[t, k]|
+//   lcq_div_cols       scaling_input                base_blockwise_quantization.py:899-912   x / s[None, :]
+//   lcq_sq_err_mean    Awq.calculate_loss           awq.py:134-145   mean(((a - b) in the tensor dtype).float()^2)
+//   lcq_awq_weight_scale  Awq.get_weight_scale      awq.py:48-72     mean_r (|W| / group max)
+//
+// All four are single-pass HBM-bound streams: 16-byte loads per lane,
+// per-thread fp32 partial sums, one small second stage.
+#include "rowquant.h"
+
+namespace {
+using namespace lcq;
+
+constexpr int PARTS_MAX = 1024;
+
+// ---- column-wise mean of |x| over T rows ------------------------------------------------
+// grid = (column blocks of 256 * N, row splits); every thread owns one 16-byte column chunk
+template <bool BF>
+__global__ __launch_bounds__(256) void absmean_stage1(const u32x4* __restrict__ x, int64_t T, int64_t K,
+                                                      float* __restrict__ part) {
+  constexpr int N = Vec<BF>::N;
+  const int64_t nch = K / N;
+  const int64_t ch = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (ch >= nch) return;
+  const int64_t rows_per = (T + gridDim.y - 1) / gridDim.y;
+  const int64_t r0 = blockIdx.y * rows_per, r1 = min(T, r0 + rows_per);
+  float acc[N];
+  #pragma unroll
+  for (int i = 0; i < N; ++i) acc[i] = 0.0f;
+  for (int64_t r = r0; r < r1; ++r) {
+    float v[N];
+    unpack<BF>(__builtin_nontemporal_load(x + r * nch + ch), v);
+    #pragma unroll
+    for (int i = 0; i < N; ++i) acc[i] += fabsf(v[i]);
+  }
+  float* p = part + (int64_t)blockIdx.y * K + ch * N;
+  #pragma unroll
+  for (int i = 0; i < N; ++i) p[i] = acc[i];
+}
+template <bool BF>
+__global__ __launch_bounds__(256) void absmean_stage2(const float* __restrict__ part, int nparts, int64_t T, int64_t K,
+                                                      void* __restrict__ out) {
+  const int64_t k = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (k >= K) return;
+  float s = 0.0f;
+  for (int p = 0; p < nparts; ++p) s += part[(int64_t)p * K + k];
+  store_scalar<BF>(out, k, rnd<BF>(s / (float)T));
+}
+
+// ---- x / s[None, :] -----------------------------------------------------------------------
+template <bool BF>
+__global__ __launch_bounds__(256) void div_cols_kernel(const u32x4* __restrict__ x, const u32x4* __restrict__ s,
+                                                       int64_t nchunks_total, int64_t nch_row, u32x4* __restrict__ out) {
+  constexpr int N = Vec<BF>::N;
+  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < nchunks_total; c += (int64_t)gridDim.x * 256) {
+    float v[N], sv[N];
+    unpack<BF>(__builtin_nontemporal_load(x + c), v);
+    unpack<BF>(s[c % nch_row], sv);
+    #pragma unroll
+    for (int i = 0; i < N; ++i) v[i] = rnd_e<BF>(v[i] / sv[i]);
+    __builtin_nontemporal_store(pack<BF>(v), out + c);
+  }
+}
+
+// ---- mean of squared differences ------------------------------------------------------------
+template <bool BF>
+__global__ __launch_bounds__(256) void sqerr_stage1(const u32x4* __restrict__ a, const u32x4* __restrict__ b,
+                                                    int64_t nchunks, double* __restrict__ part) {
+  constexpr int N = Vec<BF>::N;
+  __shared__ float sm[4];
+  float acc = 0.0f;
+  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < nchunks; c += (int64_t)gridDim.x * 256) {
+    float va[N], vb[N];
+    unpack<BF>(__builtin_nontemporal_load(a + c), va);
+    unpack<BF>(__builtin_nontemporal_load(b + c), vb);
+    #pragma unroll
+    for (int i = 0; i < N; ++i) { const float d = rnd_e<BF>(va[i] - vb[i]); acc += d * d; }
+  }
+  acc = team_sum<64>(acc);
+  if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) part[blockIdx.x] = (double)sm[0] + (double)sm[1] + (double)sm[2] + (double)sm[3];
+}
+__global__ __launch_bounds__(256) void sqerr_stage2(const double* __restrict__ part, int nparts, double n,
+                                                    float* __restrict__ out) {
+  __shared__ double sm[256];
+  double s = 0.0;
+  for (int i = threadIdx.x; i < nparts; i += 256) s += part[i];
+  sm[threadIdx.x] = s;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w) sm[threadIdx.x] += sm[threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) out[0] = (float)(sm[0] / n);
+}
+
+// ---- mean over rows of |W| / (group max of |W|) -----------------------------------------------
+// one workgroup per slab of rows; a group of g columns is shared by g/N consecutive lanes
+template <bool BF, int TEAM>
+__global__ __launch_bounds__(256) void wscale_stage1(const u32x4* __restrict__ w, int64_t R, int64_t K,
+                                                     float* __restrict__ part) {
+  constexpr int N = Vec<BF>::N;
+  const int64_t nch = K / N;
+  const int64_t rows_per = (R + gridDim.x - 1) / gridDim.x;
+  const int64_t r0 = blockIdx.x * rows_per, r1 = min(R, r0 + rows_per);
+  for (int64_t ch0 = 0; ch0 < nch; ch0 += 256) {
+    const int64_t ch = ch0 + threadIdx.x;
+    float acc[N];
+    #pragma unroll
+    for (int i = 0; i < N; ++i) acc[i] = 0.0f;
+    for (int64_t r = r0; r < r1; ++r) {
+      float v[N];
+      float mx = 0.0f;
+      if (ch < nch) {
+        unpack<BF>(w[r * nch + ch], v);
+        #pragma unroll
+        for (int i = 0; i < N; ++i) { v[i] = fabsf(v[i]); mx = fmaxf(mx, v[i]); }
+      }
+      mx = team_reduce<TEAM, true>(mx);
+      if (ch < nch) {
+        #pragma unroll
+        for (int i = 0; i < N; ++i) acc[i] += rnd_e<BF>(v[i] / mx);
+      }
+    }
+    if (ch < nch) {
+      float* p = part + (int64_t)blockIdx.x * K + ch * N;
+      #pragma unroll
+      for (int i = 0; i < N; ++i) p[i] = acc[i];
+    }
+  }
+}
+
+template <bool BF>
+int absmean(const void* x, int64_t T, int64_t K, void* out, float* part, hipStream_t st) {
+  constexpr int N = Vec<BF>::N;
+  if (K % N != 0 || ((uintptr_t)x % 16) != 0) return LCQ_EALIGN;
+  const int64_t nch = K / N;
+  int splits = (int)((T + 63) / 64);
+  if (splits > PARTS_MAX) splits = PARTS_MAX;
+  if (splits < 1) splits = 1;
+  absmean_stage1<BF><<<dim3((unsigned)((nch + 255) / 256), (unsigned)splits), dim3(256), 0, st>>>((const u32x4*)x, T, K, part);
+  absmean_stage2<BF><<<dim3((unsigned)((K + 255) / 256)), dim3(256), 0, st>>>(part, splits, T, K, out);
+  return LCQ_OK;
+}
+
+template <bool BF>
+int wscale(const void* w, int64_t R, int64_t K, int g, void* out, float* part, hipStream_t st) {
+  constexpr int N = Vec<BF>::N;
+  if (K % N != 0 || g % N != 0 || K % g != 0 || ((uintptr_t)w % 16) != 0) return LCQ_EALIGN;
+  const int team = g / N;
+  int splits = (int)((R + 15) / 16);
+  if (splits > PARTS_MAX) splits = PARTS_MAX;
+  #define LCQ_WS(T) wscale_stage1<BF, T><<<dim3((unsigned)splits), dim3(256), 0, st>>>((const u32x4*)w, R, K, part)
+  if (team == 1) LCQ_WS(1); else if (team == 2) LCQ_WS(2); else if (team == 4) LCQ_WS(4); else if (team == 8) LCQ_WS(8);
+  else if (team == 16) LCQ_WS(16); else if (team == 32) LCQ_WS(32); else if (team == 64) LCQ_WS(64);
+  else return LCQ_EINVAL;
+  #undef LCQ_WS
+  absmean_stage2<BF><<<dim3((unsigned)((K + 255) / 256)), dim3(256), 0, st>>>(part, splits, R, K, out);
+  return LCQ_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int64_t lcq_awq_workspace_bytes(int64_t K) { return (int64_t)PARTS_MAX * K * 4 + 8192 * 8; }
+
+int lcq_absmean_cols(const void* x, int dtype, int64_t T, int64_t K, void* out, void* workspace, void* stream) {
+  if (!x || !out || !workspace || T <= 0 || K <= 0) return LCQ_EINVAL;
+  hipStream_t st = (hipStream_t)stream;
+  int rc;
+  if (dtype == LCQ_F32) rc = absmean<false>(x, T, K, out, (float*)workspace, st);
+  else if (dtype == LCQ_BF16) rc = absmean<true>(x, T, K, out, (float*)workspace, st);
+  else return LCQ_EDTYPE;
+  if (rc != LCQ_OK) return rc;
+  LCQ_CHECK_LAUNCH();
+  return LCQ_OK;
+}
+
+int lcq_awq_weight_scale(const void* w, int dtype, int64_t R, int64_t K, int group_size, void* out, void* workspace,
+                         void* stream) {
+  if (!w || !out || !workspace || R <= 0 || K <= 0 || group_size <= 0) return LCQ_EINVAL;
+  hipStream_t st = (hipStream_t)stream;
+  int rc;
+  if (dtype == LCQ_F32) rc = wscale<false>(w, R, K, group_size, out, (float*)workspace, st);
+  else if (dtype == LCQ_BF16) rc = wscale<true>(w, R, K, group_size, out, (float*)workspace, st);
+  else return LCQ_EDTYPE;
+  if (rc != LCQ_OK) return rc;
+  LCQ_CHECK_LAUNCH();
+  return LCQ_OK;
+}
+
+int lcq_div_cols(const void* x, int dtype, int64_t T, int64_t K, const void* s, void* out, void* stream) {
+  if (!x || !s || !out || T <= 0 || K <= 0) return LCQ_EINVAL;
+  const int n = dtype == LCQ_BF16 ? 8 : 4;
+  if (dtype != LCQ_BF16 && dtype != LCQ_F32) return LCQ_EDTYPE;
+  if (K % n != 0 || (((uintptr_t)x | (uintptr_t)s | (uintptr_t)out) % 16) != 0) return LCQ_EALIGN;
+  const int64_t nch_row = K / n, total = T * nch_row;
+  int64_t grid = (total + 255) / 256;
+  if (grid > 65536 * 4) grid = 65536 * 4;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == LCQ_BF16) div_cols_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)x, (const u32x4*)s, total, nch_row, (u32x4*)out);
+  else div_cols_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)x, (const u32x4*)s, total, nch_row, (u32x4*)out);
+  LCQ_CHECK_LAUNCH();
+  return LCQ_OK;
+}
+
+int lcq_sq_err_mean(const void* a, const void* b, int dtype, int64_t n, float* out, void* workspace, void* stream) {
+  if (!a || !b || !out || !workspace || n <= 0) return LCQ_EINVAL;
+  const int nn = dtype == LCQ_BF16 ? 8 : 4;
+  if (dtype != LCQ_BF16 && dtype != LCQ_F32) return LCQ_EDTYPE;
+  if (n % nn != 0 || (((uintptr_t)a | (uintptr_t)b) % 16) != 0) return LCQ_EALIGN;
+  const int64_t nchunks = n / nn;
+  int64_t grid = (nchunks + 255) / 256;
+  if (grid > 8192) grid = 8192;
+  hipStream_t st = (hipStream_t)stream;
+  double* part = (double*)workspace;
+  if (dtype == LCQ_BF16) sqerr_stage1<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)a, (const u32x4*)b, nchunks, part);
+  else sqerr_stage1<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)a, (const u32x4*)b, nchunks, part);
+  sqerr_stage2<<<dim3(1), dim3(256), 0, st>>>(part, (int)grid, (double)n, out);
+  LCQ_CHECK_LAUNCH();
+  return LCQ_OK;
+}
+
+}  // extern "C"

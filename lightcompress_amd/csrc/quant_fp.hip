@@ -28,6 +28,7 @@ struct FpRow {
 template <bool BF_>
 struct FpOp {
   static constexpr bool BF = BF_;
+  static constexpr bool HAS_PRESCALE = false;
   using Row = FpRow;
   float qmax;
   int e_bits, m_bits, tie_even, subnormals;

@@ -29,12 +29,33 @@ struct IntRow {
 };
 
 // FAST: round_zp and |qmin|,qmax <= 256 (every stock configuration).
-template <bool BF_, bool FAST>
+template <bool BF_, bool FAST, bool PRESCALE = false>
 struct IntOp {
   static constexpr bool BF = BF_;
+  static constexpr bool HAS_PRESCALE = PRESCALE;
   using Row = IntRow;
   float qmin, qmax, qrange, osf;
   int sym, round_zp, is_static, scalar_qp, dq_f32, code_dtype, range_bf16, scale_f32;
+  // optional per-column factor applied first (AWQ: W * s), rows of the reshaped tensor tile a
+  // weight row of wrow_cols columns
+  const void* colscale;
+  int wrow_cols;
+
+  __device__ __forceinline__ float prescale1(float x, int64_t row, int64_t col, int64_t cols) const {
+    const int64_t c = (row * cols + col) % wrow_cols;
+    return rnd_e<BF>(x * load_scalar<BF>(colscale, c));
+  }
+  __device__ __forceinline__ u32x4 prescale(const u32x4& raw, int64_t row, int ch, int nchunks) const {
+    constexpr int N = Vec<BF>::N;
+    const int64_t c0 = ((row * nchunks + ch) * N) % wrow_cols;       // wrow_cols % N == 0 on this path
+    const u32x4 sraw = *((const u32x4*)colscale + c0 / N);
+    float v[N], sv[N];
+    unpack<BF>(raw, v);
+    unpack<BF>(sraw, sv);
+    #pragma unroll
+    for (int i = 0; i < N; ++i) v[i] = rnd_e<BF>(v[i] * sv[i]);
+    return pack<BF>(v);
+  }
 
   __device__ __forceinline__ Row finish(float s, float z) const {
     Row p;
@@ -80,7 +101,7 @@ struct IntOp {
   }
 
   __device__ __forceinline__ void store_qp(void* scales, void* zeros, int64_t row, const Row& p) const {
-    store_scalar<BF>(scales, row, p.s);
+    if (scales) store_scalar<BF>(scales, row, p.s);
     if (zeros && !sym) store_scalar<BF>(zeros, row, p.z);
   }
 
@@ -134,6 +155,7 @@ Op make_op(float qmin, float qmax, int flags, float osf, int code_dtype) {
   c.dq_f32 = 0;
   c.range_bf16 = (flags & LCQ_FLAG_RANGE_BF16) != 0;
   c.scale_f32 = (flags & LCQ_FLAG_SCALE_F32) != 0;
+  c.colscale = nullptr; c.wrow_cols = 1;
   c.code_dtype = code_dtype;
   return c;
 }
@@ -236,6 +258,33 @@ int lcq_quant_int(const void* x, int dtype, int64_t rows, int64_t cols, float qm
   if (dtype == LCQ_F32) rc = run<false>(x, rows, cols, qmin, qmax, flags, out_scale_factor, dq, codes, code_dtype, scales, zeros, st);
   else if (dtype == LCQ_BF16) rc = run<true>(x, rows, cols, qmin, qmax, flags, out_scale_factor, dq, codes, code_dtype, scales, zeros, st);
   else return LCQ_EDTYPE;
+  if (rc != LCQ_OK) return rc;
+  LCQ_CHECK_LAUNCH();
+  return LCQ_OK;
+}
+
+int lcq_awq_scale_quant(const void* w, int dtype, int64_t R, int64_t K, const void* colscale, int group_size,
+                        float qmin, float qmax, int flags, void* out, void* stream) {
+  if (!w || !colscale || !out || R <= 0 || K <= 0 || K > 0x7fffffff) return LCQ_EINVAL;
+  if (!(qmax > qmin) || (flags & (LCQ_FLAG_STATIC | LCQ_FLAG_NO_ROUND_ZP))) return LCQ_EINVAL;
+  if (qmax > 256.0f || qmin < -256.0f) return LCQ_EINVAL;
+  const int64_t cols = group_size > 0 ? group_size : K;
+  if (K % cols != 0) return LCQ_EINVAL;
+  const int64_t rows = R * (K / cols);
+  const int n = dtype == LCQ_BF16 ? 8 : 4;
+  if (cols % n != 0 || K % n != 0 || ((uintptr_t)colscale % 16) != 0) return LCQ_EALIGN;
+  hipStream_t st = (hipStream_t)stream;
+  int rc;
+  // the group scales / zeros stay in registers: fake_quantize_weight does not return them
+  if (dtype == LCQ_F32) {
+    auto op = make_op<IntOp<false, true, true>>(qmin, qmax, flags, 1.0f, LCQ_CODE_NONE);
+    op.colscale = colscale; op.wrow_cols = (int)K; op.is_static = 0;
+    rc = dispatch_rows(w, rows, cols, out, (void*)nullptr, (void*)nullptr, (void*)nullptr, op, false, st);
+  } else if (dtype == LCQ_BF16) {
+    auto op = make_op<IntOp<true, true, true>>(qmin, qmax, flags, 1.0f, LCQ_CODE_NONE);
+    op.colscale = colscale; op.wrow_cols = (int)K; op.is_static = 0;
+    rc = dispatch_rows(w, rows, cols, out, (void*)nullptr, (void*)nullptr, (void*)nullptr, op, false, st);
+  } else return LCQ_EDTYPE;
   if (rc != LCQ_OK) return rc;
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;

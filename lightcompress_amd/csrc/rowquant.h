@@ -14,6 +14,8 @@
 //   float deq(q, Row)                   dequantized value (already rounded to the output type)
 //   uint32_t byte(q)                    1-byte storage of a code (U8 / I8 / FP8)
 //   bool is_static, dq_f32; int code_dtype
+//   static constexpr bool HAS_PRESCALE; if set, prescale(chunk,row,ch,nchunks) / prescale1(x,row,col,cols)
+//   multiply the input by a per-column factor (rounded to the row type) before anything else
 #pragma once
 #include "common.h"
 #include "lcq_internal.h"
@@ -168,8 +170,10 @@ __global__ __launch_bounds__(256) void row_team_kernel(
     #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       const int ch = t + it * TEAM;
-      if (row < rows && ch < nchunks) raw[u][it] = __builtin_nontemporal_load(x + row * nchunks + ch);
-      else raw[u][it] = u32x4{0, 0, 0, 0};
+      if (row < rows && ch < nchunks) {
+        raw[u][it] = __builtin_nontemporal_load(x + row * nchunks + ch);
+        if constexpr (Op::HAS_PRESCALE) raw[u][it] = op.prescale(raw[u][it], row, ch, nchunks);
+      } else raw[u][it] = u32x4{0, 0, 0, 0};
     }
   }
 
@@ -226,6 +230,7 @@ __global__ __launch_bounds__(256) void row_block_kernel(
   for (int k = 0; k < CACHE; ++k) {
     const int ch = threadIdx.x + k * 256;
     raw[k] = (ch < nchunks) ? __builtin_nontemporal_load(xr + ch) : u32x4{0, 0, 0, 0};
+    if constexpr (Op::HAS_PRESCALE) if (ch < nchunks) raw[k] = op.prescale(raw[k], row, ch, nchunks);
   }
   typename Op::Row p;
   if (!op.is_static) {
@@ -233,7 +238,11 @@ __global__ __launch_bounds__(256) void row_block_kernel(
     #pragma unroll
     for (int k = 0; k < CACHE; ++k)
       if ((int)threadIdx.x + k * 256 < nchunks) chunk_minmax<Op>(raw[k], mn, mx);
-    for (int ch = threadIdx.x + CACHE * 256; ch < nchunks; ch += 256) chunk_minmax<Op>(xr[ch], mn, mx);
+    for (int ch = threadIdx.x + CACHE * 256; ch < nchunks; ch += 256) {
+      u32x4 r = xr[ch];
+      if constexpr (Op::HAS_PRESCALE) r = op.prescale(r, row, ch, nchunks);
+      chunk_minmax<Op>(r, mn, mx);
+    }
     mn = block_reduce<false>(mn, sm);
     mx = block_reduce<true>(mx, sm);
     p = op.make(mn, mx);
@@ -246,7 +255,11 @@ __global__ __launch_bounds__(256) void row_block_kernel(
     const int ch = threadIdx.x + k * 256;
     if (ch < nchunks) emit_chunk(op, p, raw[k], row * nchunks + ch, dq, codes);
   }
-  for (int ch = threadIdx.x + CACHE * 256; ch < nchunks; ch += 256) emit_chunk(op, p, xr[ch], row * nchunks + ch, dq, codes);
+  for (int ch = threadIdx.x + CACHE * 256; ch < nchunks; ch += 256) {
+    u32x4 r = xr[ch];
+    if constexpr (Op::HAS_PRESCALE) r = op.prescale(r, row, ch, nchunks);
+    emit_chunk(op, p, r, row * nchunks + ch, dq, codes);
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -264,7 +277,8 @@ __global__ __launch_bounds__(256) void row_scalar_kernel(
   if (!op.is_static) {
     float mn = __builtin_inff(), mx = -__builtin_inff();
     for (int64_t j = lane; j < cols; j += 64) {
-      const float v = load_scalar<BF>(x, row * cols + j);
+      float v = load_scalar<BF>(x, row * cols + j);
+      if constexpr (Op::HAS_PRESCALE) v = op.prescale1(v, row, j, cols);
       mn = nan_min(mn, v); mx = nan_max(mx, v);
     }
     mn = team_reduce<64, false>(mn);
@@ -276,7 +290,9 @@ __global__ __launch_bounds__(256) void row_scalar_kernel(
   }
   for (int64_t j = lane; j < cols; j += 64) {
     const int64_t e = row * cols + j;
-    const float q = op.code(load_scalar<BF>(x, e), p);
+    float xv = load_scalar<BF>(x, e);
+    if constexpr (Op::HAS_PRESCALE) xv = op.prescale1(xv, row, j, cols);
+    const float q = op.code(xv, p);
     if (codes) store_code1(op, codes, e, q);
     if (dq) {
       const float d = op.deq(q, p);
