@@ -83,53 +83,92 @@ __global__ __launch_bounds__(256) void build_kernel(const float* __restrict__ H,
   A[(long long)a * K + b] = v;
 }
 
-// diagonal block: Cholesky (left-looking) and inverse of the factor, all in LDS
+// Diagonal block: Cholesky factor L11 and its inverse in one elimination sweep.
+// 256 threads hold the 128x128 block of A and of B (= I, turning into L11^-1) as 8x8
+// register tiles (thread (ty, tx) owns rows 8ty.., columns 8tx..).  Step j:
+//   d = sqrt(a_jj);  column j of L = a[:, j] / d;  row j of X = b[j, :] / d   (through LDS)
+//   a[i][k] -= l_ij l_kj  (i, k > j)      b[i][:] -= l_ij x_j[:]  (i > j)
+// i.e. the right-looking Cholesky update and the forward substitution L X = I share the
+// broadcast of column j.  Two barriers and at most 128 FMAs per thread per step.
 __global__ __launch_bounds__(256) void potrf_diag_kernel(float* __restrict__ Ablk, int lda, int nb,
                                                          float* __restrict__ Dinv, PrepScalars* sc) {
-  __shared__ float Ls[NB * (NB + 1)];
-  __shared__ float Xs[NB * NB];
-  __shared__ float piv;
-  constexpr int P = NB + 1;
+  __shared__ float colbuf[NB];     // column j of L (zero above the diagonal)
+  __shared__ float rowbuf[NB];     // row j of X = L^-1
+  __shared__ float pivot;
   const int tid = threadIdx.x;
-  for (int e = tid; e < NB * NB; e += 256) {
-    const int r = e / NB, c = e % NB;
-    Ls[r * P + c] = (r < nb && c <= r) ? Ablk[(long long)r * lda + c] : 0.0f;
-    Xs[e] = 0.0f;
-  }
-  __syncthreads();
-  const int i = tid >> 1, half = tid & 1;
-  for (int j = 0; j < nb; ++j) {
-    float dot = 0.0f;
-    if (i >= j && i < nb)
-      for (int k = half; k < j; k += 2) dot += Ls[i * P + k] * Ls[j * P + k];
-    dot += lane_xor<1>(dot);
-    const float v = Ls[i * P + j] - dot;
-    if (i == j && half == 0) {
-      if (!(v > 0.0f)) sc->status = 1;
-      piv = sqrtf(v);
+  const int ty = tid >> 4, tx = tid & 15;
+  float a[8][8], x[8][8];
+  #pragma unroll
+  for (int ii = 0; ii < 8; ++ii)
+    #pragma unroll
+    for (int cc = 0; cc < 8; ++cc) {
+      const int r = 8 * ty + ii, c = 8 * tx + cc;
+      a[ii][cc] = (r < nb && c <= r) ? Ablk[(long long)r * lda + c] : ((r == c) ? 1.0f : 0.0f);   // pad with identity
+      x[ii][cc] = (r == c) ? 1.0f : 0.0f;
     }
-    __syncthreads();
-    if (half == 0 && i < nb) {
-      if (i == j) Ls[i * P + j] = piv;
-      else if (i > j) Ls[i * P + j] = v / piv;
+  for (int J = 0; J < NB / 8; ++J) {
+    if (8 * J >= nb) break;
+    #pragma unroll
+    for (int jj = 0; jj < 8; ++jj) {
+      const int j = 8 * J + jj;
+      if (ty == J && tx == J) pivot = a[jj][jj];
+      __syncthreads();
+      const float pv = pivot;
+      const float d = sqrtf(pv);
+      if (tid == 0 && !(pv > 0.0f)) sc->status = 1;
+      if (tx == J && ty >= J) {                       // column j of L
+        #pragma unroll
+        for (int ii = 0; ii < 8; ++ii) {
+          const int r = 8 * ty + ii;
+          float l = 0.0f;
+          if (r == j) l = d;
+          else if (r > j) l = a[ii][jj] / d;
+          a[ii][jj] = l;
+          colbuf[r] = l;
+        }
+      }
+      if (ty == J) {                                  // row j of X
+        #pragma unroll
+        for (int cc = 0; cc < 8; ++cc) {
+          const float v = x[jj][cc] / d;
+          x[jj][cc] = v;
+          rowbuf[8 * tx + cc] = v;
+        }
+      }
+      __syncthreads();
+      if (ty >= J) {
+        float li[8];
+        #pragma unroll
+        for (int ii = 0; ii < 8; ++ii) li[ii] = (8 * ty + ii > j) ? colbuf[8 * ty + ii] : 0.0f;
+        if (tx >= J && tx <= ty) {                    // trailing update of A (lower tiles only)
+          float lk[8];
+          #pragma unroll
+          for (int cc = 0; cc < 8; ++cc) lk[cc] = (8 * tx + cc > j) ? colbuf[8 * tx + cc] : 0.0f;
+          #pragma unroll
+          for (int ii = 0; ii < 8; ++ii)
+            #pragma unroll
+            for (int cc = 0; cc < 8; ++cc) a[ii][cc] -= li[ii] * lk[cc];
+        }
+        if (tx <= J) {                                // forward substitution: rows below j of B
+          float xr[8];
+          #pragma unroll
+          for (int cc = 0; cc < 8; ++cc) xr[cc] = rowbuf[8 * tx + cc];
+          #pragma unroll
+          for (int ii = 0; ii < 8; ++ii)
+            #pragma unroll
+            for (int cc = 0; cc < 8; ++cc) x[ii][cc] -= li[ii] * xr[cc];
+        }
+      }
     }
-    __syncthreads();
   }
-  // X = L^-1, row by row: X[r][c] = (delta_rc - sum_{k<r} L[r][k] X[k][c]) / L[r][r]
-  const int c = tid >> 1;
-  for (int r = 0; r < nb; ++r) {
-    float dot = 0.0f;
-    if (c <= r)
-      for (int k = c + half; k < r; k += 2) dot += Ls[r * P + k] * Xs[k * NB + c];
-    dot += lane_xor<1>(dot);
-    if (half == 0 && c <= r) Xs[r * NB + c] = ((r == c ? 1.0f : 0.0f) - dot) / Ls[r * P + r];
-    __syncthreads();
-  }
-  for (int e = tid; e < NB * NB; e += 256) {
-    const int r = e / NB, cc = e % NB;
-    if (r < nb && cc < nb) Ablk[(long long)r * lda + cc] = (cc <= r) ? Ls[r * P + cc] : 0.0f;
-    Dinv[e] = Xs[e];
-  }
+  #pragma unroll
+  for (int ii = 0; ii < 8; ++ii)
+    #pragma unroll
+    for (int cc = 0; cc < 8; ++cc) {
+      const int r = 8 * ty + ii, c = 8 * tx + cc;
+      if (r < nb && c < nb) Ablk[(long long)r * lda + c] = (c <= r) ? a[ii][cc] : 0.0f;
+      Dinv[r * NB + c] = (r < nb && c <= r && c < nb) ? x[ii][cc] : 0.0f;
+    }
 }
 
 // copy the inverted diagonal blocks into place

@@ -9,9 +9,10 @@
 // GEMM differs from the reference's fp32 SGEMM only in summation order.
 //
 // Shape of the kernel
-//  * one 256-thread workgroup (4 waves, 2x2) per 256x256 tile of H; each wave
-//    owns 128x128 = 4x4 blocks of v_mfma_f32_32x32x16 (256 accumulator
-//    registers per lane);
+//  * one 512-thread workgroup (8 waves, 2x4) per 256x256 tile of H; each wave
+//    owns 128x64 = 4x2 blocks of v_mfma_f32_32x32x16 (128 accumulator
+//    registers per lane), so every SIMD holds two waves that cover each
+//    other's LDS / barrier latency;
 //  * H is symmetric: only tiles on or above the diagonal are computed (the
 //    lower triangle is filled once, when H is consumed, by lcq_symmetrize);
 //  * X is streamed 32 tokens at a time through double-buffered LDS in its
@@ -48,46 +49,82 @@ __device__ __forceinline__ f32x16 mfma(const s16x8& a, const s16x8& b, const f32
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
 }
 
-// tile index -> (ti, tj) with ti <= tj, row-major over the upper triangle
-__device__ __forceinline__ void decode_upper(int idx, int nt, int& ti, int& tj) {
-  int i = 0, rowlen = nt;
-  while (idx >= rowlen) { idx -= rowlen; ++i; --rowlen; }
-  ti = i; tj = i + idx;
+// Workgroup -> tile map.  Workgroups are handed to the 8 XCDs round-robin (block b runs on
+// XCD b % 8) and each XCD has its own L2, so every XCD gets a contiguous range of a tile order
+// in which consecutive tiles form 4x8 super-blocks of the upper triangle: the 32 tiles an XCD
+// works on at one time then read 12 column stripes of X between them instead of 33.
+constexpr int SB_R = 4, SB_C = 8;
+__device__ __forceinline__ bool decode_tile(int v, int nt, int& ti, int& tj) {
+  for (int r0 = 0; r0 < nt; r0 += SB_R) {
+    const int r1 = min(r0 + SB_R, nt);
+    for (int c0 = (r0 / SB_C) * SB_C; c0 < nt; c0 += SB_C) {
+      const int c1 = min(c0 + SB_C, nt);
+      int cnt = 0;
+      for (int r = r0; r < r1; ++r) cnt += max(0, c1 - max(c0, r));
+      if (v < cnt) {
+        for (int r = r0; r < r1; ++r) {
+          const int lo = max(c0, r), n = max(0, c1 - lo);
+          if (v < n) { ti = r; tj = lo + v; return true; }
+          v -= n;
+        }
+      }
+      v -= cnt;
+    }
+  }
+  return false;
 }
 
-template <bool IS_BF16>
-__global__ __launch_bounds__(256) void hessian_kernel(float* __restrict__ H, int K, const uint16_t* __restrict__ X,
+// EDGE = false: K % 256 == 0 and T % 64 == 0, no bounds checks anywhere.
+template <bool IS_BF16, bool EDGE>
+__global__ __launch_bounds__(512) void hessian_kernel(float* __restrict__ H, int K, const uint16_t* __restrict__ X,
                                                       int T, float alpha, float beta, int nt) {
   __shared__ __attribute__((aligned(16))) char lds[2 * 2 * TILE_BYTES];
-  int ti, tj;
-  decode_upper(blockIdx.x, nt, ti, tj);
-  const bool diag = (ti == tj);
+  int ti = 0, tj = 0;
+  {
+    const int total = nt * (nt + 1) / 2, per_xcd = (total + 7) / 8;
+    const int slot = blockIdx.x >> 3, xcd = blockIdx.x & 7;
+    if (slot >= per_xcd || !decode_tile(xcd * per_xcd + slot, nt, ti, tj)) return;
+  }
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wr = wave >> 1, wc = wave & 1;
+  const int wr = wave >> 2, wc = wave & 3;
 
-  // global -> LDS staging: 32 threads cover one 512-byte token row, 8 rows per pass
-  const int ld_row = tid >> 5, ld_c16 = tid & 31;
-  const int64_t colA = (int64_t)ti * TILE + ld_c16 * 8, colB = (int64_t)tj * TILE + ld_c16 * 8;
+  // global -> LDS staging: 32 threads cover one 512-byte token row, 16 rows per pass.
+  // Per-thread element offsets inside a 32-token slab are 32-bit; the slab base is uniform.
+  const int ld_row = tid >> 5, ld_c16 = tid & 31;           // ld_row 0..15
+  const int colA = ti * TILE + ld_c16 * 8, colB = tj * TILE + ld_c16 * 8;
   const bool okA = colA < K, okB = colB < K;
-  u32x4 stA[4], stB[4];
+  constexpr int NP = 2;                     // passes of 16 token rows per slab
+  uint32_t gofA[NP], gofB[NP];
+  #pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    gofA[p] = (uint32_t)((p * 16 + ld_row) * K + colA);
+    gofB[p] = (uint32_t)((p * 16 + ld_row) * K + colB);
+  }
+  u32x4 sA0[NP], sB0[NP], sA1[NP], sB1[NP];     // two slabs of global loads stay in flight
 
-  auto gload = [&](int t0) {
+  auto gload = [&](int t0, u32x4* sa, u32x4* sb) {
+    const uint16_t* Xs = X + (int64_t)t0 * K;
     #pragma unroll
-    for (int p = 0; p < 4; ++p) {
-      const int t = t0 + p * 8 + ld_row;
-      const bool rok = t < T;
-      stA[p] = (rok && okA) ? *(const u32x4*)(X + (int64_t)t * K + colA) : u32x4{0, 0, 0, 0};
-      if (!diag) stB[p] = (rok && okB) ? *(const u32x4*)(X + (int64_t)t * K + colB) : u32x4{0, 0, 0, 0};
+    for (int p = 0; p < NP; ++p) {
+      if constexpr (EDGE) {
+        const bool rok = t0 + p * 16 + ld_row < T;
+        sa[p] = u32x4{0, 0, 0, 0};
+        sb[p] = u32x4{0, 0, 0, 0};
+        if (rok && okA) sa[p] = *(const u32x4*)(Xs + gofA[p]);
+        if (rok && okB) sb[p] = *(const u32x4*)(Xs + gofB[p]);
+      } else {
+        sa[p] = *(const u32x4*)(Xs + gofA[p]);
+        sb[p] = *(const u32x4*)(Xs + gofB[p]);
+      }
     }
   };
-  auto lstore = [&](int buf) {
-    char* a = lds + (buf * 2 + 0) * TILE_BYTES + ld_row * PITCH + ld_c16 * 16;
-    char* b = lds + (buf * 2 + 1) * TILE_BYTES + ld_row * PITCH + ld_c16 * 16;
+  char* const stp = lds + ld_row * PITCH + ld_c16 * 16;
+  auto lstore = [&](int buf, const u32x4* sa, const u32x4* sb) {
     #pragma unroll
-    for (int p = 0; p < 4; ++p) {
-      *(u32x4*)(a + p * 8 * PITCH) = stA[p];
-      if (!diag) *(u32x4*)(b + p * 8 * PITCH) = stB[p];
+    for (int p = 0; p < NP; ++p) {
+      *(u32x4*)(stp + (buf * 2 + 0) * TILE_BYTES + p * 16 * PITCH) = sa[p];
+      *(u32x4*)(stp + (buf * 2 + 1) * TILE_BYTES + p * 16 * PITCH) = sb[p];
     }
   };
 
@@ -96,63 +133,95 @@ __global__ __launch_bounds__(256) void hessian_kernel(float* __restrict__ H, int
   // receives tokens 0..3 of feature s.
   const int L = lane & 15, g16 = (lane >> 4) & 1, kh = lane >> 5;
   const int frag_off = (kh * 8 + (L >> 2)) * PITCH + (g16 * 16 + (L & 3) * 4) * 2;
-  const int offA = frag_off + wr * 128 * 2, offB = frag_off + wc * 128 * 2;
+  const char* const rdA = lds + frag_off + wr * 128 * 2;
+  const char* const rdB = lds + TILE_BYTES + frag_off + wc * 64 * 2;
 
-  f32x16 acc[4][4];
+  f32x16 acc[4][2];
   #pragma unroll
   for (int i = 0; i < 4; ++i)
     #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < 2; ++j)
       #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  const int nsteps = (T + BT - 1) / BT;
-  gload(0);
-  lstore(0);
-  __syncthreads();
-  for (int s = 0; s < nsteps; ++s) {
-    const int buf = s & 1;
-    if (s + 1 < nsteps) gload((s + 1) * BT);
-    const char* tA = lds + (buf * 2 + 0) * TILE_BYTES + offA;
-    const char* tB = lds + (buf * 2 + (diag ? 0 : 1)) * TILE_BYTES + offB;
+  auto compute = [&](int buf) {
+    const char* tA = rdA + buf * 2 * TILE_BYTES;
+    const char* tB = rdB + buf * 2 * TILE_BYTES;
     #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      s16x8 fa[4], fb[4];
+      s16x8 fa[4];
       #pragma unroll
       for (int b = 0; b < 4; ++b) {
         const s16x4 a0 = lds_tr_read(tA + ks * 16 * PITCH + b * 64);
         const s16x4 a1 = lds_tr_read(tA + ks * 16 * PITCH + 4 * PITCH + b * 64);
         fa[b] = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
-        const s16x4 b0 = lds_tr_read(tB + ks * 16 * PITCH + b * 64);
-        const s16x4 b1 = lds_tr_read(tB + ks * 16 * PITCH + 4 * PITCH + b * 64);
-        fb[b] = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7);
       }
       #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int j = 0; j < 2; ++j) {                     // one B fragment at a time keeps the register footprint small
+        const s16x4 b0 = lds_tr_read(tB + ks * 16 * PITCH + j * 64);
+        const s16x4 b1 = lds_tr_read(tB + ks * 16 * PITCH + 4 * PITCH + j * 64);
+        const s16x8 fb = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7);
         #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = mfma<IS_BF16>(fa[i], fb[j], acc[i][j]);
+        for (int i = 0; i < 4; ++i) acc[i][j] = mfma<IS_BF16>(fa[i], fb, acc[i][j]);
+      }
     }
-    if (s + 1 < nsteps) lstore(buf ^ 1);
+  };
+
+  // slabs are processed in pairs; a ragged tail is zero-filled by the EDGE loads
+  const int nsteps = ((T + 2 * BT - 1) / (2 * BT)) * 2;
+  gload(0, sA0, sB0);
+  gload(BT, sA1, sB1);
+  lstore(0, sA0, sB0);
+  __syncthreads();
+  for (int s = 0; s + 2 < nsteps; s += 2) {
+    gload((s + 2) * BT, sA0, sB0);
+    compute(0);
+    lstore(1, sA1, sB1);
+    __syncthreads();
+    gload((s + 3) * BT, sA1, sB1);
+    compute(1);
+    lstore(0, sA0, sB0);
     __syncthreads();
   }
+  compute(0);
+  lstore(1, sA1, sB1);
+  __syncthreads();
+  compute(1);
 
-  // epilogue: accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32
+  // epilogue: accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32.
+  // The old values of two 32-row bands (64 per lane) are fetched before any is used so the
+  // loads overlap; alpha == 0 (first batch) never reads H.
   const int row_l = 4 * (lane >> 5), col_l = lane & 31;
+  const int grow = ti * TILE + wr * 128 + row_l, gcol = tj * TILE + wc * 64 + col_l;
+  float* const Hb = H + (int64_t)grow * K + gcol;
+  const bool rmw = (alpha != 0.0f);
   #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int64_t gj = (int64_t)tj * TILE + wc * 128 + j * 32 + col_l;
+  for (int ih = 0; ih < 2; ++ih) {
+    float old[2][2][16];
+    if (rmw) {
       #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int64_t gi = (int64_t)ti * TILE + wr * 128 + i * 32 + 8 * (r >> 2) + row_l + (r & 3);
-        if (gi < K && gj < K) {
-          float* p = H + gi * K + gj;
-          const float v = beta * acc[i][j][r];
-          *p = (alpha != 0.0f) ? (alpha * *p + v) : v;
-        }
-      }
+      for (int i2 = 0; i2 < 2; ++i2)
+        #pragma unroll
+        for (int j = 0; j < 2; ++j)
+          #pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int dr = (ih * 2 + i2) * 32 + 8 * (r >> 2) + (r & 3), dc = j * 32;
+            const bool ok = !EDGE || ((grow + dr < K) && (gcol + dc < K));
+            old[i2][j][r] = ok ? Hb[(int64_t)dr * K + dc] : 0.0f;
+          }
     }
+    #pragma unroll
+    for (int i2 = 0; i2 < 2; ++i2)
+      #pragma unroll
+      for (int j = 0; j < 2; ++j)
+        #pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int dr = (ih * 2 + i2) * 32 + 8 * (r >> 2) + (r & 3), dc = j * 32;
+          const bool ok = !EDGE || ((grow + dr < K) && (gcol + dc < K));
+          float v = beta * acc[ih * 2 + i2][j][r];
+          if (rmw) v = alpha * old[i2][j][r] + v;
+          if (ok) Hb[(int64_t)dr * K + dc] = v;
+        }
   }
 }
 
@@ -182,13 +251,15 @@ int lcq_hessian_accum(float* H, int64_t K, const void* X, int dtype, int64_t T, 
   if (K % 8 != 0 || K > (1 << 20) || T > 0x7fffffff) return LCQ_EINVAL;
   if (((uintptr_t)X % 16) != 0 || ((uintptr_t)H % 4) != 0) return LCQ_EALIGN;
   const int nt = (int)((K + TILE - 1) / TILE);
-  const int64_t tiles = (int64_t)nt * (nt + 1) / 2;
+  const int64_t tiles = ((int64_t)nt * (nt + 1) / 2 + 7) / 8 * 8;     // 8 XCD queues of equal length
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == LCQ_BF16)
-    hessian_kernel<true><<<dim3((unsigned)tiles), dim3(256), 0, st>>>(H, (int)K, (const uint16_t*)X, (int)T, alpha, beta, nt);
-  else if (dtype == LCQ_F16)
-    hessian_kernel<false><<<dim3((unsigned)tiles), dim3(256), 0, st>>>(H, (int)K, (const uint16_t*)X, (int)T, alpha, beta, nt);
+  if (T == 0) return LCQ_OK;
+  const bool edge = (K % TILE != 0) || (T % (2 * BT) != 0);
+  #define LCQ_HESS(BF, E) hessian_kernel<BF, E><<<dim3((unsigned)tiles), dim3(512), 0, st>>>(H, (int)K, (const uint16_t*)X, (int)T, alpha, beta, nt)
+  if (dtype == LCQ_BF16) { if (edge) LCQ_HESS(true, true); else LCQ_HESS(true, false); }
+  else if (dtype == LCQ_F16) { if (edge) LCQ_HESS(false, true); else LCQ_HESS(false, false); }
   else return LCQ_EDTYPE;
+  #undef LCQ_HESS
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;
 }
