@@ -115,6 +115,7 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(float* __restrict__ Abl
       __syncthreads();
       const float pv = pivot;
       const float d = sqrtf(pv);
+      const float rinv = 1.0f / d;                      // one division per step; columns scale by multiplication
       if (tid == 0 && !(pv > 0.0f)) sc->status = 1;
       if (tx == J && ty >= J) {                       // column j of L
         #pragma unroll
@@ -122,7 +123,7 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(float* __restrict__ Abl
           const int r = 8 * ty + ii;
           float l = 0.0f;
           if (r == j) l = d;
-          else if (r > j) l = a[ii][jj] / d;
+          else if (r > j) l = a[ii][jj] * rinv;
           a[ii][jj] = l;
           colbuf[r] = l;
         }
@@ -130,7 +131,7 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(float* __restrict__ Abl
       if (ty == J) {                                  // row j of X
         #pragma unroll
         for (int cc = 0; cc < 8; ++cc) {
-          const float v = x[jj][cc] / d;
+          const float v = x[jj][cc] * rinv;
           x[jj][cc] = v;
           rowbuf[8 * tx + cc] = v;
         }
