@@ -29,6 +29,7 @@ template <bool BF_>
 struct FpOp {
   static constexpr bool BF = BF_;
   static constexpr bool HAS_PRESCALE = false;
+  static constexpr int CD = -1;
   using Row = FpRow;
   float qmax;
   int e_bits, m_bits, tie_even, subnormals;
@@ -112,10 +113,23 @@ struct FpOp {
     return grid_round(t);
   }
 
+  template <int N>
+  __device__ __forceinline__ void codes(const float* x, float* q, const Row& p) const {
+    #pragma unroll
+    for (int i = 0; i < N; ++i) q[i] = code(x[i], p);
+  }
+
   // (q - 0.0) * s in fp32, then the cast of fake_quant_* (quant.py:1107,1153)
   __device__ __forceinline__ float deq(float q, const Row& p) const {
     const float d = (q - 0.0f) * p.sm;
     return dq_f32 ? d : rnd_e<BF>(d);
+  }
+
+  __device__ __forceinline__ uint32_t pack4(const float* q) const {
+    uint32_t w = 0;
+    #pragma unroll
+    for (int j = 0; j < 4; ++j) w |= byte(q[j]) << (8 * j);
+    return w;
   }
 
   // float8 storage of an on-grid value

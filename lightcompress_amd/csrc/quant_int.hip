@@ -29,10 +29,11 @@ struct IntRow {
 };
 
 // FAST: round_zp and |qmin|,qmax <= 256 (every stock configuration).
-template <bool BF_, bool FAST, bool PRESCALE = false>
+template <bool BF_, bool FAST, bool PRESCALE = false, int CD_ = -1>
 struct IntOp {
   static constexpr bool BF = BF_;
   static constexpr bool HAS_PRESCALE = PRESCALE;
+  static constexpr int CD = CD_;
   using Row = IntRow;
   float qmin, qmax, qrange, osf;
   int sym, round_zp, is_static, scalar_qp, dq_f32, code_dtype, range_bf16, scale_f32;
@@ -62,7 +63,7 @@ struct IntOp {
     p.s = s; p.z = z;
     p.r = 1.0f / s;
     const float a = fabsf(s);
-    p.fast = (a > 8.6736174e-19f) && (a < 1.1529215e18f);   // 2^-60 .. 2^60
+    p.fast = (a > 8.6736174e-19f) && (a < 1.1529215e18f) && (fabsf(z) <= 512.0f);   // s in 2^-60 .. 2^60
     p.sdq = scale_f32 ? s * osf : rnd<BF>(s * osf);
     return p;
   }
@@ -105,25 +106,10 @@ struct IntOp {
     if (zeros && !sym) store_scalar<BF>(zeros, row, p.z);
   }
 
-  // quant, quant.py:698-707: the integer code as a float
+  // quant, quant.py:698-707: the integer code as a float (element-wise form, any configuration)
   __device__ __forceinline__ float code(float x, const Row& p) const {
     float q;
-    if constexpr (FAST) {
-      float t = x * p.r;
-      bool ok;
-      if constexpr (BF) {
-        const uint32_t low = f2u(t) & 0xffffu;              // distance to a bf16 rounding midpoint
-        ok = (low - 0x7ff8u) > 0x10u;
-      } else {
-        // |t - x/s| <= 2^-22 |t| <= 2^-12 for |t| <= 1024: safe unless within 2^-11 of a half integer
-        const float d = t - rintf(t);
-        ok = (fabsf(fabsf(d) - 0.5f) > 4.8828125e-04f) && (fabsf(t) <= 1024.0f);
-      }
-      ok = ok && p.fast;
-      if (__builtin_expect(!ok, 0)) t = x / p.s;             // IEEE quotient near a boundary
-      t = rnd_e<BF>(t);
-      q = rintf(t) + p.z;
-    } else if (round_zp) {
+    if (round_zp) {
       const float t = rnd<BF>(x / p.s);
       q = rnd<BF>(rintf(t) + p.z);
     } else {
@@ -134,6 +120,42 @@ struct IntOp {
     return __builtin_amdgcn_fmed3f(q, qmin, qmax);
   }
 
+  // One 16-byte chunk.  FAST configurations (round_zp, |qmin|,qmax <= 256, |z| <= 512) evaluate
+  // x/s as x*(1/s); the chunk falls back to IEEE divisions when any product lies so close to a
+  // rounding boundary that the true quotient could round the other way:
+  //   fp32: |t - x/s| <= 2^-22 |t|; for |t| <= 1024 that is <= 2^-12, so a product farther than
+  //         2^-11 from every half integer rounds like the quotient; beyond 1024 both land outside
+  //         the clamp range on the same side (|z| <= 512), and a huge t has d == 0;
+  //   bf16: the quotient is rounded to bf16 first; the product is safe unless its low 16 bits
+  //         are within 8 ulp of the bf16 midpoint pattern 0x8000.
+  template <int N>
+  __device__ __forceinline__ void codes(const float* x, float* q, const Row& p) const {
+    if constexpr (!FAST) {
+      #pragma unroll
+      for (int i = 0; i < N; ++i) q[i] = code(x[i], p);
+    } else {
+      float t[N];
+      bool ok = p.fast;
+      #pragma unroll
+      for (int i = 0; i < N; ++i) {
+        t[i] = x[i] * p.r;
+        if constexpr (BF) {
+          ok = ok && (((f2u(t[i]) & 0xffffu) - 0x7ff8u) > 0x10u);
+        } else {
+          const float d = t[i] - rintf(t[i]);
+          ok = ok && (fabsf(fabsf(d) - 0.5f) > 4.8828125e-04f);
+        }
+      }
+      if (__builtin_expect(!ok, 0)) {
+        #pragma unroll
+        for (int i = 0; i < N; ++i) t[i] = x[i] / p.s;
+      }
+      #pragma unroll
+      for (int i = 0; i < N; ++i)
+        q[i] = __builtin_amdgcn_fmed3f(rintf(rnd_e<BF>(t[i])) + p.z, qmin, qmax);
+    }
+  }
+
   // dequant, quant.py:709-711 (scale already multiplied by output_scale_factor)
   __device__ __forceinline__ float deq(float q, const Row& p) const {
     float d = q - p.z;                                       // exact for small integer codes
@@ -142,6 +164,17 @@ struct IntOp {
   }
 
   __device__ __forceinline__ uint32_t byte(float q) const { return (uint32_t)(int32_t)q & 0xffu; }
+  __device__ __forceinline__ uint32_t pack4(const float* q) const {
+    uint32_t w = 0;
+    if ((CD >= 0 ? CD : code_dtype) == LCQ_CODE_U8) {        // integral values in [0, 255]: v_cvt_pk_u8_f32
+      #pragma unroll
+      for (int j = 0; j < 4; ++j) w = __builtin_amdgcn_cvt_pk_u8_f32(q[j], j, w);
+    } else {
+      #pragma unroll
+      for (int j = 0; j < 4; ++j) w |= byte(q[j]) << (8 * j);
+    }
+    return w;
+  }
 };
 
 template <class Op>
@@ -168,8 +201,16 @@ int run(const void* x, int64_t rows, int64_t cols, float qmin, float qmax, int f
   if (general)
     return dispatch_rows(x, rows, cols, dq, codes, scales, zeros,
                          make_op<IntOp<BF, false>>(qmin, qmax, flags, osf, code_dtype), true, st);
-  return dispatch_rows(x, rows, cols, dq, codes, scales, zeros,
-                       make_op<IntOp<BF, true>>(qmin, qmax, flags, osf, code_dtype), false, st);
+  // the common storage formats get kernels with the store path fixed at compile time
+  #define LCQ_RUN(CDV) return dispatch_rows(x, rows, cols, dq, codes, scales, zeros, \
+                         make_op<IntOp<BF, true, false, CDV>>(qmin, qmax, flags, osf, code_dtype), false, st)
+  switch (code_dtype) {
+    case LCQ_CODE_NONE: LCQ_RUN(LCQ_CODE_NONE);
+    case LCQ_CODE_U8: LCQ_RUN(LCQ_CODE_U8);
+    case LCQ_CODE_I32: LCQ_RUN(LCQ_CODE_I32);
+    default: LCQ_RUN(-1);
+  }
+  #undef LCQ_RUN
 }
 
 // get_minmax_range (row-wise), quant.py:141-143

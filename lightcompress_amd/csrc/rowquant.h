@@ -11,9 +11,12 @@
 //   Row  load(scales, zeros, row)       static parameters
 //   void store_qp(scales, zeros, row, Row)
 //   float code(x, Row)                  quantized value as a float
+//   void codes<N>(x[N], q[N], Row)      the same for one 16-byte chunk (lets the op share work)
 //   float deq(q, Row)                   dequantized value (already rounded to the output type)
 //   uint32_t byte(q)                    1-byte storage of a code (U8 / I8 / FP8)
+//   uint32_t pack4(q[4])                four of them in one word
 //   bool is_static, dq_f32; int code_dtype
+//   static constexpr int CD             code storage fixed at compile time, or -1 (use code_dtype)
 //   static constexpr bool HAS_PRESCALE; if set, prescale(chunk,row,ch,nchunks) / prescale1(x,row,col,cols)
 //   multiply the input by a per-column factor (rounded to the row type) before anything else
 #pragma once
@@ -72,7 +75,7 @@ template <class Op>
 __device__ __forceinline__ void store_codes(const Op& op, void* codes, int64_t elem0, const float* q) {
   constexpr bool BF = Op::BF;
   constexpr int N = Vec<BF>::N;
-  const int cd = op.code_dtype;
+  const int cd = (Op::CD >= 0) ? Op::CD : op.code_dtype;       // compile-time when the op pins it
   if (cd == LCQ_CODE_I32) {
     int32_t* p = (int32_t*)codes + elem0;
     #pragma unroll
@@ -95,10 +98,7 @@ __device__ __forceinline__ void store_codes(const Op& op, void* codes, int64_t e
     uint8_t* p = (uint8_t*)codes + elem0;
     #pragma unroll
     for (int i = 0; i < N; i += 4) {
-      uint32_t w = 0;
-      #pragma unroll
-      for (int j = 0; j < 4; ++j) w |= op.byte(q[i + j]) << (8 * j);
-      *(uint32_t*)(p + i) = w;
+      *(uint32_t*)(p + i) = op.pack4(q + i);
     }
   } else if (cd == LCQ_CODE_SAME) {
     *((u32x4*)codes + elem0 / N) = pack<BF>(q);
@@ -121,8 +121,7 @@ __device__ __forceinline__ void emit_chunk(const Op& op, const typename Op::Row&
   constexpr int N = Vec<BF>::N;
   float v[N], q[N];
   unpack<BF>(r, v);
-  #pragma unroll
-  for (int i = 0; i < N; ++i) q[i] = op.code(v[i], p);
+  op.template codes<N>(v, q, p);
   if (codes) store_codes(op, codes, cidx * N, q);
   if (dq) {
     #pragma unroll
@@ -141,19 +140,32 @@ __device__ __forceinline__ void emit_chunk(const Op& op, const typename Op::Row&
   }
 }
 
+// running min / max of a chunk with v_min3 / v_max3 (which skip NaNs); `nan` remembers whether
+// any element was a NaN so the caller can poison the range like torch.amax / amin do
 template <class Op>
-__device__ __forceinline__ void chunk_minmax(const u32x4& r, float& mn, float& mx) {
+__device__ __forceinline__ void chunk_minmax(const u32x4& r, float& mn, float& mx, bool& nan) {
   constexpr int N = Vec<Op::BF>::N;
   float v[N];
   unpack<Op::BF>(r, v);
   #pragma unroll
-  for (int i = 0; i < N; ++i) { mn = nan_min(mn, v[i]); mx = nan_max(mx, v[i]); }
+  for (int i = 0; i < N; i += 2) {
+    mn = fminf(fminf(mn, v[i]), v[i + 1]);
+    mx = fmaxf(fmaxf(mx, v[i]), v[i + 1]);
+    nan = nan || (v[i] != v[i]) || (v[i + 1] != v[i + 1]);
+  }
+}
+// range of a row from the per-lane partials: NaN anywhere in the team poisons both ends
+template <int TEAM>
+__device__ __forceinline__ void team_range(float& mn, float& mx, bool nan) {
+  mn = team_reduce<TEAM, false>(nan ? __builtin_nanf("") : mn);
+  mx = team_reduce<TEAM, true>(nan ? __builtin_nanf("") : mx);
 }
 
 // ---------------------------------------------------------------------------
 // short rows: TEAM lanes per row, ITERS chunks per lane, UNR row batches per wave
 // ---------------------------------------------------------------------------
-template <class Op, int TEAM, int ITERS, int UNR>
+// FULL: every row of the grid exists and every lane owns exactly ITERS chunks (no predicates).
+template <class Op, int TEAM, int ITERS, int UNR, bool FULL>
 __global__ __launch_bounds__(256) void row_team_kernel(
     const u32x4* __restrict__ x, void* __restrict__ dq, void* __restrict__ codes,
     void* __restrict__ scales, void* __restrict__ zeros, int64_t rows, int nchunks, Op op) {
@@ -170,7 +182,7 @@ __global__ __launch_bounds__(256) void row_team_kernel(
     #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       const int ch = t + it * TEAM;
-      if (row < rows && ch < nchunks) {
+      if (FULL || (row < rows && ch < nchunks)) {
         raw[u][it] = __builtin_nontemporal_load(x + row * nchunks + ch);
         if constexpr (Op::HAS_PRESCALE) raw[u][it] = op.prescale(raw[u][it], row, ch, nchunks);
       } else raw[u][it] = u32x4{0, 0, 0, 0};
@@ -180,15 +192,15 @@ __global__ __launch_bounds__(256) void row_team_kernel(
   #pragma unroll
   for (int u = 0; u < UNR; ++u) {
     const int64_t row = row0 + (int64_t)u * RPW;
-    const bool row_ok = row < rows;
+    const bool row_ok = FULL || row < rows;
     typename Op::Row p;
     if (!op.is_static) {
       float mn = __builtin_inff(), mx = -__builtin_inff();
+      bool nan = false;
       #pragma unroll
       for (int it = 0; it < ITERS; ++it)
-        if (t + it * TEAM < nchunks) chunk_minmax<Op>(raw[u][it], mn, mx);
-      mn = team_reduce<TEAM, false>(mn);
-      mx = team_reduce<TEAM, true>(mx);
+        if (FULL || t + it * TEAM < nchunks) chunk_minmax<Op>(raw[u][it], mn, mx, nan);
+      team_range<TEAM>(mn, mx, nan);
       p = op.make(mn, mx);
       if (row_ok && t == 0) op.store_qp(scales, zeros, row, p);
     } else {
@@ -197,7 +209,7 @@ __global__ __launch_bounds__(256) void row_team_kernel(
     #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       const int ch = t + it * TEAM;
-      if (row_ok && ch < nchunks) emit_chunk(op, p, raw[u][it], row * nchunks + ch, dq, codes);
+      if (FULL || (row_ok && ch < nchunks)) emit_chunk(op, p, raw[u][it], row * nchunks + ch, dq, codes);
     }
   }
 }
@@ -235,16 +247,17 @@ __global__ __launch_bounds__(256) void row_block_kernel(
   typename Op::Row p;
   if (!op.is_static) {
     float mn = __builtin_inff(), mx = -__builtin_inff();
+    bool nan = false;
     #pragma unroll
     for (int k = 0; k < CACHE; ++k)
-      if ((int)threadIdx.x + k * 256 < nchunks) chunk_minmax<Op>(raw[k], mn, mx);
+      if ((int)threadIdx.x + k * 256 < nchunks) chunk_minmax<Op>(raw[k], mn, mx, nan);
     for (int ch = threadIdx.x + CACHE * 256; ch < nchunks; ch += 256) {
       u32x4 r = xr[ch];
       if constexpr (Op::HAS_PRESCALE) r = op.prescale(r, row, ch, nchunks);
-      chunk_minmax<Op>(r, mn, mx);
+      chunk_minmax<Op>(r, mn, mx, nan);
     }
-    mn = block_reduce<false>(mn, sm);
-    mx = block_reduce<true>(mx, sm);
+    mn = block_reduce<false>(nan ? __builtin_nanf("") : mn, sm);
+    mx = block_reduce<true>(nan ? __builtin_nanf("") : mx, sm);
     p = op.make(mn, mx);
     if (threadIdx.x == 0) op.store_qp(scales, zeros, row, p);
   } else {
@@ -312,8 +325,12 @@ void launch_team(const void* x, void* dq, void* codes, void* scales, void* zeros
   constexpr int RPW = LCQ_WAVE / TEAM;
   const int64_t rows_per_block = (int64_t)RPW * UNR * 4;
   const int64_t grid = (rows + rows_per_block - 1) / rows_per_block;
-  row_team_kernel<Op, TEAM, ITERS, UNR><<<dim3((unsigned)grid), dim3(256), 0, st>>>(
-      (const u32x4*)x, dq, codes, scales, zeros, rows, nchunks, op);
+  if (rows % rows_per_block == 0 && nchunks == TEAM * ITERS)
+    row_team_kernel<Op, TEAM, ITERS, UNR, true><<<dim3((unsigned)grid), dim3(256), 0, st>>>(
+        (const u32x4*)x, dq, codes, scales, zeros, rows, nchunks, op);
+  else
+    row_team_kernel<Op, TEAM, ITERS, UNR, false><<<dim3((unsigned)grid), dim3(256), 0, st>>>(
+        (const u32x4*)x, dq, codes, scales, zeros, rows, nchunks, op);
 }
 
 template <class Op>
