@@ -150,40 +150,20 @@ int lcq_chol_inv_upper(float* H, int64_t K, const int64_t* perm, float percdamp,
 /* One lazy-batch block of GPTQ.weight_transform, gptq.py:203-243 (columns i1 .. i1+count, count <= 128):
  * per-group scale/zero refresh (search_column_qparams, :358-366), quantize-dequantize,
  * tmp[:, i] = w, Losses[:, i], in-block error feedback; Err [R,128] receives Err1.
- *  W, tmp, Losses [R,K] fp32; U [K,K] upper factor; scales / zeros [R,G] fp32
+ *  W, tmp, Losses [R,K] fp32; Err [R, ldErr] fp32 (column i of the block -> Err[:, i]);
+ *  U [K,K] upper factor; scales / zeros [R,G] fp32
  *  dynamic groups (default): group_size > 0, G >= ceil(K/group_size), qparams are written
  *  LCQ_FLAG_STATIC: qparams are inputs; group of column c is gidx[c] (or c/group_size, or 0 if group_size == 0) */
-int lcq_gptq_block(float* W, float* tmp, float* Losses, float* Err, const float* U, int64_t R, int64_t K, int64_t i1,
-                   int count, int group_size, float qmin, float qmax, int flags, float* scales, float* zeros,
+int lcq_gptq_block(float* W, float* tmp, float* Losses, float* Err, int64_t ldErr, const float* U, int64_t R, int64_t K,
+                   int64_t i1, int count, int group_size, float qmin, float qmax, int flags, float* scales, float* zeros,
                    const int32_t* gidx, int64_t G, void* stream);
 
-/* Deferred update of gptq.py:244:  W[:, i2:] -= Err[:, :i2-i1] @ U[i1:i2, i2:]  (fp32 MFMA). */
-int lcq_gptq_trailing(float* W, const float* Err, const float* U, int64_t R, int64_t K, int64_t i1, int64_t i2,
-                      void* stream);
-
-/* ---- AWQ scale search ------------------------------------------------------- */
-
-/* Awq.fake_quantize_weight, awq.py:147-164 with scaling_weight :39-46 fused in:
- *   out = fake_quant_weight_dynamic(W * s[None, :])   (W*s rounds to the tensor type first)
- *  W, out [R, K] of `dtype`; colscale [K] of `dtype`, 16-byte aligned; group_size 0 = per_channel.
- * W is not modified (the reference multiplies in place and restores the weights afterwards). */
-int lcq_awq_scale_quant(const void* w, int dtype, int64_t R, int64_t K, const void* colscale, int group_size,
-                        float qmin, float qmax, int flags, void* out, void* stream);
-
-int64_t lcq_awq_workspace_bytes(int64_t K);
-
-/* Awq.get_act_scale, awq.py:74-85: out[k] = mean_t |x[t, k]| (fp32 accumulation, result in `dtype`). */
-int lcq_absmean_cols(const void* x, int dtype, int64_t T, int64_t K, void* out, void* workspace, void* stream);
-
-/* Awq.get_weight_scale (one layer), awq.py:58-66: out[k] = mean_r ( |W[r,k]| / max|W[r, group(k)]| ). */
-int lcq_awq_weight_scale(const void* w, int dtype, int64_t R, int64_t K, int group_size, void* out, void* workspace,
-                         void* stream);
-
-/* scaling_input, base_blockwise_quantization.py:899-912: out = x / s[None, :]. */
-int lcq_div_cols(const void* x, int dtype, int64_t T, int64_t K, const void* s, void* out, void* stream);
-
-/* Awq.calculate_loss, awq.py:134-145: out[0] = mean( float((a - b) in `dtype`)^2 ), kept on the device. */
-int lcq_sq_err_mean(const void* a, const void* b, int dtype, int64_t n, float* out, void* workspace, void* stream);
+/* Deferred update of gptq.py:244, generalised to a column window (fp32 MFMA):
+ *   W[:, j1:j2] -= Err[:, :k2-k1] @ U[k1:k2, j1:j2],   k2 <= j1.
+ * The reference's call is (k1, k2, j1, j2) = (i1, i2, i2, K); splitting the column range lets the
+ * caller apply far-away columns once per several blocks with a deeper contraction. */
+int lcq_gptq_trailing(float* W, const float* Err, int64_t ldErr, const float* U, int64_t R, int64_t K, int64_t k1,
+                      int64_t k2, int64_t j1, int64_t j2, void* stream);
 
 #ifdef __cplusplus
 }

@@ -86,15 +86,17 @@ __global__ __launch_bounds__(256) void build_kernel(const float* __restrict__ H,
 // Diagonal block: Cholesky factor L11 and its inverse in one elimination sweep.
 // 256 threads hold the 128x128 block of A and of B (= I, turning into L11^-1) as 8x8
 // register tiles (thread (ty, tx) owns rows 8ty.., columns 8tx..).  Step j:
-//   d = sqrt(a_jj);  column j of L = a[:, j] / d;  row j of X = b[j, :] / d   (through LDS)
+//   owners publish the UNSCALED column j of A and row j of B through LDS (double buffered),
+//   one barrier, then every thread derives 1/sqrt(a_jj) itself and applies
 //   a[i][k] -= l_ij l_kj  (i, k > j)      b[i][:] -= l_ij x_j[:]  (i > j)
 // i.e. the right-looking Cholesky update and the forward substitution L X = I share the
-// broadcast of column j.  Two barriers and at most 128 FMAs per thread per step.
+// broadcast of column j.  One barrier and at most 128 FMAs per thread per step.
 __global__ __launch_bounds__(256) void potrf_diag_kernel(float* __restrict__ Ablk, int lda, int nb,
                                                          float* __restrict__ Dinv, PrepScalars* sc) {
-  __shared__ float colbuf[NB];     // column j of L (zero above the diagonal)
-  __shared__ float rowbuf[NB];     // row j of X = L^-1
-  __shared__ float pivot;
+  #pragma clang fp contract(fast)   // a -= l*l as one FMA; nothing here needs op-by-op rounding
+  __shared__ float colbuf[2][NB];  // unscaled column j of A strictly below the diagonal, zero elsewhere
+  __shared__ float rowbuf[2][NB];  // unscaled row j of B
+  __shared__ float pivbuf[2];      // a_jj
   const int tid = threadIdx.x;
   const int ty = tid >> 4, tx = tid & 15;
   float a[8][8], x[8][8];
@@ -106,54 +108,54 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(float* __restrict__ Abl
       a[ii][cc] = (r < nb && c <= r) ? Ablk[(long long)r * lda + c] : ((r == c) ? 1.0f : 0.0f);   // pad with identity
       x[ii][cc] = (r == c) ? 1.0f : 0.0f;
     }
+  bool bad = false;
   for (int J = 0; J < NB / 8; ++J) {
     if (8 * J >= nb) break;
+    const bool colowner = (tx == J) && (ty >= J), diag = (tx == J) && (ty == J), rowowner = (ty == J);
     #pragma unroll
     for (int jj = 0; jj < 8; ++jj) {
-      const int j = 8 * J + jj;
-      if (ty == J && tx == J) pivot = a[jj][jj];
-      __syncthreads();
-      const float pv = pivot;
-      const float d = sqrtf(pv);
-      const float rinv = 1.0f / d;                      // one division per step; columns scale by multiplication
-      if (tid == 0 && !(pv > 0.0f)) sc->status = 1;
-      if (tx == J && ty >= J) {                       // column j of L
+      const int j = 8 * J + jj, pb = jj & 1;
+      if (colowner) {
+        // rows of the diagonal tile up to and including j publish 0, so consumers need no masks
         #pragma unroll
-        for (int ii = 0; ii < 8; ++ii) {
-          const int r = 8 * ty + ii;
-          float l = 0.0f;
-          if (r == j) l = d;
-          else if (r > j) l = a[ii][jj] * rinv;
-          a[ii][jj] = l;
-          colbuf[r] = l;
-        }
+        for (int ii = 0; ii < 8; ++ii) colbuf[pb][8 * ty + ii] = (diag && ii <= jj) ? 0.0f : a[ii][jj];
+        if (diag) pivbuf[pb] = a[jj][jj];
       }
-      if (ty == J) {                                  // row j of X
+      if (rowowner) {
         #pragma unroll
-        for (int cc = 0; cc < 8; ++cc) {
-          const float v = x[jj][cc] * rinv;
-          x[jj][cc] = v;
-          rowbuf[8 * tx + cc] = v;
-        }
+        for (int cc = 0; cc < 8; ++cc) rowbuf[pb][8 * tx + cc] = x[jj][cc];
       }
       __syncthreads();
+      const float pv = pivbuf[pb];
+      bad = bad || !(pv > 0.0f);
+      float rinv = __builtin_amdgcn_rsqf(pv);         // 1/sqrt(pivot), one Newton step to full precision
+      rinv = rinv * (1.5f - 0.5f * pv * rinv * rinv);
       if (ty >= J) {
         float li[8];
         #pragma unroll
-        for (int ii = 0; ii < 8; ++ii) li[ii] = (8 * ty + ii > j) ? colbuf[8 * ty + ii] : 0.0f;
+        for (int ii = 0; ii < 8; ++ii) li[ii] = colbuf[pb][8 * ty + ii] * rinv;
+        if (colowner) {                               // the owners keep the scaled column: L[:, j]
+          #pragma unroll
+          for (int ii = 0; ii < 8; ++ii) a[ii][jj] = li[ii];
+          if (diag) a[jj][jj] = pv * rinv;
+        }
         if (tx >= J && tx <= ty) {                    // trailing update of A (lower tiles only)
           float lk[8];
           #pragma unroll
-          for (int cc = 0; cc < 8; ++cc) lk[cc] = (8 * tx + cc > j) ? colbuf[8 * tx + cc] : 0.0f;
+          for (int cc = 0; cc < 8; ++cc) lk[cc] = colbuf[pb][8 * tx + cc] * rinv;
           #pragma unroll
           for (int ii = 0; ii < 8; ++ii)
             #pragma unroll
             for (int cc = 0; cc < 8; ++cc) a[ii][cc] -= li[ii] * lk[cc];
         }
-        if (tx <= J) {                                // forward substitution: rows below j of B
+        if (tx <= J) {                                // row j of X = B[j, :] / l_jj, then rows below j of B
           float xr[8];
           #pragma unroll
-          for (int cc = 0; cc < 8; ++cc) xr[cc] = rowbuf[8 * tx + cc];
+          for (int cc = 0; cc < 8; ++cc) xr[cc] = rowbuf[pb][8 * tx + cc] * rinv;
+          if (rowowner) {
+            #pragma unroll
+            for (int cc = 0; cc < 8; ++cc) x[jj][cc] = xr[cc];
+          }
           #pragma unroll
           for (int ii = 0; ii < 8; ++ii)
             #pragma unroll
@@ -162,6 +164,7 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(float* __restrict__ Abl
       }
     }
   }
+  if (bad && tid == 0) sc->status = 1;
   #pragma unroll
   for (int ii = 0; ii < 8; ++ii)
     #pragma unroll
@@ -220,18 +223,31 @@ int lcq_chol_inv_upper(float* H, int64_t K64, const int64_t* perm, float percdam
   }
   build_kernel<<<dim3((unsigned)((K + 255) / 256), (unsigned)K), dim3(256), 0, st>>>(H, K, (const long long*)perm, sc, A);
 
-  // blocked right-looking Cholesky
-  for (int b = 0; b < nblk; ++b) {
-    const int k0 = b * NB, nb = (K - k0 < NB) ? (K - k0) : NB;
-    float* Akk = A + (long long)k0 * K + k0;
-    float* Db = Dinv + (long long)b * NB * NB;
-    potrf_diag_kernel<<<dim3(1), dim3(256), 0, st>>>(Akk, K, nb, Db, sc);
-    const int M = K - k0 - nb;
-    if (M > 0) {
-      float* A21 = A + (long long)(k0 + nb) * K + k0;
-      float* A22 = A + (long long)(k0 + nb) * K + (k0 + nb);
-      launch_gemm<true>(GemmProblem{A21, Db, A21, M, nb, nb, K, NB, K}, 1.0f, 0.0f, 0, st);       // A21 L11^-T
-      launch_gemm<true>(GemmProblem{A21, A21, A22, M, M, nb, K, K, K}, -1.0f, 1.0f, GEMM_LOWER_TILES, st);
+  // Blocked right-looking Cholesky with two block sizes: 128-column panels are factored one by
+  // one, but their trailing update is applied only inside the current 512-column super-panel;
+  // the rest of the matrix is updated once per super-panel with a 512-deep contraction, which
+  // cuts the read-modify-write traffic on the trailing matrix fourfold.
+  constexpr int NBO = 4 * NB;
+  for (int o0 = 0; o0 < K; o0 += NBO) {
+    const int o1 = (o0 + NBO < K) ? (o0 + NBO) : K;
+    for (int k0 = o0; k0 < o1; k0 += NB) {
+      const int b = k0 / NB, nb = (K - k0 < NB) ? (K - k0) : NB;
+      float* Akk = A + (long long)k0 * K + k0;
+      float* Db = Dinv + (long long)b * NB * NB;
+      potrf_diag_kernel<<<dim3(1), dim3(256), 0, st>>>(Akk, K, nb, Db, sc);
+      const int k1 = k0 + nb, M = K - k1;
+      if (M > 0) {
+        float* A21 = A + (long long)k1 * K + k0;
+        launch_gemm<true>(GemmProblem{A21, Db, A21, M, nb, nb, K, NB, K}, 1.0f, 0.0f, 0, st);       // A21 L11^-T
+        if (o1 > k1)                                                                              // inside the super-panel
+          launch_gemm<true>(GemmProblem{A21, A21, A + (long long)k1 * K + k1, M, o1 - k1, nb, K, K, K}, -1.0f, 1.0f,
+                            GEMM_LOWER_TILES, st);
+      }
+    }
+    if (o1 < K) {                                                                                 // everything behind it
+      const float* P = A + (long long)o1 * K + o0;
+      launch_gemm<true>(GemmProblem{P, P, A + (long long)o1 * K + o1, K - o1, K - o1, o1 - o0, K, K, K}, -1.0f, 1.0f,
+                        GEMM_LOWER_TILES, st);
     }
   }
 

@@ -8,8 +8,11 @@
 //        err = (w-q)/d;  W1[:, i:] -= err (x) Hinv1[i, i:];  Err1[:, i] = err
 //     W[:, i2:] -= Err1 @ Hinv[i1:i2, i2:]
 // The reference issues >= 5 tiny launches per column; here one launch runs the
-// 128 sequential columns of a block and one fp32-MFMA launch applies the
-// deferred rank-128 update.
+// 128 sequential columns of a block and fp32-MFMA launches apply the deferred
+// update.  The update entry point takes any (contraction range, column range),
+// so the host can defer a second time: update only the next few blocks after
+// every block and everything behind them once per 1024 columns, which reads
+// and writes the bulk of W eight times less often.
 //
 // Block kernel layout: 16 lanes share one weight row, lane t keeps columns
 // 8t..8t+7 of the block in registers; a wave therefore carries 4 rows and a
@@ -31,7 +34,7 @@ constexpr int ROWS_PER_WG = 16;
 struct LoopArgs {
   float* W; float* tmp; float* Losses; float* Err; const float* U;
   float* scales; float* zeros; const int* gidx;
-  long long R; int K, i1, count, g, G;
+  long long R; int K, i1, count, g, G, ldErr;
   float qmin, qmax;
   int sym, is_static;
 };
@@ -144,7 +147,7 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
       if (col < a.count) {
         a.tmp[rbase + a.i1 + col] = otmp[c];
         a.Losses[rbase + a.i1 + col] = oloss[c];
-        a.Err[row * BS + col] = oerr[c];
+        a.Err[row * a.ldErr + col] = oerr[c];
       }
     }
   }
@@ -154,10 +157,10 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
 
 extern "C" {
 
-int lcq_gptq_block(float* W, float* tmp, float* Losses, float* Err, const float* U, int64_t R, int64_t K, int64_t i1,
-                   int count, int group_size, float qmin, float qmax, int flags, float* scales, float* zeros,
+int lcq_gptq_block(float* W, float* tmp, float* Losses, float* Err, int64_t ldErr, const float* U, int64_t R, int64_t K,
+                   int64_t i1, int count, int group_size, float qmin, float qmax, int flags, float* scales, float* zeros,
                    const int32_t* gidx, int64_t G, void* stream) {
-  if (!W || !tmp || !Losses || !Err || !U || !scales) return LCQ_EINVAL;
+  if (!W || !tmp || !Losses || !Err || !U || !scales || ldErr < count || ldErr > 0x7fffffff) return LCQ_EINVAL;
   if (R <= 0 || K <= 0 || K > 0x7fffffff || i1 < 0 || count <= 0 || count > BS || i1 + count > K) return LCQ_EINVAL;
   if (!(qmax > qmin) || G <= 0) return LCQ_EINVAL;
   const int is_static = (flags & LCQ_FLAG_STATIC) != 0;
@@ -168,20 +171,20 @@ int lcq_gptq_block(float* W, float* tmp, float* Losses, float* Err, const float*
   a.W = W; a.tmp = tmp; a.Losses = Losses; a.Err = Err; a.U = U;
   a.scales = scales; a.zeros = zeros; a.gidx = gidx;
   a.R = R; a.K = (int)K; a.i1 = (int)i1; a.count = count; a.g = group_size; a.G = (int)G;
-  a.qmin = qmin; a.qmax = qmax; a.sym = sym; a.is_static = is_static;
+  a.qmin = qmin; a.qmax = qmax; a.sym = sym; a.is_static = is_static; a.ldErr = (int)ldErr;
   const unsigned grid = (unsigned)((R + ROWS_PER_WG - 1) / ROWS_PER_WG);
   gptq_block_kernel<<<dim3(grid), dim3(256), 0, (hipStream_t)stream>>>(a);
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;
 }
 
-int lcq_gptq_trailing(float* W, const float* Err, const float* U, int64_t R, int64_t K, int64_t i1, int64_t i2,
-                      void* stream) {
+int lcq_gptq_trailing(float* W, const float* Err, int64_t ldErr, const float* U, int64_t R, int64_t K, int64_t k1,
+                      int64_t k2, int64_t j1, int64_t j2, void* stream) {
   if (!W || !Err || !U || R <= 0 || K <= 0 || K > 0x7fffffff || R > 0x7fffffff) return LCQ_EINVAL;
-  if (i1 < 0 || i2 <= i1 || i2 > K || i2 - i1 > BS) return LCQ_EINVAL;
-  if (i2 == K) return LCQ_OK;
-  // W[:, i2:] -= Err[:, :i2-i1] @ U[i1:i2, i2:]
-  GemmProblem g{Err, U + i1 * K + i2, W + i2, (int)R, (int)(K - i2), (int)(i2 - i1), BS, (int)K, (int)K};
+  if (k1 < 0 || k2 <= k1 || k2 > K || j1 < k2 || j2 < j1 || j2 > K || ldErr < k2 - k1 || ldErr > 0x7fffffff) return LCQ_EINVAL;
+  if (j1 == j2) return LCQ_OK;
+  // W[:, j1:j2] -= Err[:, :k2-k1] @ U[k1:k2, j1:j2]
+  GemmProblem g{Err, U + k1 * K + j1, W + j1, (int)R, (int)(j2 - j1), (int)(k2 - k1), (int)ldErr, (int)K, (int)K};
   launch_gemm<false>(g, -1.0f, 1.0f, 0, (hipStream_t)stream);
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;

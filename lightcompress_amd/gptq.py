@@ -25,8 +25,15 @@ import math
 
 import torch
 
+import ctypes
+
 from . import _lib as L
 from .quant import IntegerQuantizer
+
+
+def C_ptr(view):
+    """Device pointer of a (possibly strided) view's first element."""
+    return ctypes.c_void_p(view.data_ptr())
 
 
 class GPTQ:
@@ -245,18 +252,29 @@ class GPTQ:
         if not hasattr(self, '_scales') or self._scales.shape[0] != R:
             raise L.LcqError('weight_transform needs process_hessian_and_weights (or _setup_groups) first')
         flags = (L.FLAG_SYM if wq.sym else 0) | (L.FLAG_STATIC if self._static else 0)
-        Err = torch.empty((R, 128), device=W.device)
+        # Two-level deferral: after every block only the rest of the current 1024-column window is
+        # updated; the columns behind the window get one update per window (8x fewer passes over W).
+        window = 8 * self.blocksize
+        Err = torch.empty((R, window), device=W.device)
         lib = L.lib()
         st = L.stream()
         qmin, qmax = L.f32(wq.qmin), L.f32(wq.qmax)
-        for i1 in range(0, self.n_nonout, self.blocksize):
-            i2 = min(i1 + self.blocksize, self.n_nonout)
-            L.check(lib.lcq_gptq_block(L.ptr(W), L.ptr(tmp), L.ptr(Losses), L.ptr(Err), L.ptr(Hinv), L.i64(R), L.i64(K),
-                                       L.i64(i1), L.i32(i2 - i1), L.i32(self._g), qmin, qmax, L.i32(flags),
-                                       L.ptr(self._scales), L.ptr(self._zeros), L.ptr(self._gidx), L.i64(self._G), st),
-                    'lcq_gptq_block')
-            L.check(lib.lcq_gptq_trailing(L.ptr(W), L.ptr(Err), L.ptr(Hinv), L.i64(R), L.i64(K), L.i64(i1), L.i64(i2),
-                                          st), 'lcq_gptq_trailing')
+        n = self.n_nonout
+        for o0 in range(0, n, window):
+            o1 = min(o0 + window, n)
+            for i1 in range(o0, o1, self.blocksize):
+                i2 = min(i1 + self.blocksize, o1)
+                err_blk = Err[:, i1 - o0:]
+                L.check(lib.lcq_gptq_block(L.ptr(W), L.ptr(tmp), L.ptr(Losses), C_ptr(err_blk), L.i64(window), L.ptr(Hinv),
+                                           L.i64(R), L.i64(K), L.i64(i1), L.i32(i2 - i1), L.i32(self._g), qmin, qmax,
+                                           L.i32(flags), L.ptr(self._scales), L.ptr(self._zeros), L.ptr(self._gidx),
+                                           L.i64(self._G), st), 'lcq_gptq_block')
+                if i2 < o1:
+                    L.check(lib.lcq_gptq_trailing(L.ptr(W), C_ptr(err_blk), L.i64(window), L.ptr(Hinv), L.i64(R), L.i64(K),
+                                                  L.i64(i1), L.i64(i2), L.i64(i2), L.i64(o1), st), 'lcq_gptq_trailing')
+            if o1 < K:
+                L.check(lib.lcq_gptq_trailing(L.ptr(W), L.ptr(Err), L.i64(window), L.ptr(Hinv), L.i64(R), L.i64(K),
+                                              L.i64(o0), L.i64(o1), L.i64(o1), L.i64(K), st), 'lcq_gptq_trailing')
 
     # -- qparam bookkeeping (gptq.py:332-409) ---------------------------------------
     @torch.no_grad()
