@@ -14,6 +14,10 @@ Differences a caller can observe
   * one process / one GPU: the per-call all-reduce of add_batch is not issued;
   * H is kept valid on and above the diagonal only while it accumulates
     (``hessian(name)`` returns the full symmetric matrix);
+  * ``special.hessian_defer`` (default 4) add_batch calls are copied to a staging buffer and
+    folded into one launch, so ``layers_cache[name]['H']`` lags behind ``nsamples`` until
+    ``hessian(name)``, ``hessian_sorting`` or ``process_hessian_and_weights`` settles it
+    (``hessian_defer: 1`` updates H on every call);
   * per-group qparams of the loop live in two [R, G] tensors instead of a
     Python list of dicts; ``layer.buf_scales`` / ``buf_zeros`` get the same
     [R*G, 1] layout the reference writes;
@@ -59,6 +63,8 @@ class GPTQ:
         self.owq = special_config.get('owq', False)
         self.chunk_num = special_config.get('chunk_num', 1)
         self.check_positive_definite = special_config.get('check_positive_definite', True)
+        # add_batch calls folded into one Hessian launch (1 = one launch per call)
+        self.hessian_defer = int(special_config.get('hessian_defer', 4))
         if self.owq:
             raise NotImplementedError('OWQ is not on this path')
         if self.blocksize > 128:
@@ -77,6 +83,9 @@ class GPTQ:
         self.layers_cache.setdefault(name, {})
         self.layers_cache[name]['H'] = torch.zeros((K, K), device=self.dev)
         self.layers_cache[name]['nsamples'] = 0
+        self.layers_cache[name]['n_in_H'] = 0
+        for k in ('stage', 'stage_fill', 'stage_batches'):
+            self.layers_cache[name].pop(k, None)
         self.layers_cache[name]['columns'] = K
         self.layers_cache[name].pop('leader', None)
 
@@ -111,19 +120,64 @@ class GPTQ:
         assert inp.shape[0] % self.chunk_num == 0, \
             f'Error: inp.shape[1] ({inp.shape[0]}) cannot be evenly divided by chunk_num.'
         x = inp.contiguous()
-        n = cache['nsamples']
-        alpha = n / (n + tmp)
-        cache['nsamples'] = n + tmp
-        beta = 2.0 / cache['nsamples']
+        cache['nsamples'] += tmp
+        cache['upper_only'] = True
+        if self.hessian_defer <= 1:
+            self._accumulate(cache, x, tmp)
+            return
+        # Stage a copy of the tokens and fold several calls into one launch: the window
+        # H <- H*n/(n+b1) + 2/(n+b1)*S1, then H <- H*(n+b1)/(n+b1+b2) + 2/(n+b1+b2)*S2, ...
+        # telescopes to H*n/N + (2/N)*(S1+S2+...), N = n + b1 + b2 + ..., so one launch over the
+        # concatenated tokens gives the same H while reading and writing it once.
+        stage = cache.get('stage')
+        if stage is not None and (stage.dtype != x.dtype or cache['stage_fill'] + x.shape[0] > stage.shape[0]):
+            self._flush(cache)
+            if stage.dtype != x.dtype:
+                stage = None
+        if stage is None:
+            stage = torch.empty((self.hessian_defer * x.shape[0], x.shape[1]), dtype=x.dtype, device=x.device)
+            cache['stage'] = stage
+            cache['stage_fill'] = 0
+            cache['stage_batches'] = 0
+        if x.shape[0] > stage.shape[0]:
+            self._accumulate(cache, x, tmp)
+            return
+        f = cache['stage_fill']
+        stage[f:f + x.shape[0]].copy_(x)
+        cache['stage_fill'] = f + x.shape[0]
+        cache['stage_batches'] += tmp
+        if cache['stage_fill'] == stage.shape[0]:
+            self._flush(cache)
+
+    def _accumulate(self, cache, x, batches):
+        """H <- H*n/(n+b) + 2/(n+b) * x^T x for the n batches already inside H (gptq.py:279-294)."""
+        n = cache.get('n_in_H', 0)
+        alpha = n / (n + batches)
+        beta = 2.0 / (n + batches)
+        cache['n_in_H'] = n + batches
         H = cache['H']
         L.check(L.lib().lcq_hessian_accum(L.ptr(H), L.i64(H.shape[0]), L.ptr(x), L.i32(L.dtype_code(x.dtype)),
                                           L.i64(x.shape[0]), L.f32(alpha), L.f32(beta), L.stream()),
                 'lcq_hessian_accum')
-        cache['upper_only'] = True
+
+    def _flush(self, cache):
+        """Fold the staged tokens into H."""
+        if cache.get('stage_fill', 0) > 0:
+            self._accumulate(cache, cache['stage'][:cache['stage_fill']], cache['stage_batches'])
+            cache['stage_fill'] = 0
+            cache['stage_batches'] = 0
+
+    def _settle(self, name):
+        """H of `name` (or of the layer it aliases) with no tokens left in staging."""
+        cache = self.layers_cache[name]
+        lead = self.layers_cache.get(cache.get('leader', name), cache)
+        self._flush(lead)
+        lead.pop('stage', None)
+        return cache
 
     def hessian(self, name):
         """The full symmetric H of a layer (fills the lower triangle on demand)."""
-        cache = self.layers_cache[name]
+        cache = self._settle(name)
         H = cache['H']
         if cache.get('upper_only', False) or self.layers_cache.get(cache.get('leader', name), {}).get('upper_only'):
             L.check(L.lib().lcq_symmetrize(L.ptr(H), L.i64(H.shape[0]), L.stream()), 'lcq_symmetrize')
@@ -132,7 +186,7 @@ class GPTQ:
 
     def hessian_sorting(self, name):
         """gptq.py:58-64: act-order permutation from the raw diagonal."""
-        H = self.layers_cache[name]['H']
+        H = self._settle(name)['H']
         if self.actorder:
             self.perm = torch.argsort(torch.diag(H), descending=True)
 
@@ -169,7 +223,7 @@ class GPTQ:
             W = W.flatten(1)
         W = W.float().contiguous()
         R, K = W.shape
-        cache = self.layers_cache[name]
+        cache = self._settle(name) if 'H' in self.layers_cache[name] else self.layers_cache[name]
         leader = cache.get('leader', name)
         H = cache['H']
         del cache['H']

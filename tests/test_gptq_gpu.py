@@ -73,6 +73,38 @@ def test_hessian_batched_call_and_fp16(dev):
     assert float((H - ref).abs().max() / ref.abs().max()) < 1e-5
 
 
+@pytest.mark.parametrize('defer', [1, 3, 4])
+def test_hessian_deferred_launches(dev, defer):
+    """Folding several add_batch calls into one launch leaves H and nsamples as per-call updates do,
+    for ragged token counts and for inputs the caller overwrites right after the call."""
+    K = 320
+    shapes = [(1, 96), (2, 96), (1, 96), (1, 40), (1, 96), (3, 64), (1, 96), (1, 700), (1, 96)]
+    g = make_gptq(hessian_defer=defer)
+    layer = Layer(torch.zeros(8, K, device=dev))
+    g.layers_cache['l'] = {}
+    g.layer_init(layer, 'l')
+    Ho = torch.zeros(K, K)
+    n = 0
+    flat = []
+    for i, (b, T) in enumerate(shapes):
+        x = calib_batches(b, T, K, seed=1200 + i)
+        xb = torch.stack(x)
+        xd = xb.to(dev)
+        g.add_batch(layer, 'l', xd, None)
+        xd.zero_()                                  # the staged copy must not alias the caller's tensor
+        n = G.add_batch(Ho, n, xb)
+        flat.append(xb)
+        assert g.layers_cache['l']['nsamples'] == n
+    H = g.hessian('l').cpu()
+    scale = float(Ho.abs().max())
+    assert float((H - Ho).abs().max()) / scale < 1e-5
+    assert torch.equal(H, H.t())
+    # closed form: (2 / n) * sum_i X_i^T X_i over every token
+    X = torch.cat([f.reshape(-1, K) for f in flat]).double()
+    ref = (2.0 / n) * X.t() @ X
+    assert float((H.double() - ref).abs().max() / ref.abs().max()) < 1e-5
+
+
 def _chain_inputs(K, seed, dead=()):
     H = G.hessian_closed_form(calib_batches(4, max(64, K // 4), K, seed=seed)).float()
     for j in dead:
