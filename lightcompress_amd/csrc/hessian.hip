@@ -11,16 +11,20 @@
 // Shape of the kernel
 //  * one 256-thread workgroup (4 waves, 2x2) per 256x128 tile of H; each wave
 //    owns 128x64 = 4x2 blocks of v_mfma_f32_32x32x16 (128 accumulator
-//    registers per lane).  Two workgroups fit a CU (registers and 56 KiB of
+//    registers per lane).  Two workgroups fit a CU (registers and 72 KiB of
 //    LDS each), so one tile's epilogue / barriers overlap the other's MFMAs;
 //  * H is symmetric: only tiles that touch the upper triangle are computed
 //    (the lower triangle is filled once, when H is consumed, by lcq_symmetrize);
-//  * X is streamed 32 tokens at a time through double-buffered LDS in its
-//    natural [token][feature] layout; the feature-major operand layout MFMA
-//    needs (8 consecutive tokens per lane) is produced by the LDS transpose
-//    read ds_read_b64_tr_b16, so no VALU shuffles are spent on the transpose;
-//  * LDS rows are padded by 64 bytes so the four token rows a transpose read
-//    touches fall into different banks.
+//  * X is streamed 32 tokens at a time through three LDS stages in its natural
+//    [token][feature] layout by direct global->LDS loads
+//    (global_load_lds_dwordx4): no staging registers, no LDS store
+//    instructions, one barrier per 32 tokens, two slabs of loads in flight;
+//  * the feature-major operand layout MFMA needs (8 consecutive tokens per
+//    lane) is produced by the LDS transpose read ds_read_b64_tr_b16, so no
+//    VALU shuffles are spent on the transpose;
+//  * a direct load deposits a wave's 1 KiB contiguously, so LDS rows cannot be
+//    padded; the four token rows a transpose read touches are kept in
+//    different banks by an XOR swizzle of the 64-byte blocks of each row.
 #include "common.h"
 #include "lcq_internal.h"
 
@@ -35,10 +39,16 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 constexpr int TM = 256;                   // H tile rows (A operand: 256 features)
 constexpr int TN = 128;                   // H tile columns (B operand: 128 features)
 constexpr int BT = 32;                    // tokens per LDS stage
-constexpr int PITCH_A = TM * 2 + 64;      // bytes per token row in LDS
-constexpr int PITCH_B = TN * 2 + 64;
-constexpr int BYTES_A = BT * PITCH_A, BYTES_B = BT * PITCH_B;
-constexpr int STAGE_BYTES = BYTES_A + BYTES_B;
+constexpr int ROW_A = TM * 2, ROW_B = TN * 2;             // bytes per token row in LDS (no padding)
+constexpr int BYTES_A = BT * ROW_A, BYTES_B = BT * ROW_B;
+constexpr int STAGE_BYTES = BYTES_A + BYTES_B;            // 24 KiB
+constexpr int NSTAGE = 3;
+
+// source of the 16-byte pieces that lie outside X (ragged K or T): they must read as zero
+__device__ __attribute__((aligned(16))) const uint32_t zero_piece[4] = {0, 0, 0, 0};
+
+typedef const __attribute__((address_space(1))) void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
 
 __device__ __forceinline__ s16x4 lds_tr_read(const char* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p));
@@ -58,87 +68,109 @@ __device__ __forceinline__ f32x16 mfma(const s16x8& a, const s16x8& b, const f32
 // contiguous range of a tile order in which consecutive tiles form 4x8 super-blocks: the tiles
 // an XCD works on at one time then share a handful of column stripes of X.
 constexpr int SB_R = 4, SB_C = 8;
-__device__ __forceinline__ bool decode_tile(int v, int ntr, int ntc, int& ti, int& tj) {
-  for (int r0 = 0; r0 < ntr; r0 += SB_R) {
-    const int r1 = min(r0 + SB_R, ntr);
-    for (int c0 = (2 * r0 / SB_C) * SB_C; c0 < ntc; c0 += SB_C) {
-      const int c1 = min(c0 + SB_C, ntc);
-      int cnt = 0;
-      for (int r = r0; r < r1; ++r) cnt += max(0, c1 - max(c0, 2 * r));
-      if (v < cnt) {
-        for (int r = r0; r < r1; ++r) {
-          const int lo = max(c0, 2 * r), n = max(0, c1 - lo);
-          if (v < n) { ti = r; tj = lo + v; return true; }
-          v -= n;
-        }
-      }
-      v -= cnt;
-    }
+__device__ __forceinline__ void decode_tile(int v, int ntr, int ntc, int& ti, int& tj) {
+  // super-row by bisection: the tile rows before row r0 hold r0*ntc - r0*(r0-1) tiles.  (The map is
+  // evaluated by every workgroup, so it has to cost a few dozen scalar instructions, not a scan.)
+  int lo = 0, hi = (ntr - 1) / SB_R;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1, r0 = mid * SB_R;
+    if (r0 * ntc - r0 * (r0 - 1) <= v) lo = mid; else hi = mid - 1;
   }
-  return false;
+  const int r0 = lo * SB_R, nr = min(SB_R, ntr - r0);
+  v -= r0 * ntc - r0 * (r0 - 1);
+  // first super-column starts on the diagonal (2*r0 is a multiple of SB_C) and is clipped by it
+  int c0 = 2 * r0;
+  {
+    const int c1 = min(c0 + SB_C, ntc);
+    for (int r = r0; r < r0 + nr; ++r) {
+      const int n = max(0, c1 - 2 * r);
+      if (v < n) { ti = r; tj = 2 * r + v; return; }
+      v -= n;
+    }
+    c0 += SB_C;
+  }
+  // the other super-columns are full rectangles nr x SB_C, the last one nr x (ntc - c0)
+  const int q = min(v / (nr * SB_C), (ntc - c0 - 1) / SB_C);
+  v -= q * nr * SB_C;
+  c0 += q * SB_C;
+  const int w = min(SB_C, ntc - c0);
+  ti = r0 + v / w;
+  tj = c0 + v % w;
 }
 
-// EDGE = false: K % 256 == 0 and T % 64 == 0, no bounds checks anywhere.
+// EDGE = false: K % 256 == 0 and T % 32 == 0, no bounds checks anywhere.
 template <bool IS_BF16, bool EDGE>
 __global__ __launch_bounds__(256, 2) void hessian_kernel(float* __restrict__ H, int K, const uint16_t* __restrict__ X,
                                                          int T, float alpha, float beta, int ntr, int ntc, int total) {
-  __shared__ __attribute__((aligned(16))) char lds[2 * STAGE_BYTES];
+  __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE_BYTES];
   int ti = 0, tj = 0;
   {
     const int per_xcd = (total + 7) / 8;
     const int slot = blockIdx.x >> 3, xcd = blockIdx.x & 7;
-    if (slot >= per_xcd || !decode_tile(xcd * per_xcd + slot, ntr, ntc, ti, tj)) return;
+    if (slot >= per_xcd || xcd * per_xcd + slot >= total) return;
+    decode_tile(xcd * per_xcd + slot, ntr, ntc, ti, tj);
   }
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wr = wave >> 1, wc = wave & 1;
 
-  // global -> LDS staging.  A: 32 threads per 512-byte token row, 8 rows per pass, 4 passes;
-  // B: 16 threads per 256-byte token row, 16 rows per pass, 2 passes.  Per-thread element offsets
-  // inside a 32-token slab are 32-bit; the slab base is uniform.
-  const int a_row = tid >> 5, a_c16 = tid & 31, b_row = tid >> 4, b_c16 = tid & 15;
-  const int colA = ti * TM + a_c16 * 8, colB = tj * TN + b_c16 * 8;
-  const bool okA = colA < K, okB = colB < K;
+  // global -> LDS: direct loads (global_load_lds_dwordx4), no staging registers.  One wave
+  // instruction deposits 64 x 16 bytes CONTIGUOUSLY in LDS (lane l at +16 l) from per-lane global
+  // addresses: 2 token rows of the A operand (512 B each) or 4 of the B operand (256 B each).
+  // LDS rows are unpadded; bank conflicts of the transpose reads (which touch token rows r..r+3 at
+  // one 64-byte feature block) are avoided by an XOR swizzle instead: 64-byte block c of token row
+  // r is stored at block c ^ (r & 3).  The swizzle is applied on the global side (which piece a
+  // lane fetches), the LDS side stays contiguous.  Wave w loads A rows 8w..8w+7 and B rows 8w..8w+7.
   uint32_t gofA[4], gofB[2];
+  bool okA[4], okB[2];
   #pragma unroll
-  for (int p = 0; p < 4; ++p) gofA[p] = (uint32_t)((p * 8 + a_row) * K + colA);
+  for (int p = 0; p < 4; ++p) {
+    const int r = 8 * wave + 2 * p + (lane >> 5);
+    const int col = ti * TM + (((lane & 31) ^ ((r & 3) << 2)) * 8);
+    gofA[p] = (uint32_t)(r * K + col);
+    okA[p] = col < K;
+  }
   #pragma unroll
-  for (int p = 0; p < 2; ++p) gofB[p] = (uint32_t)((p * 16 + b_row) * K + colB);
-  u32x4 sA0[4], sB0[2], sA1[4], sB1[2];     // two slabs of global loads stay in flight
-
-  auto gload = [&](int t0, u32x4* sa, u32x4* sb) {
+  for (int p = 0; p < 2; ++p) {
+    const int r = 8 * wave + 4 * p + (lane >> 4);
+    const int col = tj * TN + (((lane & 15) ^ ((r & 3) << 2)) * 8);
+    gofB[p] = (uint32_t)(r * K + col);
+    okB[p] = col < K;
+  }
+  // The loads are issued from inline assembly: the compiler would otherwise wait for ALL direct
+  // loads (vmcnt(0)) before any LDS read, which serialises the pipeline.  Waits are explicit below.
+  const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
+  auto gload = [&](int t0, int stage) {
     const uint16_t* Xs = X + (int64_t)t0 * K;
+    const uint32_t dA = lds0 + stage * STAGE_BYTES + wave * 8 * ROW_A;
+    const uint32_t dB = lds0 + stage * STAGE_BYTES + BYTES_A + wave * 8 * ROW_B;
     #pragma unroll
-    for (int p = 0; p < 4; ++p) {
+    for (int p = 0; p < 6; ++p) {
+      const bool isA = p < 4;
+      const uint32_t dst = isA ? dA + p * 2 * ROW_A : dB + (p - 4) * 4 * ROW_B;
+      const uint32_t gof = isA ? gofA[p] : gofB[p - 4];
       if constexpr (EDGE) {
-        sa[p] = u32x4{0, 0, 0, 0};
-        if (okA && t0 + p * 8 + a_row < T) sa[p] = *(const u32x4*)(Xs + gofA[p]);
-      } else sa[p] = *(const u32x4*)(Xs + gofA[p]);
+        const int r = isA ? 8 * wave + 2 * p + (lane >> 5) : 8 * wave + 4 * (p - 4) + (lane >> 4);
+        const bool ok = (isA ? okA[p] : okB[p - 4]) && t0 + r < T;
+        const uint16_t* g = ok ? Xs + gof : (const uint16_t*)zero_piece;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(g) : "memory");
+      } else {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(gof * 2u), "s"(Xs) : "memory");
+      }
     }
-    #pragma unroll
-    for (int p = 0; p < 2; ++p) {
-      if constexpr (EDGE) {
-        sb[p] = u32x4{0, 0, 0, 0};
-        if (okB && t0 + p * 16 + b_row < T) sb[p] = *(const u32x4*)(Xs + gofB[p]);
-      } else sb[p] = *(const u32x4*)(Xs + gofB[p]);
-    }
-  };
-  char* const stA = lds + a_row * PITCH_A + a_c16 * 16;
-  char* const stB = lds + BYTES_A + b_row * PITCH_B + b_c16 * 16;
-  auto lstore = [&](int buf, const u32x4* sa, const u32x4* sb) {
-    #pragma unroll
-    for (int p = 0; p < 4; ++p) *(u32x4*)(stA + buf * STAGE_BYTES + p * 8 * PITCH_A) = sa[p];
-    #pragma unroll
-    for (int p = 0; p < 2; ++p) *(u32x4*)(stB + buf * STAGE_BYTES + p * 16 * PITCH_B) = sb[p];
   };
 
-  // transpose-read lane addressing (see file header): a group of 16 lanes reads a
-  // 4(token) x 16(feature) block; lane s supplies row s/4, features 4*(s%4)..+3 and
-  // receives tokens 0..3 of feature s.
+  // transpose-read lane addressing: a group of 16 lanes reads a 4(token) x 16(feature) block;
+  // lane s supplies row s/4, features 4*(s%4)..+3 and receives tokens 0..3 of feature s.
+  // Every row a lane addresses has (row & 3) == L >> 2, so its swizzled block offsets are fixed.
   const int L = lane & 15, g16 = (lane >> 4) & 1, kh = lane >> 5;
-  const int fcol = (g16 * 16 + (L & 3) * 4) * 2, frow = kh * 8 + (L >> 2);
-  const char* const rdA = lds + frow * PITCH_A + fcol + wr * 128 * 2;
-  const char* const rdB = lds + BYTES_A + frow * PITCH_B + fcol + wc * 64 * 2;
+  const int fcol = (g16 * 16 + (L & 3) * 4) * 2, frow = kh * 8 + (L >> 2), sw = L >> 2;
+  int offA[4], offB[2];
+  #pragma unroll
+  for (int b = 0; b < 4; ++b) offA[b] = frow * ROW_A + (wr * 4 + (b ^ sw)) * 64 + fcol;
+  #pragma unroll
+  for (int j = 0; j < 2; ++j) offB[j] = BYTES_A + frow * ROW_B + ((wc * 2 + j) ^ sw) * 64 + fcol;
 
   f32x16 acc[4][2];
   #pragma unroll
@@ -148,22 +180,21 @@ __global__ __launch_bounds__(256, 2) void hessian_kernel(float* __restrict__ H, 
       #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  auto compute = [&](int buf) {
-    const char* tA = rdA + buf * STAGE_BYTES;
-    const char* tB = rdB + buf * STAGE_BYTES;
+  auto compute = [&](int stage) {
+    const char* const base = lds + stage * STAGE_BYTES;
     #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
       s16x8 fa[4];
       #pragma unroll
       for (int b = 0; b < 4; ++b) {
-        const s16x4 a0 = lds_tr_read(tA + ks * 16 * PITCH_A + b * 64);
-        const s16x4 a1 = lds_tr_read(tA + ks * 16 * PITCH_A + 4 * PITCH_A + b * 64);
+        const s16x4 a0 = lds_tr_read(base + offA[b] + ks * 16 * ROW_A);
+        const s16x4 a1 = lds_tr_read(base + offA[b] + ks * 16 * ROW_A + 4 * ROW_A);
         fa[b] = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
       }
       #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        const s16x4 b0 = lds_tr_read(tB + ks * 16 * PITCH_B + j * 64);
-        const s16x4 b1 = lds_tr_read(tB + ks * 16 * PITCH_B + 4 * PITCH_B + j * 64);
+        const s16x4 b0 = lds_tr_read(base + offB[j] + ks * 16 * ROW_B);
+        const s16x4 b1 = lds_tr_read(base + offB[j] + ks * 16 * ROW_B + 4 * ROW_B);
         const s16x8 fb = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7);
         #pragma unroll
         for (int i = 0; i < 4; ++i) acc[i][j] = mfma<IS_BF16>(fa[i], fb, acc[i][j]);
@@ -171,26 +202,23 @@ __global__ __launch_bounds__(256, 2) void hessian_kernel(float* __restrict__ H, 
     }
   };
 
-  // slabs are processed in pairs; a ragged tail is zero-filled by the EDGE loads
-  const int nsteps = ((T + 2 * BT - 1) / (2 * BT)) * 2;
-  gload(0, sA0, sB0);
-  gload(BT, sA1, sB1);
-  lstore(0, sA0, sB0);
-  __syncthreads();
-  for (int s = 0; s + 2 < nsteps; s += 2) {
-    gload((s + 2) * BT, sA0, sB0);
-    compute(0);
-    lstore(1, sA1, sB1);
+  // Three LDS stages, one barrier per 32-token slab.  At the top of step s a wave waits for its
+  // own loads of slab s (those of slab s+1 may stay in flight), the barrier then makes every
+  // wave's part of slab s visible and proves that all waves are done reading slab s-1, whose stage
+  // the loads of slab s+2 overwrite.
+  const int nsteps = (T + BT - 1) / BT;
+  gload(0, 0);
+  if (nsteps > 1) gload(BT, 1);
+  int cur = 0, nxt2 = 2;
+  for (int s = 0; s < nsteps; ++s) {
+    if (s + 1 < nsteps) __builtin_amdgcn_s_waitcnt(0x0F76);     // vmcnt(6)
+    else __builtin_amdgcn_s_waitcnt(0x0F70);                    // vmcnt(0)
     __syncthreads();
-    gload((s + 3) * BT, sA1, sB1);
-    compute(1);
-    lstore(0, sA0, sB0);
-    __syncthreads();
+    if (s + 2 < nsteps) gload((s + 2) * BT, nxt2);
+    compute(cur);
+    cur = (cur == NSTAGE - 1) ? 0 : cur + 1;
+    nxt2 = (nxt2 == NSTAGE - 1) ? 0 : nxt2 + 1;
   }
-  compute(0);
-  lstore(1, sA1, sB1);
-  __syncthreads();
-  compute(1);
 
   // epilogue: accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32.
   // The old values of two 32-row bands (64 per lane) are fetched before any is used so the
@@ -260,7 +288,7 @@ int lcq_hessian_accum(float* H, int64_t K, const void* X, int dtype, int64_t T, 
   for (int r = 0; r < ntr; ++r) total += (ntc - 2 * r > 0) ? (ntc - 2 * r) : 0;
   const int64_t grid = (total + 7) / 8 * 8;                       // 8 XCD queues of equal length
   hipStream_t st = (hipStream_t)stream;
-  const bool edge = (K % TM != 0) || (T % (2 * BT) != 0);
+  const bool edge = (K % TM != 0) || (T % BT != 0);
   #define LCQ_HESS(BF, E) hessian_kernel<BF, E><<<dim3((unsigned)grid), dim3(256), 0, st>>>(H, (int)K, (const uint16_t*)X, (int)T, alpha, beta, ntr, ntc, (int)total)
   if (dtype == LCQ_BF16) { if (edge) LCQ_HESS(true, true); else LCQ_HESS(true, false); }
   else if (dtype == LCQ_F16) { if (edge) LCQ_HESS(false, true); else LCQ_HESS(false, false); }
