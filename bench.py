@@ -129,9 +129,9 @@ def gpu_main(args):
     TL = FOLD * TOK
     def hess(b):
         b = (b * FOLD) % (NB - FOLD + 1)
-        L.check(lib.lcq_hessian_accum(L.ptr(H), L.i64(K), L.ptr(x[b]), L.i32(L.BF16), L.i64(TL), L.f32(0.5),
+        L.check(lib.lcq_hessian_accum(L.ptr(H), L.i64(K), L.ptr(x[b]), L.i32(L.BF16), L.i64(TL), L.i64(K), L.f32(0.5),
                                       L.f32(0.01), st), 'hessian')
-    for b in range(4):
+    for b in range(16):
         hess(b)
     n_launch = 32
     a, b_ = ev(), ev()
@@ -141,7 +141,7 @@ def gpu_main(args):
     b_.record(); torch.cuda.synchronize()
     t_h = a.elapsed_time(b_) * 1e-3 / n_launch
     alg_flops = 2.0 * TL * K * K
-    tiles = sum(K // 128 - 2 * ti for ti in range(K // 256))          # 256x128 tiles on or above the diagonal
+    tiles = sum(K // 128 - 2 * ti for ti in range(K // 256))          # 256x128 tiles that reach the upper triangle
     exe_flops = 2.0 * TL * tiles * 256 * 128
     roofline = {'kernel': f'hessian_kernel<bf16> K=14336 T={TL}', 'bound': 'mfma', 'achieved': round(alg_flops / t_h / 1e12, 2),
                 'peak': 2500.0, 'unit': 'TFLOP/s', 'frac': round(alg_flops / t_h / 2.5e15, 4), 'traffic': None,

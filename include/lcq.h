@@ -127,10 +127,12 @@ int lcq_pack_awq(const void* w, int dtype, const void* scales, const int32_t* ze
 
 /* GPTQ.add_batch, gptq.py:253-295:  H <- alpha*H + beta * X^T X  with
  * alpha = n/(n+b), beta = 2/(n+b) (n = batches seen so far, b = batches in this call).
- *  H [K, K] fp32; X [T, K] tokens x in_features of LCQ_BF16 | LCQ_F16, 16-byte aligned; K % 8 == 0.
- * Only the 256x128 tiles that reach the upper triangle are updated: call
- * lcq_symmetrize before reading anything below the diagonal. alpha == 0 does not read H. */
-int lcq_hessian_accum(float* H, int64_t K, const void* X, int dtype, int64_t T, float alpha, float beta, void* stream);
+ *  H [K, K] fp32; X [T, K] tokens x in_features of LCQ_BF16 | LCQ_F16, 16-byte aligned; K % 8 == 0;
+ *  ldx = elements between consecutive token rows (>= K, % 8 == 0).
+ * Only the tiles that reach the upper triangle are updated: call lcq_symmetrize before reading
+ * anything below the diagonal. alpha == 0 does not read H. */
+int lcq_hessian_accum(float* H, int64_t K, const void* X, int dtype, int64_t T, int64_t ldx, float alpha, float beta,
+                      void* stream);
 
 /* H[j][i] = H[i][j] for i < j. */
 int lcq_symmetrize(float* H, int64_t K, void* stream);

@@ -9,13 +9,16 @@
 // GEMM differs from the reference's fp32 SGEMM only in summation order.
 //
 // Shape of the kernel
-//  * one 256-thread workgroup (4 waves, 2x2) per 256x128 tile of H; each wave
-//    owns 128x64 = 4x2 blocks of v_mfma_f32_32x32x16 (128 accumulator
-//    registers per lane).  Two workgroups fit a CU (registers and 72 KiB of
-//    LDS each), so one tile's epilogue / barriers overlap the other's MFMAs;
+//  * a workgroup owns a 256 x TN tile of H, TN = 128: 4 waves (2 x 2), two
+//    workgroups per CU, so one tile's barriers and epilogue overlap the other's
+//    MFMAs.  (The template also covers TN = 256 - 8 waves, one workgroup
+//    per CU, a third less operand traffic - which measured 5 % slower at
+//    K = 14336 because nothing overlaps its barriers and epilogue.)  Each wave
+//    owns 128x64 = 4x2 blocks of v_mfma_f32_32x32x16 (128 accumulator registers
+//    per lane);
 //  * H is symmetric: only tiles that touch the upper triangle are computed
 //    (the lower triangle is filled once, when H is consumed, by lcq_symmetrize);
-//  * X is streamed 32 tokens at a time through three LDS stages in its natural
+//  * X is streamed 32 tokens at a time through 3-4 LDS stages in its natural
 //    [token][feature] layout by direct global->LDS loads
 //    (global_load_lds_dwordx4): no staging registers, no LDS store
 //    instructions, one barrier per 32 tokens, two slabs of loads in flight;
@@ -37,18 +40,12 @@ typedef __attribute__((ext_vector_type(8))) short s16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
 constexpr int TM = 256;                   // H tile rows (A operand: 256 features)
-constexpr int TN = 128;                   // H tile columns (B operand: 128 features)
 constexpr int BT = 32;                    // tokens per LDS stage
-constexpr int ROW_A = TM * 2, ROW_B = TN * 2;             // bytes per token row in LDS (no padding)
-constexpr int BYTES_A = BT * ROW_A, BYTES_B = BT * ROW_B;
-constexpr int STAGE_BYTES = BYTES_A + BYTES_B;            // 24 KiB
-constexpr int NSTAGE = 3;
+constexpr int ROW_A = TM * 2;             // bytes per token row of the A operand in LDS (no padding)
+constexpr int BYTES_A = BT * ROW_A;
 
 // source of the 16-byte pieces that lie outside X (ragged K or T): they must read as zero
 __device__ __attribute__((aligned(16))) const uint32_t zero_piece[4] = {0, 0, 0, 0};
-
-typedef const __attribute__((address_space(1))) void* gptr_t;
-typedef __attribute__((address_space(3))) void* lptr_t;
 
 __device__ __forceinline__ s16x4 lds_tr_read(const char* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p));
@@ -62,29 +59,30 @@ __device__ __forceinline__ f32x16 mfma(const s16x8& a, const s16x8& b, const f32
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
 }
 
-// Workgroup -> tile map.  Tile (ti, tj) covers rows [256 ti, +256) and columns [128 tj, +128);
-// it is needed when it reaches the upper triangle: tj >= 2 ti.  Workgroups are handed to the 8
-// XCDs round-robin (block b runs on XCD b % 8) and each XCD has its own L2, so every XCD gets a
-// contiguous range of a tile order in which consecutive tiles form 4x8 super-blocks: the tiles
-// an XCD works on at one time then share a handful of column stripes of X.
-constexpr int SB_R = 4, SB_C = 8;
+// Workgroup -> tile map.  Tile (ti, tj) covers rows [256 ti, +256) and columns [TN tj, +TN); with
+// Q = 256 / TN it is needed when it reaches the upper triangle: tj >= Q ti.  Workgroups are handed
+// to the 8 XCDs round-robin (block b runs on XCD b % 8) and each XCD has its own L2, so every XCD
+// gets a contiguous range of a tile order in which consecutive tiles form super-blocks of 4 tile
+// rows x 4Q tile columns: the tiles an XCD works on at one time then share a handful of column
+// stripes of X.  The map is evaluated by every workgroup, so it is closed-form, not a scan.
+template <int Q>
 __device__ __forceinline__ void decode_tile(int v, int ntr, int ntc, int& ti, int& tj) {
-  // super-row by bisection: the tile rows before row r0 hold r0*ntc - r0*(r0-1) tiles.  (The map is
-  // evaluated by every workgroup, so it has to cost a few dozen scalar instructions, not a scan.)
+  constexpr int SB_R = 4, SB_C = 4 * Q;
+  // super-row by bisection: the tile rows before row r0 hold r0*ntc - Q*r0*(r0-1)/2 tiles
   int lo = 0, hi = (ntr - 1) / SB_R;
   while (lo < hi) {
     const int mid = (lo + hi + 1) >> 1, r0 = mid * SB_R;
-    if (r0 * ntc - r0 * (r0 - 1) <= v) lo = mid; else hi = mid - 1;
+    if (r0 * ntc - Q * (r0 * (r0 - 1) / 2) <= v) lo = mid; else hi = mid - 1;
   }
   const int r0 = lo * SB_R, nr = min(SB_R, ntr - r0);
-  v -= r0 * ntc - r0 * (r0 - 1);
-  // first super-column starts on the diagonal (2*r0 is a multiple of SB_C) and is clipped by it
-  int c0 = 2 * r0;
+  v -= r0 * ntc - Q * (r0 * (r0 - 1) / 2);
+  // first super-column starts on the diagonal (Q*r0 is a multiple of SB_C) and is clipped by it
+  int c0 = Q * r0;
   {
     const int c1 = min(c0 + SB_C, ntc);
     for (int r = r0; r < r0 + nr; ++r) {
-      const int n = max(0, c1 - 2 * r);
-      if (v < n) { ti = r; tj = 2 * r + v; return; }
+      const int n = max(0, c1 - Q * r);
+      if (v < n) { ti = r; tj = Q * r + v; return; }
       v -= n;
     }
     c0 += SB_C;
@@ -98,61 +96,79 @@ __device__ __forceinline__ void decode_tile(int v, int ntr, int ntc, int& ti, in
   tj = c0 + v % w;
 }
 
+template <int TN> struct HessCfg {
+  static constexpr int NW = 2 * TN / 64;                 // waves: 2 x TN/64
+  static constexpr int ROW_B = TN * 2;                   // bytes per token row of the B operand
+  static constexpr int STAGE = BYTES_A + BT * ROW_B;
+  static constexpr int NSTAGE = (TN == 256) ? 4 : 3;     // 128 KiB (one workgroup per CU) / 72 KiB (two)
+  static constexpr int LA = 16 / NW;                     // A wave-loads per wave and slab (2 token rows each)
+  static constexpr int RB = 1024 / ROW_B;                // token rows per B wave-load
+  static constexpr int LB = (BT / RB) / NW;              // B wave-loads per wave and slab
+  static constexpr int NL = LA + LB;
+};
+
 // EDGE = false: K % 256 == 0 and T % 32 == 0, no bounds checks anywhere.
-template <bool IS_BF16, bool EDGE>
-__global__ __launch_bounds__(256, 2) void hessian_kernel(float* __restrict__ H, int K, const uint16_t* __restrict__ X,
-                                                         int T, float alpha, float beta, int ntr, int ntc, int total) {
-  __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE_BYTES];
+template <bool IS_BF16, bool EDGE, int TN>
+__global__ __launch_bounds__(HessCfg<TN>::NW * 64, TN == 256 ? 1 : 2)
+void hessian_kernel(float* __restrict__ H, int K, const uint16_t* __restrict__ X, int ldx, int T, float alpha,
+                    float beta, int ntr, int ntc, int total) {
+  using C = HessCfg<TN>;
+  constexpr int ROW_B = C::ROW_B, STAGE = C::STAGE, NSTAGE = C::NSTAGE, LA = C::LA, LB = C::LB, RB = C::RB;
+  __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE];
   int ti = 0, tj = 0;
   {
     const int per_xcd = (total + 7) / 8;
     const int slot = blockIdx.x >> 3, xcd = blockIdx.x & 7;
     if (slot >= per_xcd || xcd * per_xcd + slot >= total) return;
-    decode_tile(xcd * per_xcd + slot, ntr, ntc, ti, tj);
+    decode_tile<TM / TN>(xcd * per_xcd + slot, ntr, ntc, ti, tj);
   }
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wr = wave >> 1, wc = wave & 1;
+  const int wr = wave / (TN / 64), wc = wave % (TN / 64);
 
   // global -> LDS: direct loads (global_load_lds_dwordx4), no staging registers.  One wave
   // instruction deposits 64 x 16 bytes CONTIGUOUSLY in LDS (lane l at +16 l) from per-lane global
-  // addresses: 2 token rows of the A operand (512 B each) or 4 of the B operand (256 B each).
+  // addresses: 2 token rows of a 512-byte-wide operand or 4 of a 256-byte-wide one.
   // LDS rows are unpadded; bank conflicts of the transpose reads (which touch token rows r..r+3 at
   // one 64-byte feature block) are avoided by an XOR swizzle instead: 64-byte block c of token row
   // r is stored at block c ^ (r & 3).  The swizzle is applied on the global side (which piece a
-  // lane fetches), the LDS side stays contiguous.  Wave w loads A rows 8w..8w+7 and B rows 8w..8w+7.
-  uint32_t gofA[4], gofB[2];
-  bool okA[4], okB[2];
+  // lane fetches), the LDS side stays contiguous.
+  uint32_t gofA[LA], gofB[LB];
+  bool okA[LA], okB[LB];
+  int rowA[LA], rowB[LB];
   #pragma unroll
-  for (int p = 0; p < 4; ++p) {
-    const int r = 8 * wave + 2 * p + (lane >> 5);
+  for (int p = 0; p < LA; ++p) {
+    const int r = 2 * (wave * LA + p) + (lane >> 5);
     const int col = ti * TM + (((lane & 31) ^ ((r & 3) << 2)) * 8);
-    gofA[p] = (uint32_t)(r * K + col);
+    rowA[p] = r;
+    gofA[p] = (uint32_t)(r * ldx + col);
     okA[p] = col < K;
   }
   #pragma unroll
-  for (int p = 0; p < 2; ++p) {
-    const int r = 8 * wave + 4 * p + (lane >> 4);
-    const int col = tj * TN + (((lane & 15) ^ ((r & 3) << 2)) * 8);
-    gofB[p] = (uint32_t)(r * K + col);
+  for (int p = 0; p < LB; ++p) {
+    constexpr int LPR = 64 / RB;                           // lanes per token row
+    const int r = RB * (wave * LB + p) + lane / LPR;
+    const int col = tj * TN + (((lane % LPR) ^ ((r & 3) << 2)) * 8);
+    rowB[p] = r;
+    gofB[p] = (uint32_t)(r * ldx + col);
     okB[p] = col < K;
   }
   // The loads are issued from inline assembly: the compiler would otherwise wait for ALL direct
   // loads (vmcnt(0)) before any LDS read, which serialises the pipeline.  Waits are explicit below.
   const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
   auto gload = [&](int t0, int stage) {
-    const uint16_t* Xs = X + (int64_t)t0 * K;
-    const uint32_t dA = lds0 + stage * STAGE_BYTES + wave * 8 * ROW_A;
-    const uint32_t dB = lds0 + stage * STAGE_BYTES + BYTES_A + wave * 8 * ROW_B;
+    const uint16_t* Xs = X + (int64_t)t0 * ldx;
+    const uint32_t dA = lds0 + stage * STAGE + wave * LA * 1024;
+    const uint32_t dB = lds0 + stage * STAGE + BYTES_A + wave * LB * 1024;
     #pragma unroll
-    for (int p = 0; p < 6; ++p) {
-      const bool isA = p < 4;
-      const uint32_t dst = isA ? dA + p * 2 * ROW_A : dB + (p - 4) * 4 * ROW_B;
-      const uint32_t gof = isA ? gofA[p] : gofB[p - 4];
+    for (int p = 0; p < LA + LB; ++p) {
+      const bool isA = p < LA;
+      const uint32_t dst = isA ? dA + p * 1024 : dB + (p - LA) * 1024;
+      const uint32_t gof = isA ? gofA[isA ? p : 0] : gofB[isA ? 0 : p - LA];
       if constexpr (EDGE) {
-        const int r = isA ? 8 * wave + 2 * p + (lane >> 5) : 8 * wave + 4 * (p - 4) + (lane >> 4);
-        const bool ok = (isA ? okA[p] : okB[p - 4]) && t0 + r < T;
+        const int r = isA ? rowA[isA ? p : 0] : rowB[isA ? 0 : p - LA];
+        const bool ok = (isA ? okA[isA ? p : 0] : okB[isA ? 0 : p - LA]) && t0 + r < T;
         const uint16_t* g = ok ? Xs + gof : (const uint16_t*)zero_piece;
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(g) : "memory");
       } else {
@@ -181,7 +197,7 @@ __global__ __launch_bounds__(256, 2) void hessian_kernel(float* __restrict__ H, 
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
   auto compute = [&](int stage) {
-    const char* const base = lds + stage * STAGE_BYTES;
+    const char* const base = lds + stage * STAGE;
     #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
       s16x8 fa[4];
@@ -202,22 +218,27 @@ __global__ __launch_bounds__(256, 2) void hessian_kernel(float* __restrict__ H, 
     }
   };
 
-  // Three LDS stages, one barrier per 32-token slab.  At the top of step s a wave waits for its
-  // own loads of slab s (those of slab s+1 may stay in flight), the barrier then makes every
-  // wave's part of slab s visible and proves that all waves are done reading slab s-1, whose stage
-  // the loads of slab s+2 overwrite.
+  // NSTAGE LDS stages, one barrier per 32-token slab.  At the top of step s a wave waits for its
+  // own loads of slab s (those of the NSTAGE-2 later slabs may stay in flight), the barrier then
+  // makes every wave's part of slab s visible and proves that all waves are done reading slab
+  // s-1, whose stage the loads of slab s+NSTAGE-1 overwrite.
   const int nsteps = (T + BT - 1) / BT;
-  gload(0, 0);
-  if (nsteps > 1) gload(BT, 1);
-  int cur = 0, nxt2 = 2;
+  #pragma unroll
+  for (int s = 0; s < NSTAGE - 1; ++s)
+    if (s < nsteps) gload(s * BT, s);
+  int cur = 0, nxt = NSTAGE - 1;
   for (int s = 0; s < nsteps; ++s) {
-    if (s + 1 < nsteps) __builtin_amdgcn_s_waitcnt(0x0F76);     // vmcnt(6)
-    else __builtin_amdgcn_s_waitcnt(0x0F70);                    // vmcnt(0)
+    const int later = min(nsteps - 1 - s, NSTAGE - 2);          // slabs that may stay in flight
+    if (later >= 2) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * C::NL));
+    else if (later == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | C::NL);
+    else __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
-    if (s + 2 < nsteps) gload((s + 2) * BT, nxt2);
+    if (s + NSTAGE - 1 < nsteps) gload((s + NSTAGE - 1) * BT, nxt);
+    __builtin_amdgcn_s_setprio(3);        // the wave that has its operands goes first: keeps the MFMA pipe fed
     compute(cur);
+    __builtin_amdgcn_s_setprio(0);
     cur = (cur == NSTAGE - 1) ? 0 : cur + 1;
-    nxt2 = (nxt2 == NSTAGE - 1) ? 0 : nxt2 + 1;
+    nxt = (nxt == NSTAGE - 1) ? 0 : nxt + 1;
   }
 
   // epilogue: accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32.
@@ -278,18 +299,21 @@ __global__ __launch_bounds__(256) void symmetrize_kernel(float* __restrict__ H, 
 
 extern "C" {
 
-int lcq_hessian_accum(float* H, int64_t K, const void* X, int dtype, int64_t T, float alpha, float beta, void* stream) {
+int lcq_hessian_accum(float* H, int64_t K, const void* X, int dtype, int64_t T, int64_t ldx, float alpha, float beta,
+                      void* stream) {
   if (!H || !X || K <= 0 || T < 0) return LCQ_EINVAL;
-  if (K % 8 != 0 || K > (1 << 20) || T > 0x7fffffff) return LCQ_EINVAL;
+  if (K % 8 != 0 || K > (1 << 20) || T > 0x7fffffff || ldx < K || ldx % 8 != 0 || ldx > (1 << 21)) return LCQ_EINVAL;
   if (((uintptr_t)X % 16) != 0 || ((uintptr_t)H % 4) != 0) return LCQ_EALIGN;
   if (T == 0) return LCQ_OK;
-  const int ntr = (int)((K + TM - 1) / TM), ntc = (int)((K + TN - 1) / TN);
+  constexpr int TN = 128;
+  const int ntr = (int)((K + TM - 1) / TM), ntc = (int)((K + TN - 1) / TN), q = TM / TN;
   int64_t total = 0;
-  for (int r = 0; r < ntr; ++r) total += (ntc - 2 * r > 0) ? (ntc - 2 * r) : 0;
+  for (int r = 0; r < ntr; ++r) total += (ntc - q * r > 0) ? (ntc - q * r) : 0;
   const int64_t grid = (total + 7) / 8 * 8;                       // 8 XCD queues of equal length
   hipStream_t st = (hipStream_t)stream;
   const bool edge = (K % TM != 0) || (T % BT != 0);
-  #define LCQ_HESS(BF, E) hessian_kernel<BF, E><<<dim3((unsigned)grid), dim3(256), 0, st>>>(H, (int)K, (const uint16_t*)X, (int)T, alpha, beta, ntr, ntc, (int)total)
+  #define LCQ_HESS(BF, E) hessian_kernel<BF, E, TN><<<dim3((unsigned)grid), dim3(HessCfg<TN>::NW * 64), 0, st>>>( \
+      H, (int)K, (const uint16_t*)X, (int)ldx, (int)T, alpha, beta, ntr, ntc, (int)total)
   if (dtype == LCQ_BF16) { if (edge) LCQ_HESS(true, true); else LCQ_HESS(true, false); }
   else if (dtype == LCQ_F16) { if (edge) LCQ_HESS(false, true); else LCQ_HESS(false, false); }
   else return LCQ_EDTYPE;

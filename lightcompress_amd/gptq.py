@@ -150,14 +150,15 @@ class GPTQ:
             self._flush(cache)
 
     def _accumulate(self, cache, x, batches):
-        """H <- H*n/(n+b) + 2/(n+b) * x^T x for the n batches already inside H (gptq.py:279-294)."""
+        """H <- H*n/(n+b) + 2/(n+b) * x^T x for the n batches already inside H (gptq.py:279-294).
+        x: [tokens, K] view with unit column stride (rows may be padded)."""
         n = cache.get('n_in_H', 0)
         alpha = n / (n + batches)
         beta = 2.0 / (n + batches)
         cache['n_in_H'] = n + batches
         H = cache['H']
         L.check(L.lib().lcq_hessian_accum(L.ptr(H), L.i64(H.shape[0]), L.ptr(x), L.i32(L.dtype_code(x.dtype)),
-                                          L.i64(x.shape[0]), L.f32(alpha), L.f32(beta), L.stream()),
+                                          L.i64(x.shape[0]), L.i64(x.stride(0)), L.f32(alpha), L.f32(beta), L.stream()),
                 'lcq_hessian_accum')
 
     def _flush(self, cache):
