@@ -54,6 +54,8 @@ extern "C" {
                                      arithmetic unrounded (a 0-dim fp32 qparam next to a bf16 tensor); results
                                      still round to the row type */
 
+#define LCQ_FLAG_ROW_QP 512       /* lcq_quant_fp_emu, STATIC only: `scales` holds one value per row */
+
 /* errors */
 #define LCQ_OK 0
 #define LCQ_EINVAL (-1)
@@ -110,6 +112,18 @@ int lcq_quant_fp(const void* x, int dtype, int64_t rows, int64_t cols, int e_bit
 /* FloatQuantizer.dequant, quant.py:1073-1075, on fp32 codes: out = (q - 0) * s in fp32. */
 int lcq_dequant_fp(const float* q, int64_t rows, int64_t cols, const void* scales, int scale_dtype, int flags,
                    float* out, void* stream);
+
+/* FloatQuantizer with use_qtorch=False: get_float_qparams (quant.py:1004-1026) + quant / dequant
+ * (:1058-1075) in one pass.  Dynamic (default): per-row ranges `min_in` / `max_in` [rows] give
+ *   maxval = max(max, -min);  bias = 2^e - log2(maxval) + log2(2 - 2^-m) - 1  and per element
+ *   xc = clamp(x, -maxval, maxval);  s = 2^(clamp(floor(log2|xc| + bias), 1) - m - bias);
+ *   q = round(xc / s + 0);  dq = (q - 0) * s
+ * LCQ_FLAG_STATIC: `scales_in` is given ([rows, cols], or [rows] with LCQ_FLAG_ROW_QP, or [1] with
+ * LCQ_FLAG_SCALAR_QP) and xc = x.  Every output is optional and has the shape and type of x, except
+ * q with LCQ_CODE_FP8 (float8 bytes, e4m3 / e5m2 only).  cols % (16 / element size) == 0. */
+int lcq_quant_fp_emu(const void* x, int dtype, int64_t rows, int64_t cols, int e_bits, int m_bits, int flags,
+                     const void* min_in, const void* max_in, const void* scales_in, void* xc, void* scales_out,
+                     void* q, int code_dtype, void* dq, void* stream);
 
 /* ---- packing ------------------------------------------------------------ */
 

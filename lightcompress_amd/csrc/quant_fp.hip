@@ -185,6 +185,80 @@ __global__ __launch_bounds__(256) void dequant_fp_kernel(const float* __restrict
   }
 }
 
+
+// ---- FloatQuantizer without qtorch: per-element power-of-two-ish steps -------------------------
+// get_float_qparams + quant + dequant, quant.py:1004-1026, 1042-1080, as one pass.  Per row
+//   maxval = max(max, -min);  bias = 2^e - log2(maxval) + log2(2 - 2^-m) - 1
+// and per element
+//   xc = min(max(x, -maxval), maxval)
+//   ls = clamp(floor(log2|xc| + bias), min=1);  s = 2^(ls - m - bias);  s == 0 -> 1
+//   q = round(xc / s + 0);  dq = (q - 0) * s
+// with a rounding to the row dtype after every operation (bf16 rows), as torch evaluates it.
+// log2 / exp2 come from the device math library: the reference's values come from another
+// vendor's library, so this path can agree with any other implementation only up to the last
+// ulp of those two functions.
+struct EmuArgs {
+  const void* x; const void* mn; const void* mx; const void* s_in;
+  void* xc; void* s_out; void* q; void* dq;
+  int64_t rows, cols;
+  float two_e, log_top, m_bits;
+  int is_static, scalar_qp, row_qp, q_fp8, e_bits;
+};
+
+template <bool BF>
+__global__ __launch_bounds__(256) void fp_emu_kernel(EmuArgs a) {
+  constexpr int N = Vec<BF>::N;
+  const int64_t cpr = a.cols / N;                          // chunks per row (host guarantees cols % N == 0)
+  const int64_t nchunks = a.rows * cpr;
+  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < nchunks; c += (int64_t)gridDim.x * 256) {
+    const int64_t row = c / cpr, e0 = c * N;
+    float v[N], xc[N], sc[N], q[N], dq[N];
+    unpack<BF>(((const u32x4*)a.x)[c], v);
+    float maxval = 0.0f, bias = 0.0f;
+    if (!a.is_static) {
+      const float mn = load_scalar<BF>(a.mn, row), mx = load_scalar<BF>(a.mx, row);
+      maxval = nan_max(mx, -mn);
+      bias = rnd<BF>(a.two_e - rnd<BF>(__builtin_log2f(maxval)));
+      bias = rnd<BF>(bias + a.log_top);
+      bias = rnd<BF>(bias - 1.0f);
+    }
+    #pragma unroll
+    for (int i = 0; i < N; ++i) {
+      float s;
+      if (a.is_static) {
+        xc[i] = v[i];
+        s = load_scalar<BF>(a.s_in, a.scalar_qp ? 0 : (a.row_qp ? row : e0 + i));
+      } else {
+        xc[i] = nan_min(nan_max(v[i], -maxval), maxval);
+        float l = rnd<BF>(__builtin_log2f(fabsf(xc[i])));
+        l = rnd<BF>(l + bias);
+        l = __builtin_floorf(l);
+        l = clamp_min_nan(l, 1.0f);
+        float ex = rnd<BF>(l - a.m_bits);
+        ex = rnd<BF>(ex - bias);
+        s = rnd<BF>(__builtin_exp2f(ex));
+      }
+      if (s == 0.0f) s = 1.0f;                             // scales[scales == 0] = 1, quant.py:1061
+      sc[i] = s;
+      float t = rnd<BF>(xc[i] / s);
+      t = t + 0.0f;
+      q[i] = __builtin_rintf(t);
+      dq[i] = rnd<BF>((q[i] - 0.0f) * s);
+    }
+    if (a.xc) ((u32x4*)a.xc)[c] = pack<BF>(xc);
+    if (a.s_out) ((u32x4*)a.s_out)[c] = pack<BF>(sc);
+    if (a.dq) ((u32x4*)a.dq)[c] = pack<BF>(dq);
+    if (a.q) {
+      if (a.q_fp8) {
+        // |q| <= 2^(m+1) - 1 is an integer, exact in float8; written with the e4m3fn / e5m2 encoder
+        FpOp<BF> enc; enc.e_bits = a.e_bits;
+        #pragma unroll
+        for (int i = 0; i < N; ++i) ((uint8_t*)a.q)[e0 + i] = (uint8_t)enc.byte(q[i]);
+      } else ((u32x4*)a.q)[c] = pack<BF>(q);
+    }
+  }
+}
+
 }  // namespace
 
 extern "C" {
@@ -224,6 +298,44 @@ int lcq_dequant_fp(const float* q, int64_t rows, int64_t cols, const void* scale
   if (scale_dtype == LCQ_F32) dequant_fp_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>(q, rows, cols, scales, out, scalar_qp);
   else if (scale_dtype == LCQ_BF16) dequant_fp_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>(q, rows, cols, scales, out, scalar_qp);
   else return LCQ_EDTYPE;
+  LCQ_CHECK_LAUNCH();
+  return LCQ_OK;
+}
+
+int lcq_quant_fp_emu(const void* x, int dtype, int64_t rows, int64_t cols, int e_bits, int m_bits, int flags,
+                     const void* min_in, const void* max_in, const void* scales_in, void* xc, void* scales_out,
+                     void* q, int code_dtype, void* dq, void* stream) {
+  if (!x || rows < 0 || cols <= 0) return LCQ_EINVAL;
+  if (rows == 0) return LCQ_OK;
+  if (e_bits < 2 || e_bits > 5 || m_bits < 1 || m_bits > 10) return LCQ_EINVAL;
+  const int is_static = (flags & LCQ_FLAG_STATIC) != 0;
+  if (is_static ? !scales_in : (!min_in || !max_in)) return LCQ_EINVAL;
+  if ((flags & (LCQ_FLAG_SCALAR_QP | LCQ_FLAG_ROW_QP)) && !is_static) return LCQ_EINVAL;
+  if (dtype != LCQ_F32 && dtype != LCQ_BF16) return LCQ_EDTYPE;
+  const int n = (dtype == LCQ_BF16) ? 8 : 4;
+  if (cols % n != 0) return LCQ_EINVAL;
+  int q_fp8 = 0;
+  if (q) {
+    if (code_dtype == LCQ_CODE_FP8) {
+      if (!((e_bits == 4 && m_bits == 3) || (e_bits == 5 && m_bits == 2))) return LCQ_EDTYPE;
+      q_fp8 = 1;
+    } else if (code_dtype != LCQ_CODE_SAME) return LCQ_EDTYPE;
+  }
+  const void* al[] = {x, xc, scales_out, dq, (q && !q_fp8) ? q : nullptr, (is_static && !(flags & (LCQ_FLAG_SCALAR_QP | LCQ_FLAG_ROW_QP))) ? scales_in : nullptr};
+  for (const void* p : al) if (p && ((uintptr_t)p % 16) != 0) return LCQ_EALIGN;
+  EmuArgs a;
+  a.x = x; a.mn = min_in; a.mx = max_in; a.s_in = scales_in; a.xc = xc; a.s_out = scales_out; a.q = q; a.dq = dq;
+  a.rows = rows; a.cols = cols;
+  a.two_e = (float)(1 << e_bits);
+  a.log_top = log2f(2.0f - exp2f(-(float)m_bits));
+  a.m_bits = (float)m_bits;
+  a.is_static = is_static; a.scalar_qp = (flags & LCQ_FLAG_SCALAR_QP) != 0; a.row_qp = (flags & LCQ_FLAG_ROW_QP) != 0;
+  a.q_fp8 = q_fp8; a.e_bits = e_bits;
+  int64_t grid = (rows * (cols / n) + 255) / 256;
+  if (grid > 262144) grid = 262144;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == LCQ_BF16) fp_emu_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>(a);
+  else fp_emu_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>(a);
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;
 }

@@ -11,8 +11,8 @@ ABI in ``include/lcq.h``.  There is no CPU path: CPU tensors raise
 
 Not carried over (they raise ``NotImplementedError``): the ``mse`` /
 ``learnable`` / ``hqq`` / ``static_hist`` calibrators, STE rounding (training
-only), the ``rounding`` override of ``fake_quant_weight_static``, ``per_block``
-granularity and ``FloatQuantizer(use_qtorch=False)``.
+only), the ``rounding`` override of ``fake_quant_weight_static`` and ``per_block``
+granularity.
 """
 from __future__ import annotations
 
@@ -436,8 +436,11 @@ class FloatQuantizer(BaseQuantizer):
         self.default_bias = 2 ** (self.e_bits - 1)
         self.dst_nbins = 2 ** self.num_bits
         self.use_qtorch = self.kwargs.get('use_qtorch')
+        self.fp_tie = self.kwargs.get('fp_tie', 'away')
+        self.fp_subnormals = self.kwargs.get('fp_subnormals', True)
         if not self.use_qtorch:
-            raise NotImplementedError('FloatQuantizer(use_qtorch=False) is not on this path')
+            self.qmin = self.qmax = None                 # quant.py:972-1002 sets them only with qtorch
+            return
         if 'float_range' in self.kwargs:
             self.qmin, self.qmax = self.kwargs['float_range']
         else:
@@ -451,8 +454,54 @@ class FloatQuantizer(BaseQuantizer):
                 self.qmin, self.qmax = finfo.min, finfo.max
         self.qmax = torch.tensor(self.qmax)
         self.qmin = torch.tensor(self.qmin)
-        self.fp_tie = self.kwargs.get('fp_tie', 'away')
-        self.fp_subnormals = self.kwargs.get('fp_subnormals', True)
+
+    # -- use_qtorch=False: per-element steps (quant.py:1004-1026) ----------------------------------
+    def _emu(self, rows_t, scales=None, want=()):
+        """One launch of lcq_quant_fp_emu -> dict with the requested outputs out of
+        'xc', 'scales', 'q', 'q_fp8', 'dq'.  scales=None: dynamic (per-row ranges of rows_t)."""
+        t = rows_t.contiguous()
+        flags = 0
+        mn = mx = s_in = None
+        if scales is None:
+            if self.granularity == 'per_tensor':
+                # the reference indexes maxval.shape[0] of a 0-dim range here (quant.py:1011)
+                raise IndexError('tuple index out of range')
+            mn, mx = self.get_minmax_range(t)
+            if self.e_bits >= 5 and t.dtype != torch.float32:
+                t, mn, mx = t.float(), mn.float(), mx.float()        # maxval.to(float32), quant.py:1014-1015
+            mn, mx = mn.contiguous(), mx.contiguous()
+            rows, cols = _rows_cols(t)
+        else:
+            scales[scales == 0] = 1                                  # quant.py:1061 mutates the caller's tensor
+            if scales.dim() > 0 and scales.dtype != t.dtype:
+                t = t.to(torch.promote_types(t.dtype, scales.dtype))
+            s_in = scales.to(t.dtype).contiguous()
+            flags |= L.FLAG_STATIC
+            if s_in.numel() == t.numel():
+                rows, cols = _rows_cols(t)
+            else:
+                rows, cols, scalar = _static_layout(t, s_in)
+                flags |= L.FLAG_SCALAR_QP if scalar else L.FLAG_ROW_QP
+        out = {}
+        for k in want:
+            if k == 'q_fp8':
+                out[k] = torch.empty(t.shape, dtype=torch.float8_e4m3fn if self.e_bits == 4 else torch.float8_e5m2,
+                                     device=t.device)
+            else:
+                out[k] = torch.empty_like(t)
+        q = out.get('q_fp8', out.get('q'))
+        L.check(L.lib().lcq_quant_fp_emu(L.ptr(t), L.dtype_code(t.dtype), L.i64(rows), L.i64(cols), L.i32(self.e_bits),
+                                         L.i32(self.m_bits), L.i32(flags), L.ptr(mn), L.ptr(mx), L.ptr(s_in),
+                                         L.ptr(out.get('xc')), L.ptr(out.get('scales')), L.ptr(q),
+                                         L.i32(L.CODE_FP8 if 'q_fp8' in out else L.CODE_SAME), L.ptr(out.get('dq')),
+                                         L.stream()), 'lcq_quant_fp_emu')
+        return out
+
+    def get_float_qparams(self, tensor, tensor_range, device):
+        """quant.py:1004-1026 -> (clamped tensor, elementwise scales); the range is recomputed from
+        `tensor` (it is what get_tensor_range returned for it)."""
+        o = self._emu(tensor, want=('xc', 'scales'))
+        return o['xc'].view(tensor.shape), o['scales'].view(tensor.shape)
 
     def _fp_flags(self):
         return ((L.FLAG_TIE_EVEN if self.fp_tie == 'even' else 0)
@@ -514,6 +563,9 @@ class FloatQuantizer(BaseQuantizer):
         if self.calib_algo != 'minmax':
             raise NotImplementedError(f'calib_algo={self.calib_algo!r}: only minmax runs on liblcq')
         tensor = self.reshape_tensor(tensor)
+        if not self.use_qtorch:
+            xc, s = self.get_float_qparams(tensor, None, tensor.device)
+            return xc, s, torch.tensor(0), None, None
         if self.granularity == 'per_tensor':
             s, z, qmax, qmin = self.get_qparams(self.get_minmax_range(tensor), tensor.device)
             return tensor, s, z, qmax, qmin
@@ -523,12 +575,28 @@ class FloatQuantizer(BaseQuantizer):
         return tensor, s, torch.tensor(0.0), self.qmax.to(tensor.device), self.qmin.to(tensor.device)
 
     def quant(self, tensor, scales, zeros, qmax, qmin):
-        """quant.py:1060-1071: fp32 values on the minifloat grid."""
+        """quant.py:1060-1071: fp32 values on the minifloat grid (qtorch) / round(t / s) in the
+        tensor's type (no qtorch)."""
+        if not self.use_qtorch:
+            return self._emu(tensor, scales, want=('q',))['q'].view(tensor.shape)
         _, codes, _ = self._launch(tensor, static=True, scales=scales, want_codes='f32')
         return codes.view(tensor.shape)
 
     def dequant(self, tensor, scales, zeros):
         """quant.py:1073-1075 on fp32 codes."""
+        if not self.use_qtorch:
+            t = tensor.contiguous()
+            s = scales.to(t.dtype).contiguous()
+            if s.numel() == t.numel():
+                rows, cols, flags = t.numel(), 1, 0
+            else:
+                rows, cols, scalar = _static_layout(t, s)
+                flags = L.FLAG_SCALAR_QP if scalar else 0
+            out = torch.empty_like(t)
+            L.check(L.lib().lcq_dequant_int(L.ptr(t), L.dtype_code(t.dtype), L.i64(rows), L.i64(cols), L.ptr(s),
+                                            L.ptr(None), L.i32(flags | L.FLAG_SYM), L.f32(1.0), L.ptr(out), L.stream()),
+                    'lcq_dequant_int')
+            return out
         t = tensor.float().contiguous()
         s = scales.contiguous()
         rows, cols, scalar = _static_layout(t, s)
@@ -539,13 +607,18 @@ class FloatQuantizer(BaseQuantizer):
         return out
 
     def quant_dequant(self, tensor, scales, zeros, qmax, qmin):
-        """quant.py:1077-1080: fp32 result (the float codes promote it)."""
+        """quant.py:1077-1080: fp32 result (the float codes promote it); the tensor's type without qtorch."""
+        if not self.use_qtorch:
+            return self._emu(tensor, scales, want=('dq',))['dq'].view(tensor.shape)
         dq, _, _ = self._launch(tensor, static=True, scales=scales, want_dq='f32')
         return dq.view(tensor.shape)
 
     def _fake(self, t, static_scales=None):
         shape, dtype = t.shape, t.dtype
         rows_t = self.reshape_tensor(t)
+        if not self.use_qtorch:
+            dq = self._emu(rows_t, static_scales, want=('dq',))['dq']
+            return self.restore_tensor(dq.view(rows_t.shape), shape).to(dtype)
         if static_scales is None:
             dq, _, _ = self._launch(rows_t, static=False, want_dq=True)
         else:
@@ -575,6 +648,16 @@ class FloatQuantizer(BaseQuantizer):
         dtype = torch.float8_e4m3fn if self.e_bits == 4 else torch.float8_e5m2
         org_w_shape = weight.shape
         rows_t = self.reshape_tensor(weight)
+        if not self.use_qtorch:
+            if static_scales is None:
+                o = self._emu(rows_t, want=('q_fp8', 'scales'))
+                scales = o['scales']
+            else:
+                o = self._emu(rows_t, static_scales, want=('q_fp8',))
+                scales = static_scales
+            codes = self.restore_tensor(o['q_fp8'].view(rows_t.shape), org_w_shape)
+            scales = scales * output_scale_factor
+            return codes, scales.view(1 if self.granularity == 'per_tensor' else (codes.shape[0], -1)), None
         if static_scales is None:
             _, codes, scales = self._launch(rows_t, static=False, want_codes=dtype)
         else:

@@ -324,3 +324,61 @@ def float_real_quant_dynamic(spec, w, output_scale_factor=1):
     q = q.to(dt)
     shp = 1 if spec.granularity == 'per_tensor' else (q.shape[0], -1)
     return q, s.view(shp), None
+
+
+# ----------------------------------------------------------------------------
+# FloatQuantizer(use_qtorch=False): per-element power-of-two-like steps
+# ----------------------------------------------------------------------------
+def float_emu_qparams(spec, rows: torch.Tensor, lo: torch.Tensor, hi: torch.Tensor):
+    """get_float_qparams, quant.py:1004-1026, one torch op per step (the two 0-dim fp32 tensors
+    the reference creates with .cuda() live on the CPU here).  Returns (clamped rows, elementwise
+    scales).  Pinned by test_oracle_quant.py: the row maximum is a fixed point, results are
+    idempotent, relative step 2**-m_bits in the normal range, fixed step below it, and an fp64
+    evaluation of the same formula on exactly representable inputs."""
+    maxval = torch.max(hi, -lo)
+    e_bits = torch.tensor(spec.e_bits, dtype=torch.float32)
+    m_bits = torch.tensor(spec.m_bits, dtype=torch.float32)
+    if maxval.shape[0] != 1 and len(maxval.shape) != len(rows.shape):
+        maxval = maxval.view([-1] + [1] * (len(rows.shape) - 1))
+    if e_bits >= 5:
+        maxval = maxval.to(dtype=torch.float32)
+    bias = 2 ** e_bits - torch.log2(maxval) + torch.log2(2 - 2 ** (-m_bits)) - 1
+    xc = torch.min(torch.max(rows, -maxval), maxval)
+    log_scales = torch.clamp(torch.floor(torch.log2(torch.abs(xc)) + bias), 1.0)
+    scales = 2.0 ** (log_scales - m_bits - bias)
+    return xc, scales
+
+
+def float_emu_quant(t, scales, zeros):
+    """quant.py:1060-1071 with round_func = torch.round."""
+    scales[scales == 0] = 1
+    return torch.round(t / scales + zeros)
+
+
+def float_emu_tensor_qparams(spec, t):
+    """get_tensor_qparams, quant.py:1042-1058 (non-qtorch branch): zeros is an int64 0-dim 0."""
+    rows = reshape_rows(spec, t)
+    lo, hi = minmax_range(spec, rows)
+    xc, scales = float_emu_qparams(spec, rows, lo, hi)
+    return xc, scales, torch.tensor(0), None, None
+
+
+def float_emu_fake_quant_dynamic(spec, w):
+    """quant.py:1099-1108 / 1141-1158 without qtorch."""
+    shape, dtype = w.shape, w.dtype
+    xc, s, z, _, _ = float_emu_tensor_qparams(spec, w)
+    q = float_emu_quant(xc, s, z)
+    out = float_dequant(q, s, z)
+    return restore_rows(spec, out, shape).to(dtype)
+
+
+def float_emu_real_quant_dynamic(spec, w, output_scale_factor=1):
+    """quant.py:1194-1220 without qtorch: integer-valued codes stored as float8, elementwise scales."""
+    assert spec.bit in ('e4m3', 'e5m2')
+    dt = torch.float8_e4m3fn if spec.e_bits == 4 else torch.float8_e5m2
+    shape = w.shape
+    xc, s, z, _, _ = float_emu_tensor_qparams(spec, w)
+    q = restore_rows(spec, float_emu_quant(xc, s, z), shape)
+    s = s * output_scale_factor
+    q = q.to(dt)
+    return q, s.view(q.shape[0], -1), None

@@ -8,6 +8,8 @@ float8 casts torch itself provides, and pack/unpack round trips.
 from fractions import Fraction
 
 import numpy as np
+import math
+
 import pytest
 import torch
 
@@ -241,6 +243,83 @@ def test_float_real_quant_is_on_grid_and_scaled_to_448():
 # --------------------------------------------------------------------------
 # packing
 # --------------------------------------------------------------------------
+def _minifloat_grid_round(y, m_bits, emin):
+    """Nearest point (ties to even) of the minifloat grid with m_bits mantissa bits whose smallest
+    normal exponent is emin, for fp64 y >= 0: built from frexp, no logarithms or powers."""
+    mant, ex = torch.frexp(y)                       # y = mant * 2**ex, mant in [0.5, 1)
+    e = torch.clamp(ex - 1, min=emin)               # binade exponent, subnormals share emin
+    step = torch.ldexp(torch.ones_like(y), e - m_bits)
+    return torch.round(y / step) * step
+
+
+@pytest.mark.parametrize('fmt', ['e4m3', 'e5m2', 'e2m1', 'e3m2'])
+@pytest.mark.parametrize('dtype', [torch.float32])
+def test_float_emulation_is_a_minifloat_grid_scaled_to_the_row_maximum(fmt, dtype):
+    """use_qtorch=False (quant.py:1004-1026): with c = rowmax / (2 - 2**-m) the formula rounds
+    x / c to the minifloat grid whose top value is 2 - 2**-m (exponent 0) and whose smallest normal
+    exponent is 2 - 2**e, subnormals below it.  Checked against a frexp-based construction of that
+    grid; fp32 log2 / exp2 put a few elements next to a binade edge or a tie on the neighbouring
+    grid point, so the comparison allows one grid step there and counts exact agreement."""
+    spec = Q.FloatSpec(fmt, 'per_channel')
+    e, m = spec.e_bits, spec.m_bits
+    w = weight_like(64, 512, seed=31).to(dtype)
+    w[:, 0] = 0.0
+    w[:, 1] = w.abs().amax(dim=1) * 2.0 ** -20      # deep in the fixed-step range
+    out = Q.float_emu_fake_quant_dynamic(spec, w.clone())
+    assert out.dtype == dtype and out.shape == w.shape
+    wd = w.double()
+    c = wd.abs().amax(dim=1, keepdim=True) / (2 - 2.0 ** -m)
+    ref = torch.sign(wd) * _minifloat_grid_round(wd.abs() / c, m, 2 - 2 ** e) * c
+    tol = 2.0 ** -7 if dtype == torch.bfloat16 else 1e-5
+    close = (out.double() - ref).abs() <= tol * ref.abs() + 1e-30
+    assert float(close.float().mean()) > (0.97 if dtype == torch.bfloat16 else 0.995)
+    step = torch.ldexp(torch.ones_like(wd), torch.clamp(torch.frexp(wd.abs() / c)[1] - 1, min=2 - 2 ** e) - m) * c
+    assert bool(((out.double() - ref).abs() <= step * (1 + 2.0 ** -6) + tol * ref.abs()).all())
+    assert bool((out[:, 0] == 0).all())
+    # the row maximum maps to the top of the grid: unchanged up to the rounding of log2 / exp2
+    top = out.double().abs().amax(dim=1)
+    assert bool(((top - wd.abs().amax(dim=1)).abs() <= tol * top).all())
+
+
+@pytest.mark.parametrize('fmt', ['e4m3', 'e2m1', 'e5m2'])
+def test_float_emulation_bf16_rounds_after_every_op(fmt):
+    """bf16 rows: every torch op of quant.py:1004-1026 / 1060-1075 computes in fp32 and rounds its
+    result to bf16 (the 0-dim fp32 e_bits / m_bits do not promote); e_bits >= 5 switches the whole
+    chain to fp32 through maxval.  An fp32 evaluation with explicit roundings must reproduce torch's
+    bf16 evaluation bit for bit - this is the arithmetic the kernel implements."""
+    spec = Q.FloatSpec(fmt, 'per_channel')
+    e, m = spec.e_bits, spec.m_bits
+    w = weight_like(32, 256, seed=33).bfloat16()
+    w[:, 3] = 0.0
+    out = Q.float_emu_fake_quant_dynamic(spec, w.clone())
+    r = (lambda t: t) if e >= 5 else (lambda t: t.bfloat16().float())
+    x = w.float()
+    maxval = torch.max(x.amax(dim=1, keepdim=True), -x.amin(dim=1, keepdim=True))
+    bias = r(r(r(float(2 ** e) - r(torch.log2(maxval))) + math.log2(2 - 2.0 ** -m)) - 1.0)
+    xc = torch.min(torch.max(x, -maxval), maxval)
+    ls = torch.clamp(torch.floor(r(r(torch.log2(xc.abs())) + bias)), min=1.0)
+    sc = r(torch.exp2(r(r(ls - m) - bias)))
+    sc[sc == 0] = 1
+    model = r(torch.round(r(xc / sc) + 0) * sc).bfloat16()
+    assert out.dtype == torch.bfloat16
+    assert_bit_equal(out, model)
+
+
+def test_float_emulation_outputs_and_real_quant_layout():
+    spec = Q.FloatSpec('e4m3', 'per_group', group_size=128)
+    w = weight_like(8, 256, seed=32)
+    xc, s, z, qmax, qmin = Q.float_emu_tensor_qparams(spec, w.clone())
+    assert xc.shape == s.shape == (16, 128) and z.dtype == torch.int64 and qmax is None and qmin is None
+    assert torch.equal(xc, w.reshape(16, 128))                    # clamping to the row's own range changes nothing
+    q = Q.float_emu_quant(xc, s, z)
+    assert float(q.abs().max()) <= 2 ** (spec.m_bits + 1) - 1 + 1  # mantissa codes (a rounded-up edge value may add 1)
+    assert torch.equal(q, torch.round(q))
+    codes, scales, zeros = Q.float_emu_real_quant_dynamic(Q.FloatSpec('e4m3', 'per_channel'), w.clone())
+    assert codes.dtype == torch.float8_e4m3fn and codes.shape == w.shape and scales.shape == w.shape and zeros is None
+    back = codes.float() * scales
+    assert float((back - Q.float_emu_fake_quant_dynamic(Q.FloatSpec('e4m3', 'per_channel'), w.clone())).abs().max()) == 0.0
+
+
 def test_pack_ct_roundtrip_and_padding():
     g = gen(14)
     codes = torch.randint(-8, 8, (5, 37), generator=g, dtype=torch.int32)

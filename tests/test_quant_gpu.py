@@ -166,6 +166,69 @@ def test_float_quant_bit_exact(dev, tie, dtype, fmt, gran, shape):
         assert_bit_equal(rs, ors, 'fp8 scales')
 
 
+def _agree(a, b):
+    return float((a.cpu().float() == b.float()).float().mean())
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('fmt,gran,shape', [('e4m3', 'per_channel', (64, 2048)), ('e4m3', 'per_group', (64, 1024)),
+                                            ('e5m2', 'per_channel', (32, 1024)), ('e2m1', 'per_group', (64, 512)),
+                                            ('e4m3', 'per_token', (96, 7168))])
+def test_float_emulation_without_qtorch(dev, dtype, fmt, gran, shape):
+    """use_qtorch=False (quant.py:1004-1026).  log2 and 2**x come from different math libraries on
+    the two sides (and from a third in the reference), so agreement is counted instead of demanded
+    bit for bit.  bf16: every op result is rounded to 8 bits, which hides last-ulp differences:
+    >= 99.9 % of the elements identical.  fp32: the per-row bias and so every scale of a row can
+    differ: one ulp of the bias (a number near 20) is 1.3e-6 of a scale 2**(.. - bias), so results
+    agree to 4e-6 relative and the mantissa codes round(x / s) are identical on >= 99.9 %.  Everything that does not pass through log2 / exp2 is bit-exact."""
+    from lightcompress_amd import FloatQuantizer
+    w = weight_like(*shape, seed=shape[1] + 1, dtype=dtype, std=0.006, outlier_frac=0.0005, outlier_mul=30)
+    w[0, :2] = torch.tensor([0.0, -0.0], dtype=dtype)
+    kw = dict(group_size=128) if gran == 'per_group' else {}
+    spec = Q.FloatSpec(fmt, gran, group_size=kw.get('group_size', 0))
+    q = FloatQuantizer(fmt, True, gran, use_qtorch=False, **kw)
+    wd = w.to(dev)
+    got, want = q.fake_quant_weight_dynamic(wd), Q.float_emu_fake_quant_dynamic(spec, w.clone())
+    assert got.dtype == want.dtype and got.shape == want.shape
+    m = spec.m_bits
+    exact = dtype == torch.bfloat16 and spec.e_bits < 5          # e5m2 computes in fp32 whatever the input
+    near = (got.cpu().double() - want.double()).abs() <= want.double().abs() * 4e-6 + 1e-30
+    assert _agree(got, want) >= 0.999 if exact else float(near.float().mean()) >= 0.999
+    assert bool(((got.cpu().double() - want.double()).abs() <= want.double().abs() * 2.0 ** -m + 1e-30).all())
+    xc, s, z, qmax, qmin = q.get_tensor_qparams(wd)
+    oxc, os_, oz, _, _ = Q.float_emu_tensor_qparams(spec, w.clone())
+    assert qmax is None and qmin is None and z.dtype == torch.int64 and int(z) == 0
+    assert_bit_equal(xc, oxc, 'clamped tensor')
+    assert s.dtype == os_.dtype
+    if exact:
+        assert _agree(s, os_) >= 0.999
+    else:
+        assert bool(((s.cpu().double() - os_.double()).abs() <= os_.double() * 4e-6).all())
+    assert _agree(q.quant(xc, s.clone(), z, None, None), Q.float_emu_quant(oxc, os_.clone(), oz)) >= 0.999
+    # given identical scales, quant / dequant / quant_dequant are plain arithmetic: bit-exact
+    sd = os_.to(dev)
+    assert_bit_equal(q.quant(xc, sd.clone(), z, None, None), Q.float_emu_quant(oxc, os_.clone(), oz), 'round(t / s)')
+    oq = Q.float_emu_quant(oxc, os_.clone(), oz)
+    assert_bit_equal(q.dequant(oq.to(dev), sd, z), Q.float_dequant(oq, os_, oz), 'q * s')
+    assert_bit_equal(q.quant_dequant(xc, sd.clone(), z, None, None), Q.float_dequant(oq, os_, oz), 'quant_dequant')
+    assert_bit_equal(q.fake_quant_weight_static(wd, dict(scales=sd.clone(), zeros=z, qmax=None, qmin=None)),
+                     Q.restore_rows(spec, Q.float_dequant(oq, os_, oz), w.shape).to(dtype), 'static fake quant')
+    if fmt in ('e4m3', 'e5m2') and gran == 'per_channel':
+        codes, rs, rz = q.real_quant_weight_dynamic(wd)
+        ocodes, ors, _ = Q.float_emu_real_quant_dynamic(spec, w.clone())
+        assert rz is None and codes.dtype == ocodes.dtype and rs.shape == ors.shape
+        assert _agree(codes.float(), ocodes.float()) >= 0.999
+        back = codes.float().cpu() * rs.float().cpu()           # codes and scales are consistent with each other
+        assert _agree(back.to(got.dtype), got.cpu()) == 1.0
+
+
+def test_float_emulation_per_tensor_raises_like_the_reference(dev):
+    from lightcompress_amd import FloatQuantizer
+    q = FloatQuantizer('e4m3', True, 'per_tensor', use_qtorch=False)
+    with pytest.raises(IndexError):                 # maxval.shape[0] of a 0-dim range, quant.py:1011
+        q.fake_quant_weight_dynamic(weight_like(8, 64, seed=5).to(dev))
+
+
 def test_float_act_fake_quant_3d(dev):
     from lightcompress_amd import FloatQuantizer
     act = (torch.randn(2, 48, 7168, generator=gen(51)) * torch.exp(torch.randn(7168, generator=gen(52)))).bfloat16()
