@@ -34,6 +34,11 @@ LINEARS = [  # name, out_features, in_features, activation stream
 SUBSETS = [['q_proj', 'k_proj', 'v_proj'], ['o_proj'], ['gate_proj', 'up_proj'], ['down_proj']]
 STREAM_K = {'attn_in': 4096, 'o_in': 4096, 'mlp_in': 4096, 'down_in': 14336}
 NB, TOK = 128, 2048
+# HBM-side bytes per launch of the two roofline kernels: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this script,
+# scaled by the same counters' reading for a copy kernel of known size (profiles/hessian_kernel_K14336_T8192.md,
+# profiles/rtn_quant_int4_g128_4096x4096_f32.md).  Counters cannot be read from inside the timed process.
+HESSIAN_TRAFFIC_BYTES = 6.861e9
+RTN_TRAFFIC_BYTES = 1.518e8
 CFG = {'weight': dict(bit=4, symmetric=False, granularity='per_group', group_size=128),
        'special': dict(actorder=True, static_groups=False, percdamp=0.01, blocksize=128, true_sequential=True)}
 
@@ -144,7 +149,8 @@ def gpu_main(args):
     tiles = sum(K // 128 - 2 * ti for ti in range(K // 256))          # 256x128 tiles that reach the upper triangle
     exe_flops = 2.0 * TL * tiles * 256 * 128
     roofline = {'kernel': f'hessian_kernel<bf16> K=14336 T={TL}', 'bound': 'mfma', 'achieved': round(alg_flops / t_h / 1e12, 2),
-                'peak': 2500.0, 'unit': 'TFLOP/s', 'frac': round(alg_flops / t_h / 2.5e15, 4), 'traffic': None,
+                'peak': 2500.0, 'unit': 'TFLOP/s', 'frac': round(alg_flops / t_h / 2.5e15, 4),
+                'traffic': HESSIAN_TRAFFIC_BYTES if FOLD == 4 else None,
                 'launch_us': round(t_h * 1e6, 2), 'executed_tflops': round(exe_flops / t_h / 1e12, 2),
                 'frac_executed': round(exe_flops / t_h / 2.5e15, 4),
                 'note': 'achieved counts the full 2*T*K^2 product; only tiles on/above the diagonal are executed'}
@@ -172,7 +178,7 @@ def gpu_main(args):
     q_bytes = 4096 * 4096 * (4 + 4 + 1) + rows * 8
     roofline_q = {'kernel': 'row_team_kernel<IntOp<f32>> 4096x4096 g128 dq+u8', 'bound': 'hbm',
                   'achieved': round(q_bytes / t_q / 1e9, 1), 'peak': 8000.0, 'unit': 'GB/s',
-                  'frac': round(q_bytes / t_q / 8e12, 4), 'traffic': None, 'launch_us': round(t_q * 1e6, 2)}
+                  'frac': round(q_bytes / t_q / 8e12, 4), 'traffic': RTN_TRAFFIC_BYTES, 'launch_us': round(t_q * 1e6, 2)}
 
     out = {
         'metric': 'gptq_w4g128_seconds_per_llama3_8b_layer', 'value': round(dt, 4), 'unit': 's',
