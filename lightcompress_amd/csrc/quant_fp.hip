@@ -29,6 +29,7 @@ template <bool BF_>
 struct FpOp {
   static constexpr bool BF = BF_;
   static constexpr bool HAS_PRESCALE = false;
+  static constexpr bool HAS_FUSED_DQ = false;
   static constexpr int CD = -1;
   using Row = FpRow;
   float qmax;
@@ -120,8 +121,9 @@ struct FpOp {
   }
 
   // (q - 0.0) * s in fp32, then the cast of fake_quant_* (quant.py:1107,1153)
+  __device__ __forceinline__ float deq_raw(float q, const Row& p) const { return (q - 0.0f) * p.sm; }
   __device__ __forceinline__ float deq(float q, const Row& p) const {
-    const float d = (q - 0.0f) * p.sm;
+    const float d = deq_raw(q, p);
     return dq_f32 ? d : rnd_e<BF>(d);
   }
 

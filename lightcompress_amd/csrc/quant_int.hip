@@ -25,7 +25,9 @@ using namespace lcq;
 
 struct IntRow {
   float s, z, r, sdq;
-  int fast;
+  float lo, hi;      // qmin - z, qmax - z: clamp bounds of the code minus the zero point
+  int fast;          // x * (1/s) + guard may replace x / s
+  int zint;          // zero point is a small integer: rint(t) + z and q - z are exact
 };
 
 // FAST: round_zp and |qmin|,qmax <= 256 (every stock configuration).
@@ -33,6 +35,7 @@ template <bool BF_, bool FAST, bool PRESCALE = false, int CD_ = -1>
 struct IntOp {
   static constexpr bool BF = BF_;
   static constexpr bool HAS_PRESCALE = PRESCALE;
+  static constexpr bool HAS_FUSED_DQ = FAST;
   static constexpr int CD = CD_;
   using Row = IntRow;
   float qmin, qmax, qrange, osf;
@@ -64,7 +67,9 @@ struct IntOp {
     p.r = 1.0f / s;
     const float a = fabsf(s);
     p.fast = (a > 8.6736174e-19f) && (a < 1.1529215e18f) && (fabsf(z) <= 512.0f);   // s in 2^-60 .. 2^60
+    p.zint = (z == rintf(z)) && (fabsf(z) <= 512.0f);       // caller-given zero points need not be integers
     p.sdq = scale_f32 ? s * osf : rnd<BF>(s * osf);
+    p.lo = qmin - z; p.hi = qmax - z;                       // exact: small integers
     return p;
   }
 
@@ -128,40 +133,71 @@ struct IntOp {
   //         the clamp range on the same side (|z| <= 512), and a huge t has d == 0;
   //   bf16: the quotient is rounded to bf16 first; the product is safe unless its low 16 bits
   //         are within 8 ulp of the bf16 midpoint pattern 0x8000.
+  // x / s for a chunk, rounded to the row type
+  template <int N>
+  __device__ __forceinline__ void quotients(const float* x, float* t, const Row& p) const {
+    bool ok = p.fast;
+    #pragma unroll
+    for (int i = 0; i < N; ++i) {
+      t[i] = x[i] * p.r;
+      if constexpr (BF) {
+        ok = ok && (((f2u(t[i]) & 0xffffu) - 0x7ff8u) > 0x10u);
+      } else {
+        const float d = t[i] - rintf(t[i]);
+        ok = ok && (fabsf(fabsf(d) - 0.5f) > 4.8828125e-04f);
+      }
+    }
+    if (__builtin_expect(!ok, 0)) {
+      #pragma unroll
+      for (int i = 0; i < N; ++i) t[i] = x[i] / p.s;
+    }
+    #pragma unroll
+    for (int i = 0; i < N; i += 2) rnd_pair<BF>(t[i], t[i + 1]);
+  }
+
   template <int N>
   __device__ __forceinline__ void codes(const float* x, float* q, const Row& p) const {
     if constexpr (!FAST) {
       #pragma unroll
       for (int i = 0; i < N; ++i) q[i] = code(x[i], p);
     } else {
-      float t[N];
-      bool ok = p.fast;
-      #pragma unroll
-      for (int i = 0; i < N; ++i) {
-        t[i] = x[i] * p.r;
-        if constexpr (BF) {
-          ok = ok && (((f2u(t[i]) & 0xffffu) - 0x7ff8u) > 0x10u);
-        } else {
-          const float d = t[i] - rintf(t[i]);
-          ok = ok && (fabsf(fabsf(d) - 0.5f) > 4.8828125e-04f);
-        }
-      }
-      if (__builtin_expect(!ok, 0)) {
+      if (__builtin_expect(!p.zint, 0)) {
         #pragma unroll
-        for (int i = 0; i < N; ++i) t[i] = x[i] / p.s;
+        for (int i = 0; i < N; ++i) q[i] = code(x[i], p);
+        return;
       }
+      float t[N];
+      quotients<N>(x, t, p);
       #pragma unroll
       for (int i = 0; i < N; ++i)
-        q[i] = __builtin_amdgcn_fmed3f(rintf(rnd_e<BF>(t[i])) + p.z, qmin, qmax);
+        q[i] = __builtin_amdgcn_fmed3f(rintf(t[i]) + p.z, qmin, qmax);
     }
   }
 
-  // dequant, quant.py:709-711 (scale already multiplied by output_scale_factor)
-  __device__ __forceinline__ float deq(float q, const Row& p) const {
-    float d = q - p.z;                                       // exact for small integer codes
-    if constexpr (BF && !FAST) d = bf16_round(d);
-    return rnd_e<BF>(d * p.sdq);
+  // fake quant without the codes (FAST only): (clamp(rint(t) + z, qmin, qmax) - z) * s equals
+  // clamp(rint(t), qmin - z, qmax - z) * s when z is a small integer (all terms exact); "+ 0" turns the
+  // -0 that rint(-0.3) leaves into the +0 that (q - z) gives.  The products are left unrounded: the
+  // caller rounds to the row type while packing.
+  template <int N>
+  __device__ __forceinline__ void fused_dq(const float* x, float* d, const Row& p) const {
+    if (__builtin_expect(!p.zint, 0)) {
+      #pragma unroll
+      for (int i = 0; i < N; ++i) d[i] = deq_raw(code(x[i], p), p);
+      return;
+    }
+    float t[N];
+    quotients<N>(x, t, p);
+    #pragma unroll
+    for (int i = 0; i < N; ++i) d[i] = (__builtin_amdgcn_fmed3f(rintf(t[i]), p.lo, p.hi) + 0.0f) * p.sdq;
   }
+
+  // dequant, quant.py:709-711 (scale already multiplied by output_scale_factor)
+  __device__ __forceinline__ float deq_raw(float q, const Row& p) const {   // before the rounding to the row type
+    float d = q - p.z;                                       // exact for small integer codes
+    if constexpr (BF) { if (!FAST || !p.zint) d = bf16_round(d); }
+    return d * p.sdq;
+  }
+  __device__ __forceinline__ float deq(float q, const Row& p) const { return rnd_e<BF>(deq_raw(q, p)); }
 
   __device__ __forceinline__ uint32_t byte(float q) const { return (uint32_t)(int32_t)q & 0xffu; }
   __device__ __forceinline__ uint32_t pack4(const float* q) const {

@@ -36,6 +36,21 @@ template <bool BF> __device__ __forceinline__ float rnd_e(float v) {
 }
 __device__ __forceinline__ float clamp_min_nan(float v, float lo) { return (v != v) ? v : fmaxf(v, lo); }
 
+// two fp32 values -> one dword of two bf16 (RNE), a single v_cvt_pk_bf16_f32
+typedef float lcq_f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 lcq_bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t bf16_pack_rne(float a, float b) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(lcq_f32x2{a, b}, lcq_bf16x2));
+}
+// round a pair to the row type in place (bf16: one convert + two unpack ops for two elements)
+template <bool BF> __device__ __forceinline__ void rnd_pair(float& a, float& b) {
+  if constexpr (BF) {
+    const uint32_t u = bf16_pack_rne(a, b);
+    a = u2f(u << 16);
+    b = u2f(u & 0xffff0000u);
+  }
+}
+
 template <bool BF>
 __device__ __forceinline__ void unpack(const u32x4& raw, float* v) {
   if constexpr (BF) {
@@ -68,6 +83,20 @@ template <bool BF>
 __device__ __forceinline__ void store_scalar(void* p, int64_t i, float v) {
   if constexpr (BF) ((uint16_t*)p)[i] = (uint16_t)(f2u(v) >> 16);
   else ((float*)p)[i] = v;
+}
+
+// values NOT yet rounded to the row type -> one 16-byte chunk, rounding (RNE) while packing
+template <bool BF>
+__device__ __forceinline__ u32x4 pack_rne(const float* v) {
+  u32x4 raw;
+  if constexpr (BF) {
+    #pragma unroll
+    for (int i = 0; i < 4; ++i) raw[i] = bf16_pack_rne(v[2 * i], v[2 * i + 1]);
+  } else {
+    #pragma unroll
+    for (int i = 0; i < 4; ++i) raw[i] = f2u(v[i]);
+  }
+  return raw;
 }
 
 // N codes of one 16-byte input chunk -> storage
@@ -121,11 +150,20 @@ __device__ __forceinline__ void emit_chunk(const Op& op, const typename Op::Row&
   constexpr int N = Vec<BF>::N;
   float v[N], q[N];
   unpack<BF>(r, v);
+  if constexpr (Op::HAS_FUSED_DQ) {
+    if (!codes) {                                            // fake quant: no detour through the codes
+      if (dq) {
+        op.template fused_dq<N>(v, q, p);
+        __builtin_nontemporal_store(pack_rne<BF>(q), (u32x4*)dq + cidx);
+      }
+      return;
+    }
+  }
   op.template codes<N>(v, q, p);
   if (codes) store_codes(op, codes, cidx * N, q);
   if (dq) {
     #pragma unroll
-    for (int i = 0; i < N; ++i) v[i] = op.deq(q[i], p);
+    for (int i = 0; i < N; ++i) v[i] = op.deq_raw(q[i], p);   // rounded to the row type by the packing below
     if (op.dq_f32) {
       #pragma unroll
       for (int i = 0; i < N; i += 4) {
@@ -135,7 +173,7 @@ __device__ __forceinline__ void emit_chunk(const Op& op, const typename Op::Row&
         __builtin_nontemporal_store(w, (u32x4*)dq + (cidx * N + i) / 4);
       }
     } else {
-      __builtin_nontemporal_store(pack<BF>(v), (u32x4*)dq + cidx);
+      __builtin_nontemporal_store(pack_rne<BF>(v), (u32x4*)dq + cidx);
     }
   }
 }
@@ -352,7 +390,7 @@ int dispatch_rows(const void* x, int64_t rows, int64_t cols, void* dq, void* cod
   else if (nchunks <= 2) LCQ_TEAM(1, 2, 2);
   else if (nchunks <= 4) LCQ_TEAM(1, 4, 1);
   else if (nchunks <= 8) LCQ_TEAM(2, 4, 1);
-  else if (nchunks <= 16) LCQ_TEAM(4, 4, 1);
+  else if (nchunks <= 16) LCQ_TEAM(8, 2, 1);       // 8 lanes x 16 B: whole 128-byte lines per row and instruction
   else if (nchunks <= 32) LCQ_TEAM(8, 4, 1);
   else if (nchunks <= 64) LCQ_TEAM(16, 4, 1);
   else if (nchunks <= 128) LCQ_TEAM(32, 4, 1);
