@@ -41,8 +41,9 @@ __device__ __forceinline__ uint32_t bf16_pack(float a, float b) {               
 __device__ __forceinline__ float f16_round(float f) { return (float)(_Float16)f; }
 
 // NaN-propagating min / max (torch.amax / clamp semantics)
-__device__ __forceinline__ float nan_max(float a, float b) { return (a != a) ? a : ((b != b) ? b : fmaxf(a, b)); }
-__device__ __forceinline__ float nan_min(float a, float b) { return (a != a) ? a : ((b != b) ? b : fminf(a, b)); }
+// (IEEE 754-2019 maximum / minimum: v_maximum3_f32 / v_minimum3_f32 on gfx950, one instruction, no branches)
+__device__ __forceinline__ float nan_max(float a, float b) { return __builtin_elementwise_maximum(a, b); }
+__device__ __forceinline__ float nan_min(float a, float b) { return __builtin_elementwise_minimum(a, b); }
 
 // ---------------------------------------------------------------------------
 // cross-lane: xor butterfly built from DPP (inside a row of 16 lanes),

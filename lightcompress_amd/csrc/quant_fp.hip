@@ -30,22 +30,25 @@ struct FpOp {
   static constexpr bool BF = BF_;
   static constexpr bool HAS_PRESCALE = false;
   static constexpr bool HAS_FUSED_DQ = false;
+  static constexpr bool HAS_CUSTOM_EMIT = true;
   static constexpr int CD = -1;
   using Row = FpRow;
-  float qmax;
+  float qmax, rqmax;
   int e_bits, m_bits, tie_even, subnormals;
   int is_static, scalar_qp, dq_f32, code_dtype, scale_f32;
   // derived
   uint32_t half, keep, max_mag;
   int drop, min_exp, max_exp;
   float min_normal;
+  int hw;            // 1: e4m3, 2: e5m2 with subnormals -> v_cvt_pk_fp8_f32 / v_cvt_pk_bf8_f32 do the rounding
+  float hw_lim;      // first magnitude the float8 type cannot hold although the emulated grid can
 
   __device__ __forceinline__ Row finish(float s) const {
     Row p;
     if (s == 0.0f) s = 1.0f;                               // scales[scales == 0] = 1, quant.py:1061
     p.sm = s;
     p.s = s;
-    p.r = 1.0f / s;
+    p.r = __builtin_amdgcn_rcpf(s);      // 1 ulp: inside the error the exactness guards of x * r allow for
     const float a = fabsf(s);
     p.fast = (a > 8.6736174e-19f) && (a < 1.1529215e18f);
     return p;
@@ -55,7 +58,12 @@ struct FpOp {
     const float cmin = BF ? 1.0013580322265625e-05f : 1e-5f;
     float a = nan_max(fabsf(mx), fabsf(mn));
     a = clamp_min_nan(a, cmin);
-    return finish(rnd<BF>(a / qmax));
+    if constexpr (BF) {                                   // a * (1/qmax) unless the product is within 8 ulp of a bf16 midpoint
+      float q = a * rqmax;
+      if (__builtin_expect(((f2u(q) & 0xffffu) - 0x7ff8u) <= 0x10u, 0)) q = a / qmax;
+      return finish(rnd<BF>(q));
+    }
+    return finish(a / qmax);
   }
   __device__ __forceinline__ Row load(const void* scales, const void*, int64_t row) const {
     const int64_t i = scalar_qp ? 0 : row;
@@ -120,6 +128,87 @@ struct FpOp {
     for (int i = 0; i < N; ++i) q[i] = code(x[i], p);
   }
 
+  // One chunk through the hardware float8 converts (OCP e4m3fn / e5m2: round to nearest even,
+  // subnormals, checked against torch's casts for every bf16 value).  Used when the whole chunk is
+  // clear of every case where the converts and the emulated grid could disagree:
+  //   * a quotient x*(1/s) too close to a rounding boundary to stand for x/s (as in code());
+  //   * |t| >= hw_lim (the grid continues past the float8 maximum), inf, NaN;
+  //   * fp32 rows: an exact tie (ties-away differs from the hardware's ties-even) or a value below
+  //     the minimum normal - both are inside the boundary test above.
+  // bf16 rows hold ties all the time (8 significant bits), so ties-away is produced by the convert
+  // itself: t is scaled by 1 + 2^-10 first.  Every tie is a bf16 number, so a bf16 value that is
+  // not a tie is at least one bf16 ulp away from the nearest one and the nudge (1/4 ulp at most)
+  // cannot carry it across; an exact tie moves to the far side.  The fma also adds the "+ zeros"
+  // of the reference, which turns -0 into +0.
+  template <int N>
+  __device__ __forceinline__ bool emit_fast(const float* x, const Row& p, int64_t cidx, void* dq, void* codes) const {
+    if (!hw) return false;
+    const int cd = code_dtype;
+    float t[N];
+    bool ok = p.fast;
+    #pragma unroll
+    for (int i = 0; i < N; ++i) {
+      t[i] = x[i] * p.r;
+      if constexpr (BF) {
+        ok = ok && (((f2u(t[i]) & 0xffffu) - 0x7ff8u) > 0x10u);
+      } else {
+        const uint32_t lowm = f2u(t[i]) & ((1u << drop) - 1u);
+        ok = ok && ((lowm - (half - 8u)) > 16u) && (fabsf(t[i]) >= 1.0001f * min_normal);
+      }
+      ok = ok && (fabsf(t[i]) < hw_lim);
+    }
+    if (__builtin_expect(!ok, 0)) return false;
+    #pragma unroll
+    for (int i = 0; i < N; i += 2) rnd_pair<BF>(t[i], t[i + 1]);
+    const float nudge = (BF && !tie_even) ? 1.0009765625f : 1.0f;
+    #pragma unroll
+    for (int i = 0; i < N; ++i) t[i] = __builtin_fmaf(t[i], nudge, 0.0f);
+    uint32_t w[N / 4];
+    #pragma unroll
+    for (int k = 0; k < N / 4; ++k) {
+      int u = 0;
+      if (hw == 1) {
+        u = __builtin_amdgcn_cvt_pk_fp8_f32(t[4 * k], t[4 * k + 1], u, false);
+        u = __builtin_amdgcn_cvt_pk_fp8_f32(t[4 * k + 2], t[4 * k + 3], u, true);
+      } else {
+        u = __builtin_amdgcn_cvt_pk_bf8_f32(t[4 * k], t[4 * k + 1], u, false);
+        u = __builtin_amdgcn_cvt_pk_bf8_f32(t[4 * k + 2], t[4 * k + 3], u, true);
+      }
+      w[k] = (uint32_t)u;
+    }
+    if (codes && cd == LCQ_CODE_FP8) {
+      if constexpr (N == 8) *(u32x2*)((uint8_t*)codes + cidx * N) = u32x2{w[0], w[1]};
+      else *(uint32_t*)((uint8_t*)codes + cidx * N) = w[0];
+    }
+    if (dq || (codes && cd == LCQ_CODE_F32)) {
+      float q[N];
+      #pragma unroll
+      for (int k = 0; k < N / 4; ++k) {
+        f32x2 lo, hi;
+        if (hw == 1) { lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[k], false); hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[k], true); }
+        else { lo = __builtin_amdgcn_cvt_pk_f32_bf8((int)w[k], false); hi = __builtin_amdgcn_cvt_pk_f32_bf8((int)w[k], true); }
+        q[4 * k] = lo[0]; q[4 * k + 1] = lo[1]; q[4 * k + 2] = hi[0]; q[4 * k + 3] = hi[1];
+      }
+      if (codes && cd == LCQ_CODE_F32) {
+        #pragma unroll
+        for (int i = 0; i < N; i += 4) *(f32x4*)((float*)codes + cidx * N + i) = f32x4{q[i], q[i + 1], q[i + 2], q[i + 3]};
+      }
+      if (dq) {
+        #pragma unroll
+        for (int i = 0; i < N; ++i) q[i] = deq_raw(q[i], p);
+        if (dq_f32) {
+          #pragma unroll
+          for (int i = 0; i < N; i += 4)
+            __builtin_nontemporal_store(u32x4{f2u(q[i]), f2u(q[i + 1]), f2u(q[i + 2]), f2u(q[i + 3])},
+                                        (u32x4*)dq + (cidx * N + i) / 4);
+        } else {
+          __builtin_nontemporal_store(pack_rne<BF>(q), (u32x4*)dq + cidx);
+        }
+      }
+    }
+    return true;
+  }
+
   // (q - 0.0) * s in fp32, then the cast of fake_quant_* (quant.py:1107,1153)
   __device__ __forceinline__ float deq_raw(float q, const Row& p) const { return (q - 0.0f) * p.sm; }
   __device__ __forceinline__ float deq(float q, const Row& p) const {
@@ -157,7 +246,7 @@ struct FpOp {
 template <bool BF>
 FpOp<BF> make_op(int e_bits, int m_bits, float qmax, int flags, int code_dtype) {
   FpOp<BF> c;
-  c.qmax = qmax; c.e_bits = e_bits; c.m_bits = m_bits;
+  c.qmax = qmax; c.rqmax = (float)(1.0 / (double)qmax); c.e_bits = e_bits; c.m_bits = m_bits;
   c.tie_even = (flags & LCQ_FLAG_TIE_EVEN) != 0;
   c.subnormals = (flags & LCQ_FLAG_NO_SUBNORMALS) == 0;
   c.is_static = (flags & LCQ_FLAG_STATIC) != 0;
@@ -172,6 +261,9 @@ FpOp<BF> make_op(int e_bits, int m_bits, float qmax, int flags, int code_dtype) 
   c.max_exp = 1 << (e_bits - 1);
   c.max_mag = ((uint32_t)(c.max_exp + 127) << 23) | (((1u << m_bits) - 1u) << c.drop);
   c.min_normal = __builtin_ldexpf(1.0f, c.min_exp);
+  c.hw = 0; c.hw_lim = 0.0f;
+  if (c.subnormals && e_bits == 4 && m_bits == 3) { c.hw = 1; c.hw_lim = 464.0f; }       // 448 is the float8 maximum
+  if (c.subnormals && e_bits == 5 && m_bits == 2) { c.hw = 2; c.hw_lim = 61440.0f; }     // 57344
   return c;
 }
 

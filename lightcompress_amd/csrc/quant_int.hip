@@ -36,9 +36,11 @@ struct IntOp {
   static constexpr bool BF = BF_;
   static constexpr bool HAS_PRESCALE = PRESCALE;
   static constexpr bool HAS_FUSED_DQ = FAST;
+  static constexpr bool HAS_CUSTOM_EMIT = false;
   static constexpr int CD = CD_;
   using Row = IntRow;
   float qmin, qmax, qrange, osf;
+  float rqmax, rqrange;         // 1 / qmax, 1 / qrange (fp32-rounded)
   int sym, round_zp, is_static, scalar_qp, dq_f32, code_dtype, range_bf16, scale_f32;
   // optional per-column factor applied first (AWQ: W * s), rows of the reshaped tensor tile a
   // weight row of wrow_cols columns
@@ -64,13 +66,26 @@ struct IntOp {
   __device__ __forceinline__ Row finish(float s, float z) const {
     Row p;
     p.s = s; p.z = z;
-    p.r = 1.0f / s;
+    p.r = __builtin_amdgcn_rcpf(s);      // 1 ulp: inside the error the exactness guards of x * r allow for
     const float a = fabsf(s);
     p.fast = (a > 8.6736174e-19f) && (a < 1.1529215e18f) && (fabsf(z) <= 512.0f);   // s in 2^-60 .. 2^60
     p.zint = (z == rintf(z)) && (fabsf(z) <= 512.0f);       // caller-given zero points need not be integers
     p.sdq = scale_f32 ? s * osf : rnd<BF>(s * osf);
     p.lo = qmin - z; p.hi = qmax - z;                       // exact: small integers
     return p;
+  }
+
+  // a / c for a per-launch constant c (rc = 1/c rounded to fp32), rounded to the row type.  bf16 rows:
+  // the product a * rc stands for the quotient unless it lies within 8 ulp of a bf16 rounding
+  // midpoint; fp32 rows need the correctly rounded quotient itself.
+  __device__ __forceinline__ float div_const(float a, float c, float rc) const {
+    if constexpr (BF) {
+      float q = a * rc;
+      if (__builtin_expect(((f2u(q) & 0xffffu) - 0x7ff8u) <= 0x10u, 0)) q = a / c;
+      return rnd<BF>(q);
+    } else {
+      return a / c;
+    }
   }
 
   // get_qparams, quant.py:544-558
@@ -80,14 +95,25 @@ struct IntOp {
     if (sym) {
       float a = nan_max(fabsf(mx), fabsf(mn));
       a = clamp_min_nan(a, cmin);
-      s = rnd<BF>(a / qmax);
+      s = div_const(a, qmax, rqmax);
       z = 0.0f;
     } else {
       float d = rnd<BF>(mx - mn);
       if (range_bf16) d = bf16_round(d);
       d = clamp_min_nan(d, cmin);
-      s = rnd<BF>(d / qrange);
-      const float t = rnd<BF>(mn / s);
+      s = div_const(d, qrange, rqrange);
+      // mn / s through the reciprocal, with the same exactness guards as the per-element quotients
+      float t = mn * __builtin_amdgcn_rcpf(s);
+      const float as = fabsf(s);
+      bool ok = (as > 8.6736174e-19f) && (as < 1.1529215e18f);
+      if constexpr (BF) {
+        ok = ok && (((f2u(t) & 0xffffu) - 0x7ff8u) > 0x10u);
+      } else {
+        const float fr = t - rintf(t);
+        ok = ok && (fabsf(fabsf(fr) - 0.5f) > 4.8828125e-04f) && (fabsf(t) <= 1024.0f) && round_zp;
+      }
+      if (__builtin_expect(!ok, 0)) t = mn / s;
+      t = rnd<BF>(t);
       if (round_zp) {
         z = rnd<BF>(qmin - rintf(t));
         z = fminf(fmaxf(z, qmin), qmax);
@@ -217,6 +243,7 @@ template <class Op>
 Op make_op(float qmin, float qmax, int flags, float osf, int code_dtype) {
   Op c;
   c.qmin = qmin; c.qmax = qmax; c.qrange = qmax - qmin; c.osf = osf;
+  c.rqmax = (float)(1.0 / (double)qmax); c.rqrange = (float)(1.0 / (double)(qmax - qmin));
   c.sym = (flags & LCQ_FLAG_SYM) != 0;
   c.round_zp = (flags & LCQ_FLAG_NO_ROUND_ZP) == 0;
   c.is_static = (flags & LCQ_FLAG_STATIC) != 0;

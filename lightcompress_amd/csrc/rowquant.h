@@ -28,13 +28,13 @@ namespace lcq {
 template <bool BF> struct Vec { static constexpr int N = BF ? 8 : 4; };
 
 template <bool BF> __device__ __forceinline__ float rnd(float v) {
-  if constexpr (BF) return bf16_round(v); else return v;
+  if constexpr (BF) return (float)(__bf16)v; else return v;
 }
 // per-element rounding: hardware RNE convert (v_cvt_pk_bf16_f32)
 template <bool BF> __device__ __forceinline__ float rnd_e(float v) {
   if constexpr (BF) return (float)(__bf16)v; else return v;
 }
-__device__ __forceinline__ float clamp_min_nan(float v, float lo) { return (v != v) ? v : fmaxf(v, lo); }
+__device__ __forceinline__ float clamp_min_nan(float v, float lo) { return nan_max(v, lo); }
 
 // two fp32 values -> one dword of two bf16 (RNE), a single v_cvt_pk_bf16_f32
 typedef float lcq_f32x2 __attribute__((ext_vector_type(2)));
@@ -178,25 +178,23 @@ __device__ __forceinline__ void emit_chunk(const Op& op, const typename Op::Row&
   }
 }
 
-// running min / max of a chunk with v_min3 / v_max3 (which skip NaNs); `nan` remembers whether
-// any element was a NaN so the caller can poison the range like torch.amax / amin do
+// running min / max of a chunk; NaN-propagating like torch.amax / amin (v_minimum3 / v_maximum3)
 template <class Op>
-__device__ __forceinline__ void chunk_minmax(const u32x4& r, float& mn, float& mx, bool& nan) {
+__device__ __forceinline__ void chunk_minmax(const u32x4& r, float& mn, float& mx) {
   constexpr int N = Vec<Op::BF>::N;
   float v[N];
   unpack<Op::BF>(r, v);
   #pragma unroll
   for (int i = 0; i < N; i += 2) {
-    mn = fminf(fminf(mn, v[i]), v[i + 1]);
-    mx = fmaxf(fmaxf(mx, v[i]), v[i + 1]);
-    nan = nan || (v[i] != v[i]) || (v[i + 1] != v[i + 1]);
+    mn = nan_min(nan_min(mn, v[i]), v[i + 1]);
+    mx = nan_max(nan_max(mx, v[i]), v[i + 1]);
   }
 }
-// range of a row from the per-lane partials: NaN anywhere in the team poisons both ends
+// range of a row from the per-lane partials
 template <int TEAM>
-__device__ __forceinline__ void team_range(float& mn, float& mx, bool nan) {
-  mn = team_reduce<TEAM, false>(nan ? __builtin_nanf("") : mn);
-  mx = team_reduce<TEAM, true>(nan ? __builtin_nanf("") : mx);
+__device__ __forceinline__ void team_range(float& mn, float& mx) {
+  mn = team_reduce<TEAM, false>(mn);
+  mx = team_reduce<TEAM, true>(mx);
 }
 
 // ---------------------------------------------------------------------------
@@ -234,11 +232,10 @@ __global__ __launch_bounds__(256) void row_team_kernel(
     typename Op::Row p;
     if (!op.is_static) {
       float mn = __builtin_inff(), mx = -__builtin_inff();
-      bool nan = false;
       #pragma unroll
       for (int it = 0; it < ITERS; ++it)
-        if (FULL || t + it * TEAM < nchunks) chunk_minmax<Op>(raw[u][it], mn, mx, nan);
-      team_range<TEAM>(mn, mx, nan);
+        if (FULL || t + it * TEAM < nchunks) chunk_minmax<Op>(raw[u][it], mn, mx);
+      team_range<TEAM>(mn, mx);
       p = op.make(mn, mx);
       if (row_ok && t == 0) op.store_qp(scales, zeros, row, p);
     } else {
@@ -285,17 +282,16 @@ __global__ __launch_bounds__(256) void row_block_kernel(
   typename Op::Row p;
   if (!op.is_static) {
     float mn = __builtin_inff(), mx = -__builtin_inff();
-    bool nan = false;
     #pragma unroll
     for (int k = 0; k < CACHE; ++k)
-      if ((int)threadIdx.x + k * 256 < nchunks) chunk_minmax<Op>(raw[k], mn, mx, nan);
+      if ((int)threadIdx.x + k * 256 < nchunks) chunk_minmax<Op>(raw[k], mn, mx);
     for (int ch = threadIdx.x + CACHE * 256; ch < nchunks; ch += 256) {
       u32x4 r = xr[ch];
       if constexpr (Op::HAS_PRESCALE) r = op.prescale(r, row, ch, nchunks);
-      chunk_minmax<Op>(r, mn, mx, nan);
+      chunk_minmax<Op>(r, mn, mx);
     }
-    mn = block_reduce<false>(nan ? __builtin_nanf("") : mn, sm);
-    mx = block_reduce<true>(nan ? __builtin_nanf("") : mx, sm);
+    mn = block_reduce<false>(mn, sm);
+    mx = block_reduce<true>(mx, sm);
     p = op.make(mn, mx);
     if (threadIdx.x == 0) op.store_qp(scales, zeros, row, p);
   } else {
