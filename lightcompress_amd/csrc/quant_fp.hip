@@ -145,19 +145,30 @@ struct FpOp {
     if (!hw) return false;
     const int cd = code_dtype;
     float t[N];
-    bool ok = p.fast;
+    bool near = !p.fast, far = false;
     #pragma unroll
     for (int i = 0; i < N; ++i) {
       t[i] = x[i] * p.r;
       if constexpr (BF) {
-        ok = ok && (((f2u(t[i]) & 0xffffu) - 0x7ff8u) > 0x10u);
+        near = near || (((f2u(t[i]) & 0xffffu) - 0x7ff8u) <= 0x10u);
       } else {
         const uint32_t lowm = f2u(t[i]) & ((1u << drop) - 1u);
-        ok = ok && ((lowm - (half - 8u)) > 16u) && (fabsf(t[i]) >= 1.0001f * min_normal);
+        far = far || ((lowm - (half - 8u)) <= 16u) || !(fabsf(t[i]) >= 1.0001f * min_normal);
       }
-      ok = ok && (fabsf(t[i]) < hw_lim);
+      far = far || !(fabsf(t[i]) < hw_lim);
     }
-    if (__builtin_expect(!ok, 0)) return false;
+    if (__builtin_expect(far, 0)) return false;              // left to the emulated grid (rare: ties of fp32 rows, inf, NaN)
+    if constexpr (BF) {
+      if (__builtin_expect(near, 0)) {                       // the product may round unlike the quotient: divide
+        #pragma unroll
+        for (int i = 0; i < N; ++i) t[i] = x[i] / p.s;
+        #pragma unroll
+        for (int i = 0; i < N; ++i) far = far || !(fabsf(t[i]) < hw_lim);
+        if (far) return false;
+      }
+    } else {
+      if (!p.fast) return false;
+    }
     #pragma unroll
     for (int i = 0; i < N; i += 2) rnd_pair<BF>(t[i], t[i + 1]);
     const float nudge = (BF && !tie_even) ? 1.0009765625f : 1.0f;

@@ -142,23 +142,15 @@ __device__ __forceinline__ void store_code1(const Op& op, void* codes, int64_t e
   else if (cd == LCQ_CODE_SAME) store_scalar<Op::BF>(codes, e, q);
 }
 
-// codes + dq of one chunk
+// codes + dq of one chunk, generic form: op.codes -> storage, op.deq_raw -> storage
 template <class Op>
-__device__ __forceinline__ void emit_chunk(const Op& op, const typename Op::Row& p, const u32x4& r, int64_t cidx,
-                                           void* dq, void* codes) {
+__device__ __forceinline__ void emit_chunk_generic(const Op& op, const typename Op::Row& p, const float* v_in, int64_t cidx,
+                                                   void* dq, void* codes) {
   constexpr bool BF = Op::BF;
   constexpr int N = Vec<BF>::N;
   float v[N], q[N];
-  unpack<BF>(r, v);
-  if constexpr (Op::HAS_FUSED_DQ) {
-    if (!codes) {                                            // fake quant: no detour through the codes
-      if (dq) {
-        op.template fused_dq<N>(v, q, p);
-        __builtin_nontemporal_store(pack_rne<BF>(q), (u32x4*)dq + cidx);
-      }
-      return;
-    }
-  }
+  #pragma unroll
+  for (int i = 0; i < N; ++i) v[i] = v_in[i];
   op.template codes<N>(v, q, p);
   if (codes) store_codes(op, codes, cidx * N, q);
   if (dq) {
@@ -176,6 +168,39 @@ __device__ __forceinline__ void emit_chunk(const Op& op, const typename Op::Row&
       __builtin_nontemporal_store(pack_rne<BF>(v), (u32x4*)dq + cidx);
     }
   }
+}
+// Returns false when the op's fast path declined the chunk (HAS_CUSTOM_EMIT only): the caller
+// then runs emit_chunk_slow on it, from ONE rolled loop, so the long generic code exists once per
+// kernel instead of once per unrolled chunk (and stays out of the instruction cache).
+template <class Op>
+__device__ __forceinline__ bool emit_chunk(const Op& op, const typename Op::Row& p, const u32x4& r, int64_t cidx,
+                                           void* dq, void* codes) {
+  constexpr bool BF = Op::BF;
+  constexpr int N = Vec<BF>::N;
+  float v[N], q[N];
+  unpack<BF>(r, v);
+  if constexpr (Op::HAS_CUSTOM_EMIT) {
+    return op.template emit_fast<N>(v, p, cidx, dq, codes);
+  } else {
+    if constexpr (Op::HAS_FUSED_DQ) {
+      if (!codes) {                                          // fake quant: no detour through the codes
+        if (dq) {
+          op.template fused_dq<N>(v, q, p);
+          __builtin_nontemporal_store(pack_rne<BF>(q), (u32x4*)dq + cidx);
+        }
+        return true;
+      }
+    }
+    emit_chunk_generic(op, p, v, cidx, dq, codes);
+    return true;
+  }
+}
+template <class Op>
+__device__ __forceinline__ void emit_chunk_slow(const Op& op, const typename Op::Row& p, const u32x4& r, int64_t cidx,
+                                                void* dq, void* codes) {
+  float v[Vec<Op::BF>::N];
+  unpack<Op::BF>(r, v);
+  emit_chunk_generic(op, p, v, cidx, dq, codes);
 }
 
 // running min / max of a chunk; NaN-propagating like torch.amax / amin (v_minimum3 / v_maximum3)
@@ -241,10 +266,22 @@ __global__ __launch_bounds__(256) void row_team_kernel(
     } else {
       p = op.load(scales, zeros, row_ok ? row : 0);
     }
+    uint32_t redo = 0;
     #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       const int ch = t + it * TEAM;
-      if (FULL || (row_ok && ch < nchunks)) emit_chunk(op, p, raw[u][it], row * nchunks + ch, dq, codes);
+      if (FULL || (row_ok && ch < nchunks))
+        if (!emit_chunk(op, p, raw[u][it], row * nchunks + ch, dq, codes)) redo |= 1u << it;
+    }
+    if constexpr (Op::HAS_CUSTOM_EMIT) {
+      #pragma unroll 1
+      for (int it = 0; redo; ++it, redo >>= 1)
+        if (redo & 1u) {
+          const int ch = t + it * TEAM;
+          u32x4 r = x[row * nchunks + ch];
+          if constexpr (Op::HAS_PRESCALE) r = op.prescale(r, row, ch, nchunks);
+          emit_chunk_slow(op, p, r, row * nchunks + ch, dq, codes);
+        }
     }
   }
 }
@@ -263,6 +300,18 @@ __device__ __forceinline__ float block_reduce(float v, float* sm) {
   float r = sm[0];
   for (int i = 1; i < nw; ++i) r = IS_MAX ? nan_max(r, sm[i]) : nan_min(r, sm[i]);
   return r;
+}
+
+// min and max of a workgroup in one round: two barriers instead of four
+__device__ __forceinline__ void block_range(float& mn, float& mx, float* sm) {
+  mn = team_reduce<64, false>(mn);
+  mx = team_reduce<64, true>(mx);
+  const int w = threadIdx.x >> 6;
+  __syncthreads();                                           // previous readers of sm are done
+  if ((threadIdx.x & 63) == 0) { sm[w] = mn; sm[4 + w] = mx; }
+  __syncthreads();
+  mn = nan_min(nan_min(sm[0], sm[1]), nan_min(sm[2], sm[3]));
+  mx = nan_max(nan_max(sm[4], sm[5]), nan_max(sm[6], sm[7]));
 }
 
 template <class Op, int CACHE>
@@ -290,22 +339,34 @@ __global__ __launch_bounds__(256) void row_block_kernel(
       if constexpr (Op::HAS_PRESCALE) r = op.prescale(r, row, ch, nchunks);
       chunk_minmax<Op>(r, mn, mx);
     }
-    mn = block_reduce<false>(mn, sm);
-    mx = block_reduce<true>(mx, sm);
+    block_range(mn, mx, sm);
     p = op.make(mn, mx);
     if (threadIdx.x == 0) op.store_qp(scales, zeros, row, p);
   } else {
     p = op.load(scales, zeros, row);
   }
+  // chunks the fast path declines are redone by the generic code in the rolled loop at the end
+  bool redo = false;
   #pragma unroll
   for (int k = 0; k < CACHE; ++k) {
     const int ch = threadIdx.x + k * 256;
-    if (ch < nchunks) emit_chunk(op, p, raw[k], row * nchunks + ch, dq, codes);
+    if (ch < nchunks) redo = !emit_chunk(op, p, raw[k], row * nchunks + ch, dq, codes) || redo;
   }
   for (int ch = threadIdx.x + CACHE * 256; ch < nchunks; ch += 256) {
     u32x4 r = xr[ch];
     if constexpr (Op::HAS_PRESCALE) r = op.prescale(r, row, ch, nchunks);
-    emit_chunk(op, p, r, row * nchunks + ch, dq, codes);
+    redo = !emit_chunk(op, p, r, row * nchunks + ch, dq, codes) || redo;
+  }
+  if constexpr (Op::HAS_CUSTOM_EMIT) {
+    if (__builtin_expect(redo, 0)) {
+      // rare: redo every chunk of this lane with the generic code (same results where the fast path ran)
+      #pragma unroll 1
+      for (int ch = threadIdx.x; ch < nchunks; ch += 256) {
+        u32x4 r = xr[ch];
+        if constexpr (Op::HAS_PRESCALE) r = op.prescale(r, row, ch, nchunks);
+        emit_chunk_slow(op, p, r, row * nchunks + ch, dq, codes);
+      }
+    }
   }
 }
 
@@ -392,7 +453,7 @@ int dispatch_rows(const void* x, int64_t rows, int64_t cols, void* dq, void* cod
   else if (nchunks <= 128) LCQ_TEAM(32, 4, 1);
   else if (nchunks <= 256) LCQ_TEAM(64, 4, 1);
   else {
-    row_block_kernel<Op, 8><<<dim3((unsigned)rows), dim3(256), 0, st>>>(
+    row_block_kernel<Op, 4><<<dim3((unsigned)rows), dim3(256), 0, st>>>(
         (const u32x4*)x, dq, codes, scales, zeros, rows, nchunks, op);
   }
   #undef LCQ_TEAM
