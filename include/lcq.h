@@ -38,6 +38,9 @@ extern "C" {
 #define LCQ_CODE_SAME 4      /* codes stored as floats of the input type (what .quant() returns) */
 #define LCQ_CODE_F32 5       /* FloatQuantizer.quant(): fp32 values on the minifloat grid */
 #define LCQ_CODE_FP8 6       /* float8_e4m3fn / float8_e5m2 bytes */
+#define LCQ_CODE_CT4 7       /* lcq_quant_int: 4-bit codes packed like VllmRealQuantLinear.pack (module_utils.py:929-955):
+                                nibble i of int32 word j of a tensor row = code[8j+i] + 8; needs -8 <= qmin, qmax <= 7
+                                and cols % 8 == 0; `codes` is int32 [rows * cols / 8] */
 
 /* flags */
 #define LCQ_FLAG_SYM 1            /* symmetric: zero point is 0 */

@@ -271,6 +271,7 @@ int run(const void* x, int64_t rows, int64_t cols, float qmin, float qmax, int f
     case LCQ_CODE_NONE: LCQ_RUN(LCQ_CODE_NONE);
     case LCQ_CODE_U8: LCQ_RUN(LCQ_CODE_U8);
     case LCQ_CODE_I32: LCQ_RUN(LCQ_CODE_I32);
+    case LCQ_CODE_CT4: LCQ_RUN(LCQ_CODE_CT4);
     default: LCQ_RUN(-1);
   }
   #undef LCQ_RUN
@@ -352,8 +353,13 @@ int lcq_quant_int(const void* x, int dtype, int64_t rows, int64_t cols, float qm
   if (!x || rows < 0 || cols <= 0 || !scales) return LCQ_EINVAL;
   if (rows == 0) return LCQ_OK;
   if (codes && !(code_dtype == LCQ_CODE_U8 || code_dtype == LCQ_CODE_I8 || code_dtype == LCQ_CODE_I32 ||
-                 code_dtype == LCQ_CODE_SAME)) return LCQ_EDTYPE;
+                 code_dtype == LCQ_CODE_SAME || code_dtype == LCQ_CODE_CT4)) return LCQ_EDTYPE;
   if (!(qmax > qmin)) return LCQ_EINVAL;
+  if (codes && code_dtype == LCQ_CODE_CT4) {
+    // only the vectorised kernels store nibbles: 16-byte chunks, codes + 8 within a nibble
+    if (qmin < -8.0f || qmax > 7.0f || (flags & LCQ_FLAG_NO_ROUND_ZP) || cols % 8 != 0) return LCQ_EINVAL;
+    if ((((uintptr_t)x | (uintptr_t)dq) % 16) != 0 || ((uintptr_t)codes % 4) != 0) return LCQ_EALIGN;
+  }
   if ((flags & LCQ_FLAG_SCALAR_QP) && !(flags & LCQ_FLAG_STATIC)) return LCQ_EINVAL;
   if ((flags & LCQ_FLAG_SCALE_F32) && !(flags & LCQ_FLAG_STATIC)) return LCQ_EINVAL;
   if (!codes) code_dtype = LCQ_CODE_NONE;

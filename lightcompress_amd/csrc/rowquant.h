@@ -131,6 +131,13 @@ __device__ __forceinline__ void store_codes(const Op& op, void* codes, int64_t e
     }
   } else if (cd == LCQ_CODE_SAME) {
     *((u32x4*)codes + elem0 / N) = pack<BF>(q);
+  } else if (cd == LCQ_CODE_CT4) {
+    // compressed-tensors nibbles: 8 codes per int32 word, a 4-element chunk fills half a word
+    uint32_t w = 0;
+    #pragma unroll
+    for (int i = 0; i < N; ++i) w |= (((uint32_t)(int32_t)q[i] + 8u) & 0xfu) << (4 * i);
+    if constexpr (N == 8) ((uint32_t*)codes)[elem0 / 8] = w;
+    else ((uint16_t*)codes)[elem0 / 4] = (uint16_t)w;
   }
 }
 template <class Op>
@@ -433,7 +440,8 @@ int dispatch_rows(const void* x, int64_t rows, int64_t cols, void* dq, void* cod
                   const Op& op, bool force_scalar, hipStream_t st) {
   constexpr int N = Vec<Op::BF>::N;
   if (rows > 0x7fffffff) return LCQ_EINVAL;
-  const bool aligned = (cols % N == 0) && (((uintptr_t)x | (uintptr_t)dq | (uintptr_t)codes) % 16 == 0);
+  const bool aligned = (cols % N == 0) && (((uintptr_t)x | (uintptr_t)dq) % 16 == 0) &&
+                       ((uintptr_t)codes % (Op::CD == LCQ_CODE_CT4 ? 4 : 16) == 0);
   if (!aligned || force_scalar) {
     const int64_t grid = (rows + 3) / 4;
     row_scalar_kernel<Op><<<dim3((unsigned)grid), dim3(256), 0, st>>>(x, dq, codes, scales, zeros, rows, cols, op);

@@ -33,6 +33,15 @@ class VllmRealQuantLinear:
                                     L.ptr(packed), L.stream()), 'lcq_pack_ct')
         return packed, scales.to(torch.float16)
 
+    @classmethod
+    @torch.no_grad()
+    def quant_pack(cls, weight, wquantizer, quant_config):
+        """pack(*wquantizer.real_quant_weight_dynamic(weight)[:2], quant_config) in one kernel: the bf16 / fp32
+        weight is read once and only the packed words and the scales are written."""
+        assert quant_config['weight']['bit'] == 4
+        packed, scales, _ = wquantizer.real_quant_pack_dynamic(weight)
+        return packed, scales.to(torch.float16)
+
 
 class AutoawqRealQuantLinear:
     @classmethod

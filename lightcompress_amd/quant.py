@@ -234,6 +234,8 @@ class IntegerQuantizer(BaseQuantizer):
         if want_codes is not None:
             if want_codes == 'same':
                 codes, cd = torch.empty_like(t), L.CODE_SAME
+            elif want_codes == 'ct4':                    # eight 4-bit codes (+8) per int32, in row order
+                codes, cd = torch.empty(t.numel() // 8, dtype=torch.int32, device=t.device), L.CODE_CT4
             else:
                 codes = torch.empty(t.shape, dtype=want_codes, device=t.device)
                 cd = {torch.int32: L.CODE_I32, torch.int8: L.CODE_I8, torch.uint8: L.CODE_U8}[want_codes]
@@ -404,6 +406,17 @@ class IntegerQuantizer(BaseQuantizer):
         _, codes, scales, zeros = self._launch(rows_t, static=False, want_codes=self._code_dtype())
         codes = self.restore_tensor(codes.view(rows_t.shape), org_w_shape)
         return self._finish_real(codes, scales, zeros, output_scale_factor)
+
+    def real_quant_pack_dynamic(self, weight):
+        """Quantize and pack in one pass: what VllmRealQuantLinear.pack(*real_quant_weight_dynamic(w)[:2])
+        returns for a symmetric 4-bit quantizer (module_utils.py:929-955 after quant.py:915-952), without
+        the int32 codes ever reaching HBM -> (int32 [R, K/8], scales [R, -1], None)."""
+        if self.bit != 4 or not self.sym or weight.dim() != 2 or weight.shape[1] % 8 != 0:
+            raise NotImplementedError('fused quantize+pack: symmetric 4-bit, 2-D weight, in_features % 8 == 0')
+        rows_t = self.reshape_tensor(weight)
+        _, packed, scales, _ = self._launch(rows_t, static=False, want_codes='ct4')
+        qparams_shape = 1 if self.granularity == 'per_tensor' else (weight.shape[0], -1)
+        return packed.view(weight.shape[0], weight.shape[1] // 8), scales.view(qparams_shape), None
 
     def __repr__(self):
         return (

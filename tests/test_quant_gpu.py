@@ -249,6 +249,29 @@ def test_pack_ct_bit_exact(dev, bits, dt, shape):
     assert torch.equal(pack_ref.unpack_ct(got.cpu(), bits, shape[1]), codes.to(torch.int32))
 
 
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('gran,shape', [('per_group', (64, 1024)), ('per_group', (2048, 7168)), ('per_channel', (96, 512)),
+                                        ('per_channel', (16, 7168))])
+def test_fused_quant_pack_equals_quant_then_pack(dev, dtype, gran, shape):
+    """One-pass quantize+pack == VllmRealQuantLinear.pack(real_quant_weight_dynamic(w)) == the oracle's pack."""
+    from lightcompress_amd import IntegerQuantizer
+    from lightcompress_amd.module_utils import VllmRealQuantLinear
+    w = weight_like(*shape, seed=shape[1] + 7, dtype=dtype, std=0.006, outlier_frac=0.0005, outlier_mul=30)
+    kw = dict(group_size=128) if gran == 'per_group' else {}
+    q = IntegerQuantizer(4, True, gran, **kw)
+    cfg = {'weight': {'bit': 4}}
+    wd = w.to(dev)
+    codes, s, z = q.real_quant_weight_dynamic(wd)
+    two_step, s16 = VllmRealQuantLinear.pack(codes, s, cfg)
+    fused, fs16 = VllmRealQuantLinear.quant_pack(wd, q, cfg)
+    assert_bit_equal(fused, two_step, 'packed words')
+    assert_bit_equal(fs16, s16, 'fp16 scales')
+    spec = Q.IntSpec(4, True, gran, group_size=kw.get('group_size', 0))
+    ocodes, os_, _ = Q.int_real_quant_dynamic(spec, w)
+    opacked, _ = pack_ref.pack_ct(ocodes, os_, 4)
+    assert_bit_equal(fused, opacked, 'oracle pack')
+
+
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize('shape', [(64, 256), (320, 1024), (2048, 512)])
 def test_gemm_pack_bit_exact(dev, dtype, shape):
