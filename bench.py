@@ -160,12 +160,12 @@ def gpu_main(args):
     nbuf = 6
     ws = [torch.randn(4096, 4096, device=dev) * 0.02 for _ in range(nbuf)]
     dq = [torch.empty_like(w) for w in ws]
-    codes = torch.empty(4096, 4096, dtype=torch.uint8, device=dev)
+    codes = [torch.empty(4096, 4096, dtype=torch.uint8, device=dev) for _ in range(nbuf)]
     rows = 4096 * 4096 // 128
     sc, zr = torch.empty(rows, 1, device=dev), torch.empty(rows, 1, device=dev)
     def rtn(i):
         L.check(lib.lcq_quant_int(L.ptr(ws[i % nbuf]), L.i32(L.F32), L.i64(rows), L.i64(128), L.f32(0), L.f32(15),
-                                  L.i32(0), L.f32(1), L.ptr(dq[i % nbuf]), L.ptr(codes), L.i32(L.CODE_U8), L.ptr(sc),
+                                  L.i32(0), L.f32(1), L.ptr(dq[i % nbuf]), L.ptr(codes[i % nbuf]), L.i32(L.CODE_U8), L.ptr(sc),
                                   L.ptr(zr), st), 'quant')
     for i in range(6):
         rtn(i)

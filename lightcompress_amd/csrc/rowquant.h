@@ -238,6 +238,10 @@ __global__ __launch_bounds__(256) void row_team_kernel(
     const u32x4* __restrict__ x, void* __restrict__ dq, void* __restrict__ codes,
     void* __restrict__ scales, void* __restrict__ zeros, int64_t rows, int nchunks, Op op) {
   constexpr int RPW = LCQ_WAVE / TEAM;                      // rows per wave per batch
+  constexpr int N = Vec<Op::BF>::N;
+  // one-byte codes of a full grid whose lanes each produce exactly 16 bytes of them
+  constexpr bool STAGED = FULL && !Op::HAS_CUSTOM_EMIT && (Op::CD == LCQ_CODE_U8 || Op::CD == LCQ_CODE_I8) && ITERS * N == 16;
+  __shared__ uint32_t stage[STAGED ? 4 * RPW * TEAM * 4 : 1];
   const int lane = threadIdx.x & 63;
   const int t = lane & (TEAM - 1);
   const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
@@ -272,6 +276,30 @@ __global__ __launch_bounds__(256) void row_team_kernel(
       if (row_ok && t == 0) op.store_qp(scales, zeros, row, p);
     } else {
       p = op.load(scales, zeros, row_ok ? row : 0);
+    }
+    if constexpr (STAGED) {
+      if (codes) {
+        // byte codes: a lane's chunks are 8*TEAM.. elements apart, so direct stores would write 4-8 byte
+        // pieces of every line; the words take a detour through LDS (same wave: no barrier) and
+        // leave as ONE 16-byte store per lane, a full line per row
+        uint32_t* const wrow = stage + (threadIdx.x >> 6) * (RPW * TEAM * 4) + (lane / TEAM) * (TEAM * 4);
+        #pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+          float v[N], q[N];
+          unpack<Op::BF>(raw[u][it], v);
+          op.template codes<N>(v, q, p);
+          #pragma unroll
+          for (int k = 0; k < N / 4; ++k) wrow[(t + it * TEAM) * (N / 4) + k] = op.pack4(q + 4 * k);
+          if (dq) {
+            #pragma unroll
+            for (int i = 0; i < N; ++i) v[i] = op.deq_raw(q[i], p);
+            __builtin_nontemporal_store(pack_rne<Op::BF>(v), (u32x4*)dq + (row * nchunks + t + it * TEAM));
+          }
+        }
+        const u32x4 w = *(const u32x4*)(wrow + t * 4);
+        *((u32x4*)((uint8_t*)codes + row * (int64_t)(TEAM * 16)) + t) = w;
+        continue;
+      }
     }
     uint32_t redo = 0;
     #pragma unroll
