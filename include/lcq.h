@@ -184,6 +184,49 @@ int lcq_gptq_block(float* W, float* tmp, float* Losses, float* Err, int64_t ldEr
 int lcq_gptq_trailing(float* W, const float* Err, int64_t ldErr, const float* U, int64_t R, int64_t K, int64_t k1,
                       int64_t k2, int64_t j1, int64_t j2, void* stream);
 
+/* ---- AWQ scale search ------------------------------------------------------- */
+
+/* Awq.fake_quantize_weight, awq.py:147-164 with scaling_weight :39-46 fused in:
+ *   out = fake_quant_weight_dynamic(W * s[None, :])   (W*s rounds to the tensor type first)
+ *  W, out [R, K] of `dtype`; colscale [K] of `dtype`, 16-byte aligned; group_size 0 = per_channel.
+ * W is not modified (the reference multiplies in place and restores the weights afterwards). */
+int lcq_awq_scale_quant(const void* w, int dtype, int64_t R, int64_t K, const void* colscale, int group_size,
+                        float qmin, float qmax, int flags, void* out, void* stream);
+
+/* workspace of lcq_absmean_cols / lcq_awq_weight_scale / lcq_sq_err_mean for K columns */
+int64_t lcq_awq_workspace_bytes(int64_t K);
+
+/* Awq.get_act_scale, awq.py:74-85: out[k] = mean_t |x[t, k]| (fp32 accumulation, result in `dtype`). */
+int lcq_absmean_cols(const void* x, int dtype, int64_t T, int64_t K, void* out, void* workspace, void* stream);
+
+/* Awq.get_weight_scale (one layer), awq.py:58-66: out[k] = mean_r ( |W[r,k]| / max|W[r, group(k)]| ). */
+int lcq_awq_weight_scale(const void* w, int dtype, int64_t R, int64_t K, int group_size, void* out, void* workspace,
+                         void* stream);
+
+/* scaling_input, base_blockwise_quantization.py:899-912: out = x / s[None, :]. */
+int lcq_div_cols(const void* x, int dtype, int64_t T, int64_t K, const void* s, void* out, void* stream);
+
+/* Awq.calculate_loss, awq.py:134-145: out[0] = mean( float((a - b) in `dtype`)^2 ), kept on the device. */
+int lcq_sq_err_mean(const void* a, const void* b, int dtype, int64_t n, float* out, void* workspace, void* stream);
+
+/* AutoClipper.auto_clip_layer, auto_clip.py:83-191 (clip_version v1, weight-only, per_group with group_size 128):
+ * for every (output row, group) the shrink step i in [0, n_steps) of the group range
+ *   max_i = org_max * (1 - i / n_grid),  min_i = org_min * (1 - i / n_grid)   (min_i = -max_i if clip_sym)
+ * that minimises  mean_t ( sum_j x[t, g, j] * (fq(clamp(w, min_i, max_i)) - w)[r, g, j] )^2 ; the first minimum wins.
+ *  w [R, K] LCQ_BF16; x [T, K] LCQ_BF16 (the sampled tokens); K % 128 == 0; G = K / 128
+ *  best_max, best_min [R, G] bf16 out;  errs [R, G, n_steps] fp32 out or NULL (the means, before their rounding to bf16)
+ *  qmin / qmax / flags (LCQ_FLAG_SYM, LCQ_FLAG_NO_ROUND_ZP): the weight quantizer of fake_quant_weight_dynamic.
+ * bf16 MFMA with fp32 accumulation: the reference's two bf16-rounded dot products are evaluated as one product with
+ * the bf16-rounded weight difference. */
+int lcq_awq_clip_search(const void* w, const void* x, int64_t R, int64_t K, int64_t T, int n_grid, int n_steps,
+                        int clip_sym, float qmin, float qmax, int flags, void* best_max, void* best_min, float* errs,
+                        void* stream);
+
+/* AutoClipper.apply_clip v1, auto_clip.py:194-211: out[r, g*gs + j] = clamp(w[r, g*gs + j], lo[r, g], hi[r, g]);
+ * w, out [R, K] of `dtype` (LCQ_F32 | LCQ_BF16), lo / hi [R, K / group_size] of `dtype`; out may alias w. */
+int lcq_clamp_groups(const void* w, int dtype, int64_t R, int64_t K, int group_size, const void* lo, const void* hi,
+                     void* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

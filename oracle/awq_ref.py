@@ -69,3 +69,71 @@ def search_scale(weights: dict, x, forward, spec, n_grid=20, version='v2'):
         if l < best_err:
             best_err, best_scales = l, s
     return best_scales, losses
+
+
+# ----------------------------------------------------------------------------
+# AutoClipper (weight-only, clip_version v1)
+# ----------------------------------------------------------------------------
+def auto_clip_layer(spec, w, inputs, clip_sym=False, n_grid=20, max_shrink=0.5, n_sample_token=512):
+    """auto_clip.py:83-191 on CPU tensors, op for op (w_only, clip_version v1): for each batch of output rows the
+    [ocb, T, G, g] products of the sampled inputs with the original and with the clamped + fake-quantized weights,
+    their sums over g, the mean squared difference over tokens, and the running `err < min_errs` selection over
+    the shrink steps.  Returns (best_max [R, G, 1], best_min [R, G, 1], errs [R, G, n_steps] as computed)."""
+    assert w.dim() == 2
+    group_size = spec.group_size if spec.granularity == 'per_group' else w.shape[1]
+    w = w.reshape(w.shape[0], 1, -1, group_size)
+    oc_batch_size = 256 if w.shape[0] % 256 == 0 else 64
+    assert w.shape[0] % oc_batch_size == 0
+    w_all = w
+    best_max_val_all, best_min_val_all, errs_all = [], [], []
+    for i_b in range(w.shape[0] // oc_batch_size):
+        w = w_all[i_b * oc_batch_size:(i_b + 1) * oc_batch_size]
+        org_max_val = w.abs().amax(dim=-1, keepdim=True) if clip_sym else w.amax(dim=-1, keepdim=True)
+        org_min_val = w.amin(dim=-1, keepdim=True)
+        best_max_val = org_max_val.clone()
+        best_min_val = org_min_val.clone()
+        min_errs = torch.ones_like(org_max_val) * 1e9
+        org_out_dict = {}
+        errs_b = []
+        for i_s in range(int(max_shrink * n_grid)):
+            err_mean = 0
+            for i in range(len(inputs)):
+                x = inputs[i]
+                x = x.view(-1, x.shape[-1])
+                x = x.reshape(1, x.shape[0], -1, group_size)
+                nst = n_sample_token if n_sample_token is not None else min(x.shape[1], 512)
+                step_size = max(1, x.shape[1] // nst)
+                x = x[:, 0::step_size]
+                if i in org_out_dict:
+                    org_out = org_out_dict[i]
+                else:
+                    org_out = (x * w).sum(dim=-1)
+                    org_out_dict[i] = org_out
+                max_val = org_max_val * (1 - i_s / n_grid)
+                min_val = -max_val if clip_sym else org_min_val * (1 - i_s / n_grid)
+                cur_w = torch.clamp(w, min_val, max_val)
+                q_w = Q.int_fake_quant_dynamic(spec, cur_w)
+                cur_out = (x * q_w).sum(dim=-1)
+                err = (cur_out - org_out).pow(2).mean(dim=1).view(min_errs.shape)
+                err_mean += err
+            err_mean /= len(inputs)
+            errs_b.append(err_mean.clone())
+            cur_best_idx = err_mean < min_errs
+            min_errs[cur_best_idx] = err_mean[cur_best_idx]
+            best_max_val[cur_best_idx] = max_val[cur_best_idx]
+            best_min_val[cur_best_idx] = min_val[cur_best_idx]
+        best_max_val_all.append(best_max_val)
+        best_min_val_all.append(best_min_val)
+        errs_all.append(torch.cat(errs_b, dim=-1))          # [ocb, 1, G, n_steps]
+    best_max_val = torch.cat(best_max_val_all, dim=0)
+    best_min_val = torch.cat(best_min_val_all, dim=0)
+    return best_max_val.squeeze(1), best_min_val.squeeze(1), torch.cat(errs_all, dim=0).squeeze(1)
+
+
+def apply_clip_v1(w, min_val, max_val, clip_sym=False):
+    """auto_clip.py:194-211: clamp the weight group-wise to the found range."""
+    org_shape = w.shape
+    x = w.reshape(*max_val.shape[:2], -1)
+    if clip_sym:
+        min_val = -max_val
+    return torch.clamp(x, min_val, max_val).reshape(org_shape)

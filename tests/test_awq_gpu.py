@@ -93,3 +93,60 @@ def test_search_scale_subset_picks_the_oracle_ratio(dev, dtype):
         assert float((best.cpu().float() - best_o.float()).abs().max()) <= 2 ** -7 * float(best_o.float().abs().max())
     # weights are back to the originals
     assert torch.equal(layers['gate'].weight.data.cpu(), w['gate'])
+
+
+# ---- AutoClipper (auto_clip.py) ---------------------------------------------------------------------
+@pytest.mark.parametrize('clip_sym,sym', [(False, False), (True, False), (False, True)])
+@pytest.mark.parametrize('R,K,T', [(64, 256, 96), (320, 512, 512), (256, 128, 700)])
+def test_auto_clip_against_oracle(dev, clip_sym, sym, R, K, T):
+    """Errors of the ten shrink steps within the bf16 noise of the reference's chain (it rounds both dot products
+    to bf16 before subtracting; the kernel multiplies the weight difference on MFMA), the same step chosen wherever
+    the oracle's own errors separate the best two by more than 3 %, ranges identical there."""
+    from lightcompress_amd import IntegerQuantizer
+    from lightcompress_amd.auto_clip import AutoClipper
+    from tests.helpers import weight_like
+    spec = Q.IntSpec(4, sym, 'per_group', group_size=128)
+    w = weight_like(R, K, seed=R + K, dtype=torch.bfloat16)
+    x = (torch.randn(T, K, generator=gen(R + T)) * torch.exp(0.5 * torch.randn(K, generator=gen(K + T)))).bfloat16()
+    nst = 512
+    obmax, obmin, oerrs = A.auto_clip_layer(spec, w, [x.clone()], clip_sym=clip_sym, n_sample_token=nst)
+    wq = IntegerQuantizer(4, sym, 'per_group', group_size=128)
+    clipper = AutoClipper(True, wq, None, 'v1', clip_sym, False, None)
+    bmax, bmin = clipper.auto_clip_layer(0, 'fc', w.to(dev), [x.to(dev)], n_sample_token=nst)
+    assert bmax.shape == obmax.shape and bmin.shape == obmin.shape and bmax.dtype == torch.bfloat16
+    errs = clipper.last_errs.cpu()
+    rel = (errs.double() - oerrs.double()).abs() / oerrs.double().clamp(min=1e-30)
+    assert float(rel.median()) < 0.02 and float(rel.quantile(0.99)) < 0.25
+    top2 = oerrs.float().topk(2, dim=-1, largest=False).values
+    clear = (top2[..., 1] > 1.03 * top2[..., 0]).unsqueeze(-1)
+    assert float(clear.float().mean()) > 0.3
+    assert torch.equal(bmax.cpu()[clear], obmax[clear]) and torch.equal(bmin.cpu()[clear], obmin[clear])
+    assert float((bmax.cpu() == obmax).float().mean()) > 0.9
+    # every answer is one of the shrunken original ranges
+    wg = w.reshape(R, K // 128, 128)
+    org = (wg.abs().amax(-1) if clip_sym else wg.amax(-1)).unsqueeze(-1)
+    cands = torch.cat([org * (1 - s / 20) for s in range(10)], dim=-1)
+    assert bool((bmax.cpu() == cands).any(-1).all())
+    # apply_clip clamps the layer weight group-wise
+    layer = torch.nn.Linear(K, R, bias=False, dtype=torch.bfloat16, device=dev)
+    layer.weight.data.copy_(w)
+    clipper.apply_clip(0, layer, bmin, bmax, 'fc')
+    assert_bit_equal(layer.weight.data, A.apply_clip_v1(w, bmin.cpu(), bmax.cpu(), clip_sym), 'apply_clip')
+
+
+def test_auto_clip_run_skips_query_key_and_rejects_other_modes(dev):
+    from lightcompress_amd import IntegerQuantizer
+    from lightcompress_amd.auto_clip import AutoClipper
+    wq = IntegerQuantizer(4, False, 'per_group', group_size=128)
+    blk = torch.nn.ModuleDict({'q_proj': torch.nn.Linear(128, 64, bias=False), 'o_proj': torch.nn.Linear(128, 64, bias=False)})
+    blk = blk.to(device=dev, dtype=torch.bfloat16)
+    q0, o0 = blk['q_proj'].weight.data.clone(), blk['o_proj'].weight.data.clone()
+    x = torch.randn(4, 32, 128, generator=gen(5)).bfloat16().to(dev)
+    AutoClipper(True, wq, None, 'v1', False, False, None).run(blk, 0, {'q_proj': [x], 'o_proj': [x[:2], x[2:]]}, 512)
+    assert torch.equal(blk['q_proj'].weight.data, q0)                    # names with q_/k_ are not clipped
+    assert not torch.equal(blk['o_proj'].weight.data, o0)
+    assert float((blk['o_proj'].weight.data.abs() <= o0.abs()).float().mean()) == 1.0
+    with pytest.raises(NotImplementedError):
+        AutoClipper(True, wq, None, 'v2', False, False, None).auto_clip_layer(0, 'o', o0, [x])
+    with pytest.raises(NotImplementedError):
+        AutoClipper(False, wq, wq, 'v1', False, False, None).auto_clip_layer(0, 'o', o0, [x])

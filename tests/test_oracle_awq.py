@@ -1,9 +1,10 @@
 """Pins the AWQ oracle without a GPU: ratio 0 is plain RTN, the scale
 normalisation, and a brute-force fp64 grid search on a tiny SwiGLU MLP."""
+import pytest
 import torch
 
 from oracle import awq_ref as A, quant_ref as Q
-from tests.helpers import gen
+from tests.helpers import gen, weight_like
 
 
 def swiglu(x, w):
@@ -69,3 +70,78 @@ def test_grid_search_matches_bruteforce_fp64():
     assert torch.allclose(best, s / (s.max() * s.min()).sqrt())
     # activation-aware scaling beats plain RTN on outlier channels
     assert min(brute) < brute[0]
+
+
+# ---- AutoClipper (auto_clip.py:83-191) ------------------------------------------------------------
+def _clip_objective_fp64(spec, w, x, n_grid=20, n_steps=10, clip_sym=False):
+    """The objective in plain fp64 math, written from its definition: for every (row, group, shrink step) the
+    mean over tokens of (x_g . (fq(clamp(w_g)) - w_g))^2, with fq evaluated by the oracle quantizer on the clamped
+    bf16 group."""
+    R, K = w.shape
+    g = spec.group_size
+    G = K // g
+    wg = w.reshape(R, G, g)
+    xg = x.reshape(-1, G, g).double()
+    out = torch.zeros(R, G, n_steps, dtype=torch.float64)
+    for s in range(n_steps):
+        hi = (wg.abs().amax(-1, keepdim=True) if clip_sym else wg.amax(-1, keepdim=True)) * (1 - s / n_grid)
+        lo = -hi if clip_sym else wg.amin(-1, keepdim=True) * (1 - s / n_grid)
+        cw = torch.clamp(wg, lo, hi)
+        qw = Q.int_fake_quant_dynamic(spec, cw.reshape(R, K)).reshape(R, G, g)
+        d = (qw.double() - wg.double())                                  # [R, G, g]
+        e = torch.einsum('tgj,rgj->rtg', xg, d)                          # [R, T, G]
+        out[:, :, s] = e.pow(2).mean(dim=1)
+    return out
+
+
+@pytest.mark.parametrize('clip_sym', [False, True])
+def test_auto_clip_oracle_tracks_the_fp64_objective(clip_sym):
+    R, K, T = 64, 256, 96
+    spec = Q.IntSpec(4, False, 'per_group', group_size=128)
+    w = weight_like(R, K, seed=61, dtype=torch.bfloat16)
+    x = (torch.randn(T, K, generator=gen(62)) * torch.exp(torch.randn(K, generator=gen(63)))).bfloat16()
+    bmax, bmin, errs = A.auto_clip_layer(spec, w, [x.clone()], clip_sym=clip_sym, n_sample_token=T)
+    assert bmax.shape == bmin.shape == (R, 2, 1) and errs.shape == (R, 2, 10)
+    ref = _clip_objective_fp64(spec, w, x, clip_sym=clip_sym)
+    # the bf16 chain (products, sums, difference, square, mean all rounded to 8 bits) follows the exact objective
+    rel = (errs.double() - ref).abs() / ref.clamp(min=1e-30)
+    assert float(rel.median()) < 0.02 and float(rel.quantile(0.99)) < 0.25
+    # the selection is the first minimum of the rounded errors, and the ranges are the shrunken originals
+    pick = torch.zeros(R, 2, dtype=torch.long)
+    best = torch.full((R, 2), 1e9).bfloat16()
+    for s in range(10):
+        better = errs[:, :, s] < best
+        best[better] = errs[:, :, s][better]
+        pick[better] = s
+    wg = w.reshape(R, 2, 128)
+    org_max = wg.abs().amax(-1) if clip_sym else wg.amax(-1)
+    want_max = torch.stack([org_max * (1 - s / 20) for s in range(10)], dim=-1).gather(-1, pick.unsqueeze(-1))
+    assert torch.equal(bmax, want_max)
+    if clip_sym:
+        assert torch.equal(bmin, -bmax)
+    # agreement with the exact argmin wherever the exact objective separates the best two steps by > 5 %
+    top2 = ref.topk(2, dim=-1, largest=False).values
+    clear = top2[..., 1] > 1.05 * top2[..., 0]
+    assert float(clear.float().mean()) > 0.3
+    assert bool((pick[clear] == ref.argmin(-1)[clear]).all())
+
+
+def test_auto_clip_oracle_known_optima():
+    """An outlier weight whose input channel is silent costs nothing to clip: the search shrinks deep.  When that channel carries all the signal, clipping only hurts: step 0 (no clipping) wins."""
+    R, K, T = 64, 128, 64
+    spec = Q.IntSpec(4, False, 'per_group', group_size=128)
+    w = (torch.randn(R, K, generator=gen(71)) * 0.02)
+    w[:, 5] = 1.0                                      # outlier column, 50 sigma
+    w[:, 9] = -1.0
+    w = w.bfloat16()
+    x = torch.randn(T, K, generator=gen(72))
+    x_silent = x.clone(); x_silent[:, 5] = 0; x_silent[:, 9] = 0
+    bmax, bmin, errs = A.auto_clip_layer(spec, w, [x_silent.bfloat16()], n_sample_token=T)
+    assert float((bmax.flatten().float() / w.float().amax(1)).mean()) < 0.7          # deep steps on average
+    assert float(errs[:, 0, 9].float().mean()) < 0.9 * float(errs[:, 0, 0].float().mean())
+    x_loud = torch.zeros(T, K); x_loud[:, 5] = x[:, 5]; x_loud[:, 9] = x[:, 9]
+    bmax, bmin, errs = A.auto_clip_layer(spec, w, [x_loud.bfloat16()], n_sample_token=T)
+    assert bool((bmax.flatten() == w.amax(1)).all()) and bool((bmin.flatten() == w.amin(1)).all())
+    # apply_clip: the weight is clamped group-wise into the found range
+    cl = A.apply_clip_v1(w, bmin, bmax)
+    assert torch.equal(cl, w)
