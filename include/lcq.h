@@ -206,6 +206,13 @@ int lcq_awq_weight_scale(const void* w, int dtype, int64_t R, int64_t K, int gro
 /* scaling_input, base_blockwise_quantization.py:899-912: out = x / s[None, :]. */
 int lcq_div_cols(const void* x, int dtype, int64_t T, int64_t K, const void* s, void* out, void* stream);
 
+/* Folding searched scales into neighbouring weights, base_blockwise_quantization.py:664-723, 772-801
+ * (scale_fc_fc, scale_ln_fcs: `fc.weight.mul_(scales.view(1, -1))`, `fc1.weight.div_(scales.view(-1, 1))`,
+ * `ln.weight.div_(scales)`):  out = x (* or /) s  with s a column vector [K] (mode 0 multiply, 1 divide) or a row
+ * vector [T] (mode 2 multiply, 3 divide) of `dtype`; x, out [T, K] of `dtype` (LCQ_F32 | LCQ_BF16), out may be x.
+ * One IEEE operation per element, rounded to `dtype`. */
+int lcq_scale_matrix(const void* x, int dtype, int64_t T, int64_t K, const void* s, int mode, void* out, void* stream);
+
 /* Awq.calculate_loss, awq.py:134-145: out[0] = mean( float((a - b) in `dtype`)^2 ), kept on the device. */
 int lcq_sq_err_mean(const void* a, const void* b, int dtype, int64_t n, float* out, void* workspace, void* stream);
 

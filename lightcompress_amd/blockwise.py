@@ -1,0 +1,117 @@
+"""Scale folding of the block-wise algorithms with the reference's method names, running on liblcq.
+
+Mirrors the members of ``BaseBlockwiseQuantization`` (llmc/compression/quantization/
+base_blockwise_quantization.py of ModelTC/LightCompress) that AWQ-style methods call after a scale search:
+``apply_scale`` (:619-636), ``scale_fc_fc`` (:664-723), ``scale_ln_fcs`` (:772-801), ``repeat_gqa_scales``
+(:613-617), ``scaling_input`` (:899-912) and ``update_input_feat`` (:914-920).  Use it as a mix-in in front of
+the reference's class, or stand-alone.
+
+Not on this path (``NotImplementedError``): fused QKV linears (``fc1.out_features == 3 * fc2.in_features``) and
+float8 block-wise checkpoints (``weight_scale_inv``).
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib as L
+
+_MUL_COLS, _DIV_COLS, _MUL_ROWS, _DIV_ROWS = 0, 1, 2, 3
+
+
+def _scale_(t, s, mode):
+    """In place: t (* or /) s along columns (mode 0 / 1) or rows (2 / 3); t [T, K] or [K]."""
+    if t.dtype == torch.float8_e4m3fn:
+        raise NotImplementedError('float8 block-wise weights are not on this path')
+    x = t.data
+    if not x.is_contiguous():
+        raise L.LcqError('in-place scaling needs a contiguous tensor')
+    x2 = x.view(1, -1) if x.dim() == 1 else x.view(-1, x.shape[-1])
+    s = s.to(device=x.device, dtype=x.dtype).contiguous().view(-1)
+    assert s.numel() == (x2.shape[1] if mode < 2 else x2.shape[0])
+    L.check(L.lib().lcq_scale_matrix(L.ptr(x2), L.i32(L.dtype_code(x.dtype)), L.i64(x2.shape[0]), L.i64(x2.shape[1]),
+                                     L.ptr(s), L.i32(mode), L.ptr(x2), L.stream()), 'lcq_scale_matrix')
+    return t
+
+
+class ScaleFolding:
+    """Expects, where GQA is used, ``num_key_value_heads``, ``head_dim``, ``num_key_value_groups``, ``has_gqa`` and
+    ``do_gqa_trans`` on ``self`` like the reference's class."""
+
+    has_gqa = False
+    do_gqa_trans = False
+
+    @torch.no_grad()
+    def repeat_gqa_scales(self, scales):
+        scales = scales.view(1, self.num_key_value_heads, self.head_dim)
+        return torch.repeat_interleave(scales, dim=1, repeats=self.num_key_value_groups)
+
+    @torch.no_grad()
+    def apply_scale(self, scales, prev_op, layers):
+        assert len(prev_op) == 1, 'Only support single prev_op. If multi prev_ops, code need to be updated.'
+        if isinstance(prev_op[0], torch.nn.Linear):
+            assert len(layers) == 1
+            self.scale_fc_fc(prev_op[0], layers[0], scales)
+        elif hasattr(prev_op[0], 'weight') and prev_op[0].weight.dim() == 1:          # LayerNorm / RMSNorm
+            self.scale_ln_fcs(prev_op[0], layers, scales)
+        else:
+            raise NotImplementedError(f'prev_op {type(prev_op[0])} not supported yet!')
+
+    @torch.no_grad()
+    def scale_fc_fc(self, fc1, fc2, scales):
+        scales = scales.to(fc1.weight.device)
+        has_bias = getattr(fc1, 'bias', None) is not None
+        if fc1.out_features == fc2.in_features * 3:
+            raise NotImplementedError('fused QKV linears are not on this path')
+        elif fc1.out_features == fc2.in_features * 2:
+            half = fc1.weight.data.shape[0] // 2
+            _scale_(fc1.weight.data[half:], scales, _DIV_ROWS)
+            if has_bias:
+                _scale_(fc1.bias.data[half:], scales, _DIV_COLS)
+        elif fc1.out_features == fc2.in_features:
+            if has_bias:
+                _scale_(fc1.bias, scales, _DIV_COLS)
+            _scale_(fc1.weight, scales, _DIV_ROWS)
+        elif self.has_gqa and self.do_gqa_trans:
+            if has_bias:
+                _scale_(fc1.bias, scales, _DIV_COLS)
+            _scale_(fc1.weight, scales, _DIV_ROWS)
+            if fc1.out_features != fc2.in_features:
+                scales = self.repeat_gqa_scales(scales)
+        else:
+            raise Exception('Can not scale this fc-fc.')
+        _scale_(fc2.weight, scales, _MUL_COLS)
+
+    @torch.no_grad()
+    def scale_ln_fcs(self, ln, fcs, scales):
+        if not isinstance(fcs, list):
+            fcs = [fcs]
+        scales = scales.to(ln.weight.device).to(ln.weight.dtype)
+        _scale_(ln.weight, scales, _DIV_COLS)
+        if getattr(ln, 'bias', None) is not None:
+            _scale_(ln.bias, scales, _DIV_COLS)
+        for fc in fcs:
+            _scale_(fc.weight, scales, _MUL_COLS)
+        for p in ln.parameters():
+            assert torch.isnan(p).sum() == 0
+        for fc in fcs:
+            for p in fc.parameters():
+                assert torch.isnan(p).sum() == 0
+
+    @torch.no_grad()
+    def scaling_input(self, x, scales, is_gqa):
+        scales_tmp = self.repeat_gqa_scales(scales) if is_gqa else scales
+        x2 = x.contiguous()
+        out = torch.empty_like(x2)
+        K = x2.shape[-1]
+        s = scales_tmp.to(device=x2.device, dtype=x2.dtype).contiguous().view(-1)
+        L.check(L.lib().lcq_scale_matrix(L.ptr(x2), L.i32(L.dtype_code(x2.dtype)), L.i64(x2.numel() // K), L.i64(K),
+                                         L.ptr(s), L.i32(_DIV_COLS), L.ptr(out), L.stream()), 'lcq_scale_matrix')
+        return out
+
+    @torch.no_grad()
+    def update_input_feat(self, scale, input_feat, layers_dict, is_gqa):
+        for layer_name in layers_dict:
+            for i in range(len(input_feat[layer_name])):
+                inp = input_feat[layer_name][i]
+                scale = scale.to(inp.device)
+                input_feat[layer_name][i] = self.scaling_input(inp, scale, is_gqa)

@@ -64,6 +64,33 @@ __global__ __launch_bounds__(256) void div_cols_kernel(const u32x4* __restrict__
   }
 }
 
+// ---- in-place capable w (*|/) s[col]  or  w (*|/) s[row] -------------------------------------
+// mode: 0 multiply by a column vector, 1 divide by a column vector, 2 multiply by a row vector, 3 divide by one
+template <bool BF>
+__global__ __launch_bounds__(256) void scale_kernel(const u32x4* x, const void* __restrict__ s, int64_t nchunks_total,
+                                                    int64_t nch_row, int mode, u32x4* out) {
+  constexpr int N = Vec<BF>::N;
+  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < nchunks_total; c += (int64_t)gridDim.x * 256) {
+    float v[N], sv[N];
+    unpack<BF>(x[c], v);
+    if (mode < 2) {
+      unpack<BF>(((const u32x4*)s)[c % nch_row], sv);
+    } else {
+      const float r = load_scalar<BF>(s, c / nch_row);
+      #pragma unroll
+      for (int i = 0; i < N; ++i) sv[i] = r;
+    }
+    if (mode & 1) {
+      #pragma unroll
+      for (int i = 0; i < N; ++i) v[i] = v[i] / sv[i];
+    } else {
+      #pragma unroll
+      for (int i = 0; i < N; ++i) v[i] = v[i] * sv[i];
+    }
+    out[c] = pack_rne<BF>(v);
+  }
+}
+
 // ---- mean of squared differences ------------------------------------------------------------
 template <bool BF>
 __global__ __launch_bounds__(256) void sqerr_stage1(const u32x4* __restrict__ a, const u32x4* __restrict__ b,
@@ -204,6 +231,21 @@ int lcq_div_cols(const void* x, int dtype, int64_t T, int64_t K, const void* s, 
   hipStream_t st = (hipStream_t)stream;
   if (dtype == LCQ_BF16) div_cols_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)x, (const u32x4*)s, total, nch_row, (u32x4*)out);
   else div_cols_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)x, (const u32x4*)s, total, nch_row, (u32x4*)out);
+  LCQ_CHECK_LAUNCH();
+  return LCQ_OK;
+}
+
+int lcq_scale_matrix(const void* x, int dtype, int64_t T, int64_t K, const void* s, int mode, void* out, void* stream) {
+  if (!x || !s || !out || T <= 0 || K <= 0 || mode < 0 || mode > 3) return LCQ_EINVAL;
+  const int n = dtype == LCQ_BF16 ? 8 : 4;
+  if (dtype != LCQ_BF16 && dtype != LCQ_F32) return LCQ_EDTYPE;
+  if (K % n != 0 || (((uintptr_t)x | (uintptr_t)out) % 16) != 0 || (mode < 2 && ((uintptr_t)s % 16) != 0)) return LCQ_EALIGN;
+  const int64_t nch_row = K / n, total = T * nch_row;
+  int64_t grid = (total + 255) / 256;
+  if (grid > 65536 * 4) grid = 65536 * 4;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == LCQ_BF16) scale_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)x, s, total, nch_row, mode, (u32x4*)out);
+  else scale_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)x, s, total, nch_row, mode, (u32x4*)out);
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;
 }

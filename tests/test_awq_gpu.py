@@ -150,3 +150,52 @@ def test_auto_clip_run_skips_query_key_and_rejects_other_modes(dev):
         AutoClipper(True, wq, None, 'v2', False, False, None).auto_clip_layer(0, 'o', o0, [x])
     with pytest.raises(NotImplementedError):
         AutoClipper(False, wq, wq, 'v1', False, False, None).auto_clip_layer(0, 'o', o0, [x])
+
+
+# ---- apply_scale / scale_fc_fc / scale_ln_fcs / update_input_feat ---------------------------------------
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+def test_scale_folding_matches_the_torch_op_sequence(dev, dtype):
+    """base_blockwise_quantization.py:619-723, 772-801, 899-920: each is a literal in-place torch op in the
+    reference (one IEEE multiply / divide per element in the tensor's type), so the CPU op is the oracle: bit-exact."""
+    from lightcompress_amd.blockwise import ScaleFolding
+    sf = ScaleFolding()
+    K, I = 256, 384
+    s = (torch.rand(K, generator=gen(1)) + 0.5).to(dtype)
+    def lin(i, o, bias, seed):
+        m = torch.nn.Linear(i, o, bias=bias, dtype=torch.float32)
+        m.weight.data = (torch.randn(o, i, generator=gen(seed)) * 0.05)
+        if bias:
+            m.bias.data = torch.randn(o, generator=gen(seed + 1)) * 0.05
+        return m.to(dtype)
+    # ln -> fcs
+    ln = torch.nn.LayerNorm(K, dtype=dtype)
+    ln.weight.data = (torch.rand(K, generator=gen(2)) + 0.5).to(dtype); ln.bias.data = torch.randn(K, generator=gen(3)).to(dtype)
+    fcs = [lin(K, I, False, 10), lin(K, I, True, 20)]
+    want_lnw, want_lnb = ln.weight.data / s, ln.bias.data / s
+    want_fc = [fc.weight.data * s.view(1, -1) for fc in fcs]
+    ln_d = ln.to(dev); fcs_d = [fc.to(dev) for fc in fcs]
+    sf.apply_scale(s.to(dev), [ln_d], fcs_d)
+    assert_bit_equal(ln_d.weight.data, want_lnw, 'ln weight'); assert_bit_equal(ln_d.bias.data, want_lnb, 'ln bias')
+    for fc, wnt in zip(fcs_d, want_fc):
+        assert_bit_equal(fc.weight.data, wnt, 'fc weight')
+    # fc -> fc, equal widths (with bias) and the gated case (fc1 twice as wide)
+    s2 = (torch.rand(I, generator=gen(4)) + 0.5).to(dtype)
+    for mult in (1, 2):
+        fc1, fc2 = lin(K, I * mult, True, 30 + mult), lin(I, K, False, 40 + mult)
+        w1, b1, w2 = fc1.weight.data.clone(), fc1.bias.data.clone(), fc2.weight.data.clone()
+        if mult == 1:
+            w1 = w1 / s2.view(-1, 1); b1 = b1 / s2
+        else:
+            w1[I:] = w1[I:] / s2.view(-1, 1); b1[I:] = b1[I:] / s2
+        w2 = w2 * s2.view(1, -1)
+        f1, f2 = fc1.to(dev), fc2.to(dev)
+        sf.apply_scale(s2.to(dev), [f1], [f2])
+        assert_bit_equal(f1.weight.data, w1, 'fc1 weight'); assert_bit_equal(f1.bias.data, b1, 'fc1 bias')
+        assert_bit_equal(f2.weight.data, w2, 'fc2 weight')
+    # cached inputs
+    x = torch.randn(3, 40, K, generator=gen(5)).to(dtype)
+    feat = {'a': [x[:2].to(dev), x[2:].to(dev)]}
+    sf.update_input_feat(s.to(dev), feat, {'a': None}, False)
+    assert_bit_equal(torch.cat(feat['a']), x / s.view(1, -1), 'scaled inputs')
+    with pytest.raises(NotImplementedError):
+        sf.scale_fc_fc(lin(K, 3 * I, False, 50).to(dev), lin(I, K, False, 51).to(dev), s2.to(dev))
