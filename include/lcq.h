@@ -57,6 +57,8 @@ extern "C" {
                                      arithmetic unrounded (a 0-dim fp32 qparam next to a bf16 tensor); results
                                      still round to the row type */
 
+#define LCQ_FLAG_CLAMP_RANGE 1024  /* lcq_fp8_block_quant: s = clamp(max|x|, 1e-5) / 448 (the FloatQuantizer path) instead of max|x| / 448 */
+#define LCQ_FLAG_TIE_AWAY 2048     /* lcq_fp8_block_quant: exact ties round away from zero instead of to even */
 #define LCQ_FLAG_ROW_QP 512       /* lcq_quant_fp_emu, STATIC only: `scales` holds one value per row */
 
 /* errors */
@@ -127,6 +129,18 @@ int lcq_dequant_fp(const float* q, int64_t rows, int64_t cols, const void* scale
 int lcq_quant_fp_emu(const void* x, int dtype, int64_t rows, int64_t cols, int e_bits, int m_bits, int flags,
                      const void* min_in, const void* max_in, const void* scales_in, void* xc, void* scales_out,
                      void* q, int code_dtype, void* dq, void* stream);
+
+/* Block-wise float8 casts: weight_cast_to_fp8 / act_quant, kernel.py:7-85 (Triton) and their fallback through
+ * FloatQuantizer(granularity='per_block'), quant.py:33-45:  per block  s = max|x| / 448 (fp32),
+ * y = float8_e4m3fn(x / s) computed in fp32.  block_rows = 128: blocks of 128 x 128 of x [M, N], scales [ceil(M/128),
+ * ceil(N/128)]; block_rows = 1: blocks of 1 x 128 (activations; N % 128 == 0), scales [M, N/128].
+ * x of `dtype` (LCQ_F32 | LCQ_BF16), y float8 bytes [M, N]. */
+int lcq_fp8_block_quant(const void* x, int dtype, int64_t M, int64_t N, int block_rows, int flags, void* y, float* scales,
+                        void* stream);
+
+/* weight_cast_to_bf16, kernel.py:88-138 / quant.py:20-31: out[i, j] = float(y[i, j]) * scales[i / 128, j / 128];
+ * out of `out_dtype` (LCQ_BF16 | LCQ_F32). */
+int lcq_fp8_block_dequant(const void* y, const float* scales, int64_t M, int64_t N, void* out, int out_dtype, void* stream);
 
 /* ---- packing ------------------------------------------------------------ */
 

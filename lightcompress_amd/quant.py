@@ -11,8 +11,8 @@ ABI in ``include/lcq.h``.  There is no CPU path: CPU tensors raise
 
 Not carried over (they raise ``NotImplementedError``): the ``mse`` /
 ``learnable`` / ``hqq`` / ``static_hist`` calibrators, STE rounding (training
-only), the ``rounding`` override of ``fake_quant_weight_static`` and ``per_block``
-granularity.
+only) and the ``rounding`` override of ``fake_quant_weight_static``.  ``per_block`` granularity runs for
+``FloatQuantizer('e4m3')`` weights only (``real_quant_weight_dynamic`` / ``fake_quant_weight_dynamic``).
 """
 from __future__ import annotations
 
@@ -40,7 +40,8 @@ class BaseQuantizer(object):
         elif self.granularity == 'per_head':
             self.head_num = self.kwargs['head_num']
         elif self.granularity == 'per_block':
-            raise NotImplementedError('per_block (FP8 block-wise checkpoints) is not part of this path')
+            assert self.calib_algo == 'minmax' and self.sym
+            self.block_size = self.kwargs['block_size']
 
         if self.kwargs.get('ste', False) or self.kwargs.get('ste_all', False):
             raise NotImplementedError('straight-through rounding is a training feature; not on this path')
@@ -627,6 +628,10 @@ class FloatQuantizer(BaseQuantizer):
         return dq.view(tensor.shape)
 
     def _fake(self, t, static_scales=None):
+        if self.granularity == 'per_block':
+            if static_scales is not None:
+                raise NotImplementedError('static per_block scales')
+            return self._per_block(t, True)
         shape, dtype = t.shape, t.dtype
         rows_t = self.reshape_tensor(t)
         if not self.use_qtorch:
@@ -656,8 +661,26 @@ class FloatQuantizer(BaseQuantizer):
         q = self._fake(weight.T if ic else weight)
         return q.T if ic else q
 
+    def _per_block(self, weight, want_dq):
+        """per_block granularity (quant.py:138-140, 634-638): 128 x 128 blocks, fp32 ranges and scales."""
+        from .kernel import FLAG_CLAMP_RANGE, FLAG_TIE_AWAY, _block_quant, _block_dequant
+        if self.bit != 'e4m3' or self.block_size != 128 or not self.use_qtorch or not self.fp_subnormals:
+            raise NotImplementedError('per_block runs for e4m3, block_size 128, use_qtorch=True')
+        if weight.dim() != 2:
+            raise NotImplementedError('per_block expects a 2-D weight')
+        flags = FLAG_CLAMP_RANGE | (0 if self.fp_tie == 'even' else FLAG_TIE_AWAY)
+        y, s = _block_quant(weight.contiguous(), 128, flags)
+        if want_dq:
+            return _block_dequant(y, s, torch.float32).to(weight.dtype)
+        return y, s
+
     def _real(self, weight, static_scales, output_scale_factor):
         assert self.bit in ['e4m3', 'e5m2'], 'Only FP8 E4M3 and E5M2 support real quant'
+        if self.granularity == 'per_block':
+            if static_scales is not None:
+                raise NotImplementedError('static per_block scales')
+            y, s = self._per_block(weight, False)
+            return y, s * output_scale_factor, None
         dtype = torch.float8_e4m3fn if self.e_bits == 4 else torch.float8_e5m2
         org_w_shape = weight.shape
         rows_t = self.reshape_tensor(weight)
@@ -697,3 +720,21 @@ class FloatQuantizer(BaseQuantizer):
             f'granularity={self.granularity},'
             f'kwargs={self.kwargs}, qmin={self.qmin}, qmax={self.qmax})'
         )
+
+
+# -- quant.py:20-45 of the reference: the block-wise float8 casts it uses where its Triton kernels do not run ----
+def weight_cast_to_bf16(weight, scale, block_size):
+    """float8 block-wise weight -> bf16: FloatQuantizer('e4m3', per_block).dequant(weight.float(), scale, 0)."""
+    from .kernel import _block_dequant
+    if block_size != 128:
+        raise NotImplementedError('block_size 128 only')
+    return _block_dequant(weight.contiguous(), scale, torch.bfloat16)
+
+
+def weight_cast_to_fp8(weight, block_size):
+    """bf16 / fp32 weight -> (float8_e4m3fn, fp32 scales [nbm, nbn]): real_quant_weight_dynamic of
+    FloatQuantizer('e4m3', per_block, use_qtorch=True): s = clamp(max|x|, 1e-5) / 448, float_quantize's
+    ties-away rounding (parameter ``fp_tie`` of FloatQuantizer; this function keeps the default)."""
+    q = FloatQuantizer('e4m3', True, 'per_block', block_size=block_size, use_qtorch=True)
+    fp8_weight, fp8_scale, _ = q.real_quant_weight_dynamic(weight)
+    return fp8_weight, fp8_scale

@@ -382,3 +382,54 @@ def float_emu_real_quant_dynamic(spec, w, output_scale_factor=1):
     s = s * output_scale_factor
     q = q.to(dt)
     return q, s.view(q.shape[0], -1), None
+
+
+# ----------------------------------------------------------------------------
+# block-wise float8 (e4m3) casts
+# ----------------------------------------------------------------------------
+def triton_weight_cast_to_fp8(x: torch.Tensor, block_size: int = 128):
+    """kernel.py:57-85 (weight_cast_to_fp8_kernel) as torch ops: per block s = max|x| / 448 in fp32,
+    y = (x.float() / s).to(float8_e4m3fn) - the cast rounds to nearest even like Triton's."""
+    M, N = x.shape
+    mb, nb = -(-M // block_size), -(-N // block_size)
+    y = torch.empty(M, N, dtype=torch.float8_e4m3fn)
+    s = torch.empty(mb, nb, dtype=torch.float32)
+    for i in range(mb):
+        for j in range(nb):
+            blk = x[i * block_size:(i + 1) * block_size, j * block_size:(j + 1) * block_size].float()
+            sc = blk.abs().max() / 448.0
+            s[i, j] = sc
+            y[i * block_size:(i + 1) * block_size, j * block_size:(j + 1) * block_size] = (blk / sc).to(torch.float8_e4m3fn)
+    return y, s
+
+
+def triton_act_quant(x: torch.Tensor, block_size: int = 128):
+    """kernel.py:7-54: one scale per block_size elements of the last dimension."""
+    xb = x.float().reshape(-1, block_size)
+    s = xb.abs().amax(dim=-1) / 448.0
+    y = (xb / s.unsqueeze(-1)).to(torch.float8_e4m3fn).reshape(x.shape)
+    return y, s.reshape(*x.shape[:-1], x.shape[-1] // block_size)
+
+
+def triton_weight_cast_to_bf16(y: torch.Tensor, s: torch.Tensor, block_size: int = 128, dtype=torch.bfloat16):
+    """kernel.py:88-138: float(y) * s per block, stored in `dtype`."""
+    M, N = y.shape
+    se = s.repeat_interleave(block_size, 0)[:M].repeat_interleave(block_size, 1)[:, :N]
+    return (y.float() * se).to(dtype)
+
+
+def float_per_block_real_quant(spec, w: torch.Tensor, block_size: int = 128):
+    """weight_cast_to_fp8 of quant.py:33-45: FloatQuantizer('e4m3', per_block).real_quant_weight_dynamic, i.e.
+    reshape_tensor (zero-padded [mb, bs, nb, bs], :634-638), abs().float() block ranges (:138-140), symmetric
+    qparams (:548-552), float_quantize on x / s in fp32 (:1060-1068), cast to float8, restore (:647-651)."""
+    m, n = w.shape
+    mb, nb = -(-m // block_size), -(-n // block_size)
+    t_padded = torch.zeros((mb * block_size, nb * block_size), dtype=w.dtype)
+    t_padded[:m, :n] = w
+    t = t_padded.view(-1, block_size, t_padded.size(1) // block_size, block_size)
+    min_val = t.abs().float().amin(dim=(1, 3), keepdim=True)
+    max_val = t.abs().float().amax(dim=(1, 3), keepdim=True)
+    scales, zeros, _, _ = float_qparams(spec, min_val, max_val)
+    q = float_quant(spec, t, scales, zeros)
+    q = q.reshape(-1, n if nb * block_size == n else nb * block_size)[:m, :n]
+    return q.to(torch.float8_e4m3fn), scales.view(scales.shape[0], scales.shape[2]), None

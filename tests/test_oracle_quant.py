@@ -353,3 +353,28 @@ def test_gemm_pack_order_bruteforce():
     # with fp16 scales the re-derived integers equal the quantizer's codes almost everywhere
     assert (iw.t() == codes).float().mean() > 0.99
     assert torch.equal(pack_ref.gemm_unpack(qzeros).t().contiguous(), z)
+
+
+def test_blockwise_fp8_oracles_scale_and_grid():
+    """Block-wise casts: the scale is max|x| / 448 of the block, the block maximum maps to +-448, every code is the
+    nearest e4m3 value of x / s (checked against the exact-rational grid search used above), zero padding of edge
+    blocks does not leak into the ranges, and dequantization is y * s."""
+    w = weight_like(200, 300, seed=81, dtype=torch.bfloat16)
+    y, s = Q.triton_weight_cast_to_fp8(w)
+    assert y.shape == (200, 300) and s.shape == (2, 3) and s.dtype == torch.float32
+    blk = w[128:, 256:].float()
+    assert float(s[1, 2]) == float(blk.abs().max() / 448.0)
+    assert float(y[128:, 256:].float().abs().max()) == 448.0
+    t = (w[:128, :128].float() / s[0, 0])
+    assert torch.equal(y[:128, :128].float(), Q.float_quantize_nearest(t, 4, 3, tie='even'))
+    back = Q.triton_weight_cast_to_bf16(y, s)
+    assert float(((back.float() - w.float()).abs() / w.float().abs().clamp(min=1e-3 * float(w.abs().max()))).max()) < 2 ** -3
+    ya, sa = Q.triton_act_quant(w[:, :256].contiguous())
+    assert sa.shape == (200, 2) and float(sa[7, 1]) == float(w[7, 128:256].float().abs().max() / 448.0)
+    # the quantizer route: same blocks, clamp(.., 1e-5), float_quantize's tie rule
+    spec = Q.FloatSpec('e4m3', 'per_block', tie='even')
+    yq, sq, z = Q.float_per_block_real_quant(spec, w)
+    assert z is None and torch.equal(sq, s) and torch.equal(yq.view(torch.uint8), y.view(torch.uint8))
+    zero = torch.zeros(128, 128, dtype=torch.bfloat16)
+    _, sz, _ = Q.float_per_block_real_quant(spec, zero)
+    assert float(sz) == float(torch.tensor(1e-5) / 448.0)

@@ -306,3 +306,42 @@ def test_full_size_rtn_properties(dev):
     spec = Q.IntSpec(4, False, 'per_group', group_size=128)
     oc, os_, oz = Q.int_real_quant_dynamic(spec, w[1000:1256])
     assert_bit_equal(codes[1000:1256], oc, 'slice codes'); assert_bit_equal(s[1000:1256], os_, 'slice scales')
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('shape', [(256, 384), (200, 296), (2048, 7168), (129, 8)])
+def test_blockwise_fp8_casts_bit_exact(dev, dtype, shape):
+    """kernel.py (Triton semantics) and the FloatQuantizer per_block route, against their oracles: codes, scales and
+    the dequantized weight bit for bit."""
+    from lightcompress_amd import kernel as K8, FloatQuantizer
+    from lightcompress_amd.quant import weight_cast_to_bf16 as q_to_bf16, weight_cast_to_fp8 as q_to_fp8
+    w = weight_like(*shape, seed=shape[1] + 3, dtype=dtype, std=0.006, outlier_frac=0.0005, outlier_mul=30)
+    w[0, :4] = torch.tensor([0.0, -0.0, 1e-9, -1e-9], dtype=dtype)
+    wd = w.to(dev)
+    y, s = K8.weight_cast_to_fp8(wd)
+    oy, os_ = Q.triton_weight_cast_to_fp8(w)
+    assert y.dtype == torch.float8_e4m3fn and s.dtype == torch.float32 and s.shape == os_.shape
+    assert_bit_equal(s, os_, 'block scales')
+    assert_bit_equal(y.view(torch.uint8), oy.view(torch.uint8), 'fp8 codes')
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        back = K8.weight_cast_to_bf16(y, s)
+    finally:
+        torch.set_default_dtype(torch.float32)
+    assert_bit_equal(back, Q.triton_weight_cast_to_bf16(oy, os_), 'block dequant')
+    assert_bit_equal(q_to_bf16(y, s, 128), Q.triton_weight_cast_to_bf16(oy, os_), 'quant.py weight_cast_to_bf16')
+    for tie in ('away', 'even'):
+        fq = FloatQuantizer('e4m3', True, 'per_block', block_size=128, use_qtorch=True, fp_tie=tie)
+        yq, sq, zq = fq.real_quant_weight_dynamic(wd)
+        oyq, osq, _ = Q.float_per_block_real_quant(Q.FloatSpec('e4m3', 'per_block', tie=tie), w)
+        assert zq is None
+        assert_bit_equal(sq, osq, 'per_block scales')
+        assert_bit_equal(yq.view(torch.uint8), oyq.view(torch.uint8), f'per_block codes tie={tie}')
+    y2, s2 = q_to_fp8(wd, 128)
+    oy2, os2, _ = Q.float_per_block_real_quant(Q.FloatSpec('e4m3', 'per_block'), w)
+    assert_bit_equal(y2.view(torch.uint8), oy2.view(torch.uint8), 'quant.py weight_cast_to_fp8')
+    if shape[1] % 128 == 0:
+        ya, sa = K8.act_quant(wd)
+        oya, osa = Q.triton_act_quant(w)
+        assert_bit_equal(sa, osa, 'act scales')
+        assert_bit_equal(ya.view(torch.uint8), oya.view(torch.uint8), 'act codes')
