@@ -1,10 +1,11 @@
-"""Packing of real-quantized weights with the reference's classmethod API.
+"""Real-quantized Linear containers and their packing, with the reference's class API.
 
-Mirrors ``VllmRealQuantLinear.pack`` (module_utils.py:929-955) and
-``AutoawqRealQuantLinear.gemm_pack`` (module_utils.py:1097-1158) of
-ModelTC/LightCompress.  The reference packs on the host (numpy round trip /
-Python loops over columns); here both layouts are one kernel over device
-memory.  The nn.Module containers around them are not part of this path.
+Mirrors ``VllmRealQuantLinear`` (module_utils.py:855-955: buffers ``weight`` / ``weight_packed``,
+``weight_scale`` / ``weight_scale_inv``, ``input_scale``, ``bias``; ``new``, ``quant_pack``, ``pack``) and
+``AutoawqRealQuantLinear`` (module_utils.py:1029-1158: buffers ``qweight``, ``scales``, ``qzeros``, ``bias``;
+``new``, ``quant_pack``, ``gemm_pack``) of ModelTC/LightCompress, so that what they hold loads in vLLM / SGLang
+(compressed-tensors) and AutoAWQ.  The reference packs on the host (numpy round trip / Python loops over
+columns); here both layouts are one kernel over device memory.
 """
 from __future__ import annotations
 
@@ -17,7 +18,68 @@ from . import _lib as L
 _CODE = {torch.int32: L.CODE_I32, torch.int8: L.CODE_I8, torch.uint8: L.CODE_U8}
 
 
-class VllmRealQuantLinear:
+def _bf16_weight(module):
+    """module_utils.py:916-921 / 1085-1090: a block-wise float8 checkpoint weight is brought back to bf16 first."""
+    if module.weight.data.dtype == torch.float8_e4m3fn:
+        from .quant import weight_cast_to_bf16
+        module.weight.data = weight_cast_to_bf16(module.weight.data, module.weight_scale_inv.data,
+                                                 module.block_size).to(torch.bfloat16)
+
+
+class _RealQuantLinear(torch.nn.Module):
+    @torch.no_grad()
+    def forward(self, x):
+        raise NotImplementedError
+
+    def _describe(self, module, weight, scales, zeros):
+        self.in_features = module.in_features
+        self.out_features = module.out_features
+        self.weight_shape, self.weight_dtype = weight.shape, weight.dtype
+        self.scales_shape, self.scales_dtype = scales.shape, scales.dtype
+        self.zeros_shape = zeros.shape if zeros is not None else None
+        self.zeros_dtype = zeros.dtype if zeros is not None else None
+
+    def _reg(self, name, value):
+        if value is not None:
+            self.register_buffer(name, value)
+        else:
+            setattr(self, name, None)
+
+
+class VllmRealQuantLinear(_RealQuantLinear):
+    def __init__(self, weight, bias, scales, input_scale, need_pack, scales_name):
+        super().__init__()
+        self.register_buffer('weight_packed' if need_pack else 'weight', weight)
+        self._reg('bias', bias)
+        self.register_buffer(scales_name, scales)
+        self.register_buffer('input_scale', input_scale)
+
+    @classmethod
+    @torch.no_grad()
+    def new(cls, module, w_q, quant_config):
+        """module_utils.py:875-911."""
+        weight, scales = cls.quant_pack(module, w_q, quant_config)
+        input_scale = module.buf_act_scales_0 if hasattr(module, 'buf_act_scales_0') else None
+        act = quant_config['act'] if 'act' in quant_config else None
+        if act is not None and act.get('static', False) and quant_config.get('quant_type', 'int-quant') == 'int-quant':
+            input_scale = input_scale.unsqueeze(0)
+        bias = module.bias.data if module.bias is not None else None
+        need_pack = quant_config['weight'].get('need_pack', False)
+        scales_name = 'weight_scale_inv' if quant_config['weight']['granularity'] == 'per_block' else 'weight_scale'
+        new_module = cls(weight, bias, scales, input_scale, need_pack, scales_name)
+        new_module._describe(module, weight, scales, None)
+        return new_module
+
+    @classmethod
+    @torch.no_grad()
+    def quant_pack(cls, module, w_q, quant_config):
+        """module_utils.py:913-927: w_q(module) -> (codes, scales, zeros), packed when need_pack."""
+        _bf16_weight(module)
+        weight, scales, zeros = w_q(module)
+        if quant_config['weight'].get('need_pack', False):
+            weight, scales = cls.pack(weight, scales, quant_config)
+        return weight, scales
+
     @classmethod
     @torch.no_grad()
     def pack(cls, weight, scales, quant_config):
@@ -35,7 +97,7 @@ class VllmRealQuantLinear:
 
     @classmethod
     @torch.no_grad()
-    def quant_pack(cls, weight, wquantizer, quant_config):
+    def quant_pack_fused(cls, weight, wquantizer, quant_config):
         """pack(*wquantizer.real_quant_weight_dynamic(weight)[:2], quant_config) in one kernel: the bf16 / fp32
         weight is read once and only the packed words and the scales are written."""
         assert quant_config['weight']['bit'] == 4
@@ -43,7 +105,35 @@ class VllmRealQuantLinear:
         return packed, scales.to(torch.float16)
 
 
-class AutoawqRealQuantLinear:
+class AutoawqRealQuantLinear(_RealQuantLinear):
+    def __init__(self, weight, bias, scales, zeros):
+        super().__init__()
+        self.register_buffer('qweight', weight)
+        self._reg('bias', bias)
+        self.register_buffer('scales', scales)
+        self._reg('qzeros', zeros)
+
+    @classmethod
+    @torch.no_grad()
+    def new(cls, module, w_q, quant_config):
+        """module_utils.py:1053-1078."""
+        weight, scales, zeros = cls.quant_pack(module, w_q, quant_config)
+        bias = module.bias.data if module.bias is not None else None
+        new_module = cls(weight, bias, scales, zeros)
+        new_module._describe(module, weight, scales, zeros)
+        return new_module
+
+    @classmethod
+    @torch.no_grad()
+    def quant_pack(cls, module, w_q, quant_config):
+        """module_utils.py:1080-1095."""
+        _bf16_weight(module)
+        _, scales, zeros = w_q(module)
+        pack_version = quant_config['weight']['pack_version']
+        if pack_version != 'gemm_pack':
+            raise NotImplementedError(f'Not support {pack_version}.')
+        return cls.gemm_pack(module, module.weight.data, scales, zeros, quant_config)
+
     @classmethod
     @torch.no_grad()
     def gemm_pack(cls, module, weight, scales, zeros, quant_config):

@@ -263,7 +263,7 @@ def test_fused_quant_pack_equals_quant_then_pack(dev, dtype, gran, shape):
     wd = w.to(dev)
     codes, s, z = q.real_quant_weight_dynamic(wd)
     two_step, s16 = VllmRealQuantLinear.pack(codes, s, cfg)
-    fused, fs16 = VllmRealQuantLinear.quant_pack(wd, q, cfg)
+    fused, fs16 = VllmRealQuantLinear.quant_pack_fused(wd, q, cfg)
     assert_bit_equal(fused, two_step, 'packed words')
     assert_bit_equal(fs16, s16, 'fp16 scales')
     spec = Q.IntSpec(4, True, gran, group_size=kw.get('group_size', 0))
