@@ -98,6 +98,13 @@ int lcq_minmax_all(const void* x, int dtype, int64_t n, void* min_out, void* max
 int lcq_qparams_int(const void* min_in, const void* max_in, int dtype, int64_t n, float qmin, float qmax, int flags,
                     void* scales, void* zeros, void* stream);
 
+/* get_mse_range, quant.py:147-205 (calib_algo 'mse'): per row the shrunken range p * (min, max), p = 1 - i / grid_n,
+ * i < steps, with the smallest sum_j |quant_dequant(x_j) - x_j| ^ norm; a better step replaces the range the next
+ * steps shrink (the reference's aliasing of best_min_val with min_val).  x [rows, cols] of `dtype`, arithmetic and
+ * outputs [rows] in fp32 (the reference upcasts with tensor.float()). */
+int lcq_mse_range(const void* x, int dtype, int64_t rows, int64_t cols, float qmin, float qmax, int flags, int steps,
+                  int grid_n, float norm, float* min_out, float* max_out, void* stream);
+
 /* dequant, quant.py:709-711: out = (q - z) * (s * out_scale_factor). */
 int lcq_dequant_int(const void* q, int dtype, int64_t rows, int64_t cols, const void* scales, const void* zeros,
                     int flags, float out_scale_factor, void* out, void* stream);

@@ -110,6 +110,42 @@ __global__ __launch_bounds__(256) void dequant_kernel(const void* __restrict__ q
   }
 }
 
+// get_mse_range, quant.py:147-205: per row, shrink steps i = 0 .. steps-1 with p = 1 - i / grid:
+//   xmin = p * cur_min, xmax = p * cur_max;  err = sum_j |quant_dequant(x_j; xmin, xmax) - x_j| ^ norm
+//   err < best  ->  best = err, cur_min = xmin, cur_max = xmax
+// cur_min / cur_max start as the row's min / max and - as in the reference, whose best_min_val / best_max_val
+// alias the range tensors - are the values the NEXT step shrinks.  All arithmetic in fp32 (tensor.float()).
+// One wave per row; the row is re-read from L1/L2 on every step.
+template <bool BF>
+__global__ __launch_bounds__(256) void mse_range_kernel(const void* __restrict__ x, int64_t rows, int64_t cols, int steps,
+                                                        int grid_n, float norm, IntOp<false, false> op,
+                                                        float* __restrict__ mn_out, float* __restrict__ mx_out) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  float mn = __builtin_inff(), mx = -__builtin_inff();
+  for (int64_t j = lane; j < cols; j += 64) {
+    const float v = load_scalar<BF>(x, row * cols + j);
+    mn = nan_min(mn, v); mx = nan_max(mx, v);
+  }
+  float cur_min = team_reduce<64, false>(mn), cur_max = team_reduce<64, true>(mx);
+  float best = __builtin_inff();
+  for (int i = 0; i < steps; ++i) {
+    const float p = (float)(1.0 - (double)i / (double)grid_n);
+    const float xmin = p * cur_min, xmax = p * cur_max;
+    const IntRow prm = op.make(xmin, xmax);
+    float err = 0.0f;
+    for (int64_t j = lane; j < cols; j += 64) {
+      const float v = load_scalar<BF>(x, row * cols + j);
+      const float d = fabsf(op.deq(op.code(v, prm), prm) - v);
+      err += __builtin_powf(d, norm);
+    }
+    err = team_sum<64>(err);
+    if (err < best) { best = err; cur_min = xmin; cur_max = xmax; }
+  }
+  if (lane == 0) { mn_out[row] = cur_min; mx_out[row] = cur_max; }
+}
+
 }  // namespace
 
 extern "C" {
@@ -136,6 +172,21 @@ int lcq_quant_int(const void* x, int dtype, int64_t rows, int64_t cols, float qm
   else if (dtype == LCQ_BF16) rc = run<true>(x, rows, cols, qmin, qmax, flags, out_scale_factor, dq, codes, code_dtype, scales, zeros, st);
   else return LCQ_EDTYPE;
   if (rc != LCQ_OK) return rc;
+  LCQ_CHECK_LAUNCH();
+  return LCQ_OK;
+}
+
+int lcq_mse_range(const void* x, int dtype, int64_t rows, int64_t cols, float qmin, float qmax, int flags, int steps,
+                  int grid_n, float norm, float* min_out, float* max_out, void* stream) {
+  if (!x || !min_out || !max_out || rows <= 0 || cols <= 0 || steps <= 0 || grid_n <= 0) return LCQ_EINVAL;
+  if (!(qmax > qmin) || (flags & LCQ_FLAG_STATIC)) return LCQ_EINVAL;
+  auto op = make_op<IntOp<false, false>>(qmin, qmax, flags, 1.0f, LCQ_CODE_NONE);
+  const int64_t grid = (rows + 3) / 4;
+  if (grid > 0x7fffffff) return LCQ_EINVAL;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == LCQ_F32) mse_range_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>(x, rows, cols, steps, grid_n, norm, op, min_out, max_out);
+  else if (dtype == LCQ_BF16) mse_range_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>(x, rows, cols, steps, grid_n, norm, op, min_out, max_out);
+  else return LCQ_EDTYPE;
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;
 }

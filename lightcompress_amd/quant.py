@@ -35,6 +35,10 @@ class BaseQuantizer(object):
         self.kwargs = kwargs
 
         self.calib_algo = self.kwargs.get('calib_algo', 'minmax')
+        # mse config (quant.py:78-81)
+        self.mse_b_num = self.kwargs.get('mse_b_num', 1)
+        self.maxshrink = self.kwargs.get('maxshrink', 0.8)
+        self.mse_grid = self.kwargs.get('mse_grid', 100)
         if self.granularity == 'per_group':
             self.group_size = self.kwargs['group_size']
         elif self.granularity == 'per_head':
@@ -51,9 +55,30 @@ class BaseQuantizer(object):
 
     # -- calibration -------------------------------------------------------
     def get_tensor_range(self, tensor, args={}):
-        if self.calib_algo != 'minmax':
-            raise NotImplementedError(f'calib_algo={self.calib_algo!r}: only minmax runs on liblcq')
-        return self.get_minmax_range(tensor)
+        if self.calib_algo == 'minmax':
+            return self.get_minmax_range(tensor)
+        if self.calib_algo == 'mse':
+            return self.get_mse_range(tensor)
+        raise NotImplementedError(f'calib_algo={self.calib_algo!r}: minmax and mse run on liblcq')
+
+    def get_mse_range(self, tensor, norm=2.4, bs=256):
+        """quant.py:147-205 -> fp32 (min_val, max_val) [rows, 1]: the shrunken range with the smallest
+        sum |quant_dequant(x) - x| ** norm per row, one kernel instead of 80 rounds of ~10 torch ops."""
+        if getattr(self, 'quant_type', 'int-quant') != 'int-quant':
+            raise NotImplementedError('get_mse_range runs for IntegerQuantizer')
+        if self.granularity == 'per_tensor' or tensor.dim() != 2:
+            raise NotImplementedError('get_mse_range runs on a 2-D reshaped tensor')
+        assert self.mse_b_num >= 1 and tensor.shape[0] % self.mse_b_num == 0, \
+            'Batch number must be divisible by tensor.shape[0],'
+        t = tensor.contiguous()
+        rows, cols = t.shape
+        mn = torch.empty((rows, 1), dtype=torch.float32, device=t.device)
+        mx = torch.empty((rows, 1), dtype=torch.float32, device=t.device)
+        L.check(L.lib().lcq_mse_range(L.ptr(t), L.dtype_code(t.dtype), L.i64(rows), L.i64(cols), L.f32(float(self.qmin)),
+                                      L.f32(float(self.qmax)), L.i32(self._int_flags()),
+                                      L.i32(int(self.maxshrink * self.mse_grid)), L.i32(int(self.mse_grid)),
+                                      L.f32(norm), L.ptr(mn), L.ptr(mx), L.stream()), 'lcq_mse_range')
+        return (mn, mx)
 
     def get_minmax_range(self, tensor):
         """quant.py:134-145 -> (min_val, max_val)."""
@@ -250,9 +275,10 @@ class IntegerQuantizer(BaseQuantizer):
     # -- reference API ----------------------------------------------------------
     def get_tensor_qparams(self, tensor, args={}):
         """quant.py:689-696 -> (tensor_reshaped, scales, zeros, qmax, qmin)."""
-        if self.calib_algo != 'minmax':
-            raise NotImplementedError(f'calib_algo={self.calib_algo!r}: only minmax runs on liblcq')
         tensor = self.reshape_tensor(tensor)
+        if self.calib_algo != 'minmax':
+            scales, zeros, qmax, qmin = self.get_qparams(self.get_tensor_range(tensor, args), tensor.device)
+            return tensor, scales, zeros, qmax, qmin
         if self.granularity == 'per_tensor':
             scales, zeros, qmax, qmin = self.get_qparams(self.get_minmax_range(tensor), tensor.device)
             return tensor, scales, zeros, qmax, qmin
@@ -298,6 +324,10 @@ class IntegerQuantizer(BaseQuantizer):
     def _fake_dynamic(self, t):
         shape, dtype = t.shape, t.dtype
         rows_t = self.reshape_tensor(t)
+        if self.calib_algo != 'minmax':                  # calibrated ranges, then the static path (quant.py:853-860)
+            rows_t, scales, zeros, qmax, qmin = self.get_tensor_qparams(t)
+            dq, _, _, _ = self._launch(rows_t, static=True, scales=scales, zeros=zeros, want_dq=True, qmin=qmin, qmax=qmax)
+            return self.restore_tensor(dq.view(rows_t.shape), shape).to(dtype)
         dq, _, _, _ = self._launch(rows_t, static=False, want_dq=True)
         return self.restore_tensor(dq.view(rows_t.shape), shape).to(dtype)
 
@@ -404,7 +434,12 @@ class IntegerQuantizer(BaseQuantizer):
         org_w_shape = weight.shape
         output_scale_factor = args.pop('output_scale_factor', 1) if 'output_scale_factor' in args else 1
         rows_t = self.reshape_tensor(weight)
-        _, codes, scales, zeros = self._launch(rows_t, static=False, want_codes=self._code_dtype())
+        if self.calib_algo != 'minmax':
+            rows_t, scales, zeros, qmax, qmin = self.get_tensor_qparams(weight)
+            _, codes, _, _ = self._launch(rows_t, static=True, scales=scales, zeros=zeros, want_codes=self._code_dtype(),
+                                          qmin=qmin, qmax=qmax)
+        else:
+            _, codes, scales, zeros = self._launch(rows_t, static=False, want_codes=self._code_dtype())
         codes = self.restore_tensor(codes.view(rows_t.shape), org_w_shape)
         return self._finish_real(codes, scales, zeros, output_scale_factor)
 

@@ -433,3 +433,38 @@ def float_per_block_real_quant(spec, w: torch.Tensor, block_size: int = 128):
     q = float_quant(spec, t, scales, zeros)
     q = q.reshape(-1, n if nb * block_size == n else nb * block_size)[:m, :n]
     return q.to(torch.float8_e4m3fn), scales.view(scales.shape[0], scales.shape[2]), None
+
+
+# ----------------------------------------------------------------------------
+# calib_algo 'mse'
+# ----------------------------------------------------------------------------
+def int_mse_range(spec, tensor: torch.Tensor, norm=2.4, maxshrink=0.8, mse_grid=100, mse_b_num=1):
+    """get_mse_range, quant.py:147-205, op for op - including its aliasing: `best_min_val, best_max_val = _min_val,
+    _max_val` are views of the range tensors, so an improving step overwrites the range that the following
+    steps shrink."""
+    assert mse_b_num >= 1 and tensor.shape[0] % mse_b_num == 0
+    bs = tensor.shape[0] // mse_b_num
+    tensor = tensor.float()
+    min_val, max_val = minmax_range(spec, tensor)
+    for b_num in range(mse_b_num):
+        _tensor = tensor[b_num * bs:(b_num + 1) * bs, :]
+        _min_val, _max_val = min_val[b_num * bs:(b_num + 1) * bs, :], max_val[b_num * bs:(b_num + 1) * bs, :]
+        best = torch.full([_tensor.shape[0]], float('inf'))
+        best_min_val, best_max_val = _min_val, _max_val
+        for i in range(int(maxshrink * mse_grid)):
+            p = 1 - i / mse_grid
+            xmin = p * _min_val
+            xmax = p * _max_val
+            scales, zeros, qmax, qmin = int_qparams(spec, xmin, xmax)
+            q_tensor = int_quant_dequant(spec, _tensor, scales, zeros, qmax, qmin)
+            q_tensor -= _tensor
+            q_tensor.abs_()
+            q_tensor.pow_(norm)
+            err = torch.sum(q_tensor, 1)
+            tmp = err < best
+            if torch.any(tmp):
+                best[tmp] = err[tmp]
+                best_min_val[tmp] = xmin[tmp]
+                best_max_val[tmp] = xmax[tmp]
+        min_val[b_num * bs:(b_num + 1) * bs, :], max_val[b_num * bs:(b_num + 1) * bs, :] = best_min_val, best_max_val
+    return min_val, max_val

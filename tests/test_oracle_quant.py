@@ -378,3 +378,28 @@ def test_blockwise_fp8_oracles_scale_and_grid():
     zero = torch.zeros(128, 128, dtype=torch.bfloat16)
     _, sz, _ = Q.float_per_block_real_quant(spec, zero)
     assert float(sz) == float(torch.tensor(1e-5) / 448.0)
+
+
+def test_mse_range_oracle_recurrence_and_optimality():
+    """get_mse_range: a plain per-row Python loop of the recurrence (shrink the CURRENT best range by p_i; accept on
+    a strictly smaller error) reproduces the vectorised oracle, the result never widens the min/max range, and its
+    |.|^2.4 error is no larger than that of plain min/max."""
+    spec = Q.IntSpec(4, False, 'per_group', group_size=128)
+    w = weight_like(16, 128, seed=91)
+    mn, mx = Q.int_mse_range(spec, w.clone())
+    assert mn.dtype == torch.float32 and mn.shape == (16, 1)
+    def err_of(row, lo, hi):
+        s, z, qmax, qmin = Q.int_qparams(spec, lo.reshape(1, 1), hi.reshape(1, 1))
+        return float((Q.int_quant_dequant(spec, row.reshape(1, -1), s, z, qmax, qmin) - row).abs().pow(2.4).sum())
+    for r in range(16):
+        row = w[r].float()
+        lo, hi, best = row.min(), row.max(), float('inf')
+        for i in range(80):
+            p = 1 - i / 100
+            xlo, xhi = p * lo, p * hi
+            e = err_of(row, xlo, xhi)
+            if e < best:
+                best, lo, hi = e, xlo, xhi
+        assert abs(float(lo) - float(mn[r])) <= 1e-6 * abs(float(lo)) and abs(float(hi) - float(mx[r])) <= 1e-6 * abs(float(hi))
+        assert float(mn[r]) >= float(row.min()) and float(mx[r]) <= float(row.max())
+        assert err_of(row, mn[r], mx[r]) <= err_of(row, row.min(), row.max()) * (1 + 1e-6)
