@@ -18,10 +18,22 @@
 // 8t..8t+7 of the block in registers; a wave therefore carries 4 rows and a
 // 256-thread workgroup 16.  Column i lives on lane i/8: every lane evaluates
 // the quantizer on its own register (same instruction stream), the owner's
-// error is broadcast inside the 16-lane team with ds_bpermute, and all lanes
-// apply the rank-1 update to their 8 columns from the Hinv block held in LDS.
-// Per-group min/max are 16-lane DPP butterflies.  tmp / Losses / Err are kept
-// in registers and written once, 32 bytes per lane.
+// error is broadcast inside the 16-lane team, and all lanes apply the rank-1
+// update to their 8 columns from the Hinv block held in LDS.
+// Per-group min/max are 16-lane DPP butterflies.
+//
+// With R = 4096 rows the kernel has one wave per SIMD on the whole chip, so its run time is the
+// length of the per-column dependency chain times 128.  That chain is kept to about ten VALU
+// operations: the quotient w/s goes through the group's reciprocal (an octet in which an owner comes
+// near a rounding boundary is replayed with true divisions), (w-q)/d through a reciprocal of the diagonal prepared in LDS (at most one ulp
+// from the quotient; it only perturbs later columns, never the rounding of this one), the broadcast
+// of the error is a DPP row_share from lane 0 instead of an LDS permute (the registers rotate by one
+// lane after every 8 columns, so the owner is always lane 0 and the loop over octets stays rolled:
+// fully unrolled it is 126 KB of straight-line code that runs at instruction-fetch speed), the U row
+// comes from addresses that do not depend on the chain, and because U is upper triangular no update
+// needs a mask.  tmp / (w-q) / err rotate along and are stored once at the end, 32 bytes per lane.
+#include <type_traits>
+
 #include "gemm_f32.h"
 #include "lcq_internal.h"
 
@@ -36,118 +48,258 @@ struct LoopArgs {
   float* scales; float* zeros; const int* gidx;
   long long R; int K, i1, count, g, G, ldErr;
   float qmin, qmax;
-  int sym, is_static;
+  int sym, is_static, aligned;
 };
 
-__device__ __forceinline__ float team16_bcast(float v, int src) {   // value of lane (lane & ~15) | src
-  return u2f((uint32_t)__builtin_amdgcn_ds_bpermute((int)(((threadIdx.x & ~15) | src) << 2), (int)f2u(v)));
+// DPP moves inside every 16-lane row: the value of lane 0, and the value of the next lane (rotation by one)
+__device__ __forceinline__ float row16_first(float v) {
+  return u2f((uint32_t)__builtin_amdgcn_update_dpp(0, (int)f2u(v), 0x150, 0xf, 0xf, true));          // row_share:0
+}
+__device__ __forceinline__ float row16_next(float v) {
+  return u2f((uint32_t)__builtin_amdgcn_update_dpp(0, (int)f2u(v), 0x12F, 0xf, 0xf, true));          // row_ror:15
 }
 
-__global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
-  __shared__ float Us[BS * BS];                  // Hinv1 = U[i1:i2, i1:i2]
-  const int tid = threadIdx.x;
-  for (int e = tid; e < BS * BS / 4; e += 256) {
-    const int r = (e * 4) / BS, c = (e * 4) % BS;
-    f32x4 v = {0.f, 0.f, 0.f, 0.f};
-    if (r < a.count) {
-      const float* p = a.U + (long long)(a.i1 + r) * a.K + a.i1 + c;
-      #pragma unroll
-      for (int k = 0; k < 4; ++k) if (c + k < a.count) v[k] = p[k];
-    }
-    *(f32x4*)(Us + e * 4) = v;
-  }
+struct ColQ {           // quantizer of the column being processed
+  float s, z, r;        // scale, zero point, 1/s
+  float lo, hi;         // qmin - z, qmax - z: clamp(round(t) + z, qmin, qmax) - z == clamp(round(t), lo, hi) for integral z
+  bool fast;            // x * r may stand for x / s (guarded) and lo / hi are exact
+};
+__device__ __forceinline__ ColQ make_colq(float s, float z, float qmin, float qmax) {
+  ColQ q;
+  q.s = s; q.z = z;
+  q.r = __builtin_amdgcn_rcpf(s);
+  q.lo = qmin - z; q.hi = qmax - z;
+  const float a = fabsf(s);
+  q.fast = (a > 8.6736174e-19f) & (a < 1.1529215e18f) & (rintf(z) == z) & (fabsf(z) <= 512.0f) & (fabsf(qmin) <= 512.0f) &
+           (fabsf(qmax) <= 512.0f);
+  return q;
+}
 
-  const int t = tid & 15;
+// A group opens at column idx: scale and zero point from the range of W[row, idx : min(idx+g, K)] as it is in
+// memory now -- trailing updates of earlier blocks applied, this block's own updates not (gptq.py:216-222 reads
+// W, not W1).
+// `held`: the team's registers when they are exactly that range (group = block, nothing updated yet).
+__device__ __forceinline__ ColQ open_group(const LoopArgs& a, int idx, int lane, long long row, bool row_ok, long long rbase,
+                                           const float (&held)[8], bool use_held) {
+  const int end = min(idx + a.g, a.K);
+  float mn = __builtin_inff(), mx = -__builtin_inff();
+  if (use_held) {
+    #pragma unroll
+    for (int c = 0; c < 8; ++c) { mn = fminf(mn, held[c]); mx = fmaxf(mx, held[c]); }
+  } else {
+    for (int col = idx + lane; col < end; col += 16) {
+      const float v = a.W[rbase + col];
+      mn = fminf(mn, v); mx = fmaxf(mx, v);
+    }
+  }
+  mn = team_reduce<16, false>(mn);
+  mx = team_reduce<16, true>(mx);
+  float s, z;
+  if (a.sym) {
+    s = fmaxf(fmaxf(fabsf(mx), fabsf(mn)), 1e-5f) / a.qmax;
+    z = 0.0f;
+  } else {
+    s = fmaxf(mx - mn, 1e-5f) / (a.qmax - a.qmin);
+    z = fminf(fmaxf(a.qmin - rintf(mn / s), a.qmin), a.qmax);
+  }
+  if (row_ok && lane == 0) {
+    a.scales[row * a.G + idx / a.g] = s;
+    if (!a.sym) a.zeros[row * a.G + idx / a.g] = z;
+  }
+  return make_colq(s, z, a.qmin, a.qmax);
+}
+
+// STATIC: scales / zero points are given (per group, or per column through gidx).  OCT: every group starts on
+// a multiple of 8 columns, so groups open only between octets and the 8 columns of an octet are straight-line code.
+template <bool STATIC, bool OCT>
+__global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
+  __shared__ float Us[BS * BS];                  // Hinv1 = U[i1:i2, i1:i2], zero outside the block and below the diagonal
+  __shared__ float Rd[BS];                       // 1 / U[i, i]
+  const int tid = threadIdx.x;
+  // full block and 16-byte aligned rows (the entry point checks the base pointers): vector loads and stores
+  const bool vec = (a.count == BS) && (a.K % 4 == 0) && (a.i1 % 4 == 0) && a.aligned;
+  if (vec) {
+    // all 16 loads of the thread in flight at once: one after the other they are 16 memory latencies,
+    // which used to be most of the kernel's run time
+    f32x4 v[16];
+    #pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const int e = tid + 256 * j, r = e >> 5, c = (e & 31) * 4;
+      v[j] = *(const f32x4*)(a.U + (long long)(a.i1 + r) * a.K + a.i1 + c);
+    }
+    #pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const int e = tid + 256 * j, r = e >> 5, c = (e & 31) * 4;
+      #pragma unroll
+      for (int k = 0; k < 4; ++k) if (c + k < r) v[j][k] = 0.0f;
+      *(f32x4*)(Us + e * 4) = v[j];
+    }
+  } else {
+    for (int e = tid; e < BS * BS / 4; e += 256) {
+      const int r = (e * 4) / BS, c = (e * 4) % BS;
+      f32x4 v = {0.f, 0.f, 0.f, 0.f};
+      if (r < a.count) {
+        const float* p = a.U + (long long)(a.i1 + r) * a.K + a.i1 + c;
+        #pragma unroll
+        for (int k = 0; k < 4; ++k) if (c + k < a.count && c + k >= r) v[k] = p[k];
+      }
+      *(f32x4*)(Us + e * 4) = v;
+    }
+  }
+  if (tid < BS) Rd[tid] = (tid < a.count) ? 1.0f / a.U[(long long)(a.i1 + tid) * a.K + a.i1 + tid] : 0.0f;
+
+  const int lane = tid & 15;                     // physical lane inside the row's team
   const long long row = (long long)blockIdx.x * ROWS_PER_WG + (tid >> 4);
   const bool row_ok = row < a.R;
   const long long rbase = (row_ok ? row : 0) * a.K;
 
-  float w[8], otmp[8], oloss[8], oerr[8];
+  // lane t starts with columns 8t..8t+7 (and, for static groups, their scales and zero points)
+  float w[8], ss[8], zz[8];
+  if (vec) {                                     // rows of W / tmp / Losses are 16-byte aligned at the block's columns
+    const f32x4 lo4 = *(const f32x4*)(a.W + rbase + a.i1 + 8 * lane), hi4 = *(const f32x4*)(a.W + rbase + a.i1 + 8 * lane + 4);
+    #pragma unroll
+    for (int k = 0; k < 4; ++k) { w[k] = row_ok ? lo4[k] : 0.0f; w[4 + k] = row_ok ? hi4[k] : 0.0f; }
+  }
   #pragma unroll
   for (int c = 0; c < 8; ++c) {
-    const int col = 8 * t + c;
-    w[c] = (row_ok && col < a.count) ? a.W[rbase + a.i1 + col] : 0.0f;
-    otmp[c] = 0.0f; oloss[c] = 0.0f; oerr[c] = 0.0f;
+    const int col = 8 * lane + c;
+    if (!vec) w[c] = (row_ok && col < a.count) ? a.W[rbase + a.i1 + col] : 0.0f;
+    ss[c] = 1.0f; zz[c] = 0.0f;
+    if (STATIC && col < a.count) {
+      const int idx = a.i1 + col;
+      const int gi = a.gidx ? a.gidx[idx] : (a.g > 0 ? idx / a.g : 0);
+      ss[c] = a.scales[(row_ok ? row : 0) * a.G + gi];
+      zz[c] = a.sym ? 0.0f : a.zeros[(row_ok ? row : 0) * a.G + gi];
+    }
+  }
+  ColQ q = make_colq(1.0f, 0.0f, a.qmin, a.qmax);
+  int nextb = 0x7fffffff;
+  if (!STATIC) {
+    nextb = (a.i1 + a.g - 1) / a.g * a.g;
+    if (a.i1 % a.g != 0)                         // the block starts inside a group opened by an earlier block
+      q = make_colq(a.scales[(row_ok ? row : 0) * a.G + a.i1 / a.g], a.sym ? 0.0f : a.zeros[(row_ok ? row : 0) * a.G + a.i1 / a.g], a.qmin, a.qmax);
   }
   __syncthreads();
 
-  float s = 1.0f, z = 0.0f;
-  const float qrange = a.qmax - a.qmin;
-  for (int to = 0; to < 16; ++to) {              // owner lane of columns 8*to .. 8*to+7
+  // Octet `to` = columns 8*to .. 8*to+7.  After every octet the registers rotate by one lane inside the team, so
+  // the owner of the current octet is always lane 0 (a constant DPP source) and lane p holds the columns of
+  // team member (p + to) mod 16.
+  // Outputs rotate with them: what lane 0 produced for octet `to` sits on lane (to - n) mod 16 after n rotations,
+  // so each lane ends up with 8 consecutive columns of tmp / (w-q) / err and stores them once.  (Stores inside the
+  // loop would make every later wait on a load wait for them too.)
+  float o_w[8], o_diff[8], o_err[8];
+  #pragma unroll
+  for (int c = 0; c < 8; ++c) { o_w[c] = 0.0f; o_diff[c] = 0.0f; o_err[c] = 0.0f; }
+  const bool first = lane == 0;
+  int n_oct = 0;
+  for (int to = 0; to < 16; ++to) {
     if (8 * to >= a.count) break;
+    ++n_oct;
+    // the octet's 8 rows of U (this lane's 8 columns of each) and reciprocal diagonals, fetched ahead of the
+    // dependency chain; rows past `count` are zero in LDS, so the 8 columns need no bound check
+    const float* ucol = Us + (8 * to) * BS + 8 * ((lane + to) & 15);
+    f32x4 u0[8], u1[8];
+    float rd[8];
     #pragma unroll
     for (int c = 0; c < 8; ++c) {
-      const int i = 8 * to + c;
-      const int idx = a.i1 + i;
-      if (i < a.count) {
-        // ---- per-group parameters (uniform branch: idx is the same for every lane) ----
-        if (a.is_static) {
-          const int gi = a.gidx ? a.gidx[idx] : (a.g > 0 ? idx / a.g : 0);
-          if (i == 0 || a.gidx || (a.g > 0 && idx % a.g == 0)) {
-            s = a.scales[(row_ok ? row : 0) * a.G + gi];
-            z = a.sym ? 0.0f : a.zeros[(row_ok ? row : 0) * a.G + gi];
-          }
-        } else if (idx % a.g == 0) {
-          // range of W[row, idx : min(idx+g, K)] as it is in memory now: trailing updates of
-          // earlier blocks applied, this block's own updates not (gptq.py:216-222 reads W, not W1)
-          const int end = min(idx + a.g, a.K);
-          float mn = __builtin_inff(), mx = -__builtin_inff();
-          for (int col = idx + t; col < end; col += 16) {
-            const float v = a.W[rbase + col];
-            mn = fminf(mn, v); mx = fmaxf(mx, v);
-          }
-          mn = team_reduce<16, false>(mn);
-          mx = team_reduce<16, true>(mx);
-          if (a.sym) {
-            s = fmaxf(fmaxf(fabsf(mx), fabsf(mn)), 1e-5f) / a.qmax;
-            z = 0.0f;
-          } else {
-            s = fmaxf(mx - mn, 1e-5f) / qrange;
-            z = fminf(fmaxf(a.qmin - rintf(mn / s), a.qmin), a.qmax);
-          }
-          if (row_ok && t == 0) {
-            a.scales[row * a.G + idx / a.g] = s;
-            if (!a.sym) a.zeros[row * a.G + idx / a.g] = z;
-          }
-        } else if (i == 0) {
-          // the block starts inside a group opened by an earlier block
-          s = a.scales[(row_ok ? row : 0) * a.G + idx / a.g];
-          z = a.sym ? 0.0f : a.zeros[(row_ok ? row : 0) * a.G + idx / a.g];
+      u0[c] = *(const f32x4*)(ucol + c * BS);
+      u1[c] = *(const f32x4*)(ucol + c * BS + 4);
+      rd[c] = Rd[8 * to + c];
+    }
+    if (!STATIC && OCT && a.i1 + 8 * to == nextb) {
+      nextb += a.g;
+      q = open_group(a, a.i1 + 8 * to, lane, row, row_ok, rbase, w, to == 0 && a.g == BS && a.count == BS);
+    }
+    // 8 columns.  Each: quantize-dequantize like clamp(round(w / s) + z, qmin, qmax), (q - z) * s in fp32 (only
+    // lane 0's result is used), err = (w - q) / d, rank-1 update of the lane's 8 columns.  U is upper triangular,
+    // so columns left of the current one see a zero factor and need no mask (the column itself turns into its
+    // quantized value, which nothing reads).
+    // The first pass takes the quotient through the reciprocal and only notes whether any owner came within 2^-11
+    // of a rounding boundary (or beyond 1024), where product and quotient may round apart; then the wave runs the
+    // octet again from the saved registers with true divisions.  That keeps every branch out of the chain.
+    auto octet = [&](auto exact_tag) -> bool {
+      constexpr bool EXACT = decltype(exact_tag)::value;
+      bool unsure = false;
+      #pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        if (STATIC) {
+          q = make_colq(ss[c], zz[c], a.qmin, a.qmax);                      // lane 0: the parameters of this column
+        } else if (!OCT && a.i1 + 8 * to + c == nextb && 8 * to + c < a.count) {
+          nextb += a.g;
+          q = open_group(a, a.i1 + 8 * to + c, lane, row, row_ok, rbase, w, false);
         }
-        // ---- quantize this lane's register c (meaningful on the owner lane) ----
-        const float d = Us[i * BS + i];
         const float wv = w[c];
-        float q = rintf(wv / s) + z;
-        q = fminf(fmaxf(q, a.qmin), a.qmax);
-        const float dq = (q - z) * s;
-        const float diff = wv - dq;
-        const float err = diff / d;
-        if (t == to) {
-          otmp[c] = wv;
-          oloss[c] = (diff * diff) / (2.0f * (d * d));
-          oerr[c] = err;
+        float diff;
+        if (EXACT) {
+          diff = wv - (__builtin_amdgcn_fmed3f(rintf(wv / q.s) + q.z, a.qmin, a.qmax) - q.z) * q.s;
+        } else {
+          const float t = wv * q.r, rt = rintf(t);
+          unsure |= !((fabsf(fabsf(t - rt) - 0.5f) > 4.8828125e-04f) & (fabsf(t) <= 1024.0f) & q.fast);
+          diff = wv - __builtin_amdgcn_fmed3f(rt, q.lo, q.hi) * q.s;
         }
-        const float eb = team16_bcast(err, to);
-        // ---- rank-1 update of the remaining columns of the block ----
-        const f32x4 u0 = *(const f32x4*)(Us + i * BS + 8 * t);
-        const f32x4 u1 = *(const f32x4*)(Us + i * BS + 8 * t + 4);
+        const float err = diff * rd[c];
+        o_w[c] = first ? wv : o_w[c];
+        o_diff[c] = first ? diff : o_diff[c];
+        o_err[c] = first ? err : o_err[c];
+        const float eb = row16_first(err);
         #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          if (8 * t + k > i) w[k] -= eb * u0[k];
-          if (8 * t + 4 + k > i) w[4 + k] -= eb * u1[k];
-        }
+        for (int k = 0; k < 4; ++k) { w[k] -= eb * u0[c][k]; w[4 + k] -= eb * u1[c][k]; }
       }
+      return unsure & first;
+    };
+    if (STATIC || OCT) {
+      float saved[8];
+      #pragma unroll
+      for (int c = 0; c < 8; ++c) saved[c] = w[c];
+      const bool unsure = octet(std::false_type{});
+      if (__builtin_expect(__builtin_amdgcn_ballot_w64(unsure) != 0, 0)) {
+        #pragma unroll
+        for (int c = 0; c < 8; ++c) w[c] = saved[c];
+        octet(std::true_type{});
+      }
+    } else {
+      octet(std::true_type{});          // groups may open inside the octet: no replay, divide throughout
+    }
+    #pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      w[c] = row16_next(w[c]);
+      o_w[c] = row16_next(o_w[c]); o_diff[c] = row16_next(o_diff[c]); o_err[c] = row16_next(o_err[c]);
+      if (STATIC) { ss[c] = row16_next(ss[c]); zz[c] = row16_next(zz[c]); }
     }
   }
 
+  const int oct = (lane + n_oct) & 15;                      // the octet whose outputs this lane holds now
   if (row_ok) {
+    float loss[8];
     #pragma unroll
     for (int c = 0; c < 8; ++c) {
-      const int col = 8 * t + c;
-      if (col < a.count) {
-        a.tmp[rbase + a.i1 + col] = otmp[c];
-        a.Losses[rbase + a.i1 + col] = oloss[c];
-        a.Err[row * a.ldErr + col] = oerr[c];
+      const float d = Us[(8 * oct + c) * BS + 8 * oct + c];
+      loss[c] = (o_diff[c] * o_diff[c]) / (2.0f * (d * d));
+    }
+    if (vec) {
+      float* pt = a.tmp + rbase + a.i1 + 8 * oct;
+      float* pl = a.Losses + rbase + a.i1 + 8 * oct;
+      *(f32x4*)pt = f32x4{o_w[0], o_w[1], o_w[2], o_w[3]};
+      *(f32x4*)(pt + 4) = f32x4{o_w[4], o_w[5], o_w[6], o_w[7]};
+      *(f32x4*)pl = f32x4{loss[0], loss[1], loss[2], loss[3]};
+      *(f32x4*)(pl + 4) = f32x4{loss[4], loss[5], loss[6], loss[7]};
+    }
+    float* pe = a.Err + row * a.ldErr + 8 * oct;
+    if (vec && a.ldErr % 4 == 0 && (reinterpret_cast<uintptr_t>(a.Err) & 15) == 0) {
+      *(f32x4*)pe = f32x4{o_err[0], o_err[1], o_err[2], o_err[3]};
+      *(f32x4*)(pe + 4) = f32x4{o_err[4], o_err[5], o_err[6], o_err[7]};
+    } else {
+      #pragma unroll
+      for (int c = 0; c < 8; ++c) if (8 * oct + c < a.count) pe[c] = o_err[c];
+    }
+    if (!vec) {
+      #pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        const int col = 8 * oct + c;
+        if (col < a.count) {
+          a.tmp[rbase + a.i1 + col] = o_w[c];
+          a.Losses[rbase + a.i1 + col] = loss[c];
+        }
       }
     }
   }
@@ -172,8 +324,13 @@ int lcq_gptq_block(float* W, float* tmp, float* Losses, float* Err, int64_t ldEr
   a.scales = scales; a.zeros = zeros; a.gidx = gidx;
   a.R = R; a.K = (int)K; a.i1 = (int)i1; a.count = count; a.g = group_size; a.G = (int)G;
   a.qmin = qmin; a.qmax = qmax; a.sym = sym; a.is_static = is_static; a.ldErr = (int)ldErr;
+  a.aligned = ((reinterpret_cast<uintptr_t>(W) | reinterpret_cast<uintptr_t>(tmp) | reinterpret_cast<uintptr_t>(Losses) |
+                reinterpret_cast<uintptr_t>(U)) & 15) == 0;
   const unsigned grid = (unsigned)((R + ROWS_PER_WG - 1) / ROWS_PER_WG);
-  gptq_block_kernel<<<dim3(grid), dim3(256), 0, (hipStream_t)stream>>>(a);
+  const bool oct = !is_static && group_size % 8 == 0 && i1 % 8 == 0;
+  if (is_static) gptq_block_kernel<true, true><<<dim3(grid), dim3(256), 0, (hipStream_t)stream>>>(a);
+  else if (oct) gptq_block_kernel<false, true><<<dim3(grid), dim3(256), 0, (hipStream_t)stream>>>(a);
+  else gptq_block_kernel<false, false><<<dim3(grid), dim3(256), 0, (hipStream_t)stream>>>(a);
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;
 }
