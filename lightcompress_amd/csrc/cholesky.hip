@@ -84,19 +84,111 @@ __global__ __launch_bounds__(256) void build_kernel(const float* __restrict__ H,
 }
 
 // Diagonal block: Cholesky factor L11 and its inverse in one elimination sweep.
-// 256 threads hold the 128x128 block of A and of B (= I, turning into L11^-1) as 8x8
-// register tiles (thread (ty, tx) owns rows 8ty.., columns 8tx..).  Step j:
-//   owners publish the UNSCALED column j of A and row j of B through LDS (double buffered),
-//   one barrier, then every thread derives 1/sqrt(a_jj) itself and applies
-//   a[i][k] -= l_ij l_kj  (i, k > j)      b[i][:] -= l_ij x_j[:]  (i > j)
-// i.e. the right-looking Cholesky update and the forward substitution L X = I share the
-// broadcast of column j.  One barrier and at most 128 FMAs per thread per step.
+// 256 threads hold the 128x128 block of A and of B (= I, turning into L11^-1) in registers, 8x8 each,
+// dealt out cyclically: thread (ty, tx) owns rows ty + 16 ii and columns tx + 16 cc.  The elimination
+// front therefore shrinks on every thread alike -- during columns 16P .. 16P+15 ("phase" P) a thread
+// updates (8-P)(9-P)/2 elements of A and (8-P)(P+1) of B per step, whichever thread it is -- where a
+// blocked layout leaves the last wave with 128 FMAs per step to the end while the first idles.
+// Step j:
+//   barrier; every thread reads the UNSCALED column j of A, row j of B and the pivot from LDS (double
+//   buffered; entries that must not take part are published as zeros, so no update needs a mask),
+//   derives 1/sqrt(a_jj) itself and applies
+//     a[i][k] -= l_ij l_kj  (i, k > j)      b[i][:] -= l_ij x_j[:]  (i > j)
+//   starting with the two register columns of A and rows of B that can hold column / row j+1, which
+//   their owners publish at once; the rest of the update then overlaps the next barrier.
+// The right-looking Cholesky update and the forward substitution L X = I share the broadcast.
+constexpr int lds_slot(int r) { return (r & 15) * 8 + (r >> 4); }   // a thread's 8 rows (columns) are contiguous
+
+template <int P>
+__device__ __forceinline__ void potrf_phase(float (&a)[8][8], float (&x)[8][8], float (*colbuf)[NB], float (*rowbuf)[NB],
+                                            float* pivbuf, int ty, int tx, bool& bad) {
+  #pragma clang fp contract(fast)   // a -= l*l as one FMA; nothing here needs op-by-op rounding
+  constexpr int P1 = (P < 7) ? P + 1 : 7;
+  #pragma unroll 1
+  for (int jl = 0; jl < 16; ++jl) {
+    const int j = 16 * P + jl, pb = j & 1;
+    __syncthreads();
+    const float pv = pivbuf[pb];
+    const f32x4 r0 = *(const f32x4*)(colbuf[pb] + 8 * ty), r1 = *(const f32x4*)(colbuf[pb] + 8 * ty + 4);
+    const f32x4 c0 = *(const f32x4*)(colbuf[pb] + 8 * tx), c1 = *(const f32x4*)(colbuf[pb] + 8 * tx + 4);
+    const f32x4 x0 = *(const f32x4*)(rowbuf[pb] + 8 * tx), x1 = *(const f32x4*)(rowbuf[pb] + 8 * tx + 4);
+    bad = bad || !(pv > 0.0f);
+    float rinv = __builtin_amdgcn_rsqf(pv);           // 1/sqrt(pivot), one Newton step to full precision
+    rinv = rinv * (1.5f - 0.5f * pv * rinv * rinv);
+    float lr[8], lc[8], xr[8];
+    #pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      lr[k] = r0[k] * rinv; lr[4 + k] = r1[k] * rinv;
+      lc[k] = c0[k] * rinv; lc[4 + k] = c1[k] * rinv;
+      xr[k] = x0[k] * rinv; xr[4 + k] = x1[k] * rinv;
+    }
+    // ---- first: what column j+1 of A and row j+1 of B can depend on ----
+    #pragma unroll
+    for (int ii = P; ii < 8; ++ii) {
+      a[ii][P] -= lr[ii] * lc[P];
+      if (P1 != P && P1 <= ii) a[ii][P1] -= lr[ii] * lc[P1];
+    }
+    #pragma unroll
+    for (int cc = 0; cc <= P; ++cc) {
+      x[P][cc] -= lr[P] * xr[cc];
+      if (P1 != P) x[P1][cc] -= lr[P1] * xr[cc];
+    }
+    // owners keep the scaled column j of L and row j of X (the published zeros left their own entries alone)
+    if (tx == jl) {
+      #pragma unroll
+      for (int ii = P; ii < 8; ++ii) {
+        const int r = ty + 16 * ii;
+        if (r > j) a[ii][P] = lr[ii];
+        else if (r == j) a[ii][P] = pv * rinv;
+      }
+    }
+    if (ty == jl) {
+      #pragma unroll
+      for (int cc = 0; cc <= P; ++cc) x[P][cc] = xr[cc];
+    }
+    // ---- publish column j+1 / row j+1 for the next step ----
+    if (j + 1 < NB) {
+      const int jn = j + 1, tn = jn & 15;
+      const bool nextphase = (jl == 15);
+      if (tx == tn) {
+        f32x4 v0, v1;
+        #pragma unroll
+        for (int ii = 0; ii < 8; ++ii) {
+          const float v = (ty + 16 * ii > jn) ? (nextphase ? a[ii][P1] : a[ii][P]) : 0.0f;
+          if (ii < 4) v0[ii] = v; else v1[ii - 4] = v;
+        }
+        *(f32x4*)(colbuf[pb ^ 1] + 8 * ty) = v0;
+        *(f32x4*)(colbuf[pb ^ 1] + 8 * ty + 4) = v1;
+        if (ty == tn) pivbuf[pb ^ 1] = nextphase ? a[P1][P1] : a[P][P];
+      }
+      if (ty == tn) {
+        f32x4 v0, v1;
+        #pragma unroll
+        for (int cc = 0; cc < 8; ++cc) {
+          const float v = (tx + 16 * cc <= jn) ? (nextphase ? x[P1][cc] : x[P][cc]) : 0.0f;
+          if (cc < 4) v0[cc] = v; else v1[cc - 4] = v;
+        }
+        *(f32x4*)(rowbuf[pb ^ 1] + 8 * tx) = v0;
+        *(f32x4*)(rowbuf[pb ^ 1] + 8 * tx + 4) = v1;
+      }
+    }
+    // ---- the rest of the update ----
+    #pragma unroll
+    for (int ii = P + 2; ii < 8; ++ii)
+      #pragma unroll
+      for (int cc = P + 2; cc <= ii; ++cc) a[ii][cc] -= lr[ii] * lc[cc];
+    #pragma unroll
+    for (int ii = P + 2; ii < 8; ++ii)
+      #pragma unroll
+      for (int cc = 0; cc <= P; ++cc) x[ii][cc] -= lr[ii] * xr[cc];
+  }
+}
+
 __global__ __launch_bounds__(256) void potrf_diag_kernel(float* __restrict__ Ablk, int lda, int nb,
                                                          float* __restrict__ Dinv, PrepScalars* sc) {
-  #pragma clang fp contract(fast)   // a -= l*l as one FMA; nothing here needs op-by-op rounding
-  __shared__ float colbuf[2][NB];  // unscaled column j of A strictly below the diagonal, zero elsewhere
-  __shared__ float rowbuf[2][NB];  // unscaled row j of B
-  __shared__ float pivbuf[2];      // a_jj
+  __shared__ __align__(16) float colbuf[2][NB];  // unscaled column j of A strictly below the diagonal, zero elsewhere
+  __shared__ __align__(16) float rowbuf[2][NB];  // unscaled row j of B up to the diagonal, zero elsewhere
+  __shared__ float pivbuf[2];                    // a_jj
   const int tid = threadIdx.x;
   const int ty = tid >> 4, tx = tid & 15;
   float a[8][8], x[8][8];
@@ -104,72 +196,35 @@ __global__ __launch_bounds__(256) void potrf_diag_kernel(float* __restrict__ Abl
   for (int ii = 0; ii < 8; ++ii)
     #pragma unroll
     for (int cc = 0; cc < 8; ++cc) {
-      const int r = 8 * ty + ii, c = 8 * tx + cc;
+      const int r = ty + 16 * ii, c = tx + 16 * cc;
       a[ii][cc] = (r < nb && c <= r) ? Ablk[(long long)r * lda + c] : ((r == c) ? 1.0f : 0.0f);   // pad with identity
       x[ii][cc] = (r == c) ? 1.0f : 0.0f;
     }
-  bool bad = false;
-  for (int J = 0; J < NB / 8; ++J) {
-    if (8 * J >= nb) break;
-    const bool colowner = (tx == J) && (ty >= J), diag = (tx == J) && (ty == J), rowowner = (ty == J);
+  // column 0 / row 0
+  if (tx == 0) {
     #pragma unroll
-    for (int jj = 0; jj < 8; ++jj) {
-      const int j = 8 * J + jj, pb = jj & 1;
-      if (colowner) {
-        // rows of the diagonal tile up to and including j publish 0, so consumers need no masks
-        #pragma unroll
-        for (int ii = 0; ii < 8; ++ii) colbuf[pb][8 * ty + ii] = (diag && ii <= jj) ? 0.0f : a[ii][jj];
-        if (diag) pivbuf[pb] = a[jj][jj];
-      }
-      if (rowowner) {
-        #pragma unroll
-        for (int cc = 0; cc < 8; ++cc) rowbuf[pb][8 * tx + cc] = x[jj][cc];
-      }
-      __syncthreads();
-      const float pv = pivbuf[pb];
-      bad = bad || !(pv > 0.0f);
-      float rinv = __builtin_amdgcn_rsqf(pv);         // 1/sqrt(pivot), one Newton step to full precision
-      rinv = rinv * (1.5f - 0.5f * pv * rinv * rinv);
-      if (ty >= J) {
-        float li[8];
-        #pragma unroll
-        for (int ii = 0; ii < 8; ++ii) li[ii] = colbuf[pb][8 * ty + ii] * rinv;
-        if (colowner) {                               // the owners keep the scaled column: L[:, j]
-          #pragma unroll
-          for (int ii = 0; ii < 8; ++ii) a[ii][jj] = li[ii];
-          if (diag) a[jj][jj] = pv * rinv;
-        }
-        if (tx >= J && tx <= ty) {                    // trailing update of A (lower tiles only)
-          float lk[8];
-          #pragma unroll
-          for (int cc = 0; cc < 8; ++cc) lk[cc] = colbuf[pb][8 * tx + cc] * rinv;
-          #pragma unroll
-          for (int ii = 0; ii < 8; ++ii)
-            #pragma unroll
-            for (int cc = 0; cc < 8; ++cc) a[ii][cc] -= li[ii] * lk[cc];
-        }
-        if (tx <= J) {                                // row j of X = B[j, :] / l_jj, then rows below j of B
-          float xr[8];
-          #pragma unroll
-          for (int cc = 0; cc < 8; ++cc) xr[cc] = rowbuf[pb][8 * tx + cc] * rinv;
-          if (rowowner) {
-            #pragma unroll
-            for (int cc = 0; cc < 8; ++cc) x[jj][cc] = xr[cc];
-          }
-          #pragma unroll
-          for (int ii = 0; ii < 8; ++ii)
-            #pragma unroll
-            for (int cc = 0; cc < 8; ++cc) x[ii][cc] -= li[ii] * xr[cc];
-        }
-      }
-    }
+    for (int ii = 0; ii < 8; ++ii) colbuf[0][8 * ty + ii] = (ty + 16 * ii > 0) ? a[ii][0] : 0.0f;
+    if (ty == 0) pivbuf[0] = a[0][0];
   }
+  if (ty == 0) {
+    #pragma unroll
+    for (int cc = 0; cc < 8; ++cc) rowbuf[0][8 * tx + cc] = (tx + 16 * cc <= 0) ? x[0][cc] : 0.0f;
+  }
+  bool bad = false;
+  potrf_phase<0>(a, x, colbuf, rowbuf, pivbuf, ty, tx, bad);
+  if (nb > 16) potrf_phase<1>(a, x, colbuf, rowbuf, pivbuf, ty, tx, bad);
+  if (nb > 32) potrf_phase<2>(a, x, colbuf, rowbuf, pivbuf, ty, tx, bad);
+  if (nb > 48) potrf_phase<3>(a, x, colbuf, rowbuf, pivbuf, ty, tx, bad);
+  if (nb > 64) potrf_phase<4>(a, x, colbuf, rowbuf, pivbuf, ty, tx, bad);
+  if (nb > 80) potrf_phase<5>(a, x, colbuf, rowbuf, pivbuf, ty, tx, bad);
+  if (nb > 96) potrf_phase<6>(a, x, colbuf, rowbuf, pivbuf, ty, tx, bad);
+  if (nb > 112) potrf_phase<7>(a, x, colbuf, rowbuf, pivbuf, ty, tx, bad);
   if (bad && tid == 0) sc->status = 1;
   #pragma unroll
   for (int ii = 0; ii < 8; ++ii)
     #pragma unroll
     for (int cc = 0; cc < 8; ++cc) {
-      const int r = 8 * ty + ii, c = 8 * tx + cc;
+      const int r = ty + 16 * ii, c = tx + 16 * cc;
       if (r < nb && c < nb) Ablk[(long long)r * lda + c] = (c <= r) ? a[ii][cc] : 0.0f;
       Dinv[r * NB + c] = (r < nb && c <= r && c < nb) ? x[ii][cc] : 0.0f;
     }

@@ -47,32 +47,35 @@ struct GemmBatch {
   int M[GEMM_MAX_BATCH], N[GEMM_MAX_BATCH], Kc[GEMM_MAX_BATCH];
 };
 
-template <bool B_T>
+template <bool B_T, int TM = GT>
 __device__ __forceinline__ void gemm_tile(const float* A, int lda, const float* B, int ldb,
                                           float* C, int ldc, int M, int N, int Kc, float alpha, float beta,
                                           int flags, int m0, int n0, float* sA, float* sB) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wr = wave >> 1, wc = wave & 1;
+  constexpr int MI = TM / 64;           // 32-row MFMA blocks per wave (waves are 2 x 2 over the TM x 128 tile)
+  constexpr int WM = TM / 2;            // rows per wave
+  constexpr int AP = TM / 32;           // float4 of the A slab per thread
 
   int kb = 0, ke = Kc;
   if (flags & GEMM_K_FROM_N) kb = (n0 / GK) * GK;
-  if (flags & GEMM_K_TO_M) ke = min(Kc, m0 + GT);
+  if (flags & GEMM_K_TO_M) ke = min(Kc, m0 + TM);
 
-  f32x16 acc[2][2];
+  f32x16 acc[MI][2];
   #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MI; ++i)
     #pragma unroll
     for (int j = 0; j < 2; ++j)
       #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
   // staging registers: A tile 128 x 32 floats = 1024 float4 -> 4 per thread; B likewise
-  f32x4 ra[4], rb[4];
+  f32x4 ra[AP], rb[4];
   auto gload = [&](int k0) {
     #pragma unroll
     for (int p = 0; p < 4; ++p) {
       const int idx = p * 256 + tid;
-      {   // A: row = idx / 8, k4 = idx % 8
+      if (p < AP) {   // A: row = idx / 8, k4 = idx % 8
         const int r = idx >> 3, k = k0 + (idx & 7) * 4;
         const int gm = m0 + r;
         f32x4 v = {0.f, 0.f, 0.f, 0.f};
@@ -118,7 +121,7 @@ __device__ __forceinline__ void gemm_tile(const float* A, int lda, const float* 
     #pragma unroll
     for (int p = 0; p < 4; ++p) {
       const int idx = p * 256 + tid;
-      {
+      if (p < AP) {
         const int r = idx >> 3, k = (idx & 7) * 4;
         #pragma unroll
         for (int e = 0; e < 4; ++e) sA[r * GPA + k + e] = ra[p][e];
@@ -143,47 +146,61 @@ __device__ __forceinline__ void gemm_tile(const float* A, int lda, const float* 
     if (k0 + GK < ke) gload(k0 + GK);      // next slab in flight while this one is multiplied
     #pragma unroll
     for (int kk = 0; kk < GK; kk += 2) {
-      float a[2], b[2];
+      float a[MI], b[2];
       #pragma unroll
-      for (int i = 0; i < 2; ++i) a[i] = sA[(wr * 64 + i * 32 + lm) * GPA + kk + lk];
+      for (int i = 0; i < MI; ++i) a[i] = sA[(wr * WM + i * 32 + lm) * GPA + kk + lk];
       #pragma unroll
       for (int j = 0; j < 2; ++j) {
         if constexpr (B_T) b[j] = sB[(wc * 64 + j * 32 + lm) * GPA + kk + lk];
         else b[j] = sB[(kk + lk) * GPB + wc * 64 + j * 32 + lm];
       }
       #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < MI; ++i)
         #pragma unroll
         for (int j = 0; j < 2; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
     }
   }
 
-  // accumulator register r of lane l: row 8*(r/4) + 4*(l/32) + r%4, column l%32
+  // accumulator register r of lane l: row 8*(r/4) + 4*(l/32) + r%4, column l%32.
+  // With beta != 0 all 16 old values of a 32x32 block are fetched before the first store: interleaved, every load
+  // would have to wait behind the store in front of it (they may alias), 64 memory latencies in a row per tile.
   #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MI; ++i)
     #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int gn = n0 + wc * 64 + j * 32 + lm;
+      const int gm0 = m0 + wr * WM + i * 32 + 4 * lk;
+      float* p0 = C + (long long)gm0 * ldc + gn;
+      float old[16];
+      if (beta != 0.0f) {
+        #pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int dm = 8 * (r >> 2) + (r & 3);
+          old[r] = (gm0 + dm < M && gn < N) ? p0[(long long)dm * ldc] : 0.0f;
+        }
+      }
       #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int gm = m0 + wr * 64 + i * 32 + 8 * (r >> 2) + 4 * lk + (r & 3);
-        if (gm < M && gn < N) {
-          float* p = C + (long long)gm * ldc + gn;
+        const int dm = 8 * (r >> 2) + (r & 3);
+        if (gm0 + dm < M && gn < N) {
           const float v = alpha * acc[i][j][r];
-          *p = (beta != 0.0f) ? (beta * *p + v) : v;
+          p0[(long long)dm * ldc] = (beta != 0.0f) ? (beta * old[r] + v) : v;
         }
       }
     }
 }
 
-template <bool B_T>
+// TM = 128 or 64 rows of C per workgroup.  The short tile is for launches that would not give every CU a
+// 128-row tile (rank-128 updates and panel solves of the blocked chains): twice the workgroups, half the serial
+// MFMA work in each.
+template <bool B_T, int TM>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmProblem g, float alpha, float beta, int flags) {
-  __shared__ float sA[GT * GPA];
+  __shared__ float sA[TM * GPA];
   __shared__ float sB[B_T ? GT * GPA : GK * GPB];
-  const int m0 = blockIdx.y * GT, n0 = blockIdx.x * GT;
-  if ((flags & GEMM_LOWER_TILES) && n0 > m0) return;
-  gemm_tile<B_T>(g.A, g.lda, g.B, g.ldb, g.C, g.ldc, g.M, g.N, g.Kc, alpha, beta, flags, m0, n0, sA, sB);
+  const int m0 = blockIdx.y * TM, n0 = blockIdx.x * GT;
+  if ((flags & GEMM_LOWER_TILES) && n0 >= m0 + TM) return;
+  gemm_tile<B_T, TM>(g.A, g.lda, g.B, g.ldb, g.C, g.ldc, g.M, g.N, g.Kc, alpha, beta, flags, m0, n0, sA, sB);
 }
 
 template <bool B_T>
@@ -201,8 +218,11 @@ __global__ __launch_bounds__(256) void gemm_f32_batched_kernel(const float* A, i
 template <bool B_T>
 inline void launch_gemm(const GemmProblem& g, float alpha, float beta, int flags, hipStream_t st) {
   if (g.M <= 0 || g.N <= 0) return;
-  const dim3 grid((unsigned)((g.N + GT - 1) / GT), (unsigned)((g.M + GT - 1) / GT));
-  gemm_f32_kernel<B_T><<<grid, dim3(256), 0, st>>>(g, alpha, beta, flags);
+  const unsigned gx = (unsigned)((g.N + GT - 1) / GT), gy = (unsigned)((g.M + GT - 1) / GT);
+  if ((long long)gx * gy <= 256)
+    gemm_f32_kernel<B_T, 64><<<dim3(gx, (unsigned)((g.M + 63) / 64)), dim3(256), 0, st>>>(g, alpha, beta, flags);
+  else
+    gemm_f32_kernel<B_T, GT><<<dim3(gx, gy), dim3(256), 0, st>>>(g, alpha, beta, flags);
 }
 
 }  // namespace lcq
