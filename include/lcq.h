@@ -105,6 +105,21 @@ int lcq_qparams_int(const void* min_in, const void* max_in, int dtype, int64_t n
 int lcq_mse_range(const void* x, int dtype, int64_t rows, int64_t cols, float qmin, float qmax, int flags, int steps,
                   int grid_n, float norm, float* min_out, float* max_out, void* stream);
 
+/* One iteration of BaseQuantizer.optimize_weights_proximal (the HQQ zero-point solver), quant.py:587-609:
+ *   W_q = clamp(round(x * inv_s + z), qmin, qmax), inv_s = 1/s;  W_r = (W_q - z) / inv_s
+ *   W_e = sign(d) relu(|d| - inv_beta |d|^(lp_norm-1)), d = x - W_r   (lp_norm == 1: |d| - inv_beta; the
+ *   reference's shrink_op reads self.beta, not the annealed beta it is handed, quant.py:94-103)
+ *   zeros_out[r] = mean_c(W_q - (x - W_e) * inv_s);  abs_err_rowsum[r] = sum_c |x - W_r|
+ *  x [rows, cols] fp32 (get_hqq_qparams casts to float first, quant.py:680); scales, zeros_in, zeros_out,
+ *  abs_err_rowsum [rows] fp32; zeros_in NULL = 0 (symmetric start); zeros_out must not alias zeros_in;
+ *  scales_roundtrip [rows] or NULL: 1/(1/s), what the reference returns as scales.
+ *  The caller owns the loop: error = sum(abs_err_rowsum) / (rows*cols), stop at the first iteration that does
+ *  not improve on the best error (the zeros of that iteration are the result). */
+int lcq_hqq_step(const float* x, int64_t rows, int64_t cols, const float* scales, const float* zeros_in, float* zeros_out,
+                 float* abs_err_rowsum, float* scales_roundtrip, float inv_beta, float lp_norm, float qmin, float qmax,
+                 void* stream);
+
+
 /* dequant, quant.py:709-711: out = (q - z) * (s * out_scale_factor). */
 int lcq_dequant_int(const void* q, int dtype, int64_t rows, int64_t cols, const void* scales, const void* zeros,
                     int flags, float out_scale_factor, void* out, void* stream);

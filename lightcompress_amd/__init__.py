@@ -5,4 +5,4 @@ The package is a thin Python mirror of the reference's class API over a C-ABI
 shared library (``liblcq.so``, declared in ``include/lcq.h``) of hand-written
 HIP kernels.  Build it with ``python -m lightcompress_amd.build``.
 """
-from .quant import FloatQuantizer, IntegerQuantizer  # noqa: F401
+from .quant import FloatQuantizer, IntegerQuantizer, Weight48IntegerQuantizer  # noqa: F401

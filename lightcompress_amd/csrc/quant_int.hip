@@ -146,6 +146,47 @@ __global__ __launch_bounds__(256) void mse_range_kernel(const void* __restrict__
   if (lane == 0) { mn_out[row] = cur_min; mx_out[row] = cur_max; }
 }
 
+// One proximal iteration of the HQQ zero-point solver (optimize_weights_proximal, quant.py:587-609):
+//   W_q = clamp(round(x * inv_s + z), qmin, qmax);  W_r = (W_q - z) / inv_s;  W_e = shrink(x - W_r)
+//   z'  = mean(W_q - (x - W_e) * inv_s)  per row;   abs_err = sum |x - W_r|  per row
+// with inv_s = 1 / s and shrink(d) = sign(d) * relu(|d| - inv_beta * |d|^(p-1))  (p == 1: |d| - inv_beta).
+// One pass over x; LANES lanes share a row and combine their partial sums with a DPP butterfly.
+template <int LANES>
+__global__ __launch_bounds__(256) void hqq_step_kernel(const float* __restrict__ x, long long rows, int cols,
+                                                       const float* __restrict__ scales, const float* __restrict__ zeros_in,
+                                                       float* __restrict__ zeros_out, float* __restrict__ abs_err,
+                                                       float* __restrict__ scales_rt, float inv_beta, float p, float qmin,
+                                                       float qmax) {
+  const int lane = threadIdx.x % LANES;
+  const long long row = (long long)blockIdx.x * (256 / LANES) + threadIdx.x / LANES;
+  const bool ok = row < rows;
+  const long long r = ok ? row : 0;
+  const float inv_s = 1.0f / scales[r];
+  const float z = zeros_in ? zeros_in[r] : 0.0f;
+  const float* xr = x + r * cols;
+  float acc_z = 0.0f, acc_e = 0.0f;
+  for (int c = lane; c < cols; c += LANES) {
+    const float v = xr[c];
+    const float wq = __builtin_amdgcn_fmed3f(rintf(v * inv_s + z), qmin, qmax);
+    const float wr = (wq - z) / inv_s;
+    const float d = v - wr;
+    const float ad = fabsf(d);
+    const float thr = (p == 1.0f) ? inv_beta : inv_beta * powf(ad, p - 1.0f);
+    const float mag = fmaxf(ad - thr, 0.0f);
+    const float sgn = (d > 0.0f) ? 1.0f : ((d < 0.0f) ? -1.0f : 0.0f);
+    const float we = sgn * mag;
+    acc_z += wq - (v - we) * inv_s;
+    acc_e += ad;
+  }
+  acc_z = team_sum<LANES>(acc_z);
+  acc_e = team_sum<LANES>(acc_e);
+  if (ok && lane == 0) {
+    zeros_out[row] = acc_z / (float)cols;
+    abs_err[row] = acc_e;
+    if (scales_rt) scales_rt[row] = 1.0f / inv_s;
+  }
+}
+
 }  // namespace
 
 extern "C" {
@@ -187,6 +228,27 @@ int lcq_mse_range(const void* x, int dtype, int64_t rows, int64_t cols, float qm
   if (dtype == LCQ_F32) mse_range_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>(x, rows, cols, steps, grid_n, norm, op, min_out, max_out);
   else if (dtype == LCQ_BF16) mse_range_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>(x, rows, cols, steps, grid_n, norm, op, min_out, max_out);
   else return LCQ_EDTYPE;
+  LCQ_CHECK_LAUNCH();
+  return LCQ_OK;
+}
+
+int lcq_hqq_step(const float* x, int64_t rows, int64_t cols, const float* scales, const float* zeros_in, float* zeros_out,
+                 float* abs_err_rowsum, float* scales_roundtrip, float inv_beta, float lp_norm, float qmin, float qmax,
+                 void* stream) {
+  if (!x || !scales || !zeros_out || !abs_err_rowsum || rows <= 0 || cols <= 0 || cols > 0x7fffffff) return LCQ_EINVAL;
+  if (!(qmax > qmin) || zeros_in == zeros_out) return LCQ_EINVAL;
+  hipStream_t st = (hipStream_t)stream;
+  if (cols <= 256) {
+    const int64_t grid = (rows + 15) / 16;
+    if (grid > 0x7fffffff) return LCQ_EINVAL;
+    hqq_step_kernel<16><<<dim3((unsigned)grid), dim3(256), 0, st>>>(x, rows, (int)cols, scales, zeros_in, zeros_out,
+                                                                     abs_err_rowsum, scales_roundtrip, inv_beta, lp_norm, qmin, qmax);
+  } else {
+    const int64_t grid = (rows + 3) / 4;
+    if (grid > 0x7fffffff) return LCQ_EINVAL;
+    hqq_step_kernel<64><<<dim3((unsigned)grid), dim3(256), 0, st>>>(x, rows, (int)cols, scales, zeros_in, zeros_out,
+                                                                     abs_err_rowsum, scales_roundtrip, inv_beta, lp_norm, qmin, qmax);
+  }
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;
 }

@@ -39,6 +39,11 @@ class BaseQuantizer(object):
         self.mse_b_num = self.kwargs.get('mse_b_num', 1)
         self.maxshrink = self.kwargs.get('maxshrink', 0.8)
         self.mse_grid = self.kwargs.get('mse_grid', 100)
+        # hqq config (quant.py:89-93)
+        self.lp_norm = self.kwargs.get('lp_norm', 0.7)
+        self.beta = self.kwargs.get('beta', 10)
+        self.kappa = self.kwargs.get('kappa', 1.01)
+        self.iters = self.kwargs.get('iters', 20)
         if self.granularity == 'per_group':
             self.group_size = self.kwargs['group_size']
         elif self.granularity == 'per_head':
@@ -59,7 +64,10 @@ class BaseQuantizer(object):
             return self.get_minmax_range(tensor)
         if self.calib_algo == 'mse':
             return self.get_mse_range(tensor)
-        raise NotImplementedError(f'calib_algo={self.calib_algo!r}: minmax and mse run on liblcq')
+        if self.calib_algo == 'learnable':
+            raise NotImplementedError("calib_algo='learnable' (sigmoid-scaled clipping, quant.py:207-221) belongs to the "
+                                      'gradient-trained methods; this path has no autograd')
+        return self.get_minmax_range(tensor)                 # quant.py:131-132: anything else falls back to minmax
 
     def get_mse_range(self, tensor, norm=2.4, bs=256):
         """quant.py:147-205 -> fp32 (min_val, max_val) [rows, 1]: the shrunken range with the smallest
@@ -120,6 +128,124 @@ class BaseQuantizer(object):
                                         L.i32(flags), L.ptr(scales),
                                         L.ptr(None if self.sym else zeros), L.stream()), 'lcq_qparams_int')
         return scales, zeros, qmax, qmin
+
+    # -- static activation calibration (quant.py:105-124, 223-262, 523-585) -------------------
+    def reshape_batch_tensors(self, act_tensors):
+        """quant.py:105-124: calibration inputs -> list (one entry per module input) of lists of tensors."""
+        assert len(act_tensors) > 0, (
+            'Calibration data is insufficient. Please provide more data to ensure '
+            'all experts in the MOE receive an adequate number of tokens.'
+        )
+        if isinstance(act_tensors[0], tuple):
+            act_tensors = [torch.stack(tensor_list) for tensor_list in zip(*act_tensors)]
+        elif len(act_tensors) == 1:
+            act_tensors[0] = [act_tensors[0][i] for i in range(act_tensors[0].size(0))]
+        else:
+            act_tensors = [act_tensors]
+        return act_tensors
+
+    def get_minmax_stats(self, act_tensors):
+        """quant.py:223-250: per input, the stacked fp32 CPU ranges of every calibration tensor (range kernels on
+        the GPU; like the reference the handful of scalars is collected on the host)."""
+        stats_min_max = {}
+        for input_idx, tensors in enumerate(act_tensors):
+            mins, maxs = [], []
+            for tensor in tensors:
+                lo, hi = self.get_minmax_range(self.reshape_tensor(tensor))
+                mins.append(lo.detach().cpu().to(torch.float32).unsqueeze(0))
+                maxs.append(hi.detach().cpu().to(torch.float32).unsqueeze(0))
+            stats_min_max[input_idx] = {'min': torch.cat(mins), 'max': torch.cat(maxs)}
+        return stats_min_max
+
+    def get_static_minmax_range(self, act_tensors):
+        """quant.py:252-262: mean of the per-tensor ranges."""
+        stats = self.get_minmax_stats(self.reshape_batch_tensors(act_tensors))
+        min_vals = [r['min'].mean(dim=0) for r in stats.values()]
+        max_vals = [r['max'].mean(dim=0) for r in stats.values()]
+        return min_vals, max_vals
+
+    def get_static_moving_minmax_range(self, act_tensors, alpha):
+        """quant.py:523-542: exponential moving average of the per-tensor ranges, in the tensors' dtype."""
+        act_tensors = self.reshape_batch_tensors(act_tensors)
+        moving_min_vals, moving_max_vals = [], []
+        for tensors in act_tensors:
+            moving_min_val, moving_max_val = None, None
+            for tensor in tensors:
+                min_val, max_val = self.get_minmax_range(self.reshape_tensor(tensor))
+                if moving_min_val is None or moving_max_val is None:
+                    moving_min_val, moving_max_val = min_val, max_val
+                else:
+                    moving_min_val = moving_min_val + alpha * (min_val - moving_min_val)
+                    moving_max_val = moving_max_val + alpha * (max_val - moving_max_val)
+            moving_min_vals.append(moving_min_val)
+            moving_max_vals.append(moving_max_val)
+        return moving_min_vals, moving_max_vals
+
+    def get_batch_tensors_qparams(self, act_tensors, alpha=0.01, args={}):
+        """quant.py:559-585 -> (scales_list, zeros_list, qmin_list, qmax_list), one entry per module input."""
+        if self.calib_algo == 'static_hist':
+            raise NotImplementedError("calib_algo='static_hist' (the histogram observer, quant.py:264-521) is host-side "
+                                      'search code outside this path; static_minmax and static_moving_minmax run on liblcq')
+        elif self.calib_algo == 'static_minmax':
+            min_vals, max_vals = self.get_static_minmax_range(act_tensors)
+        elif self.calib_algo == 'static_moving_minmax':
+            min_vals, max_vals = self.get_static_moving_minmax_range(act_tensors, alpha)
+        else:
+            raise ValueError(f'Unsupported calibration algorithm: {self.calib_algo}')
+        scales_list, zeros_list, qmin_list, qmax_list = [], [], [], []
+        for min_val, max_val in zip(min_vals, max_vals):
+            dev = min_val.device if min_val.is_cuda else torch.device('cuda', torch.cuda.current_device())
+            scales, zeros, qmax, qmin = self.get_qparams((min_val.to(dev), max_val.to(dev)), dev)
+            if not min_val.is_cuda:                          # host statistics give host qparams, as in the reference
+                scales, qmax, qmin = scales.cpu(), qmax.cpu(), qmin.cpu()
+                zeros = zeros.cpu()
+            scales_list.append(scales)
+            zeros_list.append(zeros)
+            qmin_list.append(qmin)
+            qmax_list.append(qmax)
+        return scales_list, zeros_list, qmin_list, qmax_list
+
+    # -- HQQ (quant.py:587-609) -----------------------------------------------------------------
+    def optimize_weights_proximal(self, tensor, scales, zeros, qmax, qmin):
+        """Half-quadratic zero-point refinement: every iteration is one fused pass (lcq_hqq_step) where the
+        reference runs about a dozen elementwise kernels; the loop and its early stop stay on the host, with the
+        same one scalar read-back per iteration."""
+        t = tensor.contiguous()
+        if t.dtype != torch.float32 or t.dim() != 2:
+            raise NotImplementedError('optimize_weights_proximal runs on the 2-D fp32 tensor get_hqq_qparams builds')
+        rows, cols = t.shape
+        s = scales.to(device=t.device, dtype=torch.float32).reshape(-1).contiguous()
+        if s.numel() != rows:
+            raise NotImplementedError('hqq needs one scale per row (per_channel / per_group)')
+        z_in = None if _is_cpu_zero(zeros) else zeros.to(device=t.device, dtype=torch.float32).reshape(-1).contiguous()
+        bufs = [torch.empty(rows, dtype=torch.float32, device=t.device) for _ in range(2)]
+        err_rows = torch.empty(rows, dtype=torch.float32, device=t.device)
+        scales_rt = torch.empty(rows, dtype=torch.float32, device=t.device)
+        best_error = 1e4
+        z_cur = z_in
+        for i in range(self.iters):
+            z_out = bufs[i & 1]
+            L.check(L.lib().lcq_hqq_step(L.ptr(t), L.i64(rows), L.i64(cols), L.ptr(s), L.ptr(z_cur), L.ptr(z_out),
+                                         L.ptr(err_rows), L.ptr(scales_rt), L.f32(1.0 / self.beta), L.f32(self.lp_norm),
+                                         L.f32(float(qmin)), L.f32(float(qmax)), L.stream()), 'lcq_hqq_step')
+            z_cur = z_out
+            current_error = float(err_rows.sum()) / t.numel()
+            if current_error < best_error:
+                best_error = current_error
+            else:
+                break
+        if z_cur is None:                                    # iters == 0
+            z_cur = torch.zeros(rows, dtype=torch.float32, device=t.device) if z_in is None else z_in
+            scales_rt = 1 / (1 / s)
+        return scales_rt.view(rows, 1), z_cur.view(rows, 1)
+
+    def get_hqq_qparams(self, tensor, args):
+        """quant.py:679-687."""
+        tensor = self.reshape_tensor(tensor.float())
+        tensor_range = self.get_minmax_range(tensor)
+        scales, zeros, qmax, qmin = self.get_qparams(tensor_range, tensor.device)
+        best_scales, best_zeros = self.optimize_weights_proximal(tensor, scales, zeros, qmax, qmin)
+        return tensor, best_scales, best_zeros, qmax, qmin
 
     # -- views (quant.py:611-657); torch view ops only ----------------------
     def reshape_tensor(self, tensor, allow_padding=False):
@@ -275,6 +401,8 @@ class IntegerQuantizer(BaseQuantizer):
     # -- reference API ----------------------------------------------------------
     def get_tensor_qparams(self, tensor, args={}):
         """quant.py:689-696 -> (tensor_reshaped, scales, zeros, qmax, qmin)."""
+        if self.calib_algo == 'hqq':
+            return self.get_hqq_qparams(tensor, args)
         tensor = self.reshape_tensor(tensor)
         if self.calib_algo != 'minmax':
             scales, zeros, qmax, qmin = self.get_qparams(self.get_tensor_range(tensor, args), tensor.device)
@@ -758,6 +886,87 @@ class FloatQuantizer(BaseQuantizer):
 
 
 # -- quant.py:20-45 of the reference: the block-wise float8 casts it uses where its Triton kernels do not run ----
+class Weight48IntegerQuantizer(BaseQuantizer):
+    """quant.py:1230-1367: weights to 8-bit integers, those integers to 4-bit integers (second-level
+    scales / zero points optionally confined to an integer range), and back.  Both levels run on the
+    integer quantizer's kernels: range -> lcq_minmax_rows, qparams -> lcq_qparams_int, codes kept in the
+    tensor's dtype -> lcq_quant_int, back -> lcq_dequant_int."""
+
+    def __init__(self, bit, bit4, bit8, **kwargs):
+        super().__init__(bit, None, None, **kwargs)
+        self.quant_type = 'int-quant-w48'
+        assert self.bit == 48, 'Only support 48-bit quantization'
+        self.bit_settings = {4: bit4, 8: bit8}
+        self._stage = {}
+        for b, cfg in self.bit_settings.items():
+            if 'zeros_bit' in cfg:
+                raise NotImplementedError('zeros_bit: zero points outside [qmin, qmax] are not on this path')
+            extra = {k: cfg[k] for k in ('int_range', 'group_size') if k in cfg}
+            q = IntegerQuantizer(b, cfg['symmetric'], cfg.get('granularity'), **extra)
+            self._stage[b] = q
+            cfg['qmin'], cfg['qmax'] = q.qmin, q.qmax
+            if 'scales_bit' in cfg:
+                n = cfg['scales_bit']
+                cfg['scales_qmin'] = -(2 ** (n - 1)) if cfg['scales_symmetric'] else 0
+                cfg['scales_qmax'] = 2 ** (n - 1) - 1 if cfg['scales_symmetric'] else 2 ** n - 1
+            else:
+                cfg['scales_qmin'], cfg['scales_qmax'] = -torch.inf, torch.inf
+            cfg['zeros_qmin'], cfg['zeros_qmax'] = cfg['qmin'], cfg['qmax']
+
+    def reshape_tensor(self, tensor, bit=4):
+        cfg = self.bit_settings[bit]
+        if cfg.get('granularity') == 'per_group':
+            group_size = cfg.get('group_size')
+            if tensor.shape[-1] % group_size != 0:
+                raise ValueError(f'Dimension {tensor.shape[-1]} not divisible by group size {group_size}')
+            return tensor.reshape(-1, group_size)
+        return tensor
+
+    def get_minmax_range(self, tensor):
+        cols = tensor.shape[-1]
+        t = tensor.contiguous()
+        mn = torch.empty((*t.shape[:-1], 1), dtype=t.dtype, device=t.device)
+        mx = torch.empty_like(mn)
+        L.check(L.lib().lcq_minmax_rows(L.ptr(t), L.dtype_code(t.dtype), L.i64(t.numel() // cols), L.i64(cols),
+                                        L.ptr(mn), L.ptr(mx), L.stream()), 'lcq_minmax_rows')
+        return (mn, mx)
+
+    def get_qparams(self, tensor_range, device, bit):
+        cfg = self.bit_settings[bit]
+        scales, zeros, qmax, qmin = self._stage[bit].get_qparams(tensor_range, device)
+        if 'scales_bit' in cfg:                                   # a clamp of [rows, 1] parameters
+            scales = scales.clamp(cfg['scales_qmin'], cfg['scales_qmax'])
+        return scales, zeros, qmax, qmin
+
+    def quant(self, tensor, scales, zeros, qmax, qmin):
+        return self._stage[4].quant(tensor, scales, zeros, qmax, qmin)
+
+    def dequant(self, tensor, scales, zeros):
+        return self._stage[4].dequant(tensor, scales, zeros)
+
+    def quant_dequant(self, tensor, scales, zeros, qmax, qmin):
+        return self.dequant(self.quant(tensor, scales, zeros, qmax, qmin), scales, zeros)
+
+    def fake_quant_weight_dynamic(self, weight, args={}):
+        org_shape16, org_dtype16 = weight.shape, weight.dtype
+        # 16 -> 8 bit
+        weight = self.reshape_tensor(weight, bit=8)
+        scales816, zeros816, qmax816, qmin816 = self.get_qparams(self.get_tensor_range(weight), weight.device, bit=8)
+        weight = self.quant(weight, scales816, zeros816, qmax816, qmin816)
+        # 8 -> 4 bit
+        org_shape8, org_dtype8 = weight.shape, weight.dtype
+        weight = self.reshape_tensor(weight, bit=4)
+        scales48, zeros48, qmax48, qmin48 = self.get_qparams(self.get_tensor_range(weight), weight.device, bit=4)
+        weight = self.quant(weight, scales48, zeros48, qmax48, qmin48)
+        # 4 -> 8 -> 16 bit
+        weight = self.restore_tensor(self.dequant(weight, scales48, zeros48), org_shape8).to(org_dtype8)
+        weight = self.restore_tensor(self.dequant(weight, scales816, zeros816), org_shape16).to(org_dtype16)
+        return weight
+
+    def restore_tensor(self, tensor, shape):
+        return tensor.reshape(shape) if tensor.shape != shape else tensor
+
+
 def weight_cast_to_bf16(weight, scale, block_size):
     """float8 block-wise weight -> bf16: FloatQuantizer('e4m3', per_block).dequant(weight.float(), scale, 0)."""
     from .kernel import _block_dequant

@@ -468,3 +468,130 @@ def int_mse_range(spec, tensor: torch.Tensor, norm=2.4, maxshrink=0.8, mse_grid=
                 best_max_val[tmp] = xmax[tmp]
         min_val[b_num * bs:(b_num + 1) * bs, :], max_val[b_num * bs:(b_num + 1) * bs, :] = best_min_val, best_max_val
     return min_val, max_val
+
+
+# ----------------------------------------------------------------------------
+# HQQ zero-point refinement   (quant.py:94-103, 587-609, 679-687)
+# ----------------------------------------------------------------------------
+def hqq_shrink(x: torch.Tensor, beta_ctor: float, lp_norm: float) -> torch.Tensor:
+    """shrink_op, quant.py:94-103.  Both lambdas read self.beta (the constructor value): the annealed beta the
+    solver hands them is ignored."""
+    if lp_norm == 1:
+        return torch.sign(x) * torch.nn.functional.relu(torch.abs(x) - 1.0 / beta_ctor)
+    return torch.sign(x) * torch.nn.functional.relu(
+        torch.abs(x) - (1.0 / beta_ctor) * torch.pow(torch.abs(x), lp_norm - 1))
+
+
+def hqq_optimize(tensor, scales, zeros, qmax, qmin, lp_norm=0.7, beta=10, kappa=1.01, iters=20):
+    """optimize_weights_proximal, quant.py:587-609 -> (scales, zeros, iterations run)."""
+    best_error = 1e4
+    current_beta = beta
+    scales = 1 / scales
+    n_run = 0
+    for i in range(iters):
+        n_run += 1
+        W_q = torch.round(tensor * scales + zeros).clamp(qmin, qmax)
+        W_r = (W_q - zeros) / scales
+        W_e = hqq_shrink(tensor - W_r, beta, lp_norm)
+        zeros = torch.mean(W_q - (tensor - W_e) * scales, axis=-1, keepdim=True)
+        current_beta *= kappa
+        current_error = float(torch.abs(tensor - W_r).mean())
+        if current_error < best_error:
+            best_error = current_error
+        else:
+            break
+    scales = 1 / scales
+    return scales, zeros, n_run
+
+
+def int_hqq_qparams(spec, t: torch.Tensor, **hqq):
+    """get_hqq_qparams, quant.py:679-687 -> (rows fp32, scales, zeros, qmax, qmin)."""
+    rows = reshape_rows(spec, t.float())
+    lo, hi = minmax_range(spec, rows)
+    s, z, qmax, qmin = int_qparams(spec, lo, hi)
+    s, z, _ = hqq_optimize(rows, s, z, qmax, qmin, **hqq)
+    return rows, s, z, qmax, qmin
+
+
+# ----------------------------------------------------------------------------
+# static activation calibration   (quant.py:105-124, 223-262, 523-585)
+# ----------------------------------------------------------------------------
+def _batch_lists(act_tensors):
+    if isinstance(act_tensors[0], tuple):
+        return [torch.stack(ts) for ts in zip(*act_tensors)]
+    if len(act_tensors) == 1:
+        return [[act_tensors[0][i] for i in range(act_tensors[0].size(0))]]
+    return [act_tensors]
+
+
+def static_minmax_ranges(spec, act_tensors):
+    """get_static_minmax_range, quant.py:252-262: fp32 mean of the per-tensor ranges, per module input."""
+    mins, maxs = [], []
+    for tensors in _batch_lists(act_tensors):
+        lo = torch.stack([minmax_range(spec, reshape_rows(spec, t))[0].float() for t in tensors])
+        hi = torch.stack([minmax_range(spec, reshape_rows(spec, t))[1].float() for t in tensors])
+        mins.append(lo.mean(dim=0))
+        maxs.append(hi.mean(dim=0))
+    return mins, maxs
+
+
+def static_moving_minmax_ranges(spec, act_tensors, alpha):
+    """get_static_moving_minmax_range, quant.py:523-542."""
+    mins, maxs = [], []
+    for tensors in _batch_lists(act_tensors):
+        m_lo = m_hi = None
+        for t in tensors:
+            lo, hi = minmax_range(spec, reshape_rows(spec, t))
+            if m_lo is None:
+                m_lo, m_hi = lo, hi
+            else:
+                m_lo = m_lo + alpha * (lo - m_lo)
+                m_hi = m_hi + alpha * (hi - m_hi)
+        mins.append(m_lo)
+        maxs.append(m_hi)
+    return mins, maxs
+
+
+# ----------------------------------------------------------------------------
+# Weight48IntegerQuantizer   (quant.py:1230-1367)
+# ----------------------------------------------------------------------------
+def w48_fake_quant(w: torch.Tensor, bit4: dict, bit8: dict) -> torch.Tensor:
+    """fake_quant_weight_dynamic, quant.py:1338-1367: 16 -> 8 -> 4 -> 8 -> 16 bit.  Settings: symmetric,
+    granularity ('per_group' + group_size, else rows as they are), int_range, scales_bit + scales_symmetric."""
+    def bounds(cfg, bit):
+        if 'int_range' in cfg:
+            return torch.tensor(cfg['int_range'][0]), torch.tensor(cfg['int_range'][1])
+        if cfg['symmetric']:
+            return torch.tensor(-(2 ** (bit - 1))), torch.tensor(2 ** (bit - 1) - 1)
+        return torch.tensor(0), torch.tensor(2 ** bit - 1)
+
+    def rows_of(t, cfg):
+        return t.reshape(-1, cfg['group_size']) if cfg.get('granularity') == 'per_group' else t
+
+    def qparams(t, cfg, bit):
+        qmin, qmax = bounds(cfg, bit)
+        lo, hi = t.amin(dim=-1, keepdim=True), t.amax(dim=-1, keepdim=True)
+        if cfg['symmetric']:
+            scales = torch.max(hi.abs(), lo.abs()).clamp(min=1e-5) / qmax
+            zeros = torch.tensor(0.0)
+        else:
+            scales = (hi - lo).clamp(min=1e-5) / (qmax - qmin)
+            zeros = qmin - torch.round(lo / scales)
+        if 'scales_bit' in cfg:
+            n = cfg['scales_bit']
+            s_lo, s_hi = (-(2 ** (n - 1)), 2 ** (n - 1) - 1) if cfg['scales_symmetric'] else (0, 2 ** n - 1)
+            scales = scales.clamp(s_lo, s_hi)
+        zeros = zeros.clamp(qmin, qmax)
+        return scales, zeros, qmax, qmin
+
+    shape16, dtype16 = w.shape, w.dtype
+    t = rows_of(w, bit8)
+    s8, z8, qmax8, qmin8 = qparams(t, bit8, 8)
+    t = torch.clamp(torch.round(t / s8) + z8, qmin8, qmax8)
+    shape8, dtype8 = t.shape, t.dtype
+    t = rows_of(t, bit4)
+    s4, z4, qmax4, qmin4 = qparams(t, bit4, 4)
+    t = torch.clamp(torch.round(t / s4) + z4, qmin4, qmax4)
+    t = ((t - z4) * s4).reshape(shape8).to(dtype8)
+    t = ((t - z8) * s8).reshape(shape16).to(dtype16)
+    return t

@@ -403,3 +403,96 @@ def test_mse_range_oracle_recurrence_and_optimality():
         assert abs(float(lo) - float(mn[r])) <= 1e-6 * abs(float(lo)) and abs(float(hi) - float(mx[r])) <= 1e-6 * abs(float(hi))
         assert float(mn[r]) >= float(row.min()) and float(mx[r]) <= float(row.max())
         assert err_of(row, mn[r], mx[r]) <= err_of(row, row.min(), row.max()) * (1 + 1e-6)
+
+
+# ---- secondary calibrators: HQQ, static activation ranges, W4-over-W8 ---------------------------------------
+def test_hqq_shrink_is_the_soft_threshold_and_fixed_points_hold():
+    """Pins for hqq_optimize (quant.py:587-609) that do not restate it:
+    * lp_norm = 1: shrink is the proximal map of |y|/beta, i.e. argmin_y |y|/beta + (y-x)^2/2, found here by
+      brute force over a fine grid of y;
+    * values that already lie on the quantization grid are reproduced exactly: the error is 0 in the first
+      iteration, the second one cannot improve on it and stops the loop, and the zero points do not move;
+    * with shrink = identity (lp_norm 1, beta -> inf) the update is z <- mean(W_q - W_r/s) = z for any input;
+    * the returned scales are 1/(1/s), not s."""
+    xs = torch.tensor([-1.0, -0.26, -0.05, 0.0, 0.07, 0.3, 2.0])
+    got = Q.hqq_shrink(xs, 4.0, 1)
+    ys = torch.linspace(-3, 3, 600001, dtype=torch.float64)
+    for x, g in zip(xs.tolist(), got.tolist()):
+        obj = ys.abs() / 4.0 + (ys - x) ** 2 / 2
+        assert abs(float(ys[obj.argmin()]) - g) < 2e-5
+    # p < 1: threshold |x| - |x|^(p-1)/beta, zero where that is negative (and at x = 0, where |x|^(p-1) = inf)
+    got = Q.hqq_shrink(torch.tensor([0.0, 1e-3, -0.5, 4.0]), 10, 0.7)
+    want = [0.0, 0.0, -(0.5 - 0.1 * 0.5 ** -0.3), 4.0 - 0.1 * 4.0 ** -0.3]
+    assert torch.allclose(got, torch.tensor(want), rtol=1e-6, atol=0)
+
+    s = torch.tensor([[0.25], [0.5]])
+    z0 = torch.tensor([[3.0], [7.0]])
+    k = torch.tensor([[0., 5, 15, 9, 1, 3, 12, 8], [2., 2, 14, 0, 15, 7, 7, 11]])
+    x = (k - z0) * s
+    s1, z1, n = Q.hqq_optimize(x, s, z0, torch.tensor(15), torch.tensor(0.0))
+    assert n == 2 and torch.equal(z1, z0) and torch.equal(s1, s)
+    w = torch.randn(6, 64, generator=gen(3))
+    spec = Q.IntSpec(4, False, 'per_channel')
+    lo, hi = Q.minmax_range(spec, w)
+    s, z, qmax, qmin = Q.int_qparams(spec, lo, hi)
+    _, z1, _ = Q.hqq_optimize(w, s, z, qmax, qmin, lp_norm=1, beta=1e30, iters=1)
+    assert float((z1 - z).abs().max()) < 1e-4
+    one = np.float32(1)
+    sv = next(v for v in np.arange(0.01, 1.0, 0.013, dtype=np.float32) if one / (one / v) != v)
+    sr, _, _ = Q.hqq_optimize(torch.ones(1, 4), torch.tensor([[float(sv)]]), torch.zeros(1, 1), qmax, qmin, iters=1)
+    assert np.float32(sr.item()) == one / (one / sv) and np.float32(sr.item()) != sv
+
+
+def test_static_activation_ranges_known_answers():
+    """get_static_minmax_range / get_static_moving_minmax_range (quant.py:252-262, 523-542) on inputs whose ranges
+    are known by construction."""
+    spec = Q.IntSpec(8, True, 'per_tensor')
+    ts = [torch.tensor([[-1.0, 2.0], [0.5, 0.0]]), torch.tensor([[-3.0, 1.0], [4.0, 0.0]]), torch.tensor([[0.0, 6.0], [-2.0, 1.0]])]
+    lo, hi = Q.static_minmax_ranges(spec, list(ts))
+    assert len(lo) == 1 and lo[0].item() == -2.0 and hi[0].item() == 4.0
+    lo, hi = Q.static_moving_minmax_ranges(spec, list(ts), 1.0)          # alpha 1: the last tensor
+    assert lo[0].item() == -2.0 and hi[0].item() == 6.0
+    lo, hi = Q.static_moving_minmax_ranges(spec, list(ts), 0.0)          # alpha 0: the first tensor
+    assert lo[0].item() == -1.0 and hi[0].item() == 2.0
+    lo, hi = Q.static_moving_minmax_ranges(spec, list(ts), 0.5)          # ((2+4)/2 + 6)/2
+    assert hi[0].item() == 4.5 and lo[0].item() == -2.0
+    # one stacked tensor = a batch of samples (quant.py:117-120); tuples = several module inputs (:112-115)
+    lo, hi = Q.static_minmax_ranges(spec, [torch.stack(ts)])
+    assert lo[0].item() == -2.0 and hi[0].item() == 4.0
+    lo, hi = Q.static_minmax_ranges(spec, [(ts[0], ts[1]), (ts[2], ts[0])])
+    assert len(lo) == 2 and hi[0].item() == 4.0 and hi[1].item() == 3.0
+    # per_token ranges keep their shape
+    spec_t = Q.IntSpec(8, True, 'per_token')
+    lo, hi = Q.static_minmax_ranges(spec_t, list(ts))
+    assert lo[0].shape == (2, 1) and hi[0].flatten().tolist() == [3.0, float(np.float32(5.5) / np.float32(3))]   # (2,1,6)/3, (.5,4,1)/3
+
+
+def test_w48_known_answers():
+    """Weight48IntegerQuantizer.fake_quant_weight_dynamic (quant.py:1338-1367).
+    * Lossless case: weights c*m with integer m, |m| <= 127 and max |m| = 127 give 8-bit codes m; if every group of
+      the codes spans exactly 15 with its minimum in [-15, 0], the 4-bit level has scale 1 and zero -min: the
+      output is the input.
+    * scales_bit clamps the second-level scale AFTER the zero point was computed from the unclamped one (hand
+      computed below)."""
+    c = 2.0 ** -6
+    m = torch.tensor([[-15., 0, -7, -3], [127., 112, 120, 115], [-4., 11, 0, 5], [-127., -112, -120, -125]])
+    w = (m * c).reshape(2, 8)                                   # rows [g0 g1], [g2 g3]; row maxima 127
+    b8 = dict(symmetric=True, granularity='per_channel')
+    b4 = dict(symmetric=False, granularity='per_group', group_size=4)
+    out = Q.w48_fake_quant(w, b4, b8)
+    # group 1 (112..127) and group 3 (-127..-112) have minima outside [-15, 0]: their zero points clamp and the
+    # codes saturate, so only groups 0 and 2 are lossless
+    assert torch.equal(out.reshape(4, 4)[0], w.reshape(4, 4)[0]) and torch.equal(out.reshape(4, 4)[2], w.reshape(4, 4)[2])
+    assert torch.equal(out.reshape(4, 4)[1], torch.tensor([15., 15, 15, 15]) * c)       # z=0, codes clamp to 15
+    # z = clamp(0 - round(-127), 0, 15) = 15 -> codes clamp(m + 15, 0, 15) = 0 -> (0 - 15) * 1
+    assert torch.equal(out.reshape(4, 4)[3], torch.tensor([-15., -15, -15, -15]) * c)
+    # range 30 -> scale 2, zero = -round(-30/2) = 15; scales_bit=1 (unsigned) clamps the scale to 1:
+    # codes clamp(round(m/1) + 15, 0, 15), back (code - 15) * 1
+    m2 = torch.tensor([[-30., -16, -15, -1, 0, -8, -127, 127]])
+    w2 = m2 * c
+    b4c = dict(symmetric=False, granularity='per_group', group_size=4, scales_bit=1, scales_symmetric=False)
+    out2 = Q.w48_fake_quant(w2, b4c, b8)
+    assert torch.equal(out2[0, :4], torch.tensor([-15., -15, -15, -1]) * c)
+    # bf16 weights: the 8-bit codes are held in bf16 (integers up to 127 are exact there)
+    out3 = Q.w48_fake_quant(w.bfloat16(), b4, b8)
+    assert out3.dtype == torch.bfloat16 and torch.equal(out3.float().reshape(4, 4)[0], w.reshape(4, 4)[0])
