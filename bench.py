@@ -37,8 +37,8 @@ NB, TOK = 128, 2048
 # HBM-side bytes per launch of the two roofline kernels: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this script,
 # scaled by the same counters' reading for a copy kernel of known size (profiles/hessian_kernel_K14336_T8192.md,
 # profiles/rtn_quant_int4_g128_4096x4096_f32.md).  Counters cannot be read from inside the timed process.
-HESSIAN_TRAFFIC_BYTES = 6.861e9
-RTN_TRAFFIC_BYTES = 1.518e8
+HESSIAN_TRAFFIC_BYTES = 6.890e9
+RTN_TRAFFIC_BYTES = 1.501e8
 CFG = {'weight': dict(bit=4, symmetric=False, granularity='per_group', group_size=128),
        'special': dict(actorder=True, static_groups=False, percdamp=0.01, blocksize=128, true_sequential=True)}
 
