@@ -78,7 +78,7 @@ def process_hessian_and_weights(weight: torch.Tensor, H: torch.Tensor, percdamp:
 # ---------------------------------------------------------------------------
 # lazy-batch column loop   (gptq.py:198-244)
 # ---------------------------------------------------------------------------
-def weight_transform(W, Hinv, spec, blocksize=128, static_qparams=None):
+def weight_transform(W, Hinv, spec, blocksize=128, static_qparams=None, static_groups=None):
     """Runs the loop in place on W (as the reference does) and returns
     (tmp, Losses, groups) where groups is the list of per-group
     (scale [R,1], zero [R,1]|0-dim) refreshed at every group boundary.
@@ -86,6 +86,9 @@ def weight_transform(W, Hinv, spec, blocksize=128, static_qparams=None):
     ``spec`` is an oracle IntSpec (per_group or per_channel).  For
     per_channel, ``static_qparams=(scale, zero)`` are the fixed row
     parameters the reference takes from the layer's RTN buffers.
+    ``static_groups=(scales [R,G], zeros [R,G] | None, perm | None)``: per_group with
+    ``static_groups: True`` - the RTN parameters of the ORIGINAL column order, looked up as
+    ``groups[perm[idx] // g]`` (gptq.py:143-148, 224-227); nothing is refreshed.
     """
     R, K = W.shape
     Losses = torch.zeros_like(W)
@@ -102,7 +105,14 @@ def weight_transform(W, Hinv, spec, blocksize=128, static_qparams=None):
         tmp1, Err1, Losses1 = torch.zeros_like(W1), torch.zeros_like(W1), torch.zeros_like(W1)
         for i in range(count):
             w, d = W1[:, i], Hinv1[i, i]
-            if per_group and (i1 + i) % spec.group_size == 0:
+            if per_group and static_groups is not None:
+                sg, zg, perm = static_groups
+                idx = i1 + i
+                if perm is not None:
+                    idx = int(perm[idx])
+                scale = sg[:, idx // spec.group_size].unsqueeze(1)
+                zero = torch.tensor(0.0) if zg is None else zg[:, idx // spec.group_size].unsqueeze(1)
+            elif per_group and (i1 + i) % spec.group_size == 0:
                 cols = W[:, (i1 + i): min(i1 + i + spec.group_size, K)]      # W, not W1 (gptq.py:216-222)
                 _, scale, zero, qmax, qmin = Q.int_tensor_qparams(spec, cols)
                 groups.append((scale.clone(), zero.clone()))

@@ -172,7 +172,8 @@ def _loop_case(R, K, g, blocksize, sym, seed):
 
 
 @pytest.mark.parametrize('R,K,g,bs,sym', [(64, 512, 128, 128, False), (40, 512, 128, 128, True), (32, 512, 64, 128, False),
-                                           (32, 512, 256, 128, False), (48, 384, 128, 64, False), (16, 328, 128, 128, False)])
+                                           (32, 512, 256, 128, False), (48, 384, 128, 64, False), (16, 328, 128, 128, False),
+                                           (32, 400, 100, 128, False)])     # groups that open inside an octet / a block
 def test_column_loop_against_oracle(dev, R, K, g, bs, sym):
     spec, W0, W, U = _loop_case(R, K, g, bs, sym, 5000 + K + g)
     tmp_o, Loss_o, groups = G.weight_transform(W.clone(), U, spec, blocksize=bs)
@@ -212,6 +213,41 @@ def test_per_channel_static_loop(dev):
     tmp, Losses = torch.zeros_like(Wd), torch.zeros_like(Wd)
     gp.weight_transform(Wd, U.to(dev).contiguous(), Losses, tmp)
     assert float((tmp.cpu() - tmp_o).abs().max()) < 1e-4 * float(tmp_o.abs().max())
+
+
+@pytest.mark.parametrize('actorder', [False, True])
+@pytest.mark.parametrize('sym', [False, True])
+def test_static_groups_loop(dev, actorder, sym):
+    """static_groups: True (gptq.py:143-148, 224-227): the loop takes the RTN group parameters of the original
+    column order, found through the act-order permutation, and refreshes nothing."""
+    R, K, g = 48, 512, 64
+    H = G.hessian_closed_form(calib_batches(6, 256, K, seed=9100)).float()
+    W0 = torch.randn(R, K, generator=gen(9101)) * 0.02
+    spec = Q.IntSpec(4, sym, 'per_group', group_size=g)
+    _, s0, z0, _, _ = Q.int_tensor_qparams(spec, W0)
+    perm = G.act_order(H) if actorder else None
+    W, U, _ = G.process_hessian_and_weights(W0, H, 0.01, perm)
+    sg = s0.reshape(R, K // g)
+    zg = None if sym else z0.reshape(R, K // g)
+    tmp_o, Loss_o, _ = G.weight_transform(W.clone(), U, spec, static_groups=(sg, zg, perm))
+    gp = make_gptq(actorder=actorder, static_groups=True, weight=dict(bit=4, symmetric=sym, granularity='per_group', group_size=g))
+    gp.n_nonout = gp.columns = K
+    if actorder:
+        gp.perm = perm.to(dev)
+    layer = types.SimpleNamespace(buf_scales=s0.to(dev), buf_zeros=None if sym else z0.to(dev))
+    gp._setup_groups(layer, R, K)
+    Wd = W.clone().to(dev)
+    tmp, Losses = torch.zeros_like(Wd), torch.zeros_like(Wd)
+    gp.weight_transform(Wd, U.to(dev).contiguous(), Losses, tmp)
+    tmp, Losses = tmp.cpu(), Losses.cpu()
+    assert float((tmp - tmp_o).abs().max()) < 1e-4 * float(tmp_o.abs().max())
+    cols = perm if actorder else torch.arange(K)
+    s_col = sg[:, cols // g]
+    z_col = torch.zeros_like(s_col) if sym else zg[:, cols // g]
+    code = lambda t: torch.clamp(torch.round(t / s_col) + z_col, spec.qmin, spec.qmax)
+    agree = float((code(tmp) == code(tmp_o)).float().mean())
+    assert agree >= 0.999, agree
+    assert abs(float(Losses.sum()) - float(Loss_o.sum())) <= 1e-3 * float(Loss_o.sum())
 
 
 @pytest.mark.parametrize('actorder', [False, True])

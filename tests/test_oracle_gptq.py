@@ -120,6 +120,26 @@ def test_identity_hessian_reduces_to_rtn():
     assert torch.allclose(Losses, (W0 - fq) ** 2 / 2)
 
 
+def test_static_groups_look_up_the_original_columns_group():
+    """static_groups (gptq.py:143-148, 224-227): with an identity Hinv nothing propagates, so column j of the
+    permuted loop must be quantized exactly like column perm[j] of plain RTN on the original order - a lookup by the
+    permuted position, or a refresh at group boundaries, fails this."""
+    R, K, g = 6, 256, 64
+    spec = Q.IntSpec(4, False, 'per_group', group_size=g)
+    W0 = torch.randn(R, K, generator=gen(16)) * 0.02
+    W0[:, 64:128] *= 5                                           # groups with clearly different scales
+    _, s0, z0, _, _ = Q.int_tensor_qparams(spec, W0)
+    sg, zg = s0.reshape(R, K // g), z0.reshape(R, K // g)
+    fq = Q.int_fake_quant_dynamic(spec, W0)
+    perm = torch.randperm(K, generator=gen(17))
+    for p in (None, perm):
+        Wp = W0 if p is None else W0[:, p]
+        tmp, Losses, groups = G.weight_transform(Wp.clone(), torch.eye(K), spec, static_groups=(sg, zg, p))
+        assert groups == [] and torch.equal(tmp, Wp)
+        want = fq if p is None else fq[:, p]
+        assert torch.allclose(Losses, (Wp - want) ** 2 / 2, rtol=0, atol=0)
+
+
 def test_actorder_and_layer_driver_roundtrip():
     R, K = 8, 256
     spec = Q.IntSpec(4, False, 'per_group', group_size=128)
