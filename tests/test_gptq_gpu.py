@@ -113,7 +113,7 @@ def _chain_inputs(K, seed, dead=()):
 
 
 @pytest.mark.parametrize('K,actorder,dead', [(128, False, ()), (256, True, (5,)), (384, False, ()), (1000, True, (0, 999)),
-                                             (2048, True, ())])
+                                             (2048, True, ()), (3000, False, (7,))])
 def test_cholesky_chain(dev, K, actorder, dead):
     from lightcompress_amd import _lib as L
     H = _chain_inputs(K, 4000 + K, dead)
