@@ -17,8 +17,10 @@ What changes under the API
   * the inspect-module forward itself (library GEMMs) is whatever the caller
     passes; the O(K) scale arithmetic (pow / clamp / normalise) uses torch ops
     on the [K] vector like the reference;
-  * one process / one GPU: no all_reduce / broadcast of the winner; GQA
-    (prev_op = v_proj feeding o_proj with repeated heads) is not carried over.
+  * one process / one GPU: no all_reduce / broadcast of the winner;
+  * GQA (``is_gqa``: v_proj feeding o_proj, base_blockwise_quantization.py:281-295, 614-618): the scales have
+    one entry per key/value channel and are repeated per query group before they meet o_proj's columns;
+    ``set_model_config`` takes the three sizes from a config object instead of ``self.model``.
 """
 from __future__ import annotations
 
@@ -51,10 +53,31 @@ class Awq:
 
     # -- awq.py:39-46 -----------------------------------------------------------
     @torch.no_grad()
+    def set_model_config(self, model_config=None):
+        """base_blockwise_quantization.py:281-295; ``model_config`` defaults to ``self.model.model_config``."""
+        cfg = model_config if model_config is not None else self.model.model_config
+        self.hidden_size = cfg.hidden_size
+        self.num_heads = cfg.num_attention_heads
+        self.head_dim = self.hidden_size // self.num_heads
+        if hasattr(cfg, 'intermediate_size'):
+            self.intermediate_size = cfg.intermediate_size
+        if hasattr(cfg, 'num_key_value_heads'):
+            self.num_key_value_heads = cfg.num_key_value_heads
+            self.num_key_value_groups = self.num_heads // self.num_key_value_heads
+            self.has_gqa = self.num_key_value_groups > 1
+        else:
+            self.has_gqa = False
+
+    @torch.no_grad()
+    def repeat_gqa_scales(self, scales):
+        """base_blockwise_quantization.py:614-618: [kv_heads * head_dim] -> [1, heads, head_dim] (index plumbing on a
+        vector of K values)."""
+        scales = scales.view(1, self.num_key_value_heads, self.head_dim)
+        return torch.repeat_interleave(scales, dim=1, repeats=self.num_key_value_groups)
+
     def scaling_weight(self, w, scales, is_gqa):
-        if is_gqa:
-            raise NotImplementedError('GQA scale repetition is not on this path')
-        w.mul_(scales.view(1, -1))
+        scales_tmp = self.repeat_gqa_scales(scales) if is_gqa else scales
+        w.mul_(scales_tmp.view(1, -1))
         return w
 
     # -- awq.py:48-72 -------------------------------------------------------------
@@ -98,10 +121,16 @@ class Awq:
     # -- awq.py:87-108 -----------------------------------------------------------------
     @torch.no_grad()
     def get_scales(self, prev_op, x, w_max, is_gqa, ratio, x_mean=None):
-        if is_gqa:
-            raise NotImplementedError('GQA scale search is not on this path')
-        x_tmp = self.get_act_scale(x) if x_mean is None else x_mean
-        if self.trans_version == 'v1':
+        """``x_mean``: mean|x| computed earlier (of ``prev_op(x)`` when is_gqa), so that the grid does not redo it."""
+        if x_mean is not None:
+            x_tmp = x_mean
+        elif is_gqa:
+            # statistics of v_proj's OUTPUT (its forward is the caller's library GEMM); the reference also calls
+            # get_weight_scale on v_proj here and never uses the result (awq.py:90-91, 104-105)
+            x_tmp = self.get_act_scale(prev_op(x))
+        else:
+            x_tmp = self.get_act_scale(x)
+        if self.trans_version == 'v1' and not is_gqa:
             scales = (x_tmp.pow(ratio) / w_max.pow(1 - ratio)).clamp(min=1e-4).view(-1)
         else:
             scales = x_tmp.pow(ratio).clamp(min=1e-4).view(-1)
@@ -168,7 +197,7 @@ class Awq:
 
     def fake_quantize_weight(self, fc, scales, is_gqa, layer_name):
         if is_gqa:
-            raise NotImplementedError('GQA scale search is not on this path')
+            scales = self.repeat_gqa_scales(scales).reshape(-1)
         fc.weight.data = self._scale_quant(fc.weight.data, scales)
         return fc.weight
 
@@ -181,7 +210,7 @@ class Awq:
     @torch.no_grad()
     def scaling_input(self, x, scales, is_gqa):
         if is_gqa:
-            raise NotImplementedError('GQA scale search is not on this path')
+            scales = self.repeat_gqa_scales(scales).reshape(-1)
         K = x.shape[-1]
         x2 = x.contiguous()
         s = scales.to(x.dtype).contiguous()
@@ -214,12 +243,13 @@ class Awq:
                 kwargs = subset_kwargs[i] if isinstance(subset_kwargs, list) else (subset_kwargs or {})
                 if i not in org_out_dict:
                     org_out_dict[i] = self.get_original_out(x, inspect_module, kwargs)
-                    x_mean_dict[i] = self.get_act_scale(x)
+                    x_mean_dict[i] = self.get_act_scale(prev_op(x) if is_gqa else x)
                 org_out = org_out_dict[i]
                 ratio = n * 1 / n_grid
                 scales = self.get_scales(prev_op, x, w_max, is_gqa, ratio, x_mean=x_mean_dict[i])
+                col_scales = self.repeat_gqa_scales(scales).reshape(-1) if is_gqa else scales
                 for layer_name, fc in layers_dict.items():
-                    fc.weight.data = self._scale_quant(originals[layer_name], scales)
+                    fc.weight.data = self._scale_quant(originals[layer_name], col_scales)
                 x_tmp = self.scaling_input(x, scales, is_gqa)
                 if not self.w_only:
                     x_tmp = self.fake_quantize_input(x_tmp, layers_dict)

@@ -54,20 +54,32 @@ def loss(org_out, out):
     return (org_out - out).float().pow(2).mean().item()
 
 
-def search_scale(weights: dict, x, forward, spec, n_grid=20, version='v2'):
-    """-> (best_scales, losses per grid point).  `forward(x, weights_dict)` is the inspect module."""
+def repeat_gqa(scales, kv_heads, head_dim, groups):
+    """repeat_gqa_scales, base_blockwise_quantization.py:614-618 -> flat [kv_heads * groups * head_dim]."""
+    return torch.repeat_interleave(scales.view(1, kv_heads, head_dim), dim=1, repeats=groups).reshape(-1)
+
+
+def search_scale(weights: dict, x, forward, spec, n_grid=20, version='v2', gqa=None):
+    """-> (best_scales, losses per grid point).  `forward(x, weights_dict)` is the inspect module.
+    ``gqa=(prev_op, kv_heads, head_dim, groups)``: awq.py:88-93, 104-105 with is_gqa - the scales come from the
+    statistics of prev_op(x) in the v2 form and are repeated per query group before they meet the columns."""
     w_max = weight_scale(list(weights.values()), spec) if spec.granularity == 'per_group' else None
     org_out = forward(x, weights)
     best_err, best_scales, losses = float('inf'), None, []
     for n in range(n_grid):
         ratio = n * 1 / n_grid
-        s = get_scales(x, w_max, ratio, version)
+        if gqa is not None:
+            prev_op, kvh, hd, groups = gqa
+            s_kv = get_scales(prev_op(x), None, ratio, 'v2')
+            s = repeat_gqa(s_kv, kvh, hd, groups)
+        else:
+            s = s_kv = get_scales(x, w_max, ratio, version)
         wq = {k: scale_and_fake_quant(w, s, spec) for k, w in weights.items()}
         out = forward(scaling_input(x, s), wq)
         l = loss(org_out, out)
         losses.append(l)
         if l < best_err:
-            best_err, best_scales = l, s
+            best_err, best_scales = l, s_kv
     return best_scales, losses
 
 

@@ -95,6 +95,43 @@ def test_search_scale_subset_picks_the_oracle_ratio(dev, dtype):
     assert torch.equal(layers['gate'].weight.data.cpu(), w['gate'])
 
 
+def test_search_scale_subset_gqa(dev):
+    """v_proj -> o_proj with grouped query heads (is_gqa): scales from mean|v_proj(x)|, repeated per group."""
+    dtype = torch.bfloat16
+    kvh, hd, groups = 2, 64, 4                                    # o_proj sees 8 heads x 64 = 512 columns
+    K = kvh * groups * hd
+    g = gen(31)
+    x = (torch.randn(2, 128, K, generator=g) * torch.exp(0.5 * torch.randn(K, generator=g))).to(dtype)
+    wo = (torch.randn(384, K, generator=g) * 0.02).to(dtype)
+    wv = (torch.randn(kvh * hd, K, generator=g) * 0.05).to(dtype)
+    spec = Q.IntSpec(4, False, 'per_group', group_size=128)
+    fwd = lambda xx, ww: xx @ ww['o'].t()
+    best_o, losses_o = A.search_scale({'o': wo}, x, fwd, spec, gqa=(lambda t: t @ wv.t(), kvh, hd, groups))
+    awq = make_awq()
+    awq.set_model_config(types.SimpleNamespace(hidden_size=K, num_attention_heads=kvh * groups, num_key_value_heads=kvh))
+    assert awq.has_gqa and awq.head_dim == hd and awq.num_key_value_groups == groups
+    layers = {'o': Fc(wo.to(dev))}
+    wvd = wv.to(dev)
+    best = awq.search_scale_subset(lambda t: t @ wvd.t(), layers, [x.to(dev)], lambda xx: xx @ layers['o'].weight.data.t(), True, {})
+    losses = awq.search_losses.cpu()
+    assert best.shape == (kvh * hd,) and best.dtype == dtype
+    rel = ((losses.double() - torch.tensor(losses_o).double()).abs() / torch.tensor(losses_o).double()).max()
+    assert float(rel) < 0.05, float(rel)
+    ko, kg = min(range(20), key=lambda i: losses_o[i]), int(torch.argmin(losses))
+    assert kg == ko or abs(losses_o[kg] - losses_o[ko]) <= 0.02 * losses_o[ko]
+    if kg == ko:
+        assert float((best.cpu().float() - best_o.float()).abs().max()) <= 2 ** -6 * float(best_o.float().abs().max())
+    # the pieces, bit for bit: repeated scales on the weight and on the input
+    s_kv = best_o
+    rep = A.repeat_gqa(s_kv, kvh, hd, groups)
+    assert_bit_equal(awq.scaling_input(x.to(dev), s_kv.to(dev), True), A.scaling_input(x, rep), 'x / repeated scales')
+    fc = Fc(wo.to(dev).clone())
+    assert_bit_equal(awq.fake_quantize_weight(fc, s_kv.to(dev), True, 'o').data, A.scale_and_fake_quant(wo, rep, spec),
+                     'W * repeated scales -> fake quant')
+    w2 = wo.to(dev).clone()
+    assert_bit_equal(awq.scaling_weight(w2, s_kv.to(dev), True), wo * rep.view(1, -1), 'scaling_weight')
+
+
 # ---- AutoClipper (auto_clip.py) ---------------------------------------------------------------------
 @pytest.mark.parametrize('clip_sym,sym', [(False, False), (True, False), (False, True)])
 @pytest.mark.parametrize('R,K,T', [(64, 256, 96), (320, 512, 512), (256, 128, 700)])

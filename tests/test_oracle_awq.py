@@ -145,3 +145,29 @@ def test_auto_clip_oracle_known_optima():
     # apply_clip: the weight is clamped group-wise into the found range
     cl = A.apply_clip_v1(w, bmin, bmax)
     assert torch.equal(cl, w)
+
+
+def test_gqa_search_reduces_to_the_plain_search_and_repeats_per_group():
+    """is_gqa (awq.py:88-93, 104-105; base_blockwise_quantization.py:614-618).
+    * The repeated vector indexes the key/value channel of every query channel: column c of o_proj belongs to query
+      head c // head_dim, which shares key/value head (c // head_dim) // groups (written out as a loop here).
+    * With one query head per key/value head and an identity v_proj the GQA search is the plain v2 search."""
+    kvh, hd, groups = 3, 4, 2
+    s = torch.arange(kvh * hd, dtype=torch.float32) + 1
+    rep = A.repeat_gqa(s, kvh, hd, groups)
+    want = [float(s[((c // hd) // groups) * hd + c % hd]) for c in range(kvh * groups * hd)]
+    assert rep.tolist() == want
+
+    x, w, down = tiny_case(torch.float32, seed=21, T=32, K=256, I=128)
+    spec = Q.IntSpec(4, False, 'per_group', group_size=128)
+    fwd = lambda xx, ww: xx @ ww['o'].t()
+    weights = {'o': w['gate']}
+    best, losses = A.search_scale(weights, x, fwd, spec)
+    best_g, losses_g = A.search_scale(weights, x, fwd, spec, gqa=(lambda t: t, 4, 64, 1))
+    assert losses == losses_g and torch.equal(best, best_g)
+    # genuinely grouped: 2 key/value heads serve 4 query heads; the result has one entry per key/value channel and
+    # the search still returns a minimum of its own losses
+    v = torch.randn(128, 256, generator=gen(22)) * 0.05
+    best_g, losses_g = A.search_scale(weights, x, fwd, spec, gqa=(lambda t: t @ v.t(), 2, 64, 2))
+    assert best_g.shape == (128,) and abs(float(best_g.max() * best_g.min()) - 1) < 1e-5
+    assert losses_g[0] == losses[0]                               # ratio 0: all-ones scales either way
