@@ -6,8 +6,8 @@ base_blockwise_quantization.py of ModelTC/LightCompress) that AWQ-style methods 
 (:613-617), ``scaling_input`` (:899-912) and ``update_input_feat`` (:914-920).  Use it as a mix-in in front of
 the reference's class, or stand-alone.
 
-Not on this path (``NotImplementedError``): fused QKV linears (``fc1.out_features == 3 * fc2.in_features``) and
-float8 block-wise checkpoints (``weight_scale_inv``).
+Float8 block-wise checkpoints (``weight_scale_inv``) go through the block-wise casts of ``kernel.py``: cast to bf16,
+scale, cast back, like the reference (:690-699, 711-720).
 """
 from __future__ import annotations
 
@@ -20,8 +20,6 @@ _MUL_COLS, _DIV_COLS, _MUL_ROWS, _DIV_ROWS = 0, 1, 2, 3
 
 def _scale_(t, s, mode):
     """In place: t (* or /) s along columns (mode 0 / 1) or rows (2 / 3); t [T, K] or [K]."""
-    if t.dtype == torch.float8_e4m3fn:
-        raise NotImplementedError('float8 block-wise weights are not on this path')
     x = t.data
     if not x.is_contiguous():
         raise L.LcqError('in-place scaling needs a contiguous tensor')
@@ -33,12 +31,22 @@ def _scale_(t, s, mode):
     return t
 
 
+def _scale_fp8_(fc, scales, mode, block_size):
+    """A float8 block-wise weight: bf16 <- weight * weight_scale_inv, scale, back to float8 with fresh block scales."""
+    from .kernel import weight_cast_to_bf16, weight_cast_to_fp8
+    tmp = weight_cast_to_bf16(fc.weight.data, fc.weight_scale_inv, block_size).to(torch.bfloat16)
+    _scale_(tmp, scales, mode)
+    fc.weight.data, fc.weight_scale_inv.data = weight_cast_to_fp8(tmp, block_size)
+
+
 class ScaleFolding:
     """Expects, where GQA is used, ``num_key_value_heads``, ``head_dim``, ``num_key_value_groups``, ``has_gqa`` and
-    ``do_gqa_trans`` on ``self`` like the reference's class."""
+    ``do_gqa_trans`` on ``self`` like the reference's class; for fused QKV linears ``model.get_num_attention_heads()``
+    or ``num_heads``; for float8 checkpoints ``fp8_block_size``."""
 
     has_gqa = False
     do_gqa_trans = False
+    fp8_block_size = 128
 
     @torch.no_grad()
     def repeat_gqa_scales(self, scales):
@@ -61,7 +69,20 @@ class ScaleFolding:
         scales = scales.to(fc1.weight.device)
         has_bias = getattr(fc1, 'bias', None) is not None
         if fc1.out_features == fc2.in_features * 3:
-            raise NotImplementedError('fused QKV linears are not on this path')
+            # fused QKV laid out [head][q, k, v][head_dim] along the output channels (:648-676): only the value rows
+            # are divided, row (h, 2, d) by scales[h * head_dim + d]; per head they are one contiguous block
+            model = getattr(self, 'model', None)
+            num_heads = model.get_num_attention_heads() if model is not None else self.num_heads
+            w = fc1.weight.data
+            hd = w.shape[0] // (3 * num_heads)
+            blocks = w.view(num_heads, 3, hd, w.shape[1])
+            sv = scales.view(num_heads, hd)
+            for h in range(num_heads):
+                _scale_(blocks[h, 2], sv[h], _DIV_ROWS)
+            if has_bias:
+                b = fc1.bias.data.view(num_heads, 3, hd)
+                for h in range(num_heads):
+                    _scale_(b[h, 2], sv[h], _DIV_COLS)
         elif fc1.out_features == fc2.in_features * 2:
             half = fc1.weight.data.shape[0] // 2
             _scale_(fc1.weight.data[half:], scales, _DIV_ROWS)
@@ -70,7 +91,10 @@ class ScaleFolding:
         elif fc1.out_features == fc2.in_features:
             if has_bias:
                 _scale_(fc1.bias, scales, _DIV_COLS)
-            _scale_(fc1.weight, scales, _DIV_ROWS)
+            if fc1.weight.data.dtype == torch.float8_e4m3fn:
+                _scale_fp8_(fc1, scales, _DIV_ROWS, self.fp8_block_size)
+            else:
+                _scale_(fc1.weight, scales, _DIV_ROWS)
         elif self.has_gqa and self.do_gqa_trans:
             if has_bias:
                 _scale_(fc1.bias, scales, _DIV_COLS)
@@ -79,7 +103,10 @@ class ScaleFolding:
                 scales = self.repeat_gqa_scales(scales)
         else:
             raise Exception('Can not scale this fc-fc.')
-        _scale_(fc2.weight, scales, _MUL_COLS)
+        if fc2.weight.data.dtype == torch.float8_e4m3fn:
+            _scale_fp8_(fc2, scales, _MUL_COLS, self.fp8_block_size)
+        else:
+            _scale_(fc2.weight, scales, _MUL_COLS)
 
     @torch.no_grad()
     def scale_ln_fcs(self, ln, fcs, scales):
@@ -90,12 +117,15 @@ class ScaleFolding:
         if getattr(ln, 'bias', None) is not None:
             _scale_(ln.bias, scales, _DIV_COLS)
         for fc in fcs:
-            _scale_(fc.weight, scales, _MUL_COLS)
+            if fc.weight.data.dtype == torch.float8_e4m3fn:
+                _scale_fp8_(fc, scales, _MUL_COLS, self.fp8_block_size)
+            else:
+                _scale_(fc.weight, scales, _MUL_COLS)
         for p in ln.parameters():
             assert torch.isnan(p).sum() == 0
         for fc in fcs:
             for p in fc.parameters():
-                assert torch.isnan(p).sum() == 0
+                assert torch.isnan(p.float() if p.dtype == torch.float8_e4m3fn else p).sum() == 0
 
     @torch.no_grad()
     def scaling_input(self, x, scales, is_gqa):

@@ -234,5 +234,59 @@ def test_scale_folding_matches_the_torch_op_sequence(dev, dtype):
     feat = {'a': [x[:2].to(dev), x[2:].to(dev)]}
     sf.update_input_feat(s.to(dev), feat, {'a': None}, False)
     assert_bit_equal(torch.cat(feat['a']), x / s.view(1, -1), 'scaled inputs')
-    with pytest.raises(NotImplementedError):
-        sf.scale_fc_fc(lin(K, 3 * I, False, 50).to(dev), lin(I, K, False, 51).to(dev), s2.to(dev))
+    # fused QKV, output channels laid out [head][q, k, v][head_dim] (:648-676): the reference's transposed reshapes,
+    # written here as an index loop - only value rows change, row (h, 2, d) by scales[h * hd + d]
+    heads, hd = 6, I // 6
+    sf.num_heads = heads
+    fc1, fc2 = lin(K, 3 * I, True, 50), lin(I, K, False, 51)
+    w1, b1, w2 = fc1.weight.data.clone(), fc1.bias.data.clone(), fc2.weight.data.clone()
+    for h in range(heads):
+        for d in range(hd):
+            o = (h * 3 + 2) * hd + d
+            w1[o] = w1[o] / s2[h * hd + d]
+            b1[o] = b1[o] / s2[h * hd + d]
+    w2 = w2 * s2.view(1, -1)
+    f1, f2 = fc1.to(dev), fc2.to(dev)
+    sf.scale_fc_fc(f1, f2, s2.to(dev))
+    assert_bit_equal(f1.weight.data, w1, 'fused qkv weight'); assert_bit_equal(f1.bias.data, b1, 'fused qkv bias')
+    assert_bit_equal(f2.weight.data, w2, 'fc2 after fused qkv')
+
+
+def test_scale_folding_float8_blockwise_weights(dev):
+    """Float8 block-wise checkpoints (:690-699, 711-720, 786-793): bf16 <- weight * weight_scale_inv, scale, cast back.
+    Oracle = the block-wise cast oracles around the literal bf16 torch op."""
+    from lightcompress_amd.blockwise import ScaleFolding
+    sf = ScaleFolding()
+    K, I = 256, 384
+    s = (torch.rand(I, generator=gen(61)) + 0.5).bfloat16()
+    class Fp8Linear(torch.nn.Module):
+        def __init__(self, i, o, seed):
+            super().__init__()
+            w = (torch.randn(o, i, generator=gen(seed)) * 0.05).bfloat16()
+            y, sc = Q.triton_weight_cast_to_fp8(w)
+            self.in_features, self.out_features, self.bias = i, o, None
+            self.weight = torch.nn.Parameter(y, requires_grad=False)
+            self.weight_scale_inv = torch.nn.Parameter(sc, requires_grad=False)
+    fp8_linear = Fp8Linear
+    to_dev = lambda m: m.to(dev)
+    fc1, fc2 = fp8_linear(K, I, 70), fp8_linear(I, K, 71)
+    t1 = Q.triton_weight_cast_to_bf16(fc1.weight.data, fc1.weight_scale_inv.data).to(torch.bfloat16)
+    t1.div_(s.view(-1, 1))
+    w1, sc1 = Q.triton_weight_cast_to_fp8(t1)
+    t2 = Q.triton_weight_cast_to_bf16(fc2.weight.data, fc2.weight_scale_inv.data).to(torch.bfloat16)
+    t2.mul_(s.view(1, -1))
+    w2, sc2 = Q.triton_weight_cast_to_fp8(t2)
+    ln = torch.nn.LayerNorm(I, dtype=torch.bfloat16)
+    fc3 = fp8_linear(I, K, 72)
+    t3 = Q.triton_weight_cast_to_bf16(fc3.weight.data, fc3.weight_scale_inv.data).to(torch.bfloat16)
+    t3.mul_(s.view(1, -1))
+    w3, sc3 = Q.triton_weight_cast_to_fp8(t3)
+    f1, f2, f3 = to_dev(fc1), to_dev(fc2), to_dev(fc3)
+    sf.scale_ln_fcs(ln.to(dev), [f3], s.to(dev))
+    assert_bit_equal(f3.weight.data.view(torch.uint8), w3.view(torch.uint8), 'ln -> float8 fc codes')
+    assert_bit_equal(f3.weight_scale_inv.data, sc3, 'ln -> float8 fc block scales')
+    sf.scale_fc_fc(f1, f2, s.to(dev))
+    assert_bit_equal(f1.weight.data.view(torch.uint8), w1.view(torch.uint8), 'fc1 float8 codes')
+    assert_bit_equal(f1.weight_scale_inv.data, sc1, 'fc1 block scales')
+    assert_bit_equal(f2.weight.data.view(torch.uint8), w2.view(torch.uint8), 'fc2 float8 codes')
+    assert_bit_equal(f2.weight_scale_inv.data, sc2, 'fc2 block scales')
