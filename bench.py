@@ -89,15 +89,18 @@ def gpu_main(args):
                 for n in subset:                       # every Linear's hook fires on every batch
                     gp.add_batch(layers[n], n, xb, None)
             e1 = ev(); e1.record()
-            for n in subset:
-                gp.initialize_qparams_and_prepare_weights(layers[n], n)
-                a = ev(); a.record()
-                W, U = gp.process_hessian_and_weights(layers[n], n)
-                b_ = ev(); b_.record()
-                gp.update_layer_with_transformed_weights(layers[n], W, U, n)
-                c = ev(); c.record()
-                gp.free(n)
-                marks.append(('chain_ms', a, b_)); marks.append(('loop_ms', b_, c))
+            if record is None:
+                gp.subset_transform(sub)               # the reference's driver of a subset (gptq.py:96-112)
+            else:                                      # same work one Linear at a time, with events between the phases
+                for n in subset:
+                    gp.initialize_qparams_and_prepare_weights(layers[n], n)
+                    a = ev(); a.record()
+                    W, U = gp.process_hessian_and_weights(layers[n], n)
+                    b_ = ev(); b_.record()
+                    gp.update_layer_with_transformed_weights(layers[n], W, U, n)
+                    c = ev(); c.record()
+                    gp.free(n)
+                    marks.append(('chain_ms', a, b_)); marks.append(('loop_ms', b_, c))
             marks.append(('hessian_ms', e0, e1))
         torch.cuda.synchronize()
         if record is not None:
@@ -110,11 +113,14 @@ def gpu_main(args):
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        one_layer(False, phases)
+        one_layer(False)
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / args.steps
+    # where the time goes: one more pass, one Linear at a time with events between the phases (untimed; the chains of
+    # a subset run one after the other here, in the timed pass subset_transform starts them side by side)
+    one_layer(False, phases)
     for k in phases:
-        phases[k] = round(phases[k] / args.steps, 3)
+        phases[k] = round(phases[k], 3)
 
     # same layer with one Hessian / one chain per distinct input stream (q,k,v and gate,up share)
     one_layer(True)

@@ -65,6 +65,8 @@ class GPTQ:
         self.check_positive_definite = special_config.get('check_positive_definite', True)
         # add_batch calls folded into one Hessian launch (1 = one launch per call)
         self.hessian_defer = int(special_config.get('hessian_defer', 4))
+        # subset_transform starts the Cholesky chains of all Linears of a subset side by side (False: one by one)
+        self.chain_overlap = bool(special_config.get('chain_overlap', True))
         if self.owq:
             raise NotImplementedError('OWQ is not on this path')
         if self.blocksize > 128:
@@ -195,9 +197,50 @@ class GPTQ:
     @torch.no_grad()
     def subset_transform(self, subset, input_feat=None, subset_kwargs=None):
         layers_dict = subset['layers']
+        self._chains_ahead(layers_dict)
         for name in layers_dict:
             self.layer_transform(layers_dict[name], name)
             self.free(name)
+
+    def _chains_ahead(self, layers_dict):
+        """Start the Cholesky chain of every Linear of the subset now, each on its own stream.  A chain at K = 4096 is
+        a few hundred short dependent launches (diagonal blocks, panel solves) that leave most of the chip idle, so
+        the chains of q/k/v (or gate/up) run in about the time of one.  layer_transform then finds the finished factor
+        exactly as it finds a shared one; results are the same as one by one."""
+        if not self.chain_overlap:
+            return
+        todo = []
+        for name in layers_dict:
+            cache = self.layers_cache.get(name)
+            if cache is None or 'H' not in cache:
+                continue
+            leader = cache.get('leader', name)
+            if leader in self._shared or leader in todo:
+                continue
+            todo.append(leader)
+        if len(todo) < 2:
+            return
+        if not hasattr(self, '_side_streams'):
+            self._side_streams = [torch.cuda.Stream(device=self.dev) for _ in range(3)]
+        main = torch.cuda.current_stream()
+        for i, leader in enumerate(todo):
+            H = self._settle(leader)['H']
+            K = H.shape[0]
+            perm = torch.argsort(torch.diag(H), descending=True) if self.actorder else None
+            dead = torch.diag(H) == 0
+            ws_bytes = L.lib().lcq_chol_inv_upper_workspace_bytes(L.i64(K))
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=self.dev)
+            status = torch.zeros(1, dtype=torch.int32, device=self.dev)
+            side = self._side_streams[i % len(self._side_streams)]
+            side.wait_stream(main)
+            with torch.cuda.stream(side):
+                L.check(L.lib().lcq_chol_inv_upper(L.ptr(H), L.i64(K), L.ptr(perm), L.f32(self.percdamp), L.ptr(None),
+                                                   L.i64(0), L.ptr(H), L.ptr(ws), L.i64(ws_bytes), L.ptr(status),
+                                                   L.stream()), 'lcq_chol_inv_upper')
+                done = side.record_event()
+            ws.record_stream(side)                       # freed below, reusable only after the chain has run
+            del ws
+            self._shared[leader] = dict(U=H, perm=perm, status=status, dead=dead, done=done, ahead=True)
 
     @torch.no_grad()
     def layer_transform(self, layer, name):
@@ -249,6 +292,8 @@ class GPTQ:
             if is_shared:
                 self._shared[leader] = shared
         else:
+            if 'done' in shared:                             # started by _chains_ahead on another stream
+                torch.cuda.current_stream().wait_event(shared.pop('done'))
             W.masked_fill_(shared['dead'].unsqueeze(0), 0.0)
         U = shared['U']
         self._status = shared['status']

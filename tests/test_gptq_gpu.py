@@ -320,3 +320,32 @@ def test_shared_hessian_matches_separate(dev):
         outs.append((la.weight.data.cpu(), lb.weight.data.cpu(), lb.buf_scales.cpu()))
     for x, y in zip(*outs):
         assert torch.equal(x, y)
+
+
+@pytest.mark.parametrize('actorder', [False, True])
+def test_chains_side_by_side_match_one_by_one(dev, actorder):
+    """subset_transform starts the Cholesky chains of a subset on separate streams (chain_overlap, the default); the
+    weights, scales and losses must be those of the one-by-one order, bit for bit, also with a dead column and with
+    Linears of different input widths in one subset."""
+    R = 48
+    Ks = {'a': 1536, 'b': 1536, 'c': 640}
+    xs = {K: calib_batches(4, 96, K, seed=8100 + K) for K in set(Ks.values())}
+    for K in xs:
+        for x in xs[K]:
+            x[:, 7] = 0                                           # a dead column
+    Ws = {n: (torch.randn(R, K, generator=gen(8200 + i)) * 0.02).bfloat16() for i, (n, K) in enumerate(Ks.items())}
+    outs = []
+    for overlap in (False, True):
+        gp = make_gptq(actorder=actorder, chain_overlap=overlap)
+        layers = {n: Layer(Ws[n].to(dev)) for n in Ks}
+        gp.subset_init({'layers': layers})
+        for j in range(4):
+            for n, K in Ks.items():
+                gp.add_batch(layers[n], n, xs[K][j].unsqueeze(0).bfloat16().to(dev))
+        gp.subset_transform({'layers': layers})
+        torch.cuda.synchronize()
+        assert gp._shared == {}
+        outs.append([t for n in Ks for t in (layers[n].weight.data.cpu(), layers[n].buf_scales.cpu(), layers[n].buf_zeros.cpu())]
+                    + [gp.last_error.cpu()])
+    for x, y in zip(*outs):
+        assert torch.equal(x, y)
