@@ -190,6 +190,13 @@ int lcq_hessian_accum(float* H, int64_t K, const void* X, int dtype, int64_t T, 
 /* H[j][i] = H[i][j] for i < j. */
 int lcq_symmetrize(float* H, int64_t K, void* stream);
 
+/* The weight side of GPTQ.process_hessian_and_weights, gptq.py:133-141, 150-151, in one pass:
+ *   W = weight.clone().float(); W[:, dead] = 0; W = W[:, perm]
+ *  w [R,K] fp32 / bf16 / fp16; perm [K] int64 or NULL; dead [K] bytes (non-zero = dead column, indexed in the
+ *  ORIGINAL column order) or NULL; out [R,K] fp32, must not alias w. */
+int lcq_gptq_prepare_weights(const void* w, int dtype, int64_t R, int64_t K, const int64_t* perm, const uint8_t* dead,
+                             float* out, void* stream);
+
 /* Dead columns, act-order permutation, damping and the Cholesky chain of
  * GPTQ.process_hessian_and_weights, gptq.py:139-141, 150-153, 169-174:
  *   dead = diag(H)==0; H[dead,dead] = 1; W[:,dead] = 0; H = H[perm][:,perm];

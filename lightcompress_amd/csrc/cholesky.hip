@@ -66,6 +66,26 @@ __global__ __launch_bounds__(256) void apply_dead_kernel(float* __restrict__ W, 
     if (dead[e % K]) W[e] = 0.0f;
 }
 
+// W[r, j] = dead[c] ? 0 : float(w[r, c]),  c = perm ? perm[j] : j   -- the weight clone, fp32 cast, dead-column
+// zeroing and act-order gather of process_hessian_and_weights (gptq.py:133-141, 150-151) in one pass.  A workgroup
+// takes 4 rows; reads are gathers inside a row (it stays in cache), writes are coalesced.
+template <int DT>
+__global__ __launch_bounds__(256) void prepare_w_kernel(const void* __restrict__ w, long long R, int K,
+                                                        const long long* __restrict__ perm,
+                                                        const uint8_t* __restrict__ dead, float* __restrict__ out) {
+  for (long long row = (long long)blockIdx.x * 4; row < R && row < (long long)blockIdx.x * 4 + 4; ++row) {
+    for (int j = threadIdx.x; j < K; j += 256) {
+      const long long c = perm ? perm[j] : j;
+      float v;
+      if (DT == LCQ_F32) v = ((const float*)w)[row * K + c];
+      else if (DT == LCQ_BF16) v = u2f((uint32_t)((const uint16_t*)w)[row * K + c] << 16);
+      else v = (float)((const _Float16*)w)[row * K + c];
+      if (dead && dead[c]) v = 0.0f;
+      out[row * K + j] = v;
+    }
+  }
+}
+
 // A (lower triangle, reversed + permuted + damped); strict upper triangle zeroed
 __global__ __launch_bounds__(256) void build_kernel(const float* __restrict__ H, int K, const long long* __restrict__ perm,
                                                     const PrepScalars* __restrict__ sc, float* __restrict__ A) {
@@ -255,6 +275,21 @@ extern "C" {
 int64_t lcq_chol_inv_upper_workspace_bytes(int64_t K) {
   const int64_t nblk = (K + NB - 1) / NB;
   return K * K * 4 + nblk * NB * NB * 4 + ((K + 255) / 256) * 256 + 256;
+}
+
+int lcq_gptq_prepare_weights(const void* w, int dtype, int64_t R, int64_t K, const int64_t* perm, const uint8_t* dead,
+                             float* out, void* stream) {
+  if (!w || !out || R <= 0 || K <= 0 || K > 0x7fffffff || (const void*)out == w) return LCQ_EINVAL;
+  const int64_t grid = (R + 3) / 4;
+  if (grid > 0x7fffffff) return LCQ_EINVAL;
+  hipStream_t st = (hipStream_t)stream;
+  const long long* p = (const long long*)perm;
+  if (dtype == LCQ_F32) prepare_w_kernel<LCQ_F32><<<dim3((unsigned)grid), dim3(256), 0, st>>>(w, R, (int)K, p, dead, out);
+  else if (dtype == LCQ_BF16) prepare_w_kernel<LCQ_BF16><<<dim3((unsigned)grid), dim3(256), 0, st>>>(w, R, (int)K, p, dead, out);
+  else if (dtype == LCQ_F16) prepare_w_kernel<LCQ_F16><<<dim3((unsigned)grid), dim3(256), 0, st>>>(w, R, (int)K, p, dead, out);
+  else return LCQ_EDTYPE;
+  LCQ_CHECK_LAUNCH();
+  return LCQ_OK;
 }
 
 int lcq_chol_inv_upper(float* H, int64_t K64, const int64_t* perm, float percdamp, float* W, int64_t R, float* U,

@@ -262,11 +262,11 @@ class GPTQ:
 
     def process_hessian_and_weights(self, layer, name):
         """-> (W [R,K] fp32 in processing order, Hinv: upper factor of the damped inverse)."""
-        W = layer.weight.data.clone()
-        if W.dim() > 2:
-            W = W.flatten(1)
-        W = W.float().contiguous()
-        R, K = W.shape
+        w = layer.weight.data
+        if w.dim() > 2:
+            w = w.flatten(1)
+        w = w.contiguous()
+        R, K = w.shape
         cache = self._settle(name) if 'H' in self.layers_cache[name] else self.layers_cache[name]
         leader = cache.get('leader', name)
         H = cache['H']
@@ -274,32 +274,34 @@ class GPTQ:
 
         self._setup_groups(layer, R, K)
 
-        is_shared = any(c.get('leader') == leader for n, c in self.layers_cache.items() if n != name) \
-            or leader != name
         shared = self._shared.get(leader)
         if shared is None:
+            is_shared = any(c.get('leader') == leader for n, c in self.layers_cache.items() if n != name) \
+                or leader != name
             perm = self.perm if self.actorder else None
-            # followers of a shared chain need the dead-column mask after H is gone
-            dead = (torch.diag(H) == 0) if is_shared else None
+            dead = torch.diag(H) == 0                       # before the chain rewrites H
             ws_bytes = L.lib().lcq_chol_inv_upper_workspace_bytes(L.i64(K))
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=self.dev)
             status = torch.zeros(1, dtype=torch.int32, device=self.dev)
-            L.check(L.lib().lcq_chol_inv_upper(L.ptr(H), L.i64(K), L.ptr(perm), L.f32(self.percdamp), L.ptr(W),
-                                               L.i64(R), L.ptr(H), L.ptr(ws), L.i64(ws_bytes), L.ptr(status),
+            L.check(L.lib().lcq_chol_inv_upper(L.ptr(H), L.i64(K), L.ptr(perm), L.f32(self.percdamp), L.ptr(None),
+                                               L.i64(0), L.ptr(H), L.ptr(ws), L.i64(ws_bytes), L.ptr(status),
                                                L.stream()), 'lcq_chol_inv_upper')
             del ws
             shared = dict(U=H, perm=perm, status=status, dead=dead)
             if is_shared:
                 self._shared[leader] = shared
-        else:
-            if 'done' in shared:                             # started by _chains_ahead on another stream
-                torch.cuda.current_stream().wait_event(shared.pop('done'))
-            W.masked_fill_(shared['dead'].unsqueeze(0), 0.0)
+        elif 'done' in shared:                               # started by _chains_ahead on another stream
+            torch.cuda.current_stream().wait_event(shared.pop('done'))
         U = shared['U']
         self._status = shared['status']
 
+        # weight.clone().float(), W[:, dead] = 0 and W[:, perm] in one pass
+        W = torch.empty((R, K), dtype=torch.float32, device=w.device)
+        dead_u8 = shared['dead'].view(torch.uint8)
+        L.check(L.lib().lcq_gptq_prepare_weights(L.ptr(w), L.i32(L.dtype_code(w.dtype)), L.i64(R), L.i64(K),
+                                                 L.ptr(self.perm if self.actorder else None), L.ptr(dead_u8), L.ptr(W),
+                                                 L.stream()), 'lcq_gptq_prepare_weights')
         if self.actorder:
-            W = W[:, self.perm].contiguous()
             self.invperm = torch.argsort(self.perm)
             layer.buf_perm = self.perm
             layer.buf_invperm = self.invperm
@@ -332,14 +334,18 @@ class GPTQ:
             self._static = True
 
     def update_layer_with_transformed_weights(self, layer, W, H, name):
-        Losses = torch.zeros_like(W)
-        tmp = torch.zeros_like(W)
+        Losses = torch.empty_like(W)                     # the loop writes every entry of both
+        tmp = torch.empty_like(W)
         self.weight_transform(W, H, Losses, tmp)
         self.last_error = torch.sum(Losses)              # device scalar; .item() it to log like the reference
         if self.check_positive_definite and int(self._status.item()) != 0:
             raise torch.linalg.LinAlgError('GPTQ: the damped Hessian is not positive-definite')
-        if self.actorder:
-            tmp = tmp[:, self.invperm]
+        if self.actorder:                                # tmp[:, invperm]
+            out = torch.empty_like(tmp)
+            L.check(L.lib().lcq_gptq_prepare_weights(L.ptr(tmp), L.i32(L.F32), L.i64(tmp.shape[0]), L.i64(tmp.shape[1]),
+                                                     L.ptr(self.invperm), L.ptr(None), L.ptr(out), L.stream()),
+                    'lcq_gptq_prepare_weights')
+            tmp = out
         layer.weight.data = tmp.reshape(layer.weight.shape)
         if self.wquantizer.granularity == 'per_group' and not self.static_groups:
             self.update_model_qparams(layer)
