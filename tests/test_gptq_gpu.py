@@ -349,3 +349,37 @@ def test_chains_side_by_side_match_one_by_one(dev, actorder):
                     + [gp.last_error.cpu()])
     for x, y in zip(*outs):
         assert torch.equal(x, y)
+
+
+@pytest.mark.parametrize('bit,sym,g,bs,R,K,wdtype', [
+    (3, False, 128, 128, 40, 768, torch.bfloat16),      # R not a multiple of the 16 rows of a workgroup
+    (8, True, 64, 128, 64, 640, torch.float16),         # fp16 weights, symmetric 8 bit
+    (2, False, 32, 64, 24, 512, torch.float32),         # 2 bit, small groups, half-size blocks
+    (4, False, 256, 128, 32, 1280, torch.bfloat16),     # groups wider than a block
+    (4, True, 128, 128, 130, 1152, torch.bfloat16),     # odd row count, K = 9 blocks
+])
+def test_layer_configurations(dev, bit, sym, g, bs, R, K, wdtype):
+    """layer_transform over bit widths, symmetry, group / block sizes and weight dtypes against the fp32 oracle:
+    codes >= 99.9 % equal, summed loss within 0.1 %."""
+    batches = calib_batches(6, 160, K, seed=9300 + K + bit)
+    W0 = (torch.randn(R, K, generator=gen(9301 + bit)) * 0.02).to(wdtype)
+    spec = Q.IntSpec(bit, sym, 'per_group', group_size=g)
+    Ho = torch.zeros(K, K); n = 0
+    for b in batches:
+        n = G.add_batch(Ho, n, b.unsqueeze(0))
+    ref = G.gptq_layer(W0, Ho, spec, blocksize=bs)
+    gp = make_gptq(blocksize=bs, weight=dict(bit=bit, symmetric=sym, granularity='per_group', group_size=g))
+    layer = Layer(W0.to(dev))
+    gp.subset_init({'layers': {'fc': layer}})
+    for b in batches:
+        gp.add_batch(layer, 'fc', b.unsqueeze(0).to(dev), None)
+    gp.subset_transform({'layers': {'fc': layer}})
+    Wq = layer.weight.data.cpu()
+    s = layer.buf_scales.cpu()
+    z = None if sym else layer.buf_zeros.cpu()
+    assert torch.allclose(s, ref['scales'], rtol=1e-3)
+    codes = G.codes_from(Wq, s, z, spec)
+    codes_o = G.codes_from(ref['tmp_perm'], ref['scales'], ref['zeros'], spec)
+    agree = float((codes == codes_o).float().mean())
+    assert agree >= 0.999, agree
+    assert abs(float(gp.last_error) - ref['loss']) <= 1e-3 * ref['loss']
