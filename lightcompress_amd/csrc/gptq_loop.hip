@@ -14,24 +14,27 @@
 // every block and everything behind them once per 1024 columns, which reads
 // and writes the bulk of W eight times less often.
 //
-// Block kernel layout: 16 lanes share one weight row, lane t keeps columns
-// 8t..8t+7 of the block in registers; a wave therefore carries 4 rows and a
-// 256-thread workgroup 16.  Column i lives on lane i/8: every lane evaluates
-// the quantizer on its own register (same instruction stream), the owner's
-// error is broadcast inside the 16-lane team, and all lanes apply the rank-1
-// update to their 8 columns from the Hinv block held in LDS.
-// Per-group min/max are 16-lane DPP butterflies.
+// Block kernel layout: 16 lanes share one weight row, lane t starts with columns 8t..8t+7 of the
+// block in registers; a wave therefore carries 4 rows and a 256-thread workgroup 16.  Every lane
+// evaluates the quantizer on its own register (same instruction stream), the owner's error is
+// broadcast inside the 16-lane team, and all lanes apply the rank-1 update to their 8 columns from
+// the Hinv block held in LDS.  Per-group min/max are 16-lane DPP butterflies.
 //
 // With R = 4096 rows the kernel has one wave per SIMD on the whole chip, so its run time is the
 // length of the per-column dependency chain times 128.  That chain is kept to about ten VALU
-// operations: the quotient w/s goes through the group's reciprocal (an octet in which an owner comes
-// near a rounding boundary is replayed with true divisions), (w-q)/d through a reciprocal of the diagonal prepared in LDS (at most one ulp
-// from the quotient; it only perturbs later columns, never the rounding of this one), the broadcast
-// of the error is a DPP row_share from lane 0 instead of an LDS permute (the registers rotate by one
-// lane after every 8 columns, so the owner is always lane 0 and the loop over octets stays rolled:
-// fully unrolled it is 126 KB of straight-line code that runs at instruction-fetch speed), the U row
-// comes from addresses that do not depend on the chain, and because U is upper triangular no update
-// needs a mask.  tmp / (w-q) / err rotate along and are stored once at the end, 32 bytes per lane.
+// operations:
+//  * the quotient w/s goes through the group's reciprocal; an octet (8 columns) in which an owner
+//    comes within 2^-11 of a rounding boundary is replayed with true divisions;
+//  * (w-q)/d goes through a reciprocal of the diagonal prepared in LDS (at most one ulp from the
+//    quotient; it only perturbs later columns, never the rounding of this one);
+//  * the registers rotate by one lane after every octet, so the owner is always lane 0 and the
+//    broadcast of the error is a DPP row_share:0 instead of an LDS permute, while the loop over
+//    octets stays rolled (fully unrolled it is 126 KB of straight-line code that runs at
+//    instruction-fetch speed);
+//  * the octet's rows of U are fetched from LDS ahead of the chain, and because U is stored zero
+//    below the diagonal no update needs a mask;
+//  * tmp / (w-q) / err rotate along and are stored once at the end, 32 bytes per lane: a store
+//    inside the loop would make every later wait on a load cover it too.
 #include <type_traits>
 
 #include "gemm_f32.h"
