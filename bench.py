@@ -136,7 +136,7 @@ def gpu_main(args):
     H = torch.zeros(K, K, device=dev)
     x = streams['down_in']
     lib, st = L.lib(), L.stream()
-    FOLD = GPTQ(CFG).hessian_defer                      # add_batch calls per launch, as the layer run above issues them
+    FOLD = GPTQ(CFG).hessian_fold(14336)                      # add_batch calls per launch, as the layer run above issues them
     TL = FOLD * TOK
     def hess(b):
         b = (b * FOLD) % (NB - FOLD + 1)

@@ -73,7 +73,7 @@ def test_hessian_batched_call_and_fp16(dev):
     assert float((H - ref).abs().max() / ref.abs().max()) < 1e-5
 
 
-@pytest.mark.parametrize('defer', [1, 3, 4])
+@pytest.mark.parametrize('defer', [1, 3, 4, 'auto'])
 def test_hessian_deferred_launches(dev, defer):
     """Folding several add_batch calls into one launch leaves H and nsamples as per-call updates do,
     for ragged token counts and for inputs the caller overwrites right after the call."""
