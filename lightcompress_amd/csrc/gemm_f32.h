@@ -17,6 +17,8 @@
 // (GEMM_LOWER_TILES).  Batched launches take per-problem offsets from
 // GemmBatch (blockIdx.z).
 #pragma once
+#include <type_traits>
+
 #include "common.h"
 
 namespace lcq {
@@ -47,7 +49,7 @@ struct GemmBatch {
   int M[GEMM_MAX_BATCH], N[GEMM_MAX_BATCH], Kc[GEMM_MAX_BATCH];
 };
 
-template <bool B_T, int TM = GT>
+template <bool B_T, int TM = GT, bool DEEP = false>
 __device__ __forceinline__ void gemm_tile(const float* A, int lda, const float* B, int ldb,
                                           float* C, int ldc, int M, int N, int Kc, float alpha, float beta,
                                           int flags, int m0, int n0, float* sA, float* sB) {
@@ -69,9 +71,13 @@ __device__ __forceinline__ void gemm_tile(const float* A, int lda, const float* 
       #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  // staging registers: A tile 128 x 32 floats = 1024 float4 -> 4 per thread; B likewise
-  f32x4 ra[AP], rb[4];
-  auto gload = [&](int k0) {
+  // staging registers: A tile 128 x 32 floats = 1024 float4 -> 4 per thread; B likewise.
+  // DEEP (contraction of at most 4 slabs): one register set per slab, so that all global loads of the tile are in
+  // flight at once; with one set the tile pays one memory latency per slab, which is most of a rank-128 launch.
+  constexpr int NS = DEEP ? 4 : 1;
+  f32x4 ra[NS][AP], rb[NS][4];
+  auto gload = [&](int k0, auto slot_tag) {
+    constexpr int sl = decltype(slot_tag)::value;
     #pragma unroll
     for (int p = 0; p < 4; ++p) {
       const int idx = p * 256 + tid;
@@ -87,7 +93,7 @@ __device__ __forceinline__ void gemm_tile(const float* A, int lda, const float* 
             for (int e = 0; e < 4; ++e) if (k + e < ke) v[e] = p0[e];
           }
         }
-        ra[p] = v;
+        ra[sl][p] = v;
       }
       if constexpr (B_T) {   // B[n][k]: same shape as A
         const int r = idx >> 3, k = k0 + (idx & 7) * 4;
@@ -101,7 +107,7 @@ __device__ __forceinline__ void gemm_tile(const float* A, int lda, const float* 
             for (int e = 0; e < 4; ++e) if (k + e < ke) v[e] = p0[e];
           }
         }
-        rb[p] = v;
+        rb[sl][p] = v;
       } else {               // B[k][n]: k = idx / 32, n4 = idx % 32
         const int k = k0 + (idx >> 5), n = n0 + (idx & 31) * 4;
         f32x4 v = {0.f, 0.f, 0.f, 0.f};
@@ -113,37 +119,33 @@ __device__ __forceinline__ void gemm_tile(const float* A, int lda, const float* 
             for (int e = 0; e < 4; ++e) if (n + e < N) v[e] = p0[e];
           }
         }
-        rb[p] = v;
+        rb[sl][p] = v;
       }
     }
   };
-  auto lstore = [&]() {
+  auto lstore = [&](auto slot_tag) {
+    constexpr int sl = decltype(slot_tag)::value;
     #pragma unroll
     for (int p = 0; p < 4; ++p) {
       const int idx = p * 256 + tid;
       if (p < AP) {
         const int r = idx >> 3, k = (idx & 7) * 4;
         #pragma unroll
-        for (int e = 0; e < 4; ++e) sA[r * GPA + k + e] = ra[p][e];
+        for (int e = 0; e < 4; ++e) sA[r * GPA + k + e] = ra[sl][p][e];
       }
       if constexpr (B_T) {
         const int r = idx >> 3, k = (idx & 7) * 4;
         #pragma unroll
-        for (int e = 0; e < 4; ++e) sB[r * GPA + k + e] = rb[p][e];
+        for (int e = 0; e < 4; ++e) sB[r * GPA + k + e] = rb[sl][p][e];
       } else {
         const int k = idx >> 5, n = (idx & 31) * 4;
-        *(f32x4*)(sB + k * GPB + n) = rb[p];
+        *(f32x4*)(sB + k * GPB + n) = rb[sl][p];
       }
     }
   };
 
   const int lm = lane & 31, lk = lane >> 5;
-  if (kb < ke) gload(kb);
-  for (int k0 = kb; k0 < ke; k0 += GK) {
-    __syncthreads();                       // previous slab fully consumed
-    lstore();
-    __syncthreads();
-    if (k0 + GK < ke) gload(k0 + GK);      // next slab in flight while this one is multiplied
+  auto compute = [&]() {
     #pragma unroll
     for (int kk = 0; kk < GK; kk += 2) {
       float a[MI], b[2];
@@ -159,6 +161,42 @@ __device__ __forceinline__ void gemm_tile(const float* A, int lda, const float* 
         #pragma unroll
         for (int j = 0; j < 2; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+  };
+  using S0 = std::integral_constant<int, 0>;
+  float oldc[DEEP ? MI : 1][2][16];                       // DEEP: the old C values, fetched with the operands
+  if constexpr (DEEP) {
+    gload(kb, S0{});
+    if (kb + GK < ke) gload(kb + GK, std::integral_constant<int, 1>{});
+    if (kb + 2 * GK < ke) gload(kb + 2 * GK, std::integral_constant<int, 2>{});
+    if (kb + 3 * GK < ke) gload(kb + 3 * GK, std::integral_constant<int, 3>{});
+    if (beta != 0.0f) {
+      #pragma unroll
+      for (int i = 0; i < MI; ++i)
+        #pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int gn = n0 + wc * 64 + j * 32 + lm;
+          const int gm0 = m0 + wr * WM + i * 32 + 4 * lk;
+          const float* p0 = C + (long long)gm0 * ldc + gn;
+          #pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int dm = 8 * (r >> 2) + (r & 3);
+            oldc[i][j][r] = (gm0 + dm < M && gn < N) ? p0[(long long)dm * ldc] : 0.0f;
+          }
+        }
+    }
+    __syncthreads(); lstore(S0{}); __syncthreads(); compute();
+    if (kb + GK < ke) { __syncthreads(); lstore(std::integral_constant<int, 1>{}); __syncthreads(); compute(); }
+    if (kb + 2 * GK < ke) { __syncthreads(); lstore(std::integral_constant<int, 2>{}); __syncthreads(); compute(); }
+    if (kb + 3 * GK < ke) { __syncthreads(); lstore(std::integral_constant<int, 3>{}); __syncthreads(); compute(); }
+  } else {
+    if (kb < ke) gload(kb, S0{});
+    for (int k0 = kb; k0 < ke; k0 += GK) {
+      __syncthreads();                       // previous slab fully consumed
+      lstore(S0{});
+      __syncthreads();
+      if (k0 + GK < ke) gload(k0 + GK, S0{});   // next slab in flight while this one is multiplied
+      compute();
     }
   }
 
@@ -177,7 +215,8 @@ __device__ __forceinline__ void gemm_tile(const float* A, int lda, const float* 
         #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int dm = 8 * (r >> 2) + (r & 3);
-          old[r] = (gm0 + dm < M && gn < N) ? p0[(long long)dm * ldc] : 0.0f;
+          if constexpr (DEEP) old[r] = oldc[i][j][r];
+          else old[r] = (gm0 + dm < M && gn < N) ? p0[(long long)dm * ldc] : 0.0f;
         }
       }
       #pragma unroll
@@ -194,13 +233,13 @@ __device__ __forceinline__ void gemm_tile(const float* A, int lda, const float* 
 // TM = 128 or 64 rows of C per workgroup.  The short tile is for launches that would not give every CU a
 // 128-row tile (rank-128 updates and panel solves of the blocked chains): twice the workgroups, half the serial
 // MFMA work in each.
-template <bool B_T, int TM>
+template <bool B_T, int TM, bool DEEP = false>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmProblem g, float alpha, float beta, int flags) {
   __shared__ float sA[TM * GPA];
   __shared__ float sB[B_T ? GT * GPA : GK * GPB];
   const int m0 = blockIdx.y * TM, n0 = blockIdx.x * GT;
   if ((flags & GEMM_LOWER_TILES) && n0 >= m0 + TM) return;
-  gemm_tile<B_T, TM>(g.A, g.lda, g.B, g.ldb, g.C, g.ldc, g.M, g.N, g.Kc, alpha, beta, flags, m0, n0, sA, sB);
+  gemm_tile<B_T, TM, DEEP>(g.A, g.lda, g.B, g.ldb, g.C, g.ldc, g.M, g.N, g.Kc, alpha, beta, flags, m0, n0, sA, sB);
 }
 
 template <bool B_T>
@@ -219,7 +258,9 @@ template <bool B_T>
 inline void launch_gemm(const GemmProblem& g, float alpha, float beta, int flags, hipStream_t st) {
   if (g.M <= 0 || g.N <= 0) return;
   const unsigned gx = (unsigned)((g.N + GT - 1) / GT), gy = (unsigned)((g.M + GT - 1) / GT);
-  if ((long long)gx * gy <= 256)
+  if ((long long)gx * gy <= 256 && g.Kc > 0 && g.Kc <= 4 * GK && !(flags & (GEMM_K_FROM_N | GEMM_K_TO_M)))
+    gemm_f32_kernel<B_T, 64, true><<<dim3(gx, (unsigned)((g.M + 63) / 64)), dim3(256), 0, st>>>(g, alpha, beta, flags);
+  else if ((long long)gx * gy <= 256)
     gemm_f32_kernel<B_T, 64><<<dim3(gx, (unsigned)((g.M + 63) / 64)), dim3(256), 0, st>>>(g, alpha, beta, flags);
   else
     gemm_f32_kernel<B_T, GT><<<dim3(gx, gy), dim3(256), 0, st>>>(g, alpha, beta, flags);
