@@ -18,6 +18,10 @@ What changes under the API
     passes; the O(K) scale arithmetic (pow / clamp / normalise) uses torch ops
     on the [K] vector like the reference;
   * one process / one GPU: no all_reduce / broadcast of the winner;
+  * float8 block-wise checkpoints (``weight`` float8_e4m3fn with ``weight_scale_inv``, awq.py:53-56, 148-160): the
+    weight is brought to bf16 once per search (``weight_cast_to_bf16``, the block-wise casts of kernel.py), every
+    grid point's scaled + fake-quantized weight is cast back with fresh block scales (``weight_cast_to_fp8``), and
+    both buffers are put back afterwards;
   * GQA (``is_gqa``: v_proj feeding o_proj, base_blockwise_quantization.py:281-295, 614-618): the scales have
     one entry per key/value channel and are repeated per query group before they meet o_proj's columns;
     ``set_model_config`` takes the three sizes from a config object instead of ``self.model``.
@@ -38,10 +42,18 @@ class Awq:
         self.trans_version = special_config.get('trans_version', 'v2')
         self.awq_bs = special_config.get('awq_bs', None)
         self.save_mem = special_config.get('save_mem', True)
+        # Several input tensors: the reference tests `loss_mean < best_error` inside the loop over inputs
+        # (awq.py:245-248), so the grid point is picked by the FIRST input's weighted loss (later partial sums only
+        # grow), while `best_scales` aliases `scales_mean`, which the in-place `+=` of the later inputs completes to
+        # the mean over all inputs.  'first_input' reproduces that; 'mean' compares the mean loss over all inputs.
+        self.multi_input_select = special_config.get('multi_input_select', 'first_input')
+        if self.multi_input_select not in ('first_input', 'mean'):
+            raise ValueError(f'multi_input_select: {self.multi_input_select}')
         self.wquantizer = wquantizer or IntegerQuantizer(**quant_config['weight'])
         self.aquantizer = aquantizer
         self.w_only = aquantizer is None
         self.padding_mask = None
+        self.fp8_block_size = special_config.get('fp8_block_size', 128)
         self._ws = {}
 
     def _workspace(self, K, device):
@@ -80,13 +92,29 @@ class Awq:
         w.mul_(scales_tmp.view(1, -1))
         return w
 
+    def _bf16_weight(self, fc):
+        """The layer weight; a float8 block-wise weight as bf16 (awq.py:53-56, 148-151)."""
+        w = fc.weight.data
+        if w.dtype == torch.float8_e4m3fn:
+            from .kernel import weight_cast_to_bf16
+            w = weight_cast_to_bf16(w.contiguous(), fc.weight_scale_inv.data.contiguous(), self.fp8_block_size).to(torch.bfloat16)
+        return w
+
+    def _store_weight(self, fc, w):
+        """fc.weight.data = w; for a float8 block-wise layer the block-wise cast of w (awq.py:158-162)."""
+        if fc.weight.data.dtype == torch.float8_e4m3fn:
+            from .kernel import weight_cast_to_fp8
+            fc.weight.data, fc.weight_scale_inv.data = weight_cast_to_fp8(w.contiguous(), self.fp8_block_size)
+        else:
+            fc.weight.data = w
+
     # -- awq.py:48-72 -------------------------------------------------------------
     def get_weight_scale(self, layers_dict):
         layers = list(layers_dict.values())
         total_scale = None
         wq = self.wquantizer
         for _m in layers:
-            w = _m.weight.data.contiguous()
+            w = self._bf16_weight(_m).contiguous()
             R, K = w.shape
             g = wq.group_size if wq.granularity == 'per_group' else K
             out = torch.empty(K, dtype=w.dtype, device=w.device)
@@ -182,14 +210,22 @@ class Awq:
 
     # -- awq.py:147-176 ----------------------------------------------------------------------
     def _scale_quant(self, weight, scales):
+        """fake_quant_weight_dynamic(W * s) (awq.py:147-164) into a new tensor.  Min/max calibration with rounded zero
+        points is one fused kernel; any other weight quantizer setting (calib_algo mse / hqq, round_zp False, other
+        granularities) multiplies first and then goes through the quantizer's own fake_quant_weight_dynamic."""
         wq = self.wquantizer
         w = weight.contiguous()
         R, K = w.shape
-        g = wq.group_size if wq.granularity == 'per_group' else 0
-        if wq.granularity not in ('per_group', 'per_channel'):
-            raise NotImplementedError(f'AWQ weight granularity {wq.granularity}')
-        out = torch.empty_like(w)
         s = scales.to(w.dtype).contiguous()
+        fused = (wq.calib_algo not in ('mse', 'hqq', 'learnable') and wq.round_zp
+                 and wq.granularity in ('per_group', 'per_channel') and getattr(wq, 'quant_type', '') == 'int-quant')
+        if not fused:
+            ws = torch.empty_like(w)
+            L.check(L.lib().lcq_scale_matrix(L.ptr(w), L.i32(L.dtype_code(w.dtype)), L.i64(R), L.i64(K), L.ptr(s), L.i32(0),
+                                             L.ptr(ws), L.stream()), 'lcq_scale_matrix')
+            return wq.fake_quant_weight_dynamic(ws)
+        g = wq.group_size if wq.granularity == 'per_group' else 0
+        out = torch.empty_like(w)
         L.check(L.lib().lcq_awq_scale_quant(L.ptr(w), L.i32(L.dtype_code(w.dtype)), L.i64(R), L.i64(K), L.ptr(s), L.i32(g),
                                             L.f32(wq.qmin), L.f32(wq.qmax), L.i32(L.FLAG_SYM if wq.sym else 0),
                                             L.ptr(out), L.stream()), 'lcq_awq_scale_quant')
@@ -198,7 +234,7 @@ class Awq:
     def fake_quantize_weight(self, fc, scales, is_gqa, layer_name):
         if is_gqa:
             scales = self.repeat_gqa_scales(scales).reshape(-1)
-        fc.weight.data = self._scale_quant(fc.weight.data, scales)
+        self._store_weight(fc, self._scale_quant(self._bf16_weight(fc), scales))
         return fc.weight
 
     def fake_quantize_input(self, x_tmp, layers_dict):
@@ -226,9 +262,13 @@ class Awq:
             self._bs = input[0].shape[0]
         else:
             self._bs = self.awq_bs
+        # the reference computes w_max for every version (awq.py:190) and reads it only in v1
         w_max = self.get_weight_scale(layers_dict) if self.trans_version == 'v1' else None
         n_grid = 20
-        originals = {name: fc.weight.data for name, fc in layers_dict.items()}
+        # what the reference saves and reloads as a host state dict: the tensors themselves, never modified here
+        saved = {name: (fc.weight.data, fc.weight_scale_inv.data if fc.weight.data.dtype == torch.float8_e4m3fn else None)
+                 for name, fc in layers_dict.items()}
+        originals = {name: self._bf16_weight(fc) for name, fc in layers_dict.items()}
         device = next(iter(originals.values())).device
         n_samples = input[0].shape[0] if len(input) == 1 else sum(x.shape[0] for x in input)
 
@@ -237,6 +277,7 @@ class Awq:
         for n in range(n_grid):
             loss_mean = 0
             scales_mean = 0
+            loss_select = None
             for i in range(len(input)):
                 input[i] = input[i].to(device)
                 x = input[i]
@@ -249,7 +290,7 @@ class Awq:
                 scales = self.get_scales(prev_op, x, w_max, is_gqa, ratio, x_mean=x_mean_dict[i])
                 col_scales = self.repeat_gqa_scales(scales).reshape(-1) if is_gqa else scales
                 for layer_name, fc in layers_dict.items():
-                    fc.weight.data = self._scale_quant(originals[layer_name], col_scales)
+                    self._store_weight(fc, self._scale_quant(originals[layer_name], col_scales))
                 x_tmp = self.scaling_input(x, scales, is_gqa)
                 if not self.w_only:
                     x_tmp = self.fake_quantize_input(x_tmp, layers_dict)
@@ -259,10 +300,16 @@ class Awq:
                     org_out, out = org_out * m, out * m
                 loss = self._loss_device(org_out, out)
                 loss_mean = loss_mean + x.shape[0] * 1.0 / n_samples * loss
+                if i == 0:
+                    loss_select = loss_mean
                 scales_mean = scales_mean + x.shape[0] * 1.0 / n_samples * scales
                 for layer_name, fc in layers_dict.items():      # the originals were never touched
-                    fc.weight.data = originals[layer_name]
-            loss_rows.append(loss_mean.reshape(1))
+                    fc.weight.data = saved[layer_name][0]
+                    if saved[layer_name][1] is not None:
+                        fc.weight_scale_inv.data = saved[layer_name][1]
+            if len(input) > 1 and self.multi_input_select == 'mean':
+                loss_select = loss_mean
+            loss_rows.append(loss_select.reshape(1))
             scale_rows.append(scales_mean)
         losses = torch.cat(loss_rows)
         best = torch.argmin(losses)                              # first minimum, like `loss < best_error`

@@ -52,6 +52,7 @@ struct LoopArgs {
   long long R; int K, i1, count, g, G, ldErr;
   float qmin, qmax;
   int sym, is_static, aligned;
+  int nrz;              // round_zp=False: un-rounded zero point inside the rounding, scale clamped at 1e-9 (quant.py:556-557, 702-706)
 };
 
 // DPP moves inside every 16-lane row: the value of lane 0, and the value of the next lane (rotation by one)
@@ -67,14 +68,14 @@ struct ColQ {           // quantizer of the column being processed
   float lo, hi;         // qmin - z, qmax - z: clamp(round(t) + z, qmin, qmax) - z == clamp(round(t), lo, hi) for integral z
   bool fast;            // x * r may stand for x / s (guarded) and lo / hi are exact
 };
-__device__ __forceinline__ ColQ make_colq(float s, float z, float qmin, float qmax) {
+__device__ __forceinline__ ColQ make_colq(float s, float z, float qmin, float qmax, bool nrz = false) {
   ColQ q;
   q.s = s; q.z = z;
   q.r = __builtin_amdgcn_rcpf(s);
   q.lo = qmin - z; q.hi = qmax - z;
   const float a = fabsf(s);
   q.fast = (a > 8.6736174e-19f) & (a < 1.1529215e18f) & (rintf(z) == z) & (fabsf(z) <= 512.0f) & (fabsf(qmin) <= 512.0f) &
-           (fabsf(qmax) <= 512.0f);
+           (fabsf(qmax) <= 512.0f) & !nrz;
   return q;
 }
 
@@ -103,13 +104,13 @@ __device__ __forceinline__ ColQ open_group(const LoopArgs& a, int idx, int lane,
     z = 0.0f;
   } else {
     s = fmaxf(mx - mn, 1e-5f) / (a.qmax - a.qmin);
-    z = fminf(fmaxf(a.qmin - rintf(mn / s), a.qmin), a.qmax);
+    z = a.nrz ? a.qmin - mn / s : fminf(fmaxf(a.qmin - rintf(mn / s), a.qmin), a.qmax);
   }
   if (row_ok && lane == 0) {
     a.scales[row * a.G + idx / a.g] = s;
     if (!a.sym) a.zeros[row * a.G + idx / a.g] = z;
   }
-  return make_colq(s, z, a.qmin, a.qmax);
+  return make_colq(s, z, a.qmin, a.qmax, a.nrz);
 }
 
 // STATIC: scales / zero points are given (per group, or per column through gidx).  OCT: every group starts on
@@ -180,7 +181,8 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
   if (!STATIC) {
     nextb = (a.i1 + a.g - 1) / a.g * a.g;
     if (a.i1 % a.g != 0)                         // the block starts inside a group opened by an earlier block
-      q = make_colq(a.scales[(row_ok ? row : 0) * a.G + a.i1 / a.g], a.sym ? 0.0f : a.zeros[(row_ok ? row : 0) * a.G + a.i1 / a.g], a.qmin, a.qmax);
+      q = make_colq(a.scales[(row_ok ? row : 0) * a.G + a.i1 / a.g], a.sym ? 0.0f : a.zeros[(row_ok ? row : 0) * a.G + a.i1 / a.g], a.qmin, a.qmax,
+                    a.nrz);
   }
   __syncthreads();
 
@@ -226,7 +228,7 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
       #pragma unroll
       for (int c = 0; c < 8; ++c) {
         if (STATIC) {
-          q = make_colq(ss[c], zz[c], a.qmin, a.qmax);                      // lane 0: the parameters of this column
+          q = make_colq(ss[c], zz[c], a.qmin, a.qmax, a.nrz);               // lane 0: the parameters of this column
         } else if (!OCT && a.i1 + 8 * to + c == nextb && 8 * to + c < a.count) {
           nextb += a.g;
           q = open_group(a, a.i1 + 8 * to + c, lane, row, row_ok, rbase, w, false);
@@ -234,7 +236,8 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
         const float wv = w[c];
         float diff;
         if (EXACT) {
-          diff = wv - (__builtin_amdgcn_fmed3f(rintf(wv / q.s) + q.z, a.qmin, a.qmax) - q.z) * q.s;
+          const float code = a.nrz ? rintf(wv / fmaxf(q.s, 1e-9f) + q.z) : rintf(wv / q.s) + q.z;
+          diff = wv - (__builtin_amdgcn_fmed3f(code, a.qmin, a.qmax) - q.z) * q.s;
         } else {
           const float t = wv * q.r, rt = rintf(t);
           unsure |= !((fabsf(fabsf(t - rt) - 0.5f) > 4.8828125e-04f) & (fabsf(t) <= 1024.0f) & q.fast);
@@ -327,6 +330,7 @@ int lcq_gptq_block(float* W, float* tmp, float* Losses, float* Err, int64_t ldEr
   a.scales = scales; a.zeros = zeros; a.gidx = gidx;
   a.R = R; a.K = (int)K; a.i1 = (int)i1; a.count = count; a.g = group_size; a.G = (int)G;
   a.qmin = qmin; a.qmax = qmax; a.sym = sym; a.is_static = is_static; a.ldErr = (int)ldErr;
+  a.nrz = (flags & LCQ_FLAG_NO_ROUND_ZP) != 0;
   a.aligned = ((reinterpret_cast<uintptr_t>(W) | reinterpret_cast<uintptr_t>(tmp) | reinterpret_cast<uintptr_t>(Losses) |
                 reinterpret_cast<uintptr_t>(U)) & 15) == 0;
   const unsigned grid = (unsigned)((R + ROWS_PER_WG - 1) / ROWS_PER_WG);

@@ -366,7 +366,14 @@ class GPTQ:
         wq = self.wquantizer
         if not hasattr(self, '_scales') or self._scales.shape[0] != R:
             raise L.LcqError('weight_transform needs process_hessian_and_weights (or _setup_groups) first')
-        flags = (L.FLAG_SYM if wq.sym else 0) | (L.FLAG_STATIC if self._static else 0)
+        flags = (L.FLAG_SYM if wq.sym else 0) | (0 if wq.round_zp else L.FLAG_NO_ROUND_ZP)
+        # search_column_qparams (gptq.py:358-366) is wquantizer.get_tensor_qparams: min/max ranges are found inside
+        # the block kernel; any other calibrator (mse, hqq) runs on the host side before the block that opens the
+        # group, on the same columns of W the kernel would read, and the kernel takes the result as given.
+        host_groups = (not self._static) and wq.calib_algo in ('mse', 'hqq', 'learnable')
+        if self._static or host_groups:
+            flags |= L.FLAG_STATIC
+        g = self._g
         # Two-level deferral: after every block only the rest of the current 1024-column window is
         # updated; the columns behind the window get one update per window (8x fewer passes over W).
         window = 8 * self.blocksize
@@ -377,19 +384,32 @@ class GPTQ:
         n = self.n_nonout
         for o0 in range(0, n, window):
             o1 = min(o0 + window, n)
+            # A group that opens inside the window reads its whole column range of W (gptq.py:216-222), so the
+            # per-block updates reach to the end of the last such group; the window's deep update starts there.
+            hi = o1
+            if not self._static and g > 0:
+                last_open = (o1 - 1) // g * g
+                if last_open >= o0:
+                    hi = max(o1, min(last_open + g, K))
             for i1 in range(o0, o1, self.blocksize):
                 i2 = min(i1 + self.blocksize, o1)
+                if host_groups:
+                    for idx in range((i1 + g - 1) // g * g, i2, g):
+                        _, s_, z_, _, _ = wq.get_tensor_qparams(W[:, idx:min(idx + g, K)].contiguous())
+                        self._scales[:, idx // g] = s_.reshape(-1).float()
+                        if not wq.sym:
+                            self._zeros[:, idx // g] = z_.reshape(-1).float()
                 err_blk = Err[:, i1 - o0:]
                 L.check(lib.lcq_gptq_block(L.ptr(W), L.ptr(tmp), L.ptr(Losses), C_ptr(err_blk), L.i64(window), L.ptr(Hinv),
                                            L.i64(R), L.i64(K), L.i64(i1), L.i32(i2 - i1), L.i32(self._g), qmin, qmax,
                                            L.i32(flags), L.ptr(self._scales), L.ptr(self._zeros), L.ptr(self._gidx),
                                            L.i64(self._G), st), 'lcq_gptq_block')
-                if i2 < o1:
+                if i2 < hi:
                     L.check(lib.lcq_gptq_trailing(L.ptr(W), C_ptr(err_blk), L.i64(window), L.ptr(Hinv), L.i64(R), L.i64(K),
-                                                  L.i64(i1), L.i64(i2), L.i64(i2), L.i64(o1), st), 'lcq_gptq_trailing')
-            if o1 < K:
+                                                  L.i64(i1), L.i64(i2), L.i64(i2), L.i64(hi), st), 'lcq_gptq_trailing')
+            if hi < K:
                 L.check(lib.lcq_gptq_trailing(L.ptr(W), L.ptr(Err), L.i64(window), L.ptr(Hinv), L.i64(R), L.i64(K),
-                                              L.i64(o0), L.i64(o1), L.i64(o1), L.i64(K), st), 'lcq_gptq_trailing')
+                                              L.i64(o0), L.i64(o1), L.i64(hi), L.i64(K), st), 'lcq_gptq_trailing')
 
     # -- qparam bookkeeping (gptq.py:332-409) ---------------------------------------
     @torch.no_grad()

@@ -2,8 +2,9 @@
 
 Restates awq.py of the reference on CPU tensors: get_weight_scale (:48-72),
 get_act_scale (:74-85), get_scales (:87-108), fake_quantize_weight (:147-164),
-calculate_loss (:134-145), search_scale_subset (:178-278, single input batch,
-one process) and scaling_input (base_blockwise_quantization.py:899-912).
+calculate_loss (:134-145), search_scale_subset (:178-278, one process; ``search_scale``
+for one input tensor, ``search_scale_inputs`` for several tensors / ``awq_bs``
+micro-batches) and scaling_input (base_blockwise_quantization.py:899-912).
 The inspect module is any callable taking (x, weights_dict) so the tests can
 use a SwiGLU MLP without nn.Module plumbing.
 """
@@ -81,6 +82,64 @@ def search_scale(weights: dict, x, forward, spec, n_grid=20, version='v2', gqa=N
         if l < best_err:
             best_err, best_scales = l, s_kv
     return best_scales, losses
+
+
+def search_scale_inputs(weights: dict, inputs: list, forward, spec, n_grid=20, version='v2', bs=None):
+    """search_scale_subset (awq.py:178-278) for a LIST of input tensors and micro-batches of ``bs`` samples
+    (``awq_bs``), statement for statement: ``loss_mean`` and ``scales_mean`` accumulate over the inputs, and
+    ``is_best`` is evaluated inside that loop (awq.py:245-248) - with Python floats for the losses and an in-place
+    ``+=`` on ``scales_mean`` from the second input on, so ``best_scales`` (an alias of ``scales_mean``) keeps
+    growing after it was chosen.  -> (best_scales, per grid point the list of ``loss_mean`` after each input)."""
+    bs = inputs[0].shape[0] if bs is None else bs
+
+    def act_scale_bs(x):                                     # get_act_scale, awq.py:74-85
+        if x.shape[0] == bs:
+            return x.abs().view(-1, x.shape[-1]).mean(0)
+        means = [x[k * bs:(k + 1) * bs].abs().view(-1, x.shape[-1]).mean(0) for k in range(x.shape[0] // bs)]
+        return sum(means) / len(means)
+
+    def fwd_bs(x, w):                                        # inspect_module_forward, awq.py:110-126
+        if x.shape[0] == bs:
+            return forward(x, w)
+        return torch.cat([forward(x[k * bs:(k + 1) * bs], w) for k in range(x.shape[0] // bs)], dim=0)
+
+    def loss_bs(a, b):                                       # calculate_loss, awq.py:134-145
+        if b.shape[0] == bs:
+            return (a - b).float().pow(2).mean().item()
+        total = 0.0
+        for k in range(a.shape[0] // bs):
+            total += (a[k * bs:(k + 1) * bs] - b[k * bs:(k + 1) * bs]).float().pow(2).mean().item()
+        return total / (a.shape[0] // bs)
+
+    w_max = weight_scale(list(weights.values()), spec)
+    n_samples = inputs[0].shape[0] if len(inputs) == 1 else sum(x.shape[0] for x in inputs)
+    best_error, best_scales, trace = float('inf'), None, []
+    org_out = {}
+    for n in range(n_grid):
+        loss_mean = 0
+        scales_mean = 0
+        row = []
+        for i, x in enumerate(inputs):
+            if i not in org_out:
+                org_out[i] = fwd_bs(x, weights)
+            ratio = n * 1 / n_grid
+            xm = act_scale_bs(x)
+            if version == 'v1':
+                scales = (xm.pow(ratio) / w_max.pow(1 - ratio)).clamp(min=1e-4).view(-1)
+            else:
+                scales = xm.pow(ratio).clamp(min=1e-4).view(-1)
+            scales = scales / (scales.max() * scales.min()).sqrt()
+            wq = {k: scale_and_fake_quant(w, scales, spec) for k, w in weights.items()}
+            out = fwd_bs(scaling_input(x, scales), wq)
+            l = loss_bs(org_out[i], out)
+            loss_mean += x.shape[0] * 1.0 / n_samples * l
+            scales_mean += x.shape[0] * 1.0 / n_samples * scales      # in place from the second input on
+            row.append(loss_mean)
+            if loss_mean < best_error:
+                best_error = loss_mean
+                best_scales = scales_mean
+        trace.append(row)
+    return best_scales, trace
 
 
 # ----------------------------------------------------------------------------

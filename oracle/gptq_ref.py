@@ -78,7 +78,7 @@ def process_hessian_and_weights(weight: torch.Tensor, H: torch.Tensor, percdamp:
 # ---------------------------------------------------------------------------
 # lazy-batch column loop   (gptq.py:198-244)
 # ---------------------------------------------------------------------------
-def weight_transform(W, Hinv, spec, blocksize=128, static_qparams=None, static_groups=None):
+def weight_transform(W, Hinv, spec, blocksize=128, static_qparams=None, static_groups=None, qparams_fn=None):
     """Runs the loop in place on W (as the reference does) and returns
     (tmp, Losses, groups) where groups is the list of per-group
     (scale [R,1], zero [R,1]|0-dim) refreshed at every group boundary.
@@ -89,7 +89,10 @@ def weight_transform(W, Hinv, spec, blocksize=128, static_qparams=None, static_g
     ``static_groups=(scales [R,G], zeros [R,G] | None, perm | None)``: per_group with
     ``static_groups: True`` - the RTN parameters of the ORIGINAL column order, looked up as
     ``groups[perm[idx] // g]`` (gptq.py:143-148, 224-227); nothing is refreshed.
+    ``qparams_fn(spec, cols) -> (rows, scale, zero, qmax, qmin)`` stands for ``wquantizer.get_tensor_qparams``
+    (gptq.py:358-366 calls it, so ``calib_algo`` reaches the loop); default: min/max calibration.
     """
+    qparams_fn = qparams_fn or Q.int_tensor_qparams
     R, K = W.shape
     Losses = torch.zeros_like(W)
     tmp = torch.zeros_like(W)
@@ -114,7 +117,7 @@ def weight_transform(W, Hinv, spec, blocksize=128, static_qparams=None, static_g
                 zero = torch.tensor(0.0) if zg is None else zg[:, idx // spec.group_size].unsqueeze(1)
             elif per_group and (i1 + i) % spec.group_size == 0:
                 cols = W[:, (i1 + i): min(i1 + i + spec.group_size, K)]      # W, not W1 (gptq.py:216-222)
-                _, scale, zero, qmax, qmin = Q.int_tensor_qparams(spec, cols)
+                _, scale, zero, qmax, qmin = qparams_fn(spec, cols)
                 groups.append((scale.clone(), zero.clone()))
             q = Q.int_quant_dequant(spec, w.unsqueeze(1), scale, zero, qmax, qmin).squeeze(1)
             tmp1[:, i] = w
@@ -136,12 +139,20 @@ def merge_groups(groups):
     return scales, zeros
 
 
+def mse_tensor_qparams(spec, t, **mse):
+    """get_tensor_qparams with calib_algo 'mse' (quant.py:689-696 with :147-205)."""
+    rows = Q.reshape_rows(spec, t)
+    lo, hi = Q.int_mse_range(spec, rows.clone(), **mse)
+    s, z, qmax, qmin = Q.int_qparams(spec, lo, hi)
+    return rows, s, z, qmax, qmin
+
+
 def gptq_layer(weight, H, spec, percdamp=0.01, blocksize=128, actorder=False, dtype=torch.float32,
-               static_qparams=None):
+               static_qparams=None, qparams_fn=None):
     """layer_transform (gptq.py:113-196): -> dict(weight=tmp un-permuted, scales, zeros, perm, loss, Hinv)."""
     perm = act_order(H) if actorder else None
     W, Hinv, invperm = process_hessian_and_weights(weight, H, percdamp, perm, dtype)
-    tmp, Losses, groups = weight_transform(W, Hinv, spec, blocksize, static_qparams)
+    tmp, Losses, groups = weight_transform(W, Hinv, spec, blocksize, static_qparams, qparams_fn=qparams_fn)
     out = dict(loss=float(Losses.sum()), perm=perm, Hinv=Hinv, tmp_perm=tmp)
     if actorder:
         tmp = tmp[:, invperm]

@@ -132,6 +132,142 @@ def test_search_scale_subset_gqa(dev):
     assert_bit_equal(awq.scaling_weight(w2, s_kv.to(dev), True), wo * rep.view(1, -1), 'scaling_weight')
 
 
+def _search_on_gpu(dev, awq, w, down, inputs):
+    layers = {k: Fc(v.to(dev)) for k, v in w.items()}
+    downd = down.to(dev)
+    inspect = lambda xx: swiglu(xx, {'gate': layers['gate'].weight.data, 'up': layers['up'].weight.data, 'down': downd})
+    best = awq.search_scale_subset(None, layers, [x.to(dev) for x in inputs], inspect, False, {})
+    for k in w:
+        assert torch.equal(layers[k].weight.data.cpu(), w[k])              # weights are back to the originals
+    return best, awq.search_losses.cpu()
+
+
+def _same_point(losses, losses_o, tol=0.02):
+    ko = min(range(20), key=lambda i: losses_o[i])
+    kg = int(torch.argmin(losses))
+    return kg == ko, (kg == ko or abs(losses_o[kg] - losses_o[ko]) <= tol * losses_o[ko])
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+def test_search_scale_subset_trans_version_v1(dev, dtype):
+    """trans_version v1 (awq.py:97-102): scales = mean|x|^r / w_max^(1-r), w_max from get_weight_scale."""
+    x, w, down = tiny_case(dtype, seed=18, T=192, K=512, I=640)
+    spec = Q.IntSpec(4, False, 'per_group', group_size=128)
+    fwd = lambda xx, ww: swiglu(xx, dict(ww, down=down))
+    best_o, losses_o = A.search_scale(w, x, fwd, spec, version='v1')
+    best, losses = _search_on_gpu(dev, make_awq(trans_version='v1'), w, down, [x])
+    rel = ((losses.double() - torch.tensor(losses_o).double()).abs() / torch.tensor(losses_o).double()).max()
+    assert float(rel) < (0.05 if dtype == torch.bfloat16 else 1e-3), float(rel)
+    same, near = _same_point(losses, losses_o)
+    assert near
+    if same:
+        assert float((best.cpu().float() - best_o.float()).abs().max()) <= 2 ** -6 * float(best_o.float().abs().max())
+    # v1 and v2 really differ on this case
+    _, losses_v2 = A.search_scale(w, x, fwd, spec, version='v2')
+    assert max(abs(a - b) / b for a, b in zip(losses_o[1:], losses_v2[1:])) > 1e-3
+
+
+@pytest.mark.parametrize('bs', [None, 1])
+def test_search_scale_subset_several_inputs_and_micro_batches(dev, bs):
+    """len(input) > 1 and awq_bs: the reference compares `loss_mean` after every input (awq.py:245-248), so the first
+    input's loss picks the grid point and the returned scales are the mean over the inputs at that point."""
+    dtype = torch.float32
+    x0, w, down = tiny_case(dtype, seed=21, T=96, K=512, I=640)
+    g = gen(22)
+    x1 = (torch.randn(4, 96, 512, generator=g) * torch.exp(torch.randn(512, generator=g))).to(dtype)
+    x2 = (torch.randn(2, 96, 512, generator=g) * 3).to(dtype)
+    spec = Q.IntSpec(4, False, 'per_group', group_size=128)
+    fwd = lambda xx, ww: swiglu(xx, dict(ww, down=down))
+    inputs = [x0, x1, x2]
+    best_o, trace = A.search_scale_inputs(w, inputs, fwd, spec, bs=bs)
+    first = [row[0] for row in trace]
+    special = {} if bs is None else {'awq_bs': bs}
+    best, losses = _search_on_gpu(dev, make_awq(**special), w, down, inputs)
+    rel = ((losses.double() - torch.tensor(first).double()).abs() / torch.tensor(first).double()).max()
+    assert float(rel) < 1e-3, float(rel)
+    same, near = _same_point(losses, first)
+    assert near
+    if same:
+        assert float((best.cpu() - best_o).abs().max()) <= 1e-5 * float(best_o.abs().max())
+    # the documented alternative: the mean loss over all inputs
+    best_m, losses_m = _search_on_gpu(dev, make_awq(multi_input_select='mean', **special), w, down, inputs)
+    full = [row[-1] for row in trace]
+    rel = ((losses_m.double() - torch.tensor(full).double()).abs() / torch.tensor(full).double()).max()
+    assert float(rel) < 1e-3, float(rel)
+
+
+def test_search_honours_the_weight_quantizer_settings(dev):
+    """fake_quantize_weight is wquantizer.fake_quant_weight_dynamic (awq.py:156): calib_algo mse and round_zp False
+    change the quantized weights the loss is measured on."""
+    from lightcompress_amd.awq import Awq
+    from lightcompress_amd import IntegerQuantizer
+    dtype = torch.float32
+    w = (torch.randn(96, 512, generator=gen(41)) * 0.02).to(dtype)
+    s = torch.exp(torch.randn(512, generator=gen(42)) * 0.5).to(dtype)
+    for kw, spec_kw in (({'round_zp': False}, {'round_zp': False}), ({'calib_algo': 'mse'}, {})):
+        cfg = {'weight': dict(CFG['weight'], **kw), 'special': {}}
+        got = Awq(cfg)._scale_quant(w.to(dev), s.to(dev))
+        spec = Q.IntSpec(4, False, 'per_group', group_size=128, **spec_kw)
+        ws = w.clone().mul_(s.view(1, -1))
+        if 'calib_algo' in kw:
+            rows = Q.reshape_rows(spec, ws)
+            lo, hi = Q.int_mse_range(spec, rows)
+            sc, zp, qmax, qmin = Q.int_qparams(spec, lo, hi)
+            want = Q.int_quant_dequant(spec, rows, sc, zp, qmax, qmin).reshape(ws.shape)
+            assert float((got.cpu() == want).float().mean()) > 0.98        # the shrink search may tie between steps
+        else:
+            assert_bit_equal(got, Q.int_fake_quant_dynamic(spec, ws), 'round_zp False')
+        plain = make_awq()._scale_quant(w.to(dev), s.to(dev))
+        assert not torch.equal(plain, got)
+
+
+def test_search_on_float8_blockwise_weights(dev):
+    """A block-wise float8 checkpoint (awq.py:53-56, 148-162): bf16 <- weight * weight_scale_inv, scale, fake quant,
+    cast back to float8 with fresh block scales; weight and weight_scale_inv are both restored after the search."""
+    x, w, down = tiny_case(torch.bfloat16, seed=25, T=128, K=512, I=640)
+    spec = Q.IntSpec(4, False, 'per_group', group_size=128)
+
+    class Fp8Fc:
+        def __init__(self, wt):
+            y, sc = Q.triton_weight_cast_to_fp8(wt)
+            self.weight = types.SimpleNamespace(data=y.to(dev))
+            self.weight_scale_inv = types.SimpleNamespace(data=sc.to(dev))
+    layers = {k: Fp8Fc(v) for k, v in w.items()}
+    w8 = {k: (layers[k].weight.data.cpu(), layers[k].weight_scale_inv.data.cpu()) for k in w}
+    wb = {k: Q.triton_weight_cast_to_bf16(*w8[k]).to(torch.bfloat16) for k in w}
+    awq = make_awq()
+    # one grid point's weight, bit for bit
+    s = torch.exp(torch.randn(512, generator=gen(26)) * 0.3).bfloat16()
+    fc = Fp8Fc(w['gate'])
+    awq.fake_quantize_weight(fc, s.to(dev), False, 'gate')
+    yo, so = Q.triton_weight_cast_to_fp8(A.scale_and_fake_quant(wb['gate'], s, spec))
+    assert_bit_equal(fc.weight.data.view(torch.uint8), yo.view(torch.uint8), 'float8 codes')
+    assert_bit_equal(fc.weight_scale_inv.data, so, 'block scales')
+    # get_weight_scale sees the bf16 weights
+    ws = awq.get_weight_scale(layers).cpu()
+    wo = A.weight_scale(list(wb.values()), spec)
+    assert float(((ws.double() - wo.double()).abs() / wo.double()).max()) <= 2 ** -7
+    # the search: the inspect module dequantises what the layers hold
+    downd = down.to(dev)
+    def deq(fc):
+        from lightcompress_amd.kernel import weight_cast_to_bf16
+        return weight_cast_to_bf16(fc.weight.data, fc.weight_scale_inv.data).to(torch.bfloat16)
+    inspect = lambda xx: swiglu(xx, {'gate': deq(layers['gate']), 'up': deq(layers['up']), 'down': downd})
+    def fwd(xx, ww):
+        q = {k: Q.triton_weight_cast_to_bf16(*Q.triton_weight_cast_to_fp8(v)).to(torch.bfloat16) if ww is not wb else v
+             for k, v in ww.items()}
+        return swiglu(xx, dict(q, down=down))
+    best_o, losses_o = A.search_scale(wb, x, fwd, spec)
+    best = awq.search_scale_subset(None, layers, [x.to(dev)], inspect, False, {})
+    losses = awq.search_losses.cpu()
+    rel = ((losses.double() - torch.tensor(losses_o).double()).abs() / torch.tensor(losses_o).double()).max()
+    assert float(rel) < 0.05, float(rel)
+    assert _same_point(losses, losses_o)[1]
+    for k in w:
+        assert torch.equal(layers[k].weight.data.cpu().view(torch.uint8), w8[k][0].view(torch.uint8))
+        assert torch.equal(layers[k].weight_scale_inv.data.cpu(), w8[k][1])
+
+
 # ---- AutoClipper (auto_clip.py) ---------------------------------------------------------------------
 @pytest.mark.parametrize('clip_sym,sym', [(False, False), (True, False), (False, True)])
 @pytest.mark.parametrize('R,K,T', [(64, 256, 96), (320, 512, 512), (256, 128, 700)])

@@ -10,7 +10,7 @@ import pytest
 import torch
 
 from oracle import gptq_ref as G, quant_ref as Q
-from tests.helpers import gen
+from tests.helpers import assert_bit_equal, gen
 from tests.test_oracle_gptq import calib_batches
 
 pytestmark = pytest.mark.gpu
@@ -383,3 +383,141 @@ def test_layer_configurations(dev, bit, sym, g, bs, R, K, wdtype):
     agree = float((codes == codes_o).float().mean())
     assert agree >= 0.999, agree
     assert abs(float(gp.last_error) - ref['loss']) <= 1e-3 * ref['loss']
+
+
+def _run_loop(dev, gp, W, U, R, K):
+    gp.n_nonout = gp.columns = K
+    gp._setup_groups(None, R, K)
+    Wd = W.clone().to(dev)
+    tmp, Losses = torch.zeros_like(Wd), torch.zeros_like(Wd)
+    gp.weight_transform(Wd, U.to(dev).contiguous(), Losses, tmp)
+    return tmp.cpu(), Losses.cpu(), gp._scales.cpu(), (None if gp.wquantizer.sym else gp._zeros.cpu())
+
+
+@pytest.mark.parametrize('R,K,g,bs', [(32, 1200, 100, 128),      # the group opened at 1000 runs past the 1024-column window
+                                      (32, 1100, 128, 100),      # window of 800 columns: the group at 768 crosses it
+                                      (24, 2304, 384, 128)])     # groups wider than a block that straddle windows
+def test_groups_that_cross_the_update_window(dev, R, K, g, bs):
+    """The deferred update reaches far-away columns once per 8 blocks; a group that opens inside such a window and
+    ends behind it must still see every earlier block's update in all of its columns (gptq.py:216-222, 244)."""
+    spec, W0, W, U = _loop_case(R, K, g, bs, False, 5100 + K + g)
+    tmp_o, Loss_o, groups = G.weight_transform(W.clone(), U, spec, blocksize=bs)
+    so, zo = G.merge_groups(groups)
+    gp = make_gptq(blocksize=bs, weight=dict(bit=4, symmetric=False, granularity='per_group', group_size=g))
+    tmp, Losses, s, z = _run_loop(dev, gp, W, U, R, K)
+    assert torch.allclose(s.reshape(-1, 1), so, rtol=1e-4)
+    assert torch.allclose(z.reshape(-1, 1), zo, atol=0.5)
+    assert float((z.reshape(-1, 1) != zo).float().mean()) < 2e-3
+    assert float((tmp - tmp_o).abs().max()) < 1e-4 * float(tmp_o.abs().max())
+    codes_o = G.codes_from(tmp_o, so, zo, spec)
+    codes = G.codes_from(tmp, s.reshape(-1, 1), z.reshape(-1, 1), spec)
+    assert float((codes == codes_o).float().mean()) >= 0.999
+    assert abs(float(Losses.sum()) - float(Loss_o.sum())) <= 1e-3 * float(Loss_o.sum())
+
+
+@pytest.mark.parametrize('g,bs,K', [(128, 128, 512), (64, 128, 384), (256, 128, 1280)])
+def test_loop_with_unrounded_zero_points(dev, g, bs, K):
+    """round_zp: False reaches the loop through wquantizer.get_tensor_qparams / quant_dequant (gptq.py:229, 358-366):
+    zero = qmin - min/scale un-rounded, code = clamp(round(w / max(scale, 1e-9) + zero))."""
+    R = 40
+    spec, W0, W, U = _loop_case(R, K, g, bs, False, 5300 + K + g)
+    spec.round_zp = False
+    tmp_o, Loss_o, groups = G.weight_transform(W.clone(), U, spec, blocksize=bs)
+    so, zo = G.merge_groups(groups)
+    assert float((zo != torch.round(zo)).float().mean()) > 0.9             # the zero points really are fractional
+    gp = make_gptq(blocksize=bs, weight=dict(bit=4, symmetric=False, granularity='per_group', group_size=g, round_zp=False))
+    tmp, Losses, s, z = _run_loop(dev, gp, W, U, R, K)
+    assert torch.allclose(s.reshape(-1, 1), so, rtol=1e-4)
+    assert torch.allclose(z.reshape(-1, 1), zo, rtol=1e-3, atol=1e-3)
+    assert float((tmp - tmp_o).abs().max()) < 1e-4 * float(tmp_o.abs().max())
+    codes_o = G.codes_from(tmp_o, so, zo, spec)
+    codes = G.codes_from(tmp, s.reshape(-1, 1), z.reshape(-1, 1), spec)
+    assert float((codes == codes_o).float().mean()) >= 0.999
+    assert abs(float(Losses.sum()) - float(Loss_o.sum())) <= 1e-3 * float(Loss_o.sum())
+    # and it differs from the rounded-zero-point loop, i.e. the flag is not ignored
+    gp2 = make_gptq(blocksize=bs, weight=dict(bit=4, symmetric=False, granularity='per_group', group_size=g))
+    _, _, _, z2 = _run_loop(dev, gp2, W, U, R, K)
+    assert not torch.equal(z2, z)
+
+
+@pytest.mark.parametrize('g,bs,K', [(128, 128, 512), (64, 128, 256), (256, 128, 1280)])
+def test_loop_with_mse_calibrated_groups(dev, g, bs, K):
+    """calib_algo: mse (the GPTQ recipe offers it) reaches the loop through search_column_qparams ->
+    wquantizer.get_tensor_qparams (gptq.py:358-366): every group's range is the shrunken one of get_mse_range."""
+    R = 32
+    spec, W0, W, U = _loop_case(R, K, g, bs, False, 5500 + K + g)
+    tmp_o, Loss_o, groups = G.weight_transform(W.clone(), U, spec, blocksize=bs, qparams_fn=G.mse_tensor_qparams)
+    so, zo = G.merge_groups(groups)
+    _, _, groups_mm = G.weight_transform(W.clone(), U, spec, blocksize=bs)
+    assert not torch.equal(G.merge_groups(groups_mm)[0], so)               # mse ranges differ from min/max ranges
+    gp = make_gptq(blocksize=bs, weight=dict(bit=4, symmetric=False, granularity='per_group', group_size=g, calib_algo='mse'))
+    tmp, Losses, s, z = _run_loop(dev, gp, W, U, R, K)
+    # the shrink search picks between steps whose errors can tie to within fp32 summation noise: nearly all rows
+    # choose the oracle's step, the others an adjacent one
+    same = torch.isclose(s.reshape(-1, 1), so, rtol=1e-4)
+    assert float(same.float().mean()) >= 0.98, float(same.float().mean())
+    rows_ok = same.reshape(R, -1).all(dim=1)
+    assert float(rows_ok.float().mean()) >= 0.8
+    codes_o = G.codes_from(tmp_o, so, zo, spec)
+    codes = G.codes_from(tmp, s.reshape(-1, 1), z.reshape(-1, 1), spec)
+    agree = (codes == codes_o)[rows_ok]
+    assert float(agree.float().mean()) >= 0.999                             # rows with the same ranges: same codes
+    assert abs(float(Losses.sum()) - float(Loss_o.sum())) <= 0.02 * float(Loss_o.sum())
+
+
+def test_learnable_calibration_raises(dev):
+    gp = make_gptq(weight=dict(bit=4, symmetric=False, granularity='per_group', group_size=128, calib_algo='learnable'))
+    spec, W0, W, U = _loop_case(16, 256, 128, 128, False, 5700)
+    with pytest.raises(NotImplementedError):
+        _run_loop(dev, gp, W, U, 16, 256)
+
+
+@pytest.mark.parametrize('actorder', [False, True])
+@pytest.mark.parametrize('sym', [False, True])
+def test_deploy_partials_w_q_and_w_qdq(dev, actorder, sym):
+    """w_qdq / w_q (gptq.py:411-452) on a transformed layer: static fake / real quantization of the compensated
+    weights with the loop's qparams - in processing order and un-permuted again when groups follow act-order; w_q
+    rounds the scales to the model dtype first."""
+    R, K, g = 64, 768, 128
+    batches = calib_batches(4, 256, K, seed=9500)
+    W0 = (torch.randn(R, K, generator=gen(9501)) * 0.02).bfloat16()
+    spec = Q.IntSpec(4, sym, 'per_group', group_size=g)
+    gp = make_gptq(actorder=actorder, weight=dict(bit=4, symmetric=sym, granularity='per_group', group_size=g))
+    layer = Layer(W0.to(dev))
+    gp.subset_init({'layers': {'fc': layer}})
+    for b in batches:
+        gp.add_batch(layer, 'fc', b.unsqueeze(0).to(dev), None)
+    gp.layer_transform(layer, 'fc')
+    wq = gp.wquantizer
+    layer.buf_qmax, layer.buf_qmin = wq.qmax, wq.qmin
+    Wt = layer.weight.data.cpu()
+    s = layer.buf_scales.cpu()
+    z = None if sym else layer.buf_zeros.cpu()
+    zz = torch.tensor(0.0) if sym else z
+    if sym and hasattr(layer, 'buf_zeros'):
+        del layer.buf_zeros
+    fq = gp.w_qdq(layer, wq)
+    src = Wt
+    if actorder:
+        assert gp.need_perm
+        src = Wt[:, layer.buf_perm.cpu()]
+    want = Q.int_fake_quant_static(spec, src, s, zz, spec.qmax, spec.qmin).to(torch.bfloat16)
+    if actorder:
+        want = want[:, layer.buf_invperm.cpu()]
+    assert_bit_equal(fq, want, 'w_qdq')
+    # fake-quantised values sit on the loop's grid: they reproduce the loop's codes
+    codes_loop = G.codes_from(src, s, z, spec)
+    back = Q.int_quant(spec, Q.int_fake_quant_static(spec, src, s, zz, spec.qmax, spec.qmin).reshape(-1, g), s, zz, spec.qmax,
+                       spec.qmin).reshape(R, K)
+    assert torch.equal(back, codes_loop)
+    if not actorder:                                    # real-quant export needs groups in the original order (gptq.py:455-457)
+        if sym:
+            layer.buf_zeros = torch.tensor(0.0)
+        codes, s_out, z_out = gp.w_q(layer, wq)
+        oc, os_, oz = Q.int_real_quant_static(spec, Wt, s.to(torch.bfloat16), zz, spec.qmax, spec.qmin)
+        assert_bit_equal(codes, oc, 'w_q codes')
+        assert_bit_equal(s_out, os_, 'w_q scales')
+        if sym:
+            assert z_out is None
+        else:
+            assert_bit_equal(z_out, oz, 'w_q zeros')

@@ -171,3 +171,50 @@ def test_gqa_search_reduces_to_the_plain_search_and_repeats_per_group():
     best_g, losses_g = A.search_scale(weights, x, fwd, spec, gqa=(lambda t: t @ v.t(), 2, 64, 2))
     assert best_g.shape == (128,) and abs(float(best_g.max() * best_g.min()) - 1) < 1e-5
     assert losses_g[0] == losses[0]                               # ratio 0: all-ones scales either way
+
+
+def test_several_inputs_pick_by_the_first_input_and_return_the_mean_scales():
+    """awq.py:245-248 tests `loss_mean < best_error` after EVERY input.  Losses are positive, so a partial sum after
+    the second input can never beat the record its own first term set or failed to beat: the chosen grid point is the
+    argmin of the first input's weighted loss; `best_scales` aliases `scales_mean`, which the in-place `+=` of the
+    later inputs completes to the mean over all inputs.  Shown here on the statement-for-statement restatement."""
+    dtype = torch.float32
+    x0, w, down = tiny_case(dtype, seed=11, T=48)
+    g = gen(12)
+    x1 = (torch.randn(4, 48, 256, generator=g) * torch.exp(torch.randn(256, generator=g))).to(dtype)   # other statistics
+    x2 = (torch.randn(2, 48, 256, generator=g) * 3).to(dtype)           # sample counts are multiples of the first's
+    spec = Q.IntSpec(4, False, 'per_group', group_size=128)
+    fwd = lambda xx, ww: swiglu(xx, dict(ww, down=down))
+    inputs = [x0, x1, x2]
+    best, trace = A.search_scale_inputs(w, inputs, fwd, spec)
+    first = [row[0] for row in trace]
+    full = [row[-1] for row in trace]
+    k = min(range(20), key=lambda i: first[i])
+    n = sum(x.shape[0] for x in inputs)
+    want = sum(x.shape[0] / n * A.get_scales(x, None, k / 20) for x in inputs)
+    assert torch.allclose(best, want, rtol=1e-6)
+    # the single-input search on the first tensor alone picks the same grid point
+    _, losses0 = A.search_scale(w, x0, fwd, spec)
+    assert min(range(20), key=lambda i: losses0[i]) == k
+    # and the quirk is observable: the mean loss over all inputs prefers another point in this case
+    assert all(f > a for f, a in zip(full, first))
+    assert min(range(20), key=lambda i: full[i]) != k
+
+
+def test_micro_batches_average_per_batch_statistics():
+    """awq_bs: statistics, forward and loss run per micro-batch and are averaged (awq.py:74-85, 110-145); with equal
+    micro-batches that is the statistic of the whole tensor up to rounding, so the search result is unchanged."""
+    x, w, down = tiny_case(torch.float64, seed=13, T=32)
+    x = torch.cat([x, x.flip(0) * 1.5])                       # 4 samples
+    spec = Q.IntSpec(4, False, 'per_group', group_size=128)
+    fwd = lambda xx, ww: swiglu(xx, dict(ww, down=down))
+    b_all, t_all = A.search_scale_inputs(w, [x], fwd, spec)
+    b_two, t_two = A.search_scale_inputs(w, [x], fwd, spec, bs=2)
+    assert torch.allclose(b_all, b_two, rtol=1e-12)
+    # (scales that differ in the last bit move a few codes across a rounding boundary)
+    assert all(abs(a[0] - b[0]) <= 1e-3 * abs(a[0]) for a, b in zip(t_all, t_two))
+    # v1 divides by the weight statistic: ratio 0 gives 1 / w_max (normalised), not ones
+    b_v1, _ = A.search_scale_inputs(w, [x], fwd, spec, version='v1', n_grid=1)
+    wm = A.weight_scale(list(w.values()), spec)
+    s = (1 / wm).clamp(min=1e-4)
+    assert torch.allclose(b_v1, s / (s.max() * s.min()).sqrt(), rtol=1e-12)
