@@ -68,6 +68,7 @@ extern "C" {
 #define LCQ_EDTYPE (-3)
 #define LCQ_ELAUNCH (-4)
 #define LCQ_EWORKSPACE (-5)
+#define LCQ_ESIZE (-6)        /* input larger than an entry point's stated maximum */
 
 /* ---- integer quantizer -------------------------------------------------- */
 
@@ -258,6 +259,16 @@ int lcq_scale_matrix(const void* x, int dtype, int64_t T, int64_t K, const void*
 
 /* Awq.calculate_loss, awq.py:134-145: out[0] = mean( float((a - b) in `dtype`)^2 ), kept on the device. */
 int lcq_sq_err_mean(const void* a, const void* b, int dtype, int64_t n, float* out, void* workspace, void* stream);
+
+/* lcq_sq_err_mean for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc): same kernels, same result bit for bit, but the partial sums live in a 64 KiB array that is
+ * part of the library's device image instead of a caller workspace.  No counterpart in the reference.
+ * Calls no hipMalloc / hipFree or other allocating routine; the first call on a device looks the array's address up.
+ *  n <= LCQ_SQ_ERR_STATIC_MAX_N, else LCQ_ESIZE.
+ * Every call on one GPU uses that GPU's single array: calls that overlap on one GPU (different streams) race;
+ * calls on one stream, or ordered by events, are safe.  Nothing needs clearing between calls. */
+#define LCQ_SQ_ERR_STATIC_MAX_N (((int64_t)1) << 34)
+int lcq_sq_err_mean_static(const void* a, const void* b, int dtype, int64_t n, float* out, void* stream);
 
 /* AutoClipper.auto_clip_layer, auto_clip.py:83-191 (clip_version v1, weight-only, per_group with group_size 128):
  * for every (output row, group) the shrink step i in [0, n_steps) of the group range

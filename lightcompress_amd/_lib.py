@@ -23,7 +23,7 @@ FLAG_TIE_EVEN, FLAG_NO_SUBNORMALS, FLAG_DQ_F32 = 16, 32, 64
 FLAG_RANGE_BF16, FLAG_SCALE_F32, FLAG_ROW_QP = 128, 256, 512
 
 _ERR = {-1: 'invalid argument', -2: 'misaligned pointer', -3: 'unsupported dtype', -4: 'kernel launch failed',
-        -5: 'workspace too small'}
+        -5: 'workspace too small', -6: 'input larger than the entry point\'s stated maximum'}
 
 
 class LcqError(RuntimeError):

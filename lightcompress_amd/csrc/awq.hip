@@ -8,12 +8,37 @@
 //
 // All four are single-pass HBM-bound streams: 16-byte loads per lane,
 // per-thread fp32 partial sums, one small second stage.
+#include <mutex>
+
 #include "rowquant.h"
 
 namespace {
 using namespace lcq;
 
 constexpr int PARTS_MAX = 1024;
+constexpr int SQERR_PARTS_MAX = 8192;          // workgroups (= partial sums) of a squared-error launch
+
+// Partial sums of lcq_sq_err_mean_static, 64 KiB.  Every GPU the library runs on holds its own copy of this array
+// for the life of the process.  In host code the NAME of the array is only a handle: its device address is looked
+// up once per device with hipGetSymbolAddress (static_scratch() below) and only that pointer is handed to kernels.
+static __device__ __align__(256) double scratch[SQERR_PARTS_MAX];
+
+constexpr int MAX_DEVICES = 64;
+double* scratch_ptr[MAX_DEVICES] = {};
+std::mutex scratch_mutex;
+
+// device address of `scratch` on the current device, or nullptr
+double* static_scratch() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return nullptr;
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (!scratch_ptr[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return nullptr;
+    scratch_ptr[dev] = (double*)p;
+  }
+  return scratch_ptr[dev];
+}
 
 // ---- column-wise mean of |x| over T rows ------------------------------------------------
 // grid = (column blocks of 256 * N, row splits); every thread owns one 16-byte column chunk
@@ -250,21 +275,32 @@ int lcq_scale_matrix(const void* x, int dtype, int64_t T, int64_t K, const void*
   return LCQ_OK;
 }
 
-int lcq_sq_err_mean(const void* a, const void* b, int dtype, int64_t n, float* out, void* workspace, void* stream) {
-  if (!a || !b || !out || !workspace || n <= 0) return LCQ_EINVAL;
+static int sq_err_mean_launch(const void* a, const void* b, int dtype, int64_t n, float* out, double* part, hipStream_t st) {
   const int nn = dtype == LCQ_BF16 ? 8 : 4;
   if (dtype != LCQ_BF16 && dtype != LCQ_F32) return LCQ_EDTYPE;
   if (n % nn != 0 || (((uintptr_t)a | (uintptr_t)b) % 16) != 0) return LCQ_EALIGN;
   const int64_t nchunks = n / nn;
   int64_t grid = (nchunks + 255) / 256;
-  if (grid > 8192) grid = 8192;
-  hipStream_t st = (hipStream_t)stream;
-  double* part = (double*)workspace;
+  if (grid > SQERR_PARTS_MAX) grid = SQERR_PARTS_MAX;
   if (dtype == LCQ_BF16) sqerr_stage1<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)a, (const u32x4*)b, nchunks, part);
   else sqerr_stage1<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)a, (const u32x4*)b, nchunks, part);
   sqerr_stage2<<<dim3(1), dim3(256), 0, st>>>(part, (int)grid, (double)n, out);
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;
+}
+
+int lcq_sq_err_mean(const void* a, const void* b, int dtype, int64_t n, float* out, void* workspace, void* stream) {
+  if (!a || !b || !out || !workspace || n <= 0) return LCQ_EINVAL;
+  return sq_err_mean_launch(a, b, dtype, n, out, (double*)workspace, (hipStream_t)stream);
+}
+
+int lcq_sq_err_mean_static(const void* a, const void* b, int dtype, int64_t n, float* out, void* stream) {
+  if (!a || !b || !out || n <= 0) return LCQ_EINVAL;
+  if (n > LCQ_SQ_ERR_STATIC_MAX_N) return LCQ_ESIZE;
+  double* part = static_scratch();
+  if (!part) return LCQ_ELAUNCH;
+  // stage 1 writes every partial sum that stage 2 reads (the first `grid` entries), so nothing has to start at zero
+  return sq_err_mean_launch(a, b, dtype, n, out, part, (hipStream_t)stream);
 }
 
 }  // extern "C"
