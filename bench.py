@@ -5,9 +5,10 @@ One "step" = GPTQ (w4 asym g128, act_order, damp 0.01, blocksize 128) of one
 Llama-3-8B-shape decoder layer: for each of the four activation streams
 (attention input, o_proj input, MLP input with K=4096; down_proj input with
 K=14336) 128 calibration batches of 2048 tokens go through GPTQ.add_batch of
-every Linear that sees them (q,k,v / o / gate,up / down — one Hessian per
-Linear, as the reference does), then every Linear runs the damped Cholesky
-chain and the lazy-batch column loop.  Inputs are synthetic (lognormal
+every Linear that sees them (q,k,v / o / gate,up / down; Linears that are
+handed the identical tensor share one Hessian, `seconds_separate_hessians`
+is the run with one Hessian per Linear as the reference keeps them), then
+every Linear runs the damped Cholesky chain and the lazy-batch column loop.  Inputs are synthetic (lognormal
 per-channel scaled Gaussians, random-init weights) and resident in HBM before
 the timed region.
 
@@ -73,15 +74,13 @@ def gpu_main(args):
 
     phases = {'hessian_ms': 0.0, 'chain_ms': 0.0, 'loop_ms': 0.0}
 
-    def one_layer(share, record=None):
-        gp = GPTQ(CFG)
+    def one_layer(share, record=None, check=None):
+        gp = GPTQ({'weight': CFG['weight'], 'special': dict(CFG['special'], auto_share=share)})
         layers = {n: Layer(torch.nn.Parameter(weights[n].clone(), requires_grad=False)) for n, *_ in LINEARS}
         marks = []
         for subset in SUBSETS:
             sub = {'layers': {n: layers[n] for n in subset}}
             gp.subset_init(sub)
-            if share and len(subset) > 1:
-                gp.share_input(subset)
             x = streams[[s for n, _, _, s in LINEARS if n == subset[0]][0]]
             e0 = ev(); e0.record()
             for b in range(NB):
@@ -89,8 +88,14 @@ def gpu_main(args):
                 for n in subset:                       # every Linear's hook fires on every batch
                     gp.add_batch(layers[n], n, xb, None)
             e1 = ev(); e1.record()
-            if record is None:
+            if record is None and check is None:
                 gp.subset_transform(sub)               # the reference's driver of a subset (gptq.py:96-112)
+            elif check is not None:                    # untimed: the same driver, keeping each Linear's summed loss
+                gp._chains_ahead(sub['layers'])
+                for n in subset:
+                    gp.layer_transform(layers[n], n)
+                    gp.free(n)
+                    check[n] = gp.last_error
             else:                                      # same work one Linear at a time, with events between the phases
                 for n in subset:
                     gp.initialize_qparams_and_prepare_weights(layers[n], n)
@@ -108,28 +113,44 @@ def gpu_main(args):
                 record[k] += a.elapsed_time(b_)
         return layers
 
+    # Default path: Linears that receive the very same tensor on every call (q/k/v, gate/up) share one Hessian and
+    # one Cholesky chain (detected by add_batch; results bit-identical to separate Hessians).
     for _ in range(args.warmup):
-        one_layer(False)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        one_layer(False)
-    torch.cuda.synchronize()
-    dt = (time.perf_counter() - t0) / args.steps
-    # where the time goes: one more pass, one Linear at a time with events between the phases (untimed; the chains of
-    # a subset run one after the other here, in the timed pass subset_transform starts them side by side)
-    one_layer(False, phases)
-    for k in phases:
-        phases[k] = round(phases[k], 3)
-
-    # same layer with one Hessian / one chain per distinct input stream (q,k,v and gate,up share)
-    one_layer(True)
+        one_layer(True)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
         one_layer(True)
     torch.cuda.synchronize()
-    dt_shared = (time.perf_counter() - t0) / args.steps
+    dt = (time.perf_counter() - t0) / args.steps
+    # the outputs of one more (untimed) pass must be sane: finite weights and qparams, a positive finite loss
+    losses = {}
+    checked = one_layer(True, check=losses)
+    last_error = {}
+    for n, *_ in LINEARS:
+        lay = checked[n]
+        ok = bool(torch.isfinite(lay.weight.data).all()) and bool(torch.isfinite(lay.buf_scales).all()) \
+            and bool((lay.buf_scales > 0).all()) and bool(torch.isfinite(lay.buf_zeros).all())
+        le = float(losses[n])
+        if not ok or not (le > 0 and le == le and le != float('inf')):
+            print(f'bench.py: {n}: non-finite outputs or loss {le}', file=sys.stderr)
+            sys.exit(1)
+        last_error[n] = round(le, 3)
+    del checked
+    # where the time goes: one more pass, one Linear at a time with events between the phases (untimed; the chains of
+    # a subset run one after the other here, in the timed pass subset_transform starts them side by side)
+    one_layer(True, phases)
+    for k in phases:
+        phases[k] = round(phases[k], 3)
+
+    # the reference's behaviour: one Hessian and one chain per Linear, also where the inputs are identical
+    one_layer(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        one_layer(False)
+    torch.cuda.synchronize()
+    dt_separate = (time.perf_counter() - t0) / args.steps
 
     # ---- dominant kernel: bf16 MFMA Hessian at K=14336, live HIP-event timing ------------------
     K = 14336
@@ -192,9 +213,12 @@ def gpu_main(args):
         'higher_is_better': False, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'bf16 in / fp32 accumulate',
         'data': 'synthetic',
         'config': {'workload': 'GPTQ w4 asym g128 act_order, full Llama-3-8B-shape decoder layer (q,o 4096x4096; k,v 1024x4096; '
-                               'gate,up 14336x4096; down 4096x14336), 128x2048 calib tokens per stream, one Hessian per Linear',
+                               'gate,up 14336x4096; down 4096x14336), 128x2048 calib tokens per stream, add_batch per Linear per batch; '
+                               'Linears fed the identical tensor (q,k,v / gate,up) share one Hessian (seconds_separate_hessians: '
+                               'one per Linear)',
                    'blocksize': 128, 'percdamp': 0.01},
-        'seconds_shared_hessians': round(dt_shared, 4),
+        'seconds_separate_hessians': round(dt_separate, 4),
+        'last_error': last_error,
         'breakdown_ms': phases,
         'roofline': roofline, 'roofline_quantizer': roofline_q,
     }

@@ -14,6 +14,9 @@ Differences a caller can observe
   * one process / one GPU: the per-call all-reduce of add_batch is not issued;
   * H is kept valid on and above the diagonal only while it accumulates
     (``hessian(name)`` returns the full symmetric matrix);
+  * Linears of a subset that receive the very same input tensor on every call (q/k/v, gate/up) share one Hessian
+    and one Cholesky chain (``special.auto_share``, default on; detected per call, with a fallback to separate
+    Hessians at the first call that differs; results are bit-identical either way);
   * ``special.hessian_defer`` (default 'auto': 8 for K <= 8192, else 4) add_batch calls are copied to a staging buffer and
     folded into one launch, so ``layers_cache[name]['H']`` lags behind ``nsamples`` until
     ``hessian(name)``, ``hessian_sorting`` or ``process_hessian_and_weights`` settles it
@@ -68,6 +71,8 @@ class GPTQ:
         self.hessian_defer = hd if hd == 'auto' else int(hd)
         # subset_transform starts the Cholesky chains of all Linears of a subset side by side (False: one by one)
         self.chain_overlap = bool(special_config.get('chain_overlap', True))
+        # Linears of a subset that keep receiving the very same input tensor share one Hessian and one chain
+        self.auto_share = bool(special_config.get('auto_share', True))
         if self.owq:
             raise NotImplementedError('OWQ is not on this path')
         if self.blocksize > 128:
@@ -87,7 +92,8 @@ class GPTQ:
         self.layers_cache[name]['H'] = torch.zeros((K, K), device=self.dev)
         self.layers_cache[name]['nsamples'] = 0
         self.layers_cache[name]['n_in_H'] = 0
-        for k in ('stage', 'stage_fill', 'stage_batches'):
+        self.layers_cache[name]['calls'] = 0
+        for k in ('stage', 'stage_fill', 'stage_batches', 'last_stage', 'last_key', 'last_ref', 'manual_share'):
             self.layers_cache[name].pop(k, None)
         self.layers_cache[name]['columns'] = K
         self.layers_cache[name].pop('leader', None)
@@ -106,13 +112,75 @@ class GPTQ:
         for n in names[1:]:
             self.layers_cache[n]['H'] = self.layers_cache[leader]['H']
             self.layers_cache[n]['leader'] = leader
+            self.layers_cache[n]['manual_share'] = True
         self.layers_cache[leader]['leader'] = leader
+        self.layers_cache[leader]['manual_share'] = True
+
+    @staticmethod
+    def _input_key(t):
+        """Identity of an input tensor as the hooks hand it over: same memory, same layout, same version."""
+        return (t.data_ptr(), tuple(t.shape), tuple(t.stride()), t.dtype, t._version)
+
+    def _follow(self, name, cache, key, separable):
+        """Identical inputs need one Hessian.  The hooks of q/k/v (or gate/up) receive the very same tensor on
+        every forward pass (gptq.py:246-251), so a Linear whose every call so far got the tensor that an earlier
+        Linear of the subset got for the same call follows that Linear: it owns no Hessian and no Cholesky chain
+        (the results are bit-identical to separate accumulation, the arithmetic being the same).  Returns True if
+        this call is covered by the Linear it follows.  The first call that differs ends the arrangement: the
+        follower takes a copy of the Hessian and of the staged tokens as they were before that call and goes on
+        alone."""
+        calls = cache['calls']
+        lead_name = cache.get('leader', name)
+        if cache.get('manual_share'):
+            return lead_name != name
+        if lead_name != name:                             # following: does this call match the leader's?
+            lead = self.layers_cache.get(lead_name)
+            if lead is not None and lead.get('calls', 0) == calls + 1 and lead.get('last_key') == key:
+                return True
+            self._unfollow(name, cache, lead)
+            return False
+        if not (self.auto_share and separable) or calls != 0:
+            return False
+        for other, oc in self.layers_cache.items():       # first call: is there a Linear that just got this tensor?
+            if other == name or oc.get('leader', other) != other or 'H' not in oc or oc.get('manual_share'):
+                continue
+            if oc.get('calls', 0) == 1 and oc.get('last_key') == key and oc.get('last_stage', (0, 0))[0] > 0 \
+                    and oc['H'].shape == cache['H'].shape:
+                cache['leader'] = other
+                cache['H'] = oc['H']
+                oc['leader'] = other
+                return True
+        return False
+
+    def _unfollow(self, name, cache, lead):
+        """Give a follower its own Hessian: the state of the Linear it followed, without that Linear's latest call
+        when the follower has not seen it.  (A call that is shared is always still in the staging buffer: a full
+        buffer is folded at the start of the next call, not at the end of the one that filled it.)"""
+        cache['leader'] = name
+        if lead is None or 'H' not in lead:
+            raise L.LcqError(f'{name} followed a Linear whose Hessian is gone')
+        ahead = lead['calls'] - cache['calls']            # 0 or 1
+        fill, batches = lead.get('stage_fill', 0), lead.get('stage_batches', 0)
+        if ahead:
+            t_last, b_last = lead.get('last_stage', (0, 0))
+            if t_last == 0 or fill < t_last:
+                raise L.LcqError(f'{name}: the input differs from the one of {lead.get("leader")} after a call that was '
+                                 'folded into the shared Hessian directly; set special.auto_share: False')
+            fill, batches = fill - t_last, batches - b_last
+        cache['H'] = lead['H'].clone()
+        cache['n_in_H'] = lead.get('n_in_H', 0)
+        cache['upper_only'] = lead.get('upper_only', False)
+        for k in ('stage', 'stage_fill', 'stage_batches', 'last_stage'):
+            cache.pop(k, None)
+        if fill > 0:
+            cache['stage'] = torch.empty_like(lead['stage'])
+            cache['stage'][:fill].copy_(lead['stage'][:fill])
+            cache['stage_fill'], cache['stage_batches'] = fill, batches
 
     @torch.no_grad()
     def add_batch(self, layer, name, inp, out=None):
         cache = self.layers_cache[name]
-        if cache.get('leader', name) != name:
-            return                                      # aliased: the leader accumulates
+        key = self._input_key(inp)
         if len(inp.shape) == 2:
             inp = inp.unsqueeze(0)
         tmp = inp.shape[0]
@@ -122,17 +190,26 @@ class GPTQ:
             raise NotImplementedError(f'add_batch streams bf16/fp16 activations through MFMA; got {inp.dtype}')
         assert inp.shape[0] % self.chunk_num == 0, \
             f'Error: inp.shape[1] ({inp.shape[0]}) cannot be evenly divided by chunk_num.'
-        x = inp.contiguous()
+        defer = self.hessian_fold(inp.shape[1])
+        followed = self._follow(name, cache, key, defer > 1)
+        cache['calls'] += 1
         cache['nsamples'] += tmp
+        if followed:
+            return                                      # the Linear it follows accumulates
+        cache['last_key'] = key
+        cache['last_ref'] = inp                         # keeps the memory from being handed to another tensor meanwhile
+        cache['last_stage'] = (0, 0)
+        x = inp.contiguous()
         cache['upper_only'] = True
-        defer = self.hessian_fold(x.shape[1])
         if defer <= 1:
             self._accumulate(cache, x, tmp)
             return
         # Stage a copy of the tokens and fold several calls into one launch: the window
         # H <- H*n/(n+b1) + 2/(n+b1)*S1, then H <- H*(n+b1)/(n+b1+b2) + 2/(n+b1+b2)*S2, ...
         # telescopes to H*n/N + (2/N)*(S1+S2+...), N = n + b1 + b2 + ..., so one launch over the
-        # concatenated tokens gives the same H while reading and writing it once.
+        # concatenated tokens gives the same H while reading and writing it once.  A full buffer is folded at the
+        # start of the next call that needs room (or when H is asked for), so the latest call can still be told
+        # apart from H when a follower needs the state before it.
         stage = cache.get('stage')
         if stage is not None and (stage.dtype != x.dtype or cache['stage_fill'] + x.shape[0] > stage.shape[0]):
             self._flush(cache)
@@ -150,8 +227,7 @@ class GPTQ:
         stage[f:f + x.shape[0]].copy_(x)
         cache['stage_fill'] = f + x.shape[0]
         cache['stage_batches'] += tmp
-        if cache['stage_fill'] == stage.shape[0]:
-            self._flush(cache)
+        cache['last_stage'] = (x.shape[0], tmp)
 
     def hessian_fold(self, K):
         """add_batch calls folded into one Hessian launch for a Linear with K input features.  'auto': the launch over
@@ -178,6 +254,7 @@ class GPTQ:
             self._accumulate(cache, cache['stage'][:cache['stage_fill']], cache['stage_batches'])
             cache['stage_fill'] = 0
             cache['stage_batches'] = 0
+        cache['last_stage'] = (0, 0)                     # the latest call is inside H now
 
     def _settle(self, name):
         """H of `name` (or of the layer it aliases) with no tokens left in staging."""

@@ -521,3 +521,65 @@ def test_deploy_partials_w_q_and_w_qdq(dev, actorder, sym):
             assert z_out is None
         else:
             assert_bit_equal(z_out, oz, 'w_q zeros')
+
+
+def _subset_run(dev, Ws, feeds, **special):
+    """feeds: list over calls of {name: tensor}; returns per layer (weight, scales, zeros) and the GPTQ object state."""
+    gp = make_gptq(actorder=True, **special)
+    layers = {n: Layer(w.to(dev)) for n, w in Ws.items()}
+    gp.subset_init({'layers': layers})
+    followed = {}
+    for call in feeds:
+        for n, x in call.items():
+            gp.add_batch(layers[n], n, x.data, None)               # hooks pass `inp[0].data`: a fresh alias every call
+        followed = {n: gp.layers_cache[n].get('leader', n) for n in layers}
+    Hs = {n: gp.hessian(n).clone() for n in layers}
+    gp.subset_transform({'layers': layers})
+    torch.cuda.synchronize()
+    out = {n: (layers[n].weight.data.cpu(), layers[n].buf_scales.cpu(), layers[n].buf_zeros.cpu(), Hs[n].cpu()) for n in layers}
+    return out, followed
+
+
+def test_identical_inputs_share_one_hessian_automatically(dev):
+    """q/k/v-style hooks hand the same tensor to every Linear of the subset: one Hessian accumulates, the others
+    follow, and every result is bit-identical to separate accumulation."""
+    K = 640
+    Ws = {'q': (torch.randn(64, K, generator=gen(1)) * 0.02).bfloat16(), 'k': (torch.randn(32, K, generator=gen(2)) * 0.02).bfloat16(),
+          'v': (torch.randn(32, K, generator=gen(3)) * 0.02).bfloat16(), 'other': (torch.randn(48, K, generator=gen(4)) * 0.02).bfloat16()}
+    xs = [b.to(dev) for b in calib_batches(11, 96, K, seed=8300)]
+    ys = [b.to(dev) for b in calib_batches(11, 96, K, seed=8400)]
+    feeds = [{'q': x, 'k': x, 'v': x, 'other': y} for x, y in zip(xs, ys)]
+    shared, followed = _subset_run(dev, Ws, feeds, hessian_defer=4)
+    assert followed == {'q': 'q', 'k': 'q', 'v': 'q', 'other': 'other'}
+    separate, followed2 = _subset_run(dev, Ws, feeds, hessian_defer=4, auto_share=False)
+    assert followed2 == {n: n for n in Ws}
+    for n in Ws:
+        for a, b in zip(shared[n], separate[n]):
+            assert torch.equal(a, b), n
+
+
+@pytest.mark.parametrize('split_at', [1, 4, 5, 8])
+def test_sharing_falls_back_when_an_input_differs(dev, split_at):
+    """The moment one call brings a different tensor the follower continues with its own Hessian - a copy of the
+    shared state as it was before that call - and the final results equal separate accumulation bit for bit."""
+    K = 384
+    Ws = {'a': (torch.randn(32, K, generator=gen(5)) * 0.02).bfloat16(), 'b': (torch.randn(48, K, generator=gen(6)) * 0.02).bfloat16()}
+    xs = [b.to(dev) for b in calib_batches(10, 64, K, seed=8500)]
+    other = calib_batches(1, 64, K, seed=8600)[0].to(dev)
+    feeds = [{'a': x, 'b': (other if i == split_at else x)} for i, x in enumerate(xs)]
+    shared, followed = _subset_run(dev, Ws, feeds, hessian_defer=4)
+    assert followed == {'a': 'a', 'b': 'b'}
+    separate, _ = _subset_run(dev, Ws, feeds, hessian_defer=4, auto_share=False)
+    for n in Ws:
+        for a, b in zip(shared[n], separate[n]):
+            assert torch.equal(a, b), n
+    # same memory, same shape, but modified in place between the two hooks: not the same input any more
+    gp = make_gptq(actorder=True)
+    layers = {n: Layer(w.to(dev)) for n, w in Ws.items()}
+    gp.subset_init({'layers': layers})
+    x = xs[0].clone()
+    gp.add_batch(layers['a'], 'a', x, None)
+    x.mul_(2)
+    gp.add_batch(layers['b'], 'b', x, None)
+    assert gp.layers_cache['b'].get('leader', 'b') == 'b'
+    assert torch.equal(gp.hessian('b'), 4 * gp.hessian('a'))
