@@ -188,6 +188,16 @@ int lcq_pack_awq(const void* w, int dtype, const void* scales, const int32_t* ze
 int lcq_hessian_accum(float* H, int64_t K, const void* X, int dtype, int64_t T, int64_t ldx, float alpha, float beta,
                       void* stream);
 
+/* The same update with different matrices on the two sides:  H <- alpha*H + beta * XA^T XB  on the tiles that reach
+ * the upper triangle (XA supplies the rows of H, XB the columns; both [T, K] with the same ldx and dtype).
+ * add_batch on fp32 activations (gptq.py:289 `chunk.float()`) uses it with the two bf16 halves of
+ * lcq_split_f32_bf16: X^T X = hi^T hi + hi^T lo + lo^T hi + lo^T lo. */
+int lcq_hessian_accum_ab(float* H, int64_t K, const void* XA, const void* XB, int dtype, int64_t T, int64_t ldx, float alpha,
+                         float beta, void* stream);
+
+/* x [n] fp32 -> hi = bf16(x), lo = bf16(x - hi)  ([n] bf16 each; n % 4 == 0): x == hi + lo to 2^-17 relative. */
+int lcq_split_f32_bf16(const float* x, int64_t n, void* hi, void* lo, void* stream);
+
 /* H[j][i] = H[i][j] for i < j. */
 int lcq_symmetrize(float* H, int64_t K, void* stream);
 

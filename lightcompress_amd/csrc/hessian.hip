@@ -110,8 +110,8 @@ template <int TN> struct HessCfg {
 // EDGE = false: K % 256 == 0 and T % 32 == 0, no bounds checks anywhere.
 template <bool IS_BF16, bool EDGE, int TN>
 __global__ __launch_bounds__(HessCfg<TN>::NW * 64, TN == 256 ? 1 : 2)
-void hessian_kernel(float* __restrict__ H, int K, const uint16_t* __restrict__ X, int ldx, int T, float alpha,
-                    float beta, int ntr, int ntc, int total) {
+void hessian_kernel(float* __restrict__ H, int K, const uint16_t* __restrict__ X, const uint16_t* __restrict__ XB, int ldx,
+                    int T, float alpha, float beta, int ntr, int ntc, int total) {
   using C = HessCfg<TN>;
   constexpr int ROW_B = C::ROW_B, STAGE = C::STAGE, NSTAGE = C::NSTAGE, LA = C::LA, LB = C::LB, RB = C::RB;
   __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE];
@@ -158,7 +158,8 @@ void hessian_kernel(float* __restrict__ H, int K, const uint16_t* __restrict__ X
   // loads (vmcnt(0)) before any LDS read, which serialises the pipeline.  Waits are explicit below.
   const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
   auto gload = [&](int t0, int stage) {
-    const uint16_t* Xs = X + (int64_t)t0 * ldx;
+    const uint16_t* Xs = X + (int64_t)t0 * ldx;              // rows of H come from X ...
+    const uint16_t* XsB = XB + (int64_t)t0 * ldx;            // ... columns from XB (the same matrix for X^T X)
     const uint32_t dA = lds0 + stage * STAGE + wave * LA * 1024;
     const uint32_t dB = lds0 + stage * STAGE + BYTES_A + wave * LB * 1024;
     #pragma unroll
@@ -169,10 +170,10 @@ void hessian_kernel(float* __restrict__ H, int K, const uint16_t* __restrict__ X
       if constexpr (EDGE) {
         const int r = isA ? rowA[isA ? p : 0] : rowB[isA ? 0 : p - LA];
         const bool ok = (isA ? okA[isA ? p : 0] : okB[isA ? 0 : p - LA]) && t0 + r < T;
-        const uint16_t* g = ok ? Xs + gof : (const uint16_t*)zero_piece;
+        const uint16_t* g = ok ? (isA ? Xs : XsB) + gof : (const uint16_t*)zero_piece;
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(g) : "memory");
       } else {
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(gof * 2u), "s"(Xs) : "memory");
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(gof * 2u), "s"(isA ? Xs : XsB) : "memory");
       }
     }
   };
@@ -278,6 +279,20 @@ void hessian_kernel(float* __restrict__ H, int K, const uint16_t* __restrict__ X
   }
 }
 
+// x (fp32) -> hi = bf16(x), lo = bf16(x - hi): x = hi + lo up to 2^-17 relative, and every product of two such
+// halves is exact in fp32, so fp32 activations go through the bf16 matrix pipe as four products (hi/lo x hi/lo).
+__global__ __launch_bounds__(256) void split_f32_kernel(const f32x4* __restrict__ x, int64_t n4, u32x2* __restrict__ hi,
+                                                        u32x2* __restrict__ lo) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256) {
+    const f32x4 v = __builtin_nontemporal_load(x + i);
+    float h[4], l[4];
+    #pragma unroll
+    for (int k = 0; k < 4; ++k) { h[k] = bf16_round(v[k]); l[k] = bf16_round(v[k] - h[k]); }
+    hi[i] = u32x2{bf16_pack(h[0], h[1]), bf16_pack(h[2], h[3])};
+    lo[i] = u32x2{bf16_pack(l[0], l[1]), bf16_pack(l[2], l[3])};
+  }
+}
+
 // fill the lower triangle from the upper one: H[j][i] = H[i][j], i < j
 __global__ __launch_bounds__(256) void symmetrize_kernel(float* __restrict__ H, int K) {
   __shared__ float tile[32][33];
@@ -301,9 +316,14 @@ extern "C" {
 
 int lcq_hessian_accum(float* H, int64_t K, const void* X, int dtype, int64_t T, int64_t ldx, float alpha, float beta,
                       void* stream) {
-  if (!H || !X || K <= 0 || T < 0) return LCQ_EINVAL;
+  return lcq_hessian_accum_ab(H, K, X, X, dtype, T, ldx, alpha, beta, stream);
+}
+
+int lcq_hessian_accum_ab(float* H, int64_t K, const void* X, const void* XB, int dtype, int64_t T, int64_t ldx, float alpha,
+                         float beta, void* stream) {
+  if (!H || !X || !XB || K <= 0 || T < 0) return LCQ_EINVAL;
   if (K % 8 != 0 || K > (1 << 20) || T > 0x7fffffff || ldx < K || ldx % 8 != 0 || ldx > (1 << 21)) return LCQ_EINVAL;
-  if (((uintptr_t)X % 16) != 0 || ((uintptr_t)H % 4) != 0) return LCQ_EALIGN;
+  if (((uintptr_t)X % 16) != 0 || ((uintptr_t)XB % 16) != 0 || ((uintptr_t)H % 4) != 0) return LCQ_EALIGN;
   if (T == 0) return LCQ_OK;
   constexpr int TN = 128;
   const int ntr = (int)((K + TM - 1) / TM), ntc = (int)((K + TN - 1) / TN), q = TM / TN;
@@ -313,11 +333,22 @@ int lcq_hessian_accum(float* H, int64_t K, const void* X, int dtype, int64_t T, 
   hipStream_t st = (hipStream_t)stream;
   const bool edge = (K % TM != 0) || (T % BT != 0);
   #define LCQ_HESS(BF, E) hessian_kernel<BF, E, TN><<<dim3((unsigned)grid), dim3(HessCfg<TN>::NW * 64), 0, st>>>( \
-      H, (int)K, (const uint16_t*)X, (int)ldx, (int)T, alpha, beta, ntr, ntc, (int)total)
+      H, (int)K, (const uint16_t*)X, (const uint16_t*)XB, (int)ldx, (int)T, alpha, beta, ntr, ntc, (int)total)
   if (dtype == LCQ_BF16) { if (edge) LCQ_HESS(true, true); else LCQ_HESS(true, false); }
   else if (dtype == LCQ_F16) { if (edge) LCQ_HESS(false, true); else LCQ_HESS(false, false); }
   else return LCQ_EDTYPE;
   #undef LCQ_HESS
+  LCQ_CHECK_LAUNCH();
+  return LCQ_OK;
+}
+
+int lcq_split_f32_bf16(const float* x, int64_t n, void* hi, void* lo, void* stream) {
+  if (!x || !hi || !lo || n < 0 || n % 4 != 0) return LCQ_EINVAL;
+  if ((((uintptr_t)x % 16) | ((uintptr_t)hi % 8) | ((uintptr_t)lo % 8)) != 0) return LCQ_EALIGN;
+  if (n == 0) return LCQ_OK;
+  int64_t grid = (n / 4 + 255) / 256;
+  if (grid > 65536 * 4) grid = 65536 * 4;
+  split_f32_kernel<<<dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream>>>((const f32x4*)x, n / 4, (u32x2*)hi, (u32x2*)lo);
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;
 }

@@ -24,6 +24,8 @@ Differences a caller can observe
   * per-group qparams of the loop live in two [R, G] tensors instead of a
     Python list of dicts; ``layer.buf_scales`` / ``buf_zeros`` get the same
     [R*G, 1] layout the reference writes;
+  * fp32 activations are split into two bf16 halves (x = hi + lo to 2^-17) and accumulated as the four products of
+    the halves on the bf16 matrix pipe; bf16 / fp16 activations go in as they are (their products are exact in fp32);
   * OWQ (outlier columns kept in fp16) is not carried over.
 """
 from __future__ import annotations
@@ -93,7 +95,7 @@ class GPTQ:
         self.layers_cache[name]['nsamples'] = 0
         self.layers_cache[name]['n_in_H'] = 0
         self.layers_cache[name]['calls'] = 0
-        for k in ('stage', 'stage_fill', 'stage_batches', 'last_stage', 'last_key', 'last_ref', 'manual_share'):
+        for k in ('stage', 'stage_lo', 'stage_fill', 'stage_batches', 'last_stage', 'last_key', 'last_ref', 'manual_share'):
             self.layers_cache[name].pop(k, None)
         self.layers_cache[name]['columns'] = K
         self.layers_cache[name].pop('leader', None)
@@ -170,11 +172,15 @@ class GPTQ:
         cache['H'] = lead['H'].clone()
         cache['n_in_H'] = lead.get('n_in_H', 0)
         cache['upper_only'] = lead.get('upper_only', False)
-        for k in ('stage', 'stage_fill', 'stage_batches', 'last_stage'):
+        for k in ('stage', 'stage_lo', 'stage_fill', 'stage_batches', 'last_stage'):
             cache.pop(k, None)
         if fill > 0:
             cache['stage'] = torch.empty_like(lead['stage'])
             cache['stage'][:fill].copy_(lead['stage'][:fill])
+            cache['stage_lo'] = None
+            if lead.get('stage_lo') is not None:
+                cache['stage_lo'] = torch.empty_like(lead['stage_lo'])
+                cache['stage_lo'][:fill].copy_(lead['stage_lo'][:fill])
             cache['stage_fill'], cache['stage_batches'] = fill, batches
 
     @torch.no_grad()
@@ -186,8 +192,8 @@ class GPTQ:
         tmp = inp.shape[0]
         if len(inp.shape) == 3:
             inp = inp.reshape((-1, inp.shape[-1]))
-        if inp.dtype not in (torch.bfloat16, torch.float16):
-            raise NotImplementedError(f'add_batch streams bf16/fp16 activations through MFMA; got {inp.dtype}')
+        if inp.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+            raise NotImplementedError(f'add_batch takes bf16 / fp16 / fp32 activations; got {inp.dtype}')
         assert inp.shape[0] % self.chunk_num == 0, \
             f'Error: inp.shape[1] ({inp.shape[0]}) cannot be evenly divided by chunk_num.'
         defer = self.hessian_fold(inp.shape[1])
@@ -201,8 +207,10 @@ class GPTQ:
         cache['last_stage'] = (0, 0)
         x = inp.contiguous()
         cache['upper_only'] = True
+        # fp32 activations (gptq.py:289 `chunk.float()` keeps them fp32): staged as two bf16 halves, x = hi + lo
+        sdtype = torch.bfloat16 if x.dtype == torch.float32 else x.dtype
         if defer <= 1:
-            self._accumulate(cache, x, tmp)
+            self._accumulate(cache, *self._halves(x), tmp)
             return
         # Stage a copy of the tokens and fold several calls into one launch: the window
         # H <- H*n/(n+b1) + 2/(n+b1)*S1, then H <- H*(n+b1)/(n+b1+b2) + 2/(n+b1+b2)*S2, ...
@@ -211,20 +219,26 @@ class GPTQ:
         # start of the next call that needs room (or when H is asked for), so the latest call can still be told
         # apart from H when a follower needs the state before it.
         stage = cache.get('stage')
-        if stage is not None and (stage.dtype != x.dtype or cache['stage_fill'] + x.shape[0] > stage.shape[0]):
+        split = x.dtype == torch.float32
+        if stage is not None and (stage.dtype != sdtype or split != (cache.get('stage_lo') is not None)
+                                  or cache['stage_fill'] + x.shape[0] > stage.shape[0]):
             self._flush(cache)
-            if stage.dtype != x.dtype:
+            if stage.dtype != sdtype or split != (cache.get('stage_lo') is not None):
                 stage = None
         if stage is None:
-            stage = torch.empty((defer * x.shape[0], x.shape[1]), dtype=x.dtype, device=x.device)
+            stage = torch.empty((defer * x.shape[0], x.shape[1]), dtype=sdtype, device=x.device)
             cache['stage'] = stage
+            cache['stage_lo'] = torch.empty_like(stage) if split else None
             cache['stage_fill'] = 0
             cache['stage_batches'] = 0
         if x.shape[0] > stage.shape[0]:
-            self._accumulate(cache, x, tmp)
+            self._accumulate(cache, *self._halves(x), tmp)
             return
         f = cache['stage_fill']
-        stage[f:f + x.shape[0]].copy_(x)
+        if split:
+            self._halves(x, stage[f:f + x.shape[0]], cache['stage_lo'][f:f + x.shape[0]])
+        else:
+            stage[f:f + x.shape[0]].copy_(x)
         cache['stage_fill'] = f + x.shape[0]
         cache['stage_batches'] += tmp
         cache['last_stage'] = (x.shape[0], tmp)
@@ -236,22 +250,40 @@ class GPTQ:
             return 8 if K <= 8192 else 4
         return self.hessian_defer
 
-    def _accumulate(self, cache, x, batches):
+    def _halves(self, x, hi=None, lo=None):
+        """(x, None) for 16-bit activations; for fp32 the two bf16 halves hi = bf16(x), lo = bf16(x - hi)."""
+        if x.dtype != torch.float32:
+            return x, None
+        hi = torch.empty(x.shape, dtype=torch.bfloat16, device=x.device) if hi is None else hi
+        lo = torch.empty(x.shape, dtype=torch.bfloat16, device=x.device) if lo is None else lo
+        L.check(L.lib().lcq_split_f32_bf16(L.ptr(x), L.i64(x.numel()), L.ptr(hi), L.ptr(lo), L.stream()), 'lcq_split_f32_bf16')
+        return hi, lo
+
+    def _accumulate(self, cache, x, x_lo, batches):
         """H <- H*n/(n+b) + 2/(n+b) * x^T x for the n batches already inside H (gptq.py:279-294).
-        x: [tokens, K] view with unit column stride (rows may be padded)."""
+        x: [tokens, K] view with unit column stride (rows may be padded); x_lo: the low halves of fp32 activations
+        (then x holds the high halves and x^T x is the sum of the four products of the halves)."""
         n = cache.get('n_in_H', 0)
         alpha = n / (n + batches)
         beta = 2.0 / (n + batches)
         cache['n_in_H'] = n + batches
         H = cache['H']
-        L.check(L.lib().lcq_hessian_accum(L.ptr(H), L.i64(H.shape[0]), L.ptr(x), L.i32(L.dtype_code(x.dtype)),
-                                          L.i64(x.shape[0]), L.i64(x.stride(0)), L.f32(alpha), L.f32(beta), L.stream()),
-                'lcq_hessian_accum')
+        lib, code = L.lib(), L.i32(L.dtype_code(x.dtype))
+        dims = (L.i64(x.shape[0]), L.i64(x.stride(0)))
+        if x_lo is None:
+            L.check(lib.lcq_hessian_accum(L.ptr(H), L.i64(H.shape[0]), L.ptr(x), code, *dims, L.f32(alpha), L.f32(beta),
+                                          L.stream()), 'lcq_hessian_accum')
+            return
+        for a, b, al in ((x_lo, x_lo, alpha), (x, x_lo, 1.0), (x_lo, x, 1.0), (x, x, 1.0)):      # small terms first
+            L.check(lib.lcq_hessian_accum_ab(L.ptr(H), L.i64(H.shape[0]), L.ptr(a), L.ptr(b), code, *dims, L.f32(al),
+                                             L.f32(beta), L.stream()), 'lcq_hessian_accum_ab')
 
     def _flush(self, cache):
         """Fold the staged tokens into H."""
         if cache.get('stage_fill', 0) > 0:
-            self._accumulate(cache, cache['stage'][:cache['stage_fill']], cache['stage_batches'])
+            lo = cache.get('stage_lo')
+            self._accumulate(cache, cache['stage'][:cache['stage_fill']], None if lo is None else lo[:cache['stage_fill']],
+                             cache['stage_batches'])
             cache['stage_fill'] = 0
             cache['stage_batches'] = 0
         cache['last_stage'] = (0, 0)                     # the latest call is inside H now
@@ -262,6 +294,7 @@ class GPTQ:
         lead = self.layers_cache.get(cache.get('leader', name), cache)
         self._flush(lead)
         lead.pop('stage', None)
+        lead.pop('stage_lo', None)
         return cache
 
     def hessian(self, name):

@@ -583,3 +583,32 @@ def test_sharing_falls_back_when_an_input_differs(dev, split_at):
     gp.add_batch(layers['b'], 'b', x, None)
     assert gp.layers_cache['b'].get('leader', 'b') == 'b'
     assert torch.equal(gp.hessian('b'), 4 * gp.hessian('a'))
+
+
+@pytest.mark.parametrize('defer', [1, 'auto'])
+@pytest.mark.parametrize('K,T,nb', [(512, 100, 5), (1000, 33, 3), (2048, 512, 2)])
+def test_hessian_from_fp32_activations(dev, K, T, nb, defer):
+    """add_batch upcasts with .float() (gptq.py:289), so fp32 activations count in full precision: the kernel takes
+    them as two bf16 halves (four exact products) and must stay within 1e-5 of the fp64 closed form and of the fp32
+    oracle - rounding the activations to bf16 first would not."""
+    g = gen(8700 + K)
+    sigma = torch.exp(torch.randn(K, generator=g))
+    batches = [torch.randn(T, K, generator=g) * sigma for _ in range(nb)]
+    gp = make_gptq(hessian_defer=defer)
+    layer = Layer(torch.zeros(8, K, device=dev))
+    gp.layers_cache['l'] = {}
+    gp.layer_init(layer, 'l')
+    Ho, n = torch.zeros(K, K), 0
+    for b in batches:
+        gp.add_batch(layer, 'l', b.unsqueeze(0).to(dev), None)
+        n = G.add_batch(Ho, n, b.unsqueeze(0))
+    H = gp.hessian('l').cpu()
+    ref64 = G.hessian_closed_form(batches)
+    scale = float(ref64.abs().max())
+    assert float((H.double() - ref64).abs().max()) / scale < 1e-5
+    assert float((H - Ho).abs().max()) / scale < 1e-5
+    assert float((H.double() - ref64).norm() / ref64.norm()) < 1e-5
+    assert torch.equal(H, H.t())
+    # the bf16-rounded activations are a different matrix at this tolerance
+    rounded = G.hessian_closed_form([b.bfloat16() for b in batches])
+    assert float((rounded - ref64).abs().max()) / scale > 1e-4
