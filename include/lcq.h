@@ -293,6 +293,16 @@ int lcq_awq_clip_search(const void* w, const void* x, int64_t R, int64_t K, int6
                         int clip_sym, float qmin, float qmax, int flags, void* best_max, void* best_min, float* errs,
                         void* stream);
 
+/* The grouped products of AutoClipper.auto_clip_layer, auto_clip.py:141,160: `(x * w).sum(dim=-1)` with
+ * x [1, T, G, gs] and w [R, 1, G, gs]:  out[r, g, t] = round(sum_j round(x[t, g*gs + j] * w[r, g*gs + j])) - every
+ * product rounded to the tensors' type as the materialised product tensor is, fp32 accumulation, one final rounding
+ * (the reference's [R, T, G] result, stored with the token index fastest).
+ * With org != NULL (such sums for the original weights, same layout) nothing is stored in `out` (may be NULL) and
+ *   err[r, g] = round(mean_t round(round(out - org)^2))        auto_clip.py:163, `(cur_out - org_out).pow(2).mean(dim=1)`
+ *  x [T, K], w [R, K], out / org [R, K / group_size, T], err [R, K / group_size], all of `dtype` (LCQ_F32 | LCQ_BF16). */
+int lcq_group_dots(const void* x, const void* w, int dtype, int64_t R, int64_t K, int64_t T, int group_size, void* out,
+                   const void* org, void* err, void* stream);
+
 /* AutoClipper.apply_clip v1, auto_clip.py:194-211: out[r, g*gs + j] = clamp(w[r, g*gs + j], lo[r, g], hi[r, g]);
  * w, out [R, K] of `dtype` (LCQ_F32 | LCQ_BF16), lo / hi [R, K / group_size] of `dtype`; out may alias w. */
 int lcq_clamp_groups(const void* w, int dtype, int64_t R, int64_t K, int group_size, const void* lo, const void* hi,

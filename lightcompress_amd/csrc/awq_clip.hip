@@ -141,9 +141,141 @@ __global__ __launch_bounds__(256) void clamp_groups_kernel(const u32x4* __restri
   }
 }
 
+// the same clamp element by element, for group sizes that do not fill 16-byte chunks
+template <bool BF>
+__global__ __launch_bounds__(256) void clamp_groups_scalar_kernel(const void* __restrict__ w, int64_t n, int gs,
+                                                                  const void* __restrict__ lo, const void* __restrict__ hi,
+                                                                  void* __restrict__ out) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    const int64_t grp = i / gs;
+    store_scalar<BF>(out, i, nan_min(nan_max(load_scalar<BF>(w, i), load_scalar<BF>(lo, grp)), load_scalar<BF>(hi, grp)));
+  }
+}
+
+// out[r, g, t] = round( sum_j round(x[t, g*gs + j] * w[r, g*gs + j]) ): the reference's (x * w).sum(dim=-1) of
+// auto_clip.py:141,160 on x [1, T, G, gs] and w [R, 1, G, gs] - the product tensor is materialised in the tensors'
+// type there (every product rounded), the sum accumulates in fp32 and rounds once.  General in the group size, the
+// element type and which tensors are multiplied, so it serves every configuration the MFMA search kernel leaves out
+// (activation fake-quant, learnable ranges, other group sizes) and reproduces the reference's rounding sequence.
+// With `org` (the same sums for the original weights) the sums are not stored; the kernel goes on to
+//   err[r, g] = round( mean_t round( round(out - org)^2 ) )                    (auto_clip.py:163)
+// One workgroup: 64 rows x one group, looping over 64-token tiles and 128-column chunks staged in LDS as fp32; thread
+// (ty, tx) = (tid / 16, tid % 16) owns rows ty + 16 a and tokens tx + 16 b (a, b = 0..3): 8 LDS reads per 16 products.
+constexpr int GD_J = 128, GD_P = GD_J + 1, GD_M = 64;
+template <bool BF>
+__device__ __forceinline__ void gd_stage(float (*S)[GD_P], const void* __restrict__ src, int row0, int nrows, int K,
+                                         int64_t col0, int nj, bool vec, int tid) {
+  constexpr int N = Vec<BF>::N;
+  if (vec) {                                                // 16-byte pieces: K, the group offset and nj are multiples of N
+    for (int e = tid; e < GD_M * (GD_J / N); e += 256) {
+      const int rr = e / (GD_J / N), c = (e % (GD_J / N)) * N;
+      float v[N];
+      #pragma unroll
+      for (int i = 0; i < N; ++i) v[i] = 0.0f;
+      if (rr + row0 < nrows && c < nj) {
+        const char* p = (const char*)src + ((int64_t)(row0 + rr) * K + col0 + c) * (BF ? 2 : 4);
+        unpack<BF>(*(const u32x4*)p, v);
+      }
+      #pragma unroll
+      for (int i = 0; i < N; ++i) S[rr][c + i] = v[i];
+    }
+  } else {
+    for (int e = tid; e < GD_M * GD_J; e += 256) {
+      const int rr = e / GD_J, j = e % GD_J;
+      S[rr][j] = (j < nj && row0 + rr < nrows) ? load_scalar<BF>(src, (int64_t)(row0 + rr) * K + col0 + j) : 0.0f;
+    }
+  }
+}
+
+template <bool BF>
+__global__ __launch_bounds__(256) void group_dots_kernel(const void* __restrict__ x, const void* __restrict__ w, int R, int K,
+                                                         int T, int gs, int vec, void* __restrict__ out,
+                                                         const void* __restrict__ org, void* __restrict__ err) {
+  __shared__ float Xs[GD_M][GD_P], Ws[GD_M][GD_P];
+  const int tid = threadIdx.x, G = K / gs, g = blockIdx.y;
+  const int r0 = blockIdx.x * GD_M, ty = tid >> 4, tx = tid & 15;
+  const bool one_chunk = gs <= GD_J;
+  float esum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (one_chunk) gd_stage<BF>(Ws, w, r0, R, K, (int64_t)g * gs, gs, vec, tid);
+  for (int t0 = 0; t0 < T; t0 += GD_M) {
+    float acc[4][4];
+    #pragma unroll
+    for (int a = 0; a < 4; ++a)
+      #pragma unroll
+      for (int b = 0; b < 4; ++b) acc[a][b] = 0.0f;
+    for (int j0 = 0; j0 < gs; j0 += GD_J) {
+      const int nj = min(GD_J, gs - j0);
+      __syncthreads();
+      gd_stage<BF>(Xs, x, t0, T, K, (int64_t)g * gs + j0, nj, vec, tid);
+      if (!one_chunk) gd_stage<BF>(Ws, w, r0, R, K, (int64_t)g * gs + j0, nj, vec, tid);
+      __syncthreads();
+      for (int j = 0; j < nj; ++j) {
+        float wv[4], xv[4];
+        #pragma unroll
+        for (int a = 0; a < 4; ++a) wv[a] = Ws[ty + 16 * a][j];
+        #pragma unroll
+        for (int b = 0; b < 4; ++b) xv[b] = Xs[tx + 16 * b][j];
+        #pragma unroll
+        for (int a = 0; a < 4; ++a)
+          #pragma unroll
+          for (int b = 0; b < 4; b += 2) {
+            float p0 = xv[b] * wv[a], p1 = xv[b + 1] * wv[a];
+            rnd_pair<BF>(p0, p1);
+            acc[a][b] += p0;
+            acc[a][b + 1] += p1;
+          }
+      }
+    }
+    #pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const int r = r0 + ty + 16 * a;
+      #pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int t = t0 + tx + 16 * b;
+        if (r < R && t < T) {
+          const int64_t at = ((int64_t)r * G + g) * T + t;
+          const float v = rnd_e<BF>(acc[a][b]);
+          if (org) {
+            const float d = rnd_e<BF>(v - load_scalar<BF>(org, at));
+            esum[a] += rnd_e<BF>(d * d);
+          } else {
+            store_scalar<BF>(out, at, v);
+          }
+        }
+      }
+    }
+  }
+  if (org) {
+    #pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const float s = team_sum<16>(esum[a]);
+      const int r = r0 + ty + 16 * a;
+      if (tx == 0 && r < R) store_scalar<BF>(err, (int64_t)r * G + g, rnd_e<BF>(s * (1.0f / (float)T)));
+    }
+  }
+}
+
 }  // namespace
 
 extern "C" {
+
+int lcq_group_dots(const void* x, const void* w, int dtype, int64_t R, int64_t K, int64_t T, int group_size, void* out,
+                   const void* org, void* err, void* stream) {
+  if (!x || !w || R <= 0 || K <= 0 || T <= 0 || group_size <= 0 || K % group_size != 0) return LCQ_EINVAL;
+  if ((org && !err) || (!org && !out)) return LCQ_EINVAL;
+  if (R > 0x7fffffff || K > 0x7fffffff || T > 0x7fffffff || K / group_size > 65535) return LCQ_EINVAL;
+  if (dtype != LCQ_BF16 && dtype != LCQ_F32) return LCQ_EDTYPE;
+  const int n = dtype == LCQ_BF16 ? 8 : 4;
+  const int vec = (K % n == 0 && group_size % n == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0) ? 1 : 0;
+  const dim3 grid((unsigned)((R + GD_M - 1) / GD_M), (unsigned)(K / group_size));
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == LCQ_BF16)
+    group_dots_kernel<true><<<grid, dim3(256), 0, st>>>(x, w, (int)R, (int)K, (int)T, group_size, vec, out, org, err);
+  else
+    group_dots_kernel<false><<<grid, dim3(256), 0, st>>>(x, w, (int)R, (int)K, (int)T, group_size, vec, out, org, err);
+  LCQ_CHECK_LAUNCH();
+  return LCQ_OK;
+}
 
 int lcq_awq_clip_search(const void* w, const void* x, int64_t R, int64_t K, int64_t T, int n_grid, int n_steps,
                         int clip_sym, float qmin, float qmax, int flags, void* best_max, void* best_min, float* errs,
@@ -171,12 +303,18 @@ int lcq_clamp_groups(const void* w, int dtype, int64_t R, int64_t K, int group_s
   if (!w || !lo || !hi || !out || R <= 0 || K <= 0 || group_size <= 0 || K % group_size != 0) return LCQ_EINVAL;
   if (dtype != LCQ_F32 && dtype != LCQ_BF16) return LCQ_EDTYPE;
   const int n = dtype == LCQ_BF16 ? 8 : 4;
-  if (group_size % n != 0) return LCQ_EINVAL;
-  if ((((uintptr_t)w | (uintptr_t)out) % 16) != 0) return LCQ_EALIGN;
+  hipStream_t st = (hipStream_t)stream;
+  if (group_size % n != 0 || (((uintptr_t)w | (uintptr_t)out) % 16) != 0) {
+    int64_t grid = (R * K + 255) / 256;
+    if (grid > 262144) grid = 262144;
+    if (dtype == LCQ_BF16) clamp_groups_scalar_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>(w, R * K, group_size, lo, hi, out);
+    else clamp_groups_scalar_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>(w, R * K, group_size, lo, hi, out);
+    LCQ_CHECK_LAUNCH();
+    return LCQ_OK;
+  }
   const int64_t nchunks = R * K / n;
   int64_t grid = (nchunks + 255) / 256;
   if (grid > 262144) grid = 262144;
-  hipStream_t st = (hipStream_t)stream;
   if (dtype == LCQ_BF16) clamp_groups_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)w, nchunks, group_size / n, lo, hi, (u32x4*)out);
   else clamp_groups_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)w, nchunks, group_size / n, lo, hi, (u32x4*)out);
   LCQ_CHECK_LAUNCH();

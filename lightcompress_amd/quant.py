@@ -9,9 +9,10 @@ Every arithmetic method launches hand-written gfx950 kernels through the C
 ABI in ``include/lcq.h``.  There is no CPU path: CPU tensors raise
 ``LcqError``.  Reshapes/views, index mixing and dtype casts stay in torch.
 
-Not carried over (they raise ``NotImplementedError``): the ``mse`` /
-``learnable`` / ``hqq`` / ``static_hist`` calibrators, STE rounding (training
-only) and the ``rounding`` override of ``fake_quant_weight_static``.  ``per_block`` granularity runs for
+``calib_algo``: ``minmax``, ``mse``, ``hqq``, ``learnable`` (the sigmoid-scaled range with GIVEN factors; training
+them needs autograd and is not here), ``static_minmax`` / ``static_moving_minmax`` for activations.
+Not carried over (they raise ``NotImplementedError``): STE rounding (training only) and the ``rounding`` override of
+``fake_quant_weight_static``.  ``per_block`` granularity runs for
 ``FloatQuantizer('e4m3')`` weights only (``real_quant_weight_dynamic`` / ``fake_quant_weight_dynamic``).
 """
 from __future__ import annotations
@@ -55,6 +56,7 @@ class BaseQuantizer(object):
         if self.kwargs.get('ste', False) or self.kwargs.get('ste_all', False):
             raise NotImplementedError('straight-through rounding is a training feature; not on this path')
         self.round_func = torch.round
+        self.sigmoid = torch.nn.Sigmoid()
         self.ste_all = False
         self.round_zp = self.kwargs.get('round_zp', True)
 
@@ -65,9 +67,26 @@ class BaseQuantizer(object):
         if self.calib_algo == 'mse':
             return self.get_mse_range(tensor)
         if self.calib_algo == 'learnable':
-            raise NotImplementedError("calib_algo='learnable' (sigmoid-scaled clipping, quant.py:207-221) belongs to the "
-                                      'gradient-trained methods; this path has no autograd')
+            return self.get_learnable_range(tensor, **args)
         return self.get_minmax_range(tensor)                 # quant.py:131-132: anything else falls back to minmax
+
+    def get_learnable_range(self, tensor, lowbound_factor=None, upbound_factor=None):
+        """quant.py:207-221: the min/max range scaled by sigmoid(factor).  The factors are inputs here (found by
+        AutoClipper v2 or loaded); training them needs autograd and is not on this path.  Range kernels on the
+        tensor, the handful of per-row scalars in torch like the reference."""
+        min_val, max_val = self.get_minmax_range(tensor)
+        if self.sym:
+            if upbound_factor is not None:
+                abs_max = torch.max(max_val.abs(), min_val.abs())
+                abs_max = abs_max.clamp(min=1e-5)
+                abs_max = self.sigmoid(upbound_factor) * abs_max
+                min_val = -abs_max
+                max_val = abs_max
+        else:
+            if upbound_factor is not None and lowbound_factor is not None:
+                min_val = self.sigmoid(lowbound_factor) * min_val
+                max_val = self.sigmoid(upbound_factor) * max_val
+        return (min_val, max_val)
 
     def get_mse_range(self, tensor, norm=2.4, bs=256):
         """quant.py:147-205 -> fp32 (min_val, max_val) [rows, 1]: the shrunken range with the smallest
@@ -449,11 +468,13 @@ class IntegerQuantizer(BaseQuantizer):
                                    osf=output_scale_factor, qmin=qmin, qmax=qmax)
         return dq.view(tensor.shape)
 
-    def _fake_dynamic(self, t):
+    def _fake_dynamic(self, t, args={}):
         shape, dtype = t.shape, t.dtype
         rows_t = self.reshape_tensor(t)
         if self.calib_algo != 'minmax':                  # calibrated ranges, then the static path (quant.py:853-860)
-            rows_t, scales, zeros, qmax, qmin = self.get_tensor_qparams(t)
+            rargs = {k: args[k] for k in ('lowbound_factor', 'upbound_factor') if k in args} \
+                if self.calib_algo == 'learnable' else {}
+            rows_t, scales, zeros, qmax, qmin = self.get_tensor_qparams(t, rargs)
             dq, _, _, _ = self._launch(rows_t, static=True, scales=scales, zeros=zeros, want_dq=True, qmin=qmin, qmax=qmax)
             return self.restore_tensor(dq.view(rows_t.shape), shape).to(dtype)
         dq, _, _, _ = self._launch(rows_t, static=False, want_dq=True)
@@ -526,7 +547,7 @@ class IntegerQuantizer(BaseQuantizer):
     def fake_quant_weight_dynamic(self, weight, args={}):
         """quant.py:832-868."""
         q_weight, fp_weight = self._weight_view(weight, args)
-        q_weight = self._fake_dynamic(q_weight)
+        q_weight = self._fake_dynamic(q_weight, args)
         return self._weight_merge(weight, q_weight, fp_weight, args)
 
     def _code_dtype(self):

@@ -143,13 +143,55 @@ def search_scale_inputs(weights: dict, inputs: list, forward, spec, n_grid=20, v
 
 
 # ----------------------------------------------------------------------------
-# AutoClipper (weight-only, clip_version v1)
+# AutoClipper
 # ----------------------------------------------------------------------------
-def auto_clip_layer(spec, w, inputs, clip_sym=False, n_grid=20, max_shrink=0.5, n_sample_token=512):
-    """auto_clip.py:83-191 on CPU tensors, op for op (w_only, clip_version v1): for each batch of output rows the
-    [ocb, T, G, g] products of the sampled inputs with the original and with the clamped + fake-quantized weights,
-    their sums over g, the mean squared difference over tokens, and the running `err < min_errs` selection over
-    the shrink steps.  Returns (best_max [R, G, 1], best_min [R, G, 1], errs [R, G, n_steps] as computed)."""
+def _logit(x):
+    return torch.log(x / (1 - x))                       # auto_clip.py:42
+
+
+def learnable_range(spec, tensor, lowbound_factor=None, upbound_factor=None):
+    """get_learnable_range, quant.py:207-221: the min/max range scaled by sigmoid(factor)."""
+    min_val, max_val = Q.minmax_range(spec, tensor)
+    if spec.symmetric:
+        if upbound_factor is not None:
+            abs_max = torch.max(max_val.abs(), min_val.abs())
+            abs_max = abs_max.clamp(min=1e-5)
+            abs_max = torch.sigmoid(upbound_factor) * abs_max
+            min_val = -abs_max
+            max_val = abs_max
+    else:
+        if upbound_factor is not None and lowbound_factor is not None:
+            min_val = torch.sigmoid(lowbound_factor) * min_val
+            max_val = torch.sigmoid(upbound_factor) * max_val
+    return min_val, max_val
+
+
+def clip_fake_quantize_weight(spec, w, min_val, max_val, org_min_val, org_max_val, clip_version='v1'):
+    """AutoClipper.fake_quantize_weight, auto_clip.py:258-274, on w [ocb, 1, G, gs].  v2 quantizes with the qparams of
+    the learnable range; the reference's static fake quant flattens w to [ocb * G, gs] rows first, which only
+    broadcasts against the [ocb, 1, G, 1] qparams when they hold one entry per row in the same order - written here
+    with the qparams flattened the same way (identical for per_channel, G = 1; the reference fails for G > 1)."""
+    if clip_version == 'v1':
+        cur_w = torch.clamp(w, min_val, max_val)
+        return Q.int_fake_quant_dynamic(spec, cur_w)
+    low_factor = _logit(min_val / org_min_val)
+    up_factor = _logit(max_val / org_max_val)
+    lo, hi = learnable_range(spec, w, low_factor, up_factor)
+    scales, zeros, qmax, qmin = Q.int_qparams(spec, lo, hi)
+    rows = Q.reshape_rows(spec, w)
+    zr = zeros if zeros.dim() == 0 else zeros.reshape(-1, 1)
+    out = Q.int_quant_dequant(spec, rows.reshape(-1, rows.shape[-1]), scales.reshape(-1, 1), zr, qmax, qmin)
+    return out.reshape(w.shape).to(w.dtype)
+
+
+def auto_clip_layer(spec, w, inputs, clip_sym=False, n_grid=20, max_shrink=0.5, n_sample_token=512,
+                    clip_version='v1', aspec=None, eps=0.0):
+    """auto_clip.py:83-191 on CPU tensors, op for op: for each batch of output rows the [ocb, T, G, g] products of the
+    sampled inputs with the original and with the clamped (v1) / range-scaled (v2) fake-quantized weights, their sums
+    over g, the mean squared difference over tokens, and the running `err < min_errs` selection over the shrink
+    steps.  `aspec` (an IntSpec, per_token) switches the activation fake quant of w_only=False on: it sees
+    [1, T, G, g], i.e. one range per token AND group.  Returns (best_max [R, G, 1], best_min [R, G, 1],
+    errs [R, G, n_steps] as computed)."""
     assert w.dim() == 2
     group_size = spec.group_size if spec.granularity == 'per_group' else w.shape[1]
     w = w.reshape(w.shape[0], 1, -1, group_size)
@@ -167,6 +209,9 @@ def auto_clip_layer(spec, w, inputs, clip_sym=False, n_grid=20, max_shrink=0.5, 
         org_out_dict = {}
         errs_b = []
         for i_s in range(int(max_shrink * n_grid)):
+            if i_s == 0:
+                if clip_version == 'v2' and aspec is not None:
+                    i_s += eps
             err_mean = 0
             for i in range(len(inputs)):
                 x = inputs[i]
@@ -182,9 +227,9 @@ def auto_clip_layer(spec, w, inputs, clip_sym=False, n_grid=20, max_shrink=0.5, 
                     org_out_dict[i] = org_out
                 max_val = org_max_val * (1 - i_s / n_grid)
                 min_val = -max_val if clip_sym else org_min_val * (1 - i_s / n_grid)
-                cur_w = torch.clamp(w, min_val, max_val)
-                q_w = Q.int_fake_quant_dynamic(spec, cur_w)
-                cur_out = (x * q_w).sum(dim=-1)
+                q_w = clip_fake_quantize_weight(spec, w, min_val, max_val, org_min_val, org_max_val, clip_version)
+                q_x = Q.int_fake_quant_dynamic(aspec, x) if aspec is not None else x
+                cur_out = (q_x * q_w).sum(dim=-1)
                 err = (cur_out - org_out).pow(2).mean(dim=1).view(min_errs.shape)
                 err_mean += err
             err_mean /= len(inputs)
@@ -199,6 +244,21 @@ def auto_clip_layer(spec, w, inputs, clip_sym=False, n_grid=20, max_shrink=0.5, 
     best_max_val = torch.cat(best_max_val_all, dim=0)
     best_min_val = torch.cat(best_min_val_all, dim=0)
     return best_max_val.squeeze(1), best_min_val.squeeze(1), torch.cat(errs_all, dim=0).squeeze(1)
+
+
+def clip_factor(spec, w, min_val, max_val, clip_sym=False):
+    """AutoClipper.get_clip_factor, auto_clip.py:231-256 -> (up_factor, low_factor) shaped like the quantizer's ranges."""
+    org_min_val, org_max_val = Q.minmax_range(spec, Q.reshape_rows(spec, w))
+    org_val_shape = org_max_val.shape
+    if clip_sym:
+        abs_max_val = torch.max(org_max_val.abs(), org_min_val.abs()).clamp(min=1e-5)
+        abs_max_val = abs_max_val.reshape(*max_val.shape[:2], -1)
+        return _logit(max_val / abs_max_val).reshape(org_val_shape), None
+    org_max_val = org_max_val.reshape(*max_val.shape[:2], -1)
+    up = _logit(max_val / org_max_val).reshape(org_val_shape)
+    org_min_val = org_min_val.reshape(*min_val.shape[:2], -1)
+    low = _logit(min_val / org_min_val).reshape(org_val_shape)
+    return up, low
 
 
 def apply_clip_v1(w, min_val, max_val, clip_sym=False):

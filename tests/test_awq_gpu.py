@@ -271,8 +271,8 @@ def test_search_on_float8_blockwise_weights(dev):
 # ---- AutoClipper (auto_clip.py) ---------------------------------------------------------------------
 @pytest.mark.parametrize('clip_sym,sym', [(False, False), (True, False), (False, True)])
 @pytest.mark.parametrize('R,K,T', [(64, 256, 96), (320, 512, 512), (256, 128, 700)])
-def test_auto_clip_against_oracle(dev, clip_sym, sym, R, K, T):
-    """Errors of the ten shrink steps within the bf16 noise of the reference's chain (it rounds both dot products
+def test_auto_clip_mfma_kernel_against_oracle(dev, clip_sym, sym, R, K, T):
+    """AutoClipper.fast = True.  Errors of the ten shrink steps within the bf16 noise of the reference's chain (it rounds both dot products
     to bf16 before subtracting; the kernel multiplies the weight difference on MFMA), the same step chosen wherever
     the oracle's own errors separate the best two by more than 3 %, ranges identical there."""
     from lightcompress_amd import IntegerQuantizer
@@ -285,6 +285,7 @@ def test_auto_clip_against_oracle(dev, clip_sym, sym, R, K, T):
     obmax, obmin, oerrs = A.auto_clip_layer(spec, w, [x.clone()], clip_sym=clip_sym, n_sample_token=nst)
     wq = IntegerQuantizer(4, sym, 'per_group', group_size=128)
     clipper = AutoClipper(True, wq, None, 'v1', clip_sym, False, None)
+    clipper.fast = True
     bmax, bmin = clipper.auto_clip_layer(0, 'fc', w.to(dev), [x.to(dev)], n_sample_token=nst)
     assert bmax.shape == obmax.shape and bmin.shape == obmin.shape and bmax.dtype == torch.bfloat16
     errs = clipper.last_errs.cpu()
@@ -307,9 +308,101 @@ def test_auto_clip_against_oracle(dev, clip_sym, sym, R, K, T):
     assert_bit_equal(layer.weight.data, A.apply_clip_v1(w, bmin.cpu(), bmax.cpu(), clip_sym), 'apply_clip')
 
 
-def test_auto_clip_run_skips_query_key_and_rejects_other_modes(dev):
+_CLIP_CASES = [
+    # version, w_only, weight spec (bit, sym, granularity, group), clip_sym, dtype, R, K, token counts of the inputs
+    ('v1', True, (4, False, 'per_group', 128), False, torch.bfloat16, 320, 512, [512]),
+    ('v1', True, (4, False, 'per_group', 128), True, torch.bfloat16, 64, 256, [96]),
+    ('v1', True, (4, True, 'per_group', 64), False, torch.bfloat16, 128, 320, [200, 75]),
+    ('v1', True, (3, False, 'per_group', 32), False, torch.float32, 64, 96, [130]),
+    ('v1', True, (4, False, 'per_channel', 0), False, torch.bfloat16, 64, 300, [64]),
+    ('v1', False, (4, False, 'per_group', 128), False, torch.bfloat16, 256, 256, [300]),
+    ('v2', False, (8, True, 'per_channel', 0), True, torch.bfloat16, 64, 384, [100]),
+    ('v2', True, (4, False, 'per_channel', 0), False, torch.float32, 64, 256, [80, 80]),
+    ('v2', False, (4, False, 'per_group', 128), False, torch.bfloat16, 64, 256, [64]),
+]
+
+
+@pytest.mark.parametrize('ver,w_only,wspec,clip_sym,dtype,R,K,Ts', _CLIP_CASES)
+def test_auto_clip_reference_rounding_sequence(dev, ver, w_only, wspec, clip_sym, dtype, R, K, Ts):
+    """The default search path against the op-for-op oracle: the same products rounded to the tensors' type, the same
+    rounded sums, difference, square and mean.  What is left is the order of the fp32 additions inside a group sum
+    and inside the mean over tokens (torch's reduction order on the CPU differs from the kernel's): a sum that lands
+    within 1e-7 of a rounding boundary may round the other way.  Bar (bf16): at least 99 % of the 10 errors per (row,
+    group) identical bit for bit, every error within two units of its last place (fp32: within 5e-4 relative), the same range on at least 99 % of the
+    groups, and wherever the range differs the oracle's own error of the step chosen here is within two units of
+    the last place of its minimum (a tie at the precision of the comparison)."""
     from lightcompress_amd import IntegerQuantizer
     from lightcompress_amd.auto_clip import AutoClipper
+    from tests.helpers import weight_like
+    bit, sym, gran, g = wspec
+    spec = Q.IntSpec(bit, sym, gran, group_size=g)
+    aspec = None if w_only else Q.IntSpec(8, True, 'per_token')
+    w = weight_like(R, K, seed=R + K, dtype=dtype)
+    xs = [(torch.randn(T, K, generator=gen(R + T + i)) * torch.exp(0.5 * torch.randn(K, generator=gen(K + T)))).to(dtype)
+          for i, T in enumerate(Ts)]
+    nst = 128
+    obmax, obmin, oerrs = A.auto_clip_layer(spec, w, [x.clone() for x in xs], clip_sym=clip_sym, n_sample_token=nst,
+                                            clip_version=ver, aspec=aspec)
+    wq = IntegerQuantizer(bit, sym, gran, group_size=g) if gran == 'per_group' else IntegerQuantizer(bit, sym, gran)
+    aq = None if w_only else IntegerQuantizer(8, True, 'per_token')
+    clipper = AutoClipper(w_only, wq, aq, ver, clip_sym, True, None)
+    bmax, bmin = clipper.auto_clip_layer(0, 'fc', w.to(dev), [x.to(dev) for x in xs], n_sample_token=nst)
+    assert bmax.shape == obmax.shape and bmin.shape == obmin.shape and bmax.dtype == dtype
+    errs, oe = clipper.last_errs.cpu().double(), oerrs.double()
+    # fp32 tensors round nothing away: there the summation order shows in every error (cancellation in out - org)
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.5e-4
+    if dtype == torch.bfloat16:
+        same = ((errs == oe) | (errs.isnan() & oe.isnan())).float().mean()
+        assert float(same) > 0.99, float(same)
+    fin = oe.isfinite()
+    assert bool(((errs - oe).abs()[fin] <= 2 * ulp * oe.abs()[fin]).all())
+    eq = (bmax.cpu() == obmax) & (bmin.cpu() == obmin)
+    assert float(eq.float().mean()) > 0.99, float(eq.float().mean())
+    if not bool(eq.all()):
+        G = obmax.shape[1]
+        hi0 = (w.reshape(R, G, -1).abs().amax(-1) if clip_sym else w.reshape(R, G, -1).amax(-1)).unsqueeze(-1)
+        cands = torch.cat([hi0 * (1 - s / 20) for s in range(10)], dim=-1)
+        step = (cands == bmax.cpu()).float().argmax(-1)
+        picked = oe.gather(-1, step.unsqueeze(-1)).squeeze(-1)
+        best = oe.min(-1).values
+        bad = ~eq.squeeze(-1)
+        assert bool((picked[bad] <= best[bad] * (1 + 4 * ulp)).all())
+    # apply_clip: v1 clamps the weight group-wise, v2 stores the sigmoid factors of the found range
+    layer = torch.nn.Linear(K, R, bias=False, dtype=dtype, device=dev)
+    layer.weight.data.copy_(w)
+    clipper.apply_clip(3, layer, bmin, bmax, 'fc')
+    if ver == 'v1':
+        assert_bit_equal(layer.weight.data, A.apply_clip_v1(w, bmin.cpu(), bmax.cpu(), clip_sym), 'apply_clip')
+    else:
+        up, low = A.clip_factor(spec, w, bmin.cpu(), bmax.cpu(), clip_sym)
+        tol = dict(rtol=2e-2, atol=2e-2) if dtype == torch.bfloat16 else dict(rtol=1e-4, atol=1e-5)
+        got_up = layer.buf_upbound_factor.cpu()
+        fin = up.isfinite()
+        assert got_up.shape == up.shape and torch.equal(got_up.isfinite(), fin)
+        assert torch.allclose(got_up[fin].float(), up[fin].float(), **tol)
+        assert (layer.buf_lowbound_factor is None) == (low is None)
+        assert clipper.weight_clips[3]['fc.weight_quantizer.upbound_factor'].shape == up.shape
+        # the stored factors drive calib_algo='learnable' (quant.py:207-221) to the clipped quantization
+        lq = IntegerQuantizer(bit, sym, gran, group_size=g, calib_algo='learnable') if gran == 'per_group' else \
+            IntegerQuantizer(bit, sym, gran, calib_algo='learnable')
+        args = {'upbound_factor': layer.buf_upbound_factor, 'lowbound_factor': layer.buf_lowbound_factor}
+        got = lq.fake_quant_weight_dynamic(layer.weight.data, args)
+        # sigmoid comes from two math libraries (GPU / CPU torch): the range within an ulp of the oracle's, then the
+        # quantization of the oracle on the GPU's range bit for bit
+        lo_g, hi_g = lq.get_learnable_range(lq.reshape_tensor(layer.weight.data), **args)
+        lo_l, hi_l = A.learnable_range(spec, Q.reshape_rows(spec, w), None if low is None else layer.buf_lowbound_factor.cpu(),
+                                       got_up)
+        rt = 1e-2 if dtype == torch.bfloat16 else 1e-6
+        assert torch.allclose(hi_g.cpu().float(), hi_l.float(), rtol=rt) and torch.allclose(lo_g.cpu().float(), lo_l.float(), rtol=rt)
+        sc, z, qmax, qmin = Q.int_qparams(spec, lo_g.cpu(), hi_g.cpu())
+        want = Q.int_fake_quant_static(spec, w, sc, z, qmax, qmin)
+        assert_bit_equal(got, want, 'learnable fake quant')
+
+
+def test_auto_clip_run_skips_query_key_and_handles_float8_weights(dev):
+    from lightcompress_amd import IntegerQuantizer
+    from lightcompress_amd.auto_clip import AutoClipper
+    from lightcompress_amd.kernel import weight_cast_to_fp8
     wq = IntegerQuantizer(4, False, 'per_group', group_size=128)
     blk = torch.nn.ModuleDict({'q_proj': torch.nn.Linear(128, 64, bias=False), 'o_proj': torch.nn.Linear(128, 64, bias=False)})
     blk = blk.to(device=dev, dtype=torch.bfloat16)
@@ -319,10 +412,22 @@ def test_auto_clip_run_skips_query_key_and_rejects_other_modes(dev):
     assert torch.equal(blk['q_proj'].weight.data, q0)                    # names with q_/k_ are not clipped
     assert not torch.equal(blk['o_proj'].weight.data, o0)
     assert float((blk['o_proj'].weight.data.abs() <= o0.abs()).float().mean()) == 1.0
+    # v2 registers the factor buffers, None on the skipped layers
+    blk['o_proj'].weight.data.copy_(o0)
+    AutoClipper(True, wq, None, 'v2', False, False, None).run(blk, 0, {'q_proj': [x], 'o_proj': [x]}, 512)
+    assert blk['q_proj'].buf_upbound_factor is None and blk['o_proj'].buf_upbound_factor.shape == (64, 1)
+    assert torch.equal(blk['o_proj'].weight.data, o0)                    # v2 leaves the weight alone
     with pytest.raises(NotImplementedError):
-        AutoClipper(True, wq, None, 'v2', False, False, None).auto_clip_layer(0, 'o', o0, [x])
-    with pytest.raises(NotImplementedError):
-        AutoClipper(False, wq, wq, 'v1', False, False, None).auto_clip_layer(0, 'o', o0, [x])
+        AutoClipper(True, IntegerQuantizer(4, False, 'per_tensor'), None, 'v1', False, False, None).auto_clip_layer(0, 'o', o0, [x])
+    # a block-wise float8 layer is searched on its bf16 weights and cast back (auto_clip.py:48-81)
+    fp8 = torch.nn.Linear(256, 128, bias=False).to(device=dev, dtype=torch.bfloat16)
+    w8, s8 = weight_cast_to_fp8(fp8.weight.data.contiguous())
+    fp8.weight.data = w8
+    fp8.register_buffer('weight_scale_inv', s8)
+    xb = torch.randn(64, 256, generator=gen(6)).bfloat16().to(dev)
+    AutoClipper(True, wq, None, 'v1', False, False, None).run(torch.nn.ModuleDict({'o_proj': fp8}), 0, {'o_proj': [xb]}, 512)
+    assert fp8.weight.data.dtype == torch.float8_e4m3fn and fp8.weight_scale_inv.shape == s8.shape
+    assert bool((fp8.weight_scale_inv <= s8).all()) and bool(fp8.weight_scale_inv.isfinite().all())
 
 
 # ---- apply_scale / scale_fc_fc / scale_ln_fcs / update_input_feat ---------------------------------------

@@ -147,6 +147,75 @@ def test_auto_clip_oracle_known_optima():
     assert torch.equal(cl, w)
 
 
+def test_auto_clip_oracle_v2_is_the_range_scaled_quantizer():
+    """clip_version v2 (auto_clip.py:263-272): sigmoid(logit(r)) = r, so the learnable range is the shrunken min/max
+    range and the weight is quantized UNclamped against it (the code clamp cuts the tails).  Pinned in fp32 by that
+    closed form written without logit/sigmoid; step 0 (logit(1) = inf, sigmoid = 1) is plain min/max fake quant; and
+    the factors of get_clip_factor map back to the found range."""
+    R, K, T = 64, 256, 48
+    w = weight_like(R, K, seed=81)
+    x = torch.randn(T, K, generator=gen(82)) * torch.exp(0.5 * torch.randn(K, generator=gen(83)))
+    for spec, clip_sym in [(Q.IntSpec(4, False, 'per_channel'), False), (Q.IntSpec(8, True, 'per_channel'), True),
+                           (Q.IntSpec(4, False, 'per_group', group_size=128), False)]:
+        gs = spec.group_size if spec.granularity == 'per_group' else K
+        G = K // gs
+        bmax, bmin, errs = A.auto_clip_layer(spec, w, [x.clone()], clip_sym=clip_sym, n_sample_token=T, clip_version='v2')
+        assert bmax.shape == (R, G, 1) and errs.shape == (R, G, 10)
+        wg, xg = w.reshape(R, G, gs), x.reshape(T, G, gs)
+        org = torch.einsum('tgj,rgj->rtg', xg.double(), wg.double())
+        hi0 = wg.abs().amax(-1, keepdim=True) if clip_sym else wg.amax(-1, keepdim=True)
+        lo0 = wg.amin(-1, keepdim=True)
+        want = torch.zeros(R, G, 10, dtype=torch.float64)
+        for s in range(10):
+            hi = hi0 * (1 - s / 20)
+            lo = -hi if clip_sym else lo0 * (1 - s / 20)
+            if spec.symmetric:                                      # get_learnable_range, sym: +-factor * max(|min|, |max|)
+                amax = torch.max(wg.amax(-1, keepdim=True).abs(), lo0.abs()).clamp(min=1e-5)
+                hi = (hi / hi0) * amax
+                lo = -hi
+            sc, z, qmax, qmin = Q.int_qparams(spec, lo, hi)
+            q = Q.int_quant_dequant(spec, wg, sc, z, qmax, qmin)
+            want[:, :, s] = (torch.einsum('tgj,rgj->rtg', xg.double(), q.double()) - org).pow(2).mean(1)
+        rel = (errs.double() - want).abs() / want.clamp(min=1e-30)
+        assert float(rel.median()) < 1e-3 and float(rel.quantile(0.99)) < 0.05, (float(rel.median()), float(rel.max()))
+        # step 0 is the plain fake quant of the unclipped weight
+        e0 = (torch.einsum('tgj,rgj->rtg', xg.double(), Q.int_fake_quant_dynamic(spec, w).reshape(R, G, gs).double()) - org).pow(2).mean(1)
+        if not clip_sym or spec.symmetric:
+            assert torch.allclose(errs[:, :, 0].double(), e0, rtol=1e-3, atol=1e-12)
+        # the stored factors give the found range back through the learnable range
+        up, low = A.clip_factor(spec, w, bmin, bmax, clip_sym)
+        lo_l, hi_l = A.learnable_range(spec, Q.reshape_rows(spec, w), low, up)
+        if spec.symmetric == clip_sym:
+            assert torch.allclose(hi_l.reshape(bmax.shape), bmax, rtol=1e-5)
+            if not clip_sym:
+                assert torch.allclose(lo_l.reshape(bmin.shape), bmin, rtol=1e-5)
+
+
+def test_auto_clip_oracle_with_activation_quantization():
+    """w_only=False: the activations are fake-quantized as [1, T, G, gs], i.e. one range per token and group
+    (per_token reshapes nothing, the range reduces the last axis).  Pinned by that per-(token, group) closed form and
+    by the 16-bit limit in which activation quantization is the identity."""
+    R, K, T = 64, 256, 32
+    spec = Q.IntSpec(4, False, 'per_group', group_size=128)
+    w = weight_like(R, K, seed=91)
+    x = torch.randn(T, K, generator=gen(92))
+    a8 = Q.IntSpec(8, True, 'per_token')
+    qx = Q.int_fake_quant_dynamic(a8, x.reshape(1, T, 2, 128))
+    rows = x.reshape(T * 2, 128)
+    sc = rows.abs().amax(-1, keepdim=True).clamp(min=1e-5) / 127
+    assert torch.equal(qx.reshape(T * 2, 128), torch.clamp(torch.round(rows / sc), -128, 127) * sc)
+    _, _, e_w = A.auto_clip_layer(spec, w, [x.clone()], n_sample_token=T)
+    _, _, e_a16 = A.auto_clip_layer(spec, w, [x.clone()], n_sample_token=T, aspec=Q.IntSpec(16, True, 'per_token'))
+    _, _, e_a8 = A.auto_clip_layer(spec, w, [x.clone()], n_sample_token=T, aspec=a8)
+    assert torch.allclose(e_a16, e_w, rtol=2e-3)
+    # the 8-bit error is the objective evaluated with qx on the quantized side only
+    wg = w.reshape(R, 2, 128)
+    org = torch.einsum('tgj,rgj->rtg', x.reshape(T, 2, 128).double(), wg.double())
+    q0 = Q.int_fake_quant_dynamic(spec, w).reshape(R, 2, 128)
+    want0 = (torch.einsum('tgj,rgj->rtg', qx.reshape(T, 2, 128).double(), q0.double()) - org).pow(2).mean(1)
+    assert torch.allclose(e_a8[:, :, 0].double(), want0, rtol=1e-3)
+
+
 def test_gqa_search_reduces_to_the_plain_search_and_repeats_per_group():
     """is_gqa (awq.py:88-93, 104-105; base_blockwise_quantization.py:614-618).
     * The repeated vector indexes the key/value channel of every query channel: column c of o_proj belongs to query
