@@ -95,6 +95,12 @@ int lcq_minmax_rows(const void* x, int dtype, int64_t rows, int64_t cols, void* 
 int64_t lcq_minmax_all_workspace_bytes(void);
 int lcq_minmax_all(const void* x, int dtype, int64_t n, void* min_out, void* max_out, void* workspace, void* stream);
 
+/* The torch.histc(tensor.float(), bins, min, max) of get_static_hist_range, quant.py:461-511 (calib_algo
+ * 'static_hist'): hist[b] = number of elements with lo <= v <= hi and b = (int)((v - lo) * bins / (hi - lo)) in fp32
+ * (b == bins counts into the last bin); lo == hi widens the range to [lo - 1, hi + 1] as torch does.
+ *  x [n] of `dtype` (LCQ_F32 | LCQ_BF16 | LCQ_F16), counts: workspace of `bins` uint32, hist [bins] fp32; bins <= 8192. */
+int lcq_histc(const void* x, int dtype, int64_t n, int bins, float lo, float hi, void* counts, float* hist, void* stream);
+
 /* get_qparams, quant.py:544-558, on n explicit (min, max) pairs. */
 int lcq_qparams_int(const void* min_in, const void* max_in, int dtype, int64_t n, float qmin, float qmax, int flags,
                     void* scales, void* zeros, void* stream);

@@ -10,7 +10,7 @@ ABI in ``include/lcq.h``.  There is no CPU path: CPU tensors raise
 ``LcqError``.  Reshapes/views, index mixing and dtype casts stay in torch.
 
 ``calib_algo``: ``minmax``, ``mse``, ``hqq``, ``learnable`` (the sigmoid-scaled range with GIVEN factors; training
-them needs autograd and is not here), ``static_minmax`` / ``static_moving_minmax`` for activations.
+them needs autograd and is not here), ``static_minmax`` / ``static_moving_minmax`` / ``static_hist`` for activations.
 Not carried over (they raise ``NotImplementedError``): STE rounding (training only) and the ``rounding`` override of
 ``fake_quant_weight_static``.  ``per_block`` granularity runs for
 ``FloatQuantizer('e4m3')`` weights only (``real_quant_weight_dynamic`` / ``fake_quant_weight_dynamic``).
@@ -40,6 +40,9 @@ class BaseQuantizer(object):
         self.mse_b_num = self.kwargs.get('mse_b_num', 1)
         self.maxshrink = self.kwargs.get('maxshrink', 0.8)
         self.mse_grid = self.kwargs.get('mse_grid', 100)
+        # hist config (quant.py:83-87)
+        self.bins = self.kwargs.get('bins', 2048)
+        self.upsample_rate = 16
         # hqq config (quant.py:89-93)
         self.lp_norm = self.kwargs.get('lp_norm', 0.7)
         self.beta = self.kwargs.get('beta', 10)
@@ -183,6 +186,121 @@ class BaseQuantizer(object):
         max_vals = [r['max'].mean(dim=0) for r in stats.values()]
         return min_vals, max_vals
 
+    # -- histogram observer (calib_algo 'static_hist', quant.py:264-521) ---------------------------------------
+    # The passes over the activations (range, histogram) are kernels.  What follows them works on `bins` numbers per
+    # module input and stays host-side fp32 torch arithmetic on CPU tensors, as in the reference, whose histograms
+    # live on the CPU as well (quant.py:468): the search below compares sums that differ in their last bits, so it
+    # keeps the reference's operation order.
+    def _histc(self, tensor, lo, hi):
+        t = tensor.contiguous()
+        counts = torch.empty(self.bins, dtype=torch.int32, device=t.device)
+        hist = torch.empty(self.bins, dtype=torch.float32, device=t.device)
+        L.check(L.lib().lcq_histc(L.ptr(t), L.dtype_code(t.dtype), L.i64(t.numel()), L.i32(self.bins), L.f32(lo),
+                                  L.f32(hi), L.ptr(counts), L.ptr(hist), L.stream()), 'lcq_histc')
+        return hist.cpu()
+
+    def get_quantization_error(self, histogram, min_val, max_val, next_start_bin, next_end_bin):
+        """quant.py:279-328: L2 error of quantizing the histogram's mass with 2**bit levels spread over the source
+        bins next_start_bin..next_end_bin; every source bin is a uniform density."""
+        bin_width = (max_val.item() - min_val.item()) / self.bins
+        dst_bin_width = bin_width * (next_end_bin - next_start_bin + 1) / self.dst_nbins
+        if dst_bin_width == 0.0:
+            return 0.0
+        half = dst_bin_width / 2
+        cube = lambda a, b: (b * b * b - a * a * a) / 3                       # integral of x^2 over [a, b]
+        begin = (torch.arange(self.bins) - next_start_bin) * bin_width      # source bin edges from the first level's start
+        end = begin + bin_width
+        first = torch.clamp(torch.div(begin, dst_bin_width, rounding_mode='floor'), 0, self.dst_nbins - 1)
+        last = torch.clamp(torch.div(end, dst_bin_width, rounding_mode='floor'), 0, self.dst_nbins - 1)
+        density = histogram / bin_width
+        norm = torch.zeros(self.bins)
+        norm += density * cube(begin - (first + 0.5) * dst_bin_width, torch.ones(self.bins) * half)
+        norm += (last - first - 1) * (density * cube(torch.tensor(-half), torch.tensor(half)))
+        norm += density * cube(torch.tensor(-half), end - (last * dst_bin_width + half))
+        return norm.sum().item()
+
+    def _upscale_histogram(self, histogram, orig_min, orig_max, update_min, update_max):
+        """quant.py:330-366: the old histogram, `upsample_rate` sub-bins per bin, dropped into the bins of the
+        wider range."""
+        fine = histogram.repeat_interleave(self.upsample_rate) / self.upsample_rate
+        n_fine = self.bins * self.upsample_rate
+        mids = torch.linspace(orig_min, orig_max, n_fine + 1)[:-1] + 0.5 * ((orig_max - orig_min) / n_fine)
+        edges = torch.linspace(update_min, update_max, self.bins + 1)
+        where = torch.bucketize(mids, edges, right=True) - 1
+        where[where >= self.bins] = self.bins - 1
+        where[where < 0] = 0
+        return torch.bincount(where, weights=fine, minlength=self.bins)
+
+    def _combine_histograms(self, orig_hist, orig_min, orig_max, update_hist, update_min, update_max):
+        """quant.py:368-400."""
+        if update_min == orig_min and update_max == orig_max:
+            return orig_hist + update_hist
+        if orig_min == orig_max:                               # a single value so far: its bin, weighted (quant.py:380-388)
+            one = torch.histc(orig_min, bins=self.bins, min=update_min, max=update_max) * torch.sum(update_hist)
+            return one + update_hist
+        assert update_min <= orig_min
+        assert update_max >= orig_max
+        return update_hist + self._upscale_histogram(orig_hist, orig_min, orig_max, update_min, update_max)
+
+    def get_hist_threshold(self, histogram, min_val, max_val):
+        """quant.py:402-459: shrink the range one quantile step (1e-8 of the mass) at a time from whichever side
+        gives up fewer bins, until the quantization error stops falling."""
+        assert histogram.size()[0] == self.bins, 'bins mismatch'
+        bin_width = (max_val - min_val) / self.bins
+        total = torch.sum(histogram).item()
+        csum = torch.cumsum(histogram, dim=0).tolist()         # fp32 values; a 0-dim fp32 tensor compares with a
+        f32 = lambda v: torch.tensor(v, dtype=torch.float32).item()       # python number in fp32
+        stepsize = 1e-8
+        alpha, beta = 0.0, 1.0
+        start_bin, end_bin = 0, self.bins - 1
+        norm_min = float('inf')
+        while alpha < beta:
+            next_alpha, next_beta = alpha + stepsize, beta - stepsize
+            lo_mass, hi_mass = f32(next_alpha * total), f32(next_beta * total)
+            left, right = start_bin, end_bin
+            while left < end_bin and csum[left] < lo_mass:
+                left += 1
+            while right > start_bin and csum[right] > hi_mass:
+                right -= 1
+            next_start_bin, next_end_bin = start_bin, end_bin
+            if (left - start_bin) > (end_bin - right):
+                next_start_bin, alpha = left, next_alpha
+            else:
+                next_end_bin, beta = right, next_beta
+            if next_start_bin == start_bin and next_end_bin == end_bin:
+                continue
+            norm = self.get_quantization_error(histogram, min_val, max_val, next_start_bin, next_end_bin)
+            if norm > norm_min:
+                break
+            norm_min = norm
+            start_bin, end_bin = next_start_bin, next_end_bin
+        return min_val + bin_width * start_bin, min_val + bin_width * (end_bin + 1)
+
+    def get_static_hist_range(self, act_tensors):
+        """quant.py:461-521 -> (min_vals, max_vals), 0-dim fp32 CPU tensors, one per module input."""
+        act_tensors = self.reshape_batch_tensors(act_tensors)
+        stats = self.get_minmax_stats(act_tensors)
+        new_min_vals, new_max_vals = [], []
+        for input_idx, tensors in enumerate(act_tensors):
+            histogram, min_val, max_val = None, None, None
+            for idx, tensor in enumerate(tensors):
+                x_min, x_max = stats[input_idx]['min'][idx], stats[input_idx]['max'][idx]
+                if histogram is None:
+                    histogram = self._histc(tensor, x_min.item(), x_max.item())
+                    min_val, max_val = x_min, x_max
+                    continue
+                new_min, new_max = torch.min(min_val, x_min), torch.max(max_val, x_max)
+                update = self._histc(tensor, new_min.item(), new_max.item())
+                if new_min == min_val and new_max == max_val:
+                    histogram = histogram + update
+                else:
+                    histogram = self._combine_histograms(histogram, min_val, max_val, update, new_min, new_max)
+                min_val, max_val = new_min, new_max
+            new_min, new_max = self.get_hist_threshold(histogram, min_val, max_val)
+            new_min_vals.append(new_min)
+            new_max_vals.append(new_max)
+        return new_min_vals, new_max_vals
+
     def get_static_moving_minmax_range(self, act_tensors, alpha):
         """quant.py:523-542: exponential moving average of the per-tensor ranges, in the tensors' dtype."""
         act_tensors = self.reshape_batch_tensors(act_tensors)
@@ -203,8 +321,10 @@ class BaseQuantizer(object):
     def get_batch_tensors_qparams(self, act_tensors, alpha=0.01, args={}):
         """quant.py:559-585 -> (scales_list, zeros_list, qmin_list, qmax_list), one entry per module input."""
         if self.calib_algo == 'static_hist':
-            raise NotImplementedError("calib_algo='static_hist' (the histogram observer, quant.py:264-521) is host-side "
-                                      'search code outside this path; static_minmax and static_moving_minmax run on liblcq')
+            assert (
+                self.sym is True and self.granularity == 'per_tensor'
+            ), 'Only support per tensor static symmetric int quantize.'
+            min_vals, max_vals = self.get_static_hist_range(act_tensors)
         elif self.calib_algo == 'static_minmax':
             min_vals, max_vals = self.get_static_minmax_range(act_tensors)
         elif self.calib_algo == 'static_moving_minmax':

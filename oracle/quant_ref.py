@@ -553,6 +553,135 @@ def static_moving_minmax_ranges(spec, act_tensors, alpha):
 
 
 # ----------------------------------------------------------------------------
+# histogram observer, calib_algo 'static_hist'   (quant.py:264-521)
+# ----------------------------------------------------------------------------
+def histc_device(x: torch.Tensor, bins: int, lo: float, hi: float) -> torch.Tensor:
+    """torch.histc as torch's DEVICE kernel bins (the reference's activations are on the GPU, quant.py:473-487):
+    bin = (int)((v - lo) * bins / (hi - lo)) in fp32, multiply first, the top edge counted into the last bin,
+    values outside [lo, hi] dropped, lo == hi widened by one to each side.  Restated from ATen's published
+    SummaryOps kernel; the CPU torch.histc divides first and so differs on values next to a bin edge - the
+    test pins this function against it up to exactly those values.  PARITY UNPINNED for the order of the
+    multiply and the divide: no device torch.histc is available to check it against."""
+    lo32, hi32 = np.float32(lo), np.float32(hi)
+    if lo32 == hi32:
+        lo32, hi32 = lo32 - np.float32(1), hi32 + np.float32(1)
+    v = x.detach().float().flatten().numpy()
+    v = v[(v >= lo32) & (v <= hi32)]
+    b = ((v - lo32) * np.float32(bins) / (hi32 - lo32)).astype(np.int64)
+    b[b == bins] = bins - 1
+    return torch.from_numpy(np.bincount(b, minlength=bins).astype(np.float32))
+
+
+def hist_quantization_error(hist, min_val, max_val, start_bin, end_bin, bins, dst_nbins):
+    """get_quantization_error + get_norm, quant.py:264-328, op for op on CPU fp32 tensors."""
+    def get_norm(delta_begin, delta_end, density):
+        norm = (delta_end * delta_end * delta_end - delta_begin * delta_begin * delta_begin) / 3
+        return density * norm
+    bin_width = (max_val.item() - min_val.item()) / bins
+    dst_bin_width = bin_width * (end_bin - start_bin + 1) / dst_nbins
+    if dst_bin_width == 0.0:
+        return 0.0
+    src_bin = torch.arange(bins)
+    src_bin_begin = (src_bin - start_bin) * bin_width
+    src_bin_end = src_bin_begin + bin_width
+    dst_bin_of_begin = torch.clamp(torch.div(src_bin_begin, dst_bin_width, rounding_mode='floor'), 0, dst_nbins - 1)
+    dst_bin_of_begin_center = (dst_bin_of_begin + 0.5) * dst_bin_width
+    dst_bin_of_end = torch.clamp(torch.div(src_bin_end, dst_bin_width, rounding_mode='floor'), 0, dst_nbins - 1)
+    density = hist / bin_width
+    norm = torch.zeros(bins)
+    delta_begin = src_bin_begin - dst_bin_of_begin_center
+    delta_end = dst_bin_width / 2
+    norm += get_norm(delta_begin, torch.ones(bins) * delta_end, density)
+    norm += (dst_bin_of_end - dst_bin_of_begin - 1) * get_norm(torch.tensor(-dst_bin_width / 2),
+                                                              torch.tensor(dst_bin_width / 2), density)
+    dst_bin_of_end_center = dst_bin_of_end * dst_bin_width + dst_bin_width / 2
+    delta_begin = -dst_bin_width / 2
+    delta_end = src_bin_end - dst_bin_of_end_center
+    norm += get_norm(torch.tensor(delta_begin), delta_end, density)
+    return norm.sum().item()
+
+
+def hist_combine(orig_hist, orig_min, orig_max, update_hist, update_min, update_max, bins, upsample_rate=16):
+    """_combine_histograms + _upscale_histogram, quant.py:330-400."""
+    if update_min == orig_min and update_max == orig_max:
+        return orig_hist + update_hist
+    if orig_min == orig_max:
+        bin_value = torch.sum(update_hist)
+        return torch.histc(orig_min, bins=bins, min=update_min, max=update_max) * bin_value + update_hist
+    assert update_min <= orig_min and update_max >= orig_max
+    histogram = orig_hist.repeat_interleave(upsample_rate) / upsample_rate
+    bin_size = (orig_max - orig_min) / (bins * upsample_rate)
+    mid_points = torch.linspace(orig_min, orig_max, bins * upsample_rate + 1)[:-1] + 0.5 * bin_size
+    boundaries = torch.linspace(update_min, update_max, bins + 1)
+    bucket = torch.bucketize(mid_points, boundaries, right=True) - 1
+    bucket[bucket >= bins] = bins - 1
+    bucket[bucket < 0] = 0
+    return update_hist + torch.bincount(bucket, weights=histogram, minlength=bins)
+
+
+def hist_threshold(hist, min_val, max_val, bins, dst_nbins):
+    """get_hist_threshold, quant.py:402-459, the loop as written.  Its `cSum[i] < next_alpha * total` compares a 0-dim
+    fp32 tensor with a python number, which torch evaluates in fp32: written here as a comparison of python floats
+    with the right-hand side rounded to fp32 (the loop takes one step per 1e-8 of the mass, millions for a
+    histogram with heavy edge bins; as tensor operations that is minutes)."""
+    bin_width = (max_val - min_val) / bins
+    total = torch.sum(hist).item()
+    cSum = torch.cumsum(hist, dim=0).tolist()
+    f32 = lambda v: float(np.float32(v))
+    stepsize = 1e-8
+    alpha, beta = 0.0, 1.0
+    start_bin, end_bin = 0, bins - 1
+    norm_min = float('inf')
+    while alpha < beta:
+        next_alpha = alpha + stepsize
+        next_beta = beta - stepsize
+        left, right = start_bin, end_bin
+        while left < end_bin and cSum[left] < f32(next_alpha * total):
+            left = left + 1
+        while right > start_bin and cSum[right] > f32(next_beta * total):
+            right = right - 1
+        next_start_bin, next_end_bin = start_bin, end_bin
+        if (left - start_bin) > (end_bin - right):
+            next_start_bin = left
+            alpha = next_alpha
+        else:
+            next_end_bin = right
+            beta = next_beta
+        if next_start_bin == start_bin and next_end_bin == end_bin:
+            continue
+        norm = hist_quantization_error(hist, min_val, max_val, next_start_bin, next_end_bin, bins, dst_nbins)
+        if norm > norm_min:
+            break
+        norm_min = norm
+        start_bin, end_bin = next_start_bin, next_end_bin
+    return min_val + bin_width * start_bin, min_val + bin_width * (end_bin + 1)
+
+
+def static_hist_ranges(act_tensors, bit, bins=2048):
+    """get_static_hist_range, quant.py:461-521 (per_tensor, symmetric - what get_batch_tensors_qparams asserts)."""
+    mins, maxs = [], []
+    for tensors in _batch_lists(act_tensors):
+        hist = min_val = max_val = None
+        for t in tensors:
+            x_min, x_max = torch.min(t).float(), torch.max(t).float()
+            if hist is None:
+                hist = histc_device(t, bins, x_min.item(), x_max.item())
+                min_val, max_val = x_min, x_max
+                continue
+            new_min, new_max = torch.min(min_val, x_min), torch.max(max_val, x_max)
+            upd = histc_device(t, bins, new_min.item(), new_max.item())
+            if new_min == min_val and new_max == max_val:
+                hist = hist + upd
+            else:
+                hist = hist_combine(hist, min_val, max_val, upd, new_min, new_max, bins)
+            min_val, max_val = new_min, new_max
+        lo, hi = hist_threshold(hist, min_val, max_val, bins, 2 ** bit)
+        mins.append(lo)
+        maxs.append(hi)
+    return mins, maxs
+
+
+# ----------------------------------------------------------------------------
 # Weight48IntegerQuantizer   (quant.py:1230-1367)
 # ----------------------------------------------------------------------------
 def w48_fake_quant(w: torch.Tensor, bit4: dict, bit8: dict) -> torch.Tensor:

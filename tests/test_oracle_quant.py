@@ -467,6 +467,64 @@ def test_static_activation_ranges_known_answers():
     assert lo[0].shape == (2, 1) and hi[0].flatten().tolist() == [3.0, float(np.float32(5.5) / np.float32(3))]   # (2,1,6)/3, (.5,4,1)/3
 
 
+def test_hist_observer_oracle():
+    """static_hist (quant.py:264-521).  Histogram: integer data on integer edges is unambiguous; on real data the
+    device formula equals the CPU torch.histc except for values within a few ulp of a bin edge.  Quantization error:
+    the closed-form integrals against a numerical integration of (x - nearest level)^2 over every source bin in
+    fp64.  Combination: mass is conserved, and a range that doubles exactly folds pairs of bins.  Threshold: a
+    uniform histogram loses exactly the one bin of the unconditional first step, a far outlier is cut off, the result tightens the range monotonically."""
+    g = gen(5)
+    x = torch.randint(0, 64, (5000,), generator=g).float()
+    h = Q.histc_device(x, 64, 0.0, 64.0)
+    assert torch.equal(h, torch.bincount(x.long(), minlength=64).float())
+    assert float(Q.histc_device(torch.tensor([64.0, 64.0, -1.0, 65.0]), 64, 0.0, 64.0)[63]) == 2.0      # top edge in, outside out
+    assert float(Q.histc_device(torch.full((7,), 3.0), 8, 3.0, 3.0).sum()) == 7.0                       # lo == hi widened
+    y = torch.randn(200000, generator=g)
+    hd, hc = Q.histc_device(y, 2048, y.min().item(), y.max().item()), torch.histc(y, 2048, min=y.min().item(), max=y.max().item())
+    assert float(hd.sum()) == float(hc.sum()) == 200000 and float((hd - hc).abs().sum()) <= 20
+
+    bins, levels = 128, 16
+    hist = torch.rand(bins, generator=g) * 100
+    lo, hi = torch.tensor(-1.5), torch.tensor(2.5)
+    bw = 4.0 / bins
+    for sb, eb in [(0, bins - 1), (10, 100), (40, 41), (0, 5)]:
+        dw = bw * (eb - sb + 1) / levels
+        sub = 400
+        pos = ((torch.arange(bins * sub, dtype=torch.float64) + 0.5) / sub - sb) * bw          # from the first level's start
+        lvl = torch.clamp(torch.floor(pos / dw), 0, levels - 1)
+        err = (pos - (lvl + 0.5) * dw) ** 2
+        want = float((err.view(bins, sub).mean(1) * hist.double()).sum())
+        got = Q.hist_quantization_error(hist, lo, hi, sb, eb, bins, levels)
+        assert abs(got - want) < 2e-3 * want, (sb, eb, got, want)
+
+    h0 = torch.rand(bins, generator=g) * 10
+    up = torch.zeros(bins)
+    wide = Q.hist_combine(h0, torch.tensor(0.0), torch.tensor(1.0), up, torch.tensor(0.0), torch.tensor(2.0), bins)
+    assert abs(float(wide.sum()) - float(h0.sum())) < 1e-3
+    assert torch.allclose(wide[:bins // 2], h0.view(-1, 2).sum(1), rtol=1e-5) and float(wide[bins // 2:].abs().sum()) == 0.0
+    same = Q.hist_combine(h0, torch.tensor(0.0), torch.tensor(1.0), h0, torch.tensor(0.0), torch.tensor(1.0), bins)
+    assert torch.equal(same, h0 + h0)
+
+    assert not bool(torch.tensor(0.1) > 0.1) and bool(torch.tensor(0.1).double() > 0.1)      # tensor-vs-number compares in fp32
+    flat = torch.full((256,), 1000.0)
+    a, b = Q.hist_threshold(flat, torch.tensor(-1.0), torch.tensor(1.0), 256, 256)
+    # one level per bin: any cut only adds clipping error - but the first cut is always taken (norm_min starts at
+    # infinity), from the right on a tie; the second one is refused
+    assert float(a) == -1.0 and float(b) == 1.0 - 2.0 / 256
+    spike = torch.zeros(256)
+    spike[:32] = 1000.0
+    spike[255] = 1.0                                                     # one outlier far to the right
+    a, b = Q.hist_threshold(spike, torch.tensor(0.0), torch.tensor(256.0), 256, 16)
+    # the quantile walk first drops the outlier's bin (unconditionally), then jumps to the last bin whose cumulated
+    # mass is below the full body: 31 of its 32 bins; giving up another 1000-count bin is refused
+    assert float(a) == 0.0 and float(b) == 31.0
+    acts = [torch.randn(4, 300, 64, generator=g) * (1 + i) for i in range(3)]
+    lo3, hi3 = Q.static_hist_ranges(acts, 8)
+    full_lo, full_hi = min(float(t.min()) for t in acts), max(float(t.max()) for t in acts)
+    assert len(lo3) == 1 and full_lo <= float(lo3[0]) < float(hi3[0]) <= full_hi
+    assert float(hi3[0]) - float(lo3[0]) < full_hi - full_lo
+
+
 def test_w48_known_answers():
     """Weight48IntegerQuantizer.fake_quant_weight_dynamic (quant.py:1338-1367).
     * Lossless case: weights c*m with integer m, |m| <= 127 and max |m| = 127 give 8-bit codes m; if every group of

@@ -456,8 +456,62 @@ def test_static_activation_calibration(dev):
     lo, hi = q.get_static_minmax_range([acts[0].to(dev)])
     olo, ohi = Q.static_minmax_ranges(spec, [acts[0]])
     assert_bit_equal(lo[0], olo[0], 'batch tensor min')
-    with pytest.raises(NotImplementedError):
-        IntegerQuantizer(8, True, 'per_tensor', calib_algo='static_hist').get_batch_tensors_qparams([acts[0].to(dev)])
+    with pytest.raises(AssertionError):                       # quant.py:563-566: per-tensor symmetric only
+        IntegerQuantizer(8, False, 'per_tensor', calib_algo='static_hist').get_batch_tensors_qparams([acts[0].to(dev)])
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
+def test_histogram_kernel(dev, dtype):
+    """lcq_histc against the device binning formula of torch.histc: counts identical, for ragged lengths, values on
+    and outside the edges, a constant tensor (range widened by one), and more than 2^24 hits in one bin."""
+    from lightcompress_amd import IntegerQuantizer
+    q = IntegerQuantizer(8, True, 'per_tensor', calib_algo='static_hist')
+    g = gen(21)
+    for n, bins in [(100003, 2048), (4096 * 33 + 5, 512), (7, 16)]:
+        q.bins = bins
+        x = (torch.randn(n, generator=g) * 3).to(dtype)
+        lo, hi = float(x.min()), float(x.max())
+        for a, b in [(lo, hi), (lo * 0.5, hi * 0.25), (lo - 1.0, hi + 2.5)]:
+            got = q._histc(x.to(dev), a, b)
+            want = Q.histc_device(x, bins, a, b)
+            assert torch.equal(got, want), (n, bins, a, b, int((got != want).sum()))
+    q.bins = 64
+    c = torch.full((1000,), 2.5, dtype=dtype)
+    assert torch.equal(q._histc(c.to(dev), 2.5, 2.5), Q.histc_device(c, 64, 2.5, 2.5))
+    if dtype == torch.bfloat16:
+        big = torch.zeros(1 << 25, dtype=dtype, device=dev)
+        big[::1024] = 1.0
+        h = q._histc(big, 0.0, 1.0)
+        assert float(h[0]) == float((1 << 25) - (1 << 15)) and float(h[63]) == float(1 << 15) and float(h[1:63].sum()) == 0.0
+
+
+def test_static_hist_calibration(dev):
+    """calib_algo='static_hist' (quant.py:264-521, 563-567): the thresholded range and the qparams equal the oracle's
+    bit for bit - tensors of growing range (the histogram is re-binned), of equal range, a batch in one tensor, two
+    module inputs, fp32 and bf16 activations."""
+    from lightcompress_amd import IntegerQuantizer
+    g = gen(31)
+    spec = Q.IntSpec(8, True, 'per_tensor')
+    grow = [torch.randn(2, 200, 128, generator=g).bfloat16() * (1 + i) for i in range(4)]
+    same = [torch.randn(300, 64, generator=g).clamp(-2, 2) for _ in range(3)]
+    for t in same:
+        t[0, 0], t[0, 1] = -2.0, 2.0
+    shrink = [torch.randn(128, 96, generator=g) * s for s in (4.0, 1.0, 2.0)]
+    for acts in (grow, same, shrink, [grow[0]]):
+        q = IntegerQuantizer(8, True, 'per_tensor', calib_algo='static_hist')
+        lo, hi = q.get_static_hist_range([a.to(dev) for a in acts])
+        olo, ohi = Q.static_hist_ranges([a.clone() for a in acts], 8)
+        assert len(lo) == len(olo) == 1
+        assert_bit_equal(lo[0], olo[0], 'hist min'); assert_bit_equal(hi[0], ohi[0], 'hist max')
+        sl, zl, qminl, qmaxl = q.get_batch_tensors_qparams([a.to(dev) for a in acts])
+        os_, oz, oqmax, oqmin = Q.int_qparams(spec, olo[0], ohi[0])
+        assert and_bit(sl[0], os_) and float(qmaxl[0]) == 127.0 and float(qminl[0]) == -128.0
+    pairs = [(grow[0][0], same[0]), (grow[1][0], same[1])]
+    q = IntegerQuantizer(4, True, 'per_tensor', calib_algo='static_hist', bins=512)
+    sl, _, _, _ = q.get_batch_tensors_qparams([(a.to(dev), b.to(dev)) for a, b in pairs])
+    olo, ohi = Q.static_hist_ranges(pairs, 4, bins=512)
+    spec4 = Q.IntSpec(4, True, 'per_tensor')
+    assert len(sl) == 2 and and_bit(sl[0], Q.int_qparams(spec4, olo[0], ohi[0])[0]) and and_bit(sl[1], Q.int_qparams(spec4, olo[1], ohi[1])[0])
 
 
 def and_bit(a, b):
