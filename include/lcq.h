@@ -231,10 +231,12 @@ int lcq_chol_inv_upper(float* H, int64_t K, const int64_t* perm, float percdamp,
  * tmp[:, i] = w, Losses[:, i], in-block error feedback; Err [R,128] receives Err1.
  *  W, tmp, Losses [R,K] fp32; Err [R, ldErr] fp32 (column i of the block -> Err[:, i]);
  *  U [K,K] upper factor; scales / zeros [R,G] fp32
- *  dynamic groups (default): group_size > 0, G >= ceil(K/group_size), qparams are written
- *  LCQ_FLAG_STATIC: qparams are inputs; group of column c is gidx[c] (or c/group_size, or 0 if group_size == 0) */
+ *  dynamic groups (default): group_size > 0, G >= ceil(n_quant/group_size), qparams are written
+ *  LCQ_FLAG_STATIC: qparams are inputs; group of column c is gidx[c] (or c/group_size, or 0 if group_size == 0)
+ *  n_quant: the columns [0, n_quant) are quantized, a group's range ends there at the latest (gptq.py:218-221,
+ *  `self.columns - self.n_out`); K without OWQ outlier columns */
 int lcq_gptq_block(float* W, float* tmp, float* Losses, float* Err, int64_t ldErr, const float* U, int64_t R, int64_t K,
-                   int64_t i1, int count, int group_size, float qmin, float qmax, int flags, float* scales, float* zeros,
+                   int64_t n_quant, int64_t i1, int count, int group_size, float qmin, float qmax, int flags, float* scales, float* zeros,
                    const int32_t* gidx, int64_t G, void* stream);
 
 /* Deferred update of gptq.py:244, generalised to a column window (fp32 MFMA):

@@ -49,7 +49,7 @@ constexpr int ROWS_PER_WG = 16;
 struct LoopArgs {
   float* W; float* tmp; float* Losses; float* Err; const float* U;
   float* scales; float* zeros; const int* gidx;
-  long long R; int K, i1, count, g, G, ldErr;
+  long long R; int K, Kq, i1, count, g, G, ldErr;      // Kq: columns that are quantized (K unless outlier columns are kept)
   float qmin, qmax;
   int sym, is_static, aligned;
   int nrz;              // round_zp=False: un-rounded zero point inside the rounding, scale clamped at 1e-9 (quant.py:556-557, 702-706)
@@ -85,7 +85,7 @@ __device__ __forceinline__ ColQ make_colq(float s, float z, float qmin, float qm
 // `held`: the team's registers when they are exactly that range (group = block, nothing updated yet).
 __device__ __forceinline__ ColQ open_group(const LoopArgs& a, int idx, int lane, long long row, bool row_ok, long long rbase,
                                            const float (&held)[8], bool use_held) {
-  const int end = min(idx + a.g, a.K);
+  const int end = min(idx + a.g, a.Kq);
   float mn = __builtin_inff(), mx = -__builtin_inff();
   if (use_held) {
     #pragma unroll
@@ -316,19 +316,20 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
 extern "C" {
 
 int lcq_gptq_block(float* W, float* tmp, float* Losses, float* Err, int64_t ldErr, const float* U, int64_t R, int64_t K,
-                   int64_t i1, int count, int group_size, float qmin, float qmax, int flags, float* scales, float* zeros,
+                   int64_t n_quant, int64_t i1, int count, int group_size, float qmin, float qmax, int flags, float* scales, float* zeros,
                    const int32_t* gidx, int64_t G, void* stream) {
   if (!W || !tmp || !Losses || !Err || !U || !scales || ldErr < count || ldErr > 0x7fffffff) return LCQ_EINVAL;
-  if (R <= 0 || K <= 0 || K > 0x7fffffff || i1 < 0 || count <= 0 || count > BS || i1 + count > K) return LCQ_EINVAL;
+  if (R <= 0 || K <= 0 || K > 0x7fffffff || i1 < 0 || count <= 0 || count > BS) return LCQ_EINVAL;
+  if (n_quant <= 0 || n_quant > K || i1 + count > n_quant) return LCQ_EINVAL;
   if (!(qmax > qmin) || G <= 0) return LCQ_EINVAL;
   const int is_static = (flags & LCQ_FLAG_STATIC) != 0;
   const int sym = (flags & LCQ_FLAG_SYM) != 0;
-  if (!is_static && (group_size <= 0 || G < (K + group_size - 1) / group_size)) return LCQ_EINVAL;
+  if (!is_static && (group_size <= 0 || G < (n_quant + group_size - 1) / group_size)) return LCQ_EINVAL;
   if (!sym && !zeros) return LCQ_EINVAL;
   LoopArgs a;
   a.W = W; a.tmp = tmp; a.Losses = Losses; a.Err = Err; a.U = U;
   a.scales = scales; a.zeros = zeros; a.gidx = gidx;
-  a.R = R; a.K = (int)K; a.i1 = (int)i1; a.count = count; a.g = group_size; a.G = (int)G;
+  a.R = R; a.K = (int)K; a.Kq = (int)n_quant; a.i1 = (int)i1; a.count = count; a.g = group_size; a.G = (int)G;
   a.qmin = qmin; a.qmax = qmax; a.sym = sym; a.is_static = is_static; a.ldErr = (int)ldErr;
   a.nrz = (flags & LCQ_FLAG_NO_ROUND_ZP) != 0;
   a.aligned = ((reinterpret_cast<uintptr_t>(W) | reinterpret_cast<uintptr_t>(tmp) | reinterpret_cast<uintptr_t>(Losses) |

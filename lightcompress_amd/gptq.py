@@ -26,7 +26,8 @@ Differences a caller can observe
     [R*G, 1] layout the reference writes;
   * fp32 activations are split into two bf16 halves (x = hi + lo to 2^-17) and accumulated as the four products of
     the halves on the bf16 matrix pipe; bf16 / fp16 activations go in as they are (their products are exact in fp32);
-  * OWQ (outlier columns kept in fp16) is not carried over.
+  * OWQ (`special.owq`): the Linears' outlier counts come from `special.n_outs` plus `set_block_linears(names)`
+    (the reference reads the order from its model wrapper), or from a dict; Hessians and chains are not shared.
 """
 from __future__ import annotations
 
@@ -75,15 +76,23 @@ class GPTQ:
         self.chain_overlap = bool(special_config.get('chain_overlap', True))
         # Linears of a subset that keep receiving the very same input tensor share one Hessian and one chain
         self.auto_share = bool(special_config.get('auto_share', True))
-        if self.owq:
-            raise NotImplementedError('OWQ is not on this path')
+        if self.owq:                                     # gptq.py:47-50
+            self.n_outs = special_config['n_outs']
+            self.static_groups = False
+            self.actorder = False
         if self.blocksize > 128:
             raise NotImplementedError('blocksize above 128 is not supported by the column-loop kernel')
         self.need_perm = (
             self.wquantizer.granularity == 'per_group'
             and not self.static_groups
             and self.actorder
-        )
+        ) or self.owq
+
+    def set_block_linears(self, names):
+        """OWQ: `special.n_outs` lists the number of outlier columns per Linear in the order the model names the
+        Linears of a block (gptq.py:88-92, `n_out_dict`); `names` is that order.  A dict name -> count in `n_outs`
+        needs no call."""
+        self.n_out_dict = {name: self.n_outs[i] for i, name in enumerate(names)}
 
     # -- Hessian (gptq.py:253-308) ---------------------------------------------
     @torch.no_grad()
@@ -141,7 +150,7 @@ class GPTQ:
                 return True
             self._unfollow(name, cache, lead)
             return False
-        if not (self.auto_share and separable) or calls != 0:
+        if not (self.auto_share and separable) or calls != 0 or self.owq:
             return False
         for other, oc in self.layers_cache.items():       # first call: is there a Linear that just got this tensor?
             if other == name or oc.get('leader', other) != other or 'H' not in oc or oc.get('manual_share'):
@@ -309,8 +318,16 @@ class GPTQ:
     def hessian_sorting(self, name):
         """gptq.py:58-64: act-order permutation from the raw diagonal."""
         H = self._settle(name)['H']
-        if self.actorder:
-            self.perm = torch.argsort(torch.diag(H), descending=True)
+        if not self.owq:
+            if self.actorder:
+                self.perm = torch.argsort(torch.diag(H), descending=True)
+            return
+        # OWQ (gptq.py:66-83; its act-order branch is unreachable, add_quant_config switches act-order off):
+        # the n_out columns with the largest Hessian diagonal go last, the others keep their order
+        temp_mask = torch.full([self.columns], True, device=self.dev)
+        descending_ids = torch.argsort(torch.diag(H), descending=True)
+        temp_mask[descending_ids[: self.n_out]] = False
+        self.perm = torch.cat([torch.arange(self.columns, device=self.dev)[temp_mask], descending_ids[: self.n_out]])
 
     # -- per-layer driver (gptq.py:96-196) -----------------------------------------
     @torch.no_grad()
@@ -326,7 +343,7 @@ class GPTQ:
         a few hundred short dependent launches (diagonal blocks, panel solves) that leave most of the chip idle, so
         the chains of q/k/v (or gate/up) run in about the time of one.  layer_transform then finds the finished factor
         exactly as it finds a shared one; results are the same as one by one."""
-        if not self.chain_overlap:
+        if not self.chain_overlap or self.owq:           # OWQ: every Linear has its own column order
             return
         todo = []
         for name in layers_dict:
@@ -370,13 +387,19 @@ class GPTQ:
     def initialize_qparams_and_prepare_weights(self, layer, name):
         self.qparams = {}
         self.columns = self.layers_cache[name]['columns']
-        self.n_out = 0
-        self.n_nonout = self.columns
+        if self.owq:
+            nd = self.n_outs if isinstance(self.n_outs, dict) else getattr(self, 'n_out_dict', None)
+            if nd is None:
+                raise L.LcqError('OWQ: call set_block_linears(names) first (or give special.n_outs as a dict)')
+            self.n_out = nd[name]
+        else:
+            self.n_out = 0
+        self.n_nonout = self.columns - self.n_out
         cache = self.layers_cache[name]
         leader = cache.get('leader', name)
-        if leader in self._shared:
+        if leader in self._shared and not self.owq:
             self.perm = self._shared[leader].get('perm')
-        elif self.actorder:
+        elif self.actorder or self.owq:
             self.hessian_sorting(name)
 
     def process_hessian_and_weights(self, layer, name):
@@ -397,7 +420,7 @@ class GPTQ:
         if shared is None:
             is_shared = any(c.get('leader') == leader for n, c in self.layers_cache.items() if n != name) \
                 or leader != name
-            perm = self.perm if self.actorder else None
+            perm = self.perm if (self.actorder or self.owq) else None
             dead = torch.diag(H) == 0                       # before the chain rewrites H
             ws_bytes = L.lib().lcq_chol_inv_upper_workspace_bytes(L.i64(K))
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=self.dev)
@@ -418,12 +441,18 @@ class GPTQ:
         W = torch.empty((R, K), dtype=torch.float32, device=w.device)
         dead_u8 = shared['dead'].view(torch.uint8)
         L.check(L.lib().lcq_gptq_prepare_weights(L.ptr(w), L.i32(L.dtype_code(w.dtype)), L.i64(R), L.i64(K),
-                                                 L.ptr(self.perm if self.actorder else None), L.ptr(dead_u8), L.ptr(W),
-                                                 L.stream()), 'lcq_gptq_prepare_weights')
-        if self.actorder:
+                                                 L.ptr(self.perm if (self.actorder or self.owq) else None), L.ptr(dead_u8),
+                                                 L.ptr(W), L.stream()), 'lcq_gptq_prepare_weights')
+        if self.actorder or self.owq:
             self.invperm = torch.argsort(self.perm)
             layer.buf_perm = self.perm
             layer.buf_invperm = self.invperm
+            if self.owq:                                    # gptq.py:158-167
+                layer.buf_n_nonout = torch.tensor(self.n_nonout)
+                if self.wquantizer.granularity == 'per_channel':
+                    _, layer.buf_scales, layer.buf_zeros, _, _ = self.wquantizer.get_tensor_qparams(
+                        W[:, : self.n_nonout].contiguous())
+                    self._setup_groups(layer, R, K)
         return W, U
 
     def _setup_groups(self, layer, R, K):
@@ -432,7 +461,7 @@ class GPTQ:
         self._gidx = None
         if wq.granularity == 'per_group':
             g = wq.group_size
-            G = math.ceil(K / g)
+            G = math.ceil(self.n_nonout / g)             # groups of the quantized columns (all K without OWQ)
             self._g, self._G = g, G
             if self.static_groups:
                 self._scales = layer.buf_scales.reshape(R, G).float().contiguous()
@@ -459,7 +488,11 @@ class GPTQ:
         self.last_error = torch.sum(Losses)              # device scalar; .item() it to log like the reference
         if self.check_positive_definite and int(self._status.item()) != 0:
             raise torch.linalg.LinAlgError('GPTQ: the damped Hessian is not positive-definite')
-        if self.actorder:                                # tmp[:, invperm]
+        if self.owq and self.n_out > 0:                  # the outlier columns stay in floating point, with the
+            tmp[:, self.n_nonout:] = W[:, self.n_nonout:]      # updates of the loop (gptq.py:187-188)
+            Losses[:, self.n_nonout:] = 0
+            self.last_error = torch.sum(Losses)
+        if self.actorder or self.owq:                    # tmp[:, invperm]
             out = torch.empty_like(tmp)
             L.check(L.lib().lcq_gptq_prepare_weights(L.ptr(tmp), L.i32(L.F32), L.i64(tmp.shape[0]), L.i64(tmp.shape[1]),
                                                      L.ptr(self.invperm), L.ptr(None), L.ptr(out), L.stream()),
@@ -500,18 +533,18 @@ class GPTQ:
             if not self._static and g > 0:
                 last_open = (o1 - 1) // g * g
                 if last_open >= o0:
-                    hi = max(o1, min(last_open + g, K))
+                    hi = max(o1, min(last_open + g, n))
             for i1 in range(o0, o1, self.blocksize):
                 i2 = min(i1 + self.blocksize, o1)
                 if host_groups:
                     for idx in range((i1 + g - 1) // g * g, i2, g):
-                        _, s_, z_, _, _ = wq.get_tensor_qparams(W[:, idx:min(idx + g, K)].contiguous())
+                        _, s_, z_, _, _ = wq.get_tensor_qparams(W[:, idx:min(idx + g, n)].contiguous())
                         self._scales[:, idx // g] = s_.reshape(-1).float()
                         if not wq.sym:
                             self._zeros[:, idx // g] = z_.reshape(-1).float()
                 err_blk = Err[:, i1 - o0:]
                 L.check(lib.lcq_gptq_block(L.ptr(W), L.ptr(tmp), L.ptr(Losses), C_ptr(err_blk), L.i64(window), L.ptr(Hinv),
-                                           L.i64(R), L.i64(K), L.i64(i1), L.i32(i2 - i1), L.i32(self._g), qmin, qmax,
+                                           L.i64(R), L.i64(K), L.i64(n), L.i64(i1), L.i32(i2 - i1), L.i32(self._g), qmin, qmax,
                                            L.i32(flags), L.ptr(self._scales), L.ptr(self._zeros), L.ptr(self._gidx),
                                            L.i64(self._G), st), 'lcq_gptq_block')
                 if i2 < hi:
@@ -569,7 +602,11 @@ class GPTQ:
         args['zeros'] = module.buf_zeros if hasattr(module, 'buf_zeros') else None
         args['qmax'] = module.buf_qmax
         args['qmin'] = module.buf_qmin
+        if self.owq:
+            fp_weight = weight[:, module.buf_n_nonout:]
         weight = wquantizer.fake_quant_weight_static(weight, args).to(self.model_dtype)
+        if self.owq:
+            weight[:, module.buf_n_nonout:] = fp_weight.to(self.model_dtype)
         if self.need_perm:
             weight = weight[:, module.buf_invperm]
         return weight

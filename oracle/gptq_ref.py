@@ -53,6 +53,16 @@ def act_order(H: torch.Tensor) -> torch.Tensor:
     return torch.argsort(torch.diag(H), descending=True)
 
 
+def owq_order(H: torch.Tensor, n_out: int) -> torch.Tensor:
+    """hessian_sorting with owq, gptq.py:66-83 (act-order is off whenever owq is on, :47-50): the n_out columns with
+    the largest diagonal move to the end, the rest keep their order."""
+    K = H.shape[0]
+    mask = torch.full([K], True)
+    descending_ids = torch.argsort(torch.diag(H), descending=True)
+    mask[descending_ids[:n_out]] = False
+    return torch.cat([torch.arange(K)[mask], descending_ids[:n_out]])
+
+
 def process_hessian_and_weights(weight: torch.Tensor, H: torch.Tensor, percdamp: float, perm=None,
                                 dtype=torch.float32):
     """-> (W [R,K] in `dtype`, Hinv upper Cholesky factor of the damped inverse, invperm|None)."""
@@ -78,7 +88,7 @@ def process_hessian_and_weights(weight: torch.Tensor, H: torch.Tensor, percdamp:
 # ---------------------------------------------------------------------------
 # lazy-batch column loop   (gptq.py:198-244)
 # ---------------------------------------------------------------------------
-def weight_transform(W, Hinv, spec, blocksize=128, static_qparams=None, static_groups=None, qparams_fn=None):
+def weight_transform(W, Hinv, spec, blocksize=128, static_qparams=None, static_groups=None, qparams_fn=None, n_out=0):
     """Runs the loop in place on W (as the reference does) and returns
     (tmp, Losses, groups) where groups is the list of per-group
     (scale [R,1], zero [R,1]|0-dim) refreshed at every group boundary.
@@ -91,6 +101,8 @@ def weight_transform(W, Hinv, spec, blocksize=128, static_qparams=None, static_g
     ``groups[perm[idx] // g]`` (gptq.py:143-148, 224-227); nothing is refreshed.
     ``qparams_fn(spec, cols) -> (rows, scale, zero, qmax, qmin)`` stands for ``wquantizer.get_tensor_qparams``
     (gptq.py:358-366 calls it, so ``calib_algo`` reaches the loop); default: min/max calibration.
+    ``n_out``: OWQ - the last n_out columns are not quantized (the loop and the group ranges stop before them) but
+    still receive every block's update.
     """
     qparams_fn = qparams_fn or Q.int_tensor_qparams
     R, K = W.shape
@@ -101,8 +113,9 @@ def weight_transform(W, Hinv, spec, blocksize=128, static_qparams=None, static_g
     if not per_group:
         scale, zero = static_qparams
     qmax, qmin = spec.qmax, spec.qmin
-    for i1 in range(0, K, blocksize):
-        i2 = min(i1 + blocksize, K)
+    n_nonout = K - n_out
+    for i1 in range(0, n_nonout, blocksize):
+        i2 = min(i1 + blocksize, n_nonout)
         count = i2 - i1
         W1, Hinv1 = W[:, i1:i2].clone(), Hinv[i1:i2, i1:i2]
         tmp1, Err1, Losses1 = torch.zeros_like(W1), torch.zeros_like(W1), torch.zeros_like(W1)
@@ -116,7 +129,7 @@ def weight_transform(W, Hinv, spec, blocksize=128, static_qparams=None, static_g
                 scale = sg[:, idx // spec.group_size].unsqueeze(1)
                 zero = torch.tensor(0.0) if zg is None else zg[:, idx // spec.group_size].unsqueeze(1)
             elif per_group and (i1 + i) % spec.group_size == 0:
-                cols = W[:, (i1 + i): min(i1 + i + spec.group_size, K)]      # W, not W1 (gptq.py:216-222)
+                cols = W[:, (i1 + i): min(i1 + i + spec.group_size, K - n_out)]      # W, not W1 (gptq.py:216-222)
                 _, scale, zero, qmax, qmin = qparams_fn(spec, cols)
                 groups.append((scale.clone(), zero.clone()))
             q = Q.int_quant_dequant(spec, w.unsqueeze(1), scale, zero, qmax, qmin).squeeze(1)
@@ -148,13 +161,23 @@ def mse_tensor_qparams(spec, t, **mse):
 
 
 def gptq_layer(weight, H, spec, percdamp=0.01, blocksize=128, actorder=False, dtype=torch.float32,
-               static_qparams=None, qparams_fn=None):
-    """layer_transform (gptq.py:113-196): -> dict(weight=tmp un-permuted, scales, zeros, perm, loss, Hinv)."""
-    perm = act_order(H) if actorder else None
+               static_qparams=None, qparams_fn=None, owq_n_out=None):
+    """layer_transform (gptq.py:113-196): -> dict(weight=tmp un-permuted, scales, zeros, perm, loss, Hinv).
+    ``owq_n_out`` (an int) switches OWQ on: outlier-last column order, per_channel qparams from the non-outlier
+    columns of the permuted weight (:158-167), outlier columns written back un-quantized (:187-188)."""
+    owq = owq_n_out is not None
+    n_out = owq_n_out if owq else 0
+    perm = owq_order(H, n_out) if owq else (act_order(H) if actorder else None)
     W, Hinv, invperm = process_hessian_and_weights(weight, H, percdamp, perm, dtype)
-    tmp, Losses, groups = weight_transform(W, Hinv, spec, blocksize, static_qparams, qparams_fn=qparams_fn)
+    if owq and spec.granularity == 'per_channel':
+        _, s_, z_, _, _ = Q.int_tensor_qparams(spec, W[:, :W.shape[1] - n_out])
+        static_qparams = (s_, z_)
+    tmp, Losses, groups = weight_transform(W, Hinv, spec, blocksize, static_qparams, qparams_fn=qparams_fn, n_out=n_out)
     out = dict(loss=float(Losses.sum()), perm=perm, Hinv=Hinv, tmp_perm=tmp)
-    if actorder:
+    if owq:
+        tmp[:, W.shape[1] - n_out:] = W[:, W.shape[1] - n_out:]
+        out['static_qparams'] = static_qparams
+    if actorder or owq:
         tmp = tmp[:, invperm]
     out['weight'] = tmp
     if groups:

@@ -465,11 +465,16 @@ def test_loop_with_mse_calibrated_groups(dev, g, bs, K):
     assert abs(float(Losses.sum()) - float(Loss_o.sum())) <= 0.02 * float(Loss_o.sum())
 
 
-def test_learnable_calibration_raises(dev):
-    gp = make_gptq(weight=dict(bit=4, symmetric=False, granularity='per_group', group_size=128, calib_algo='learnable'))
+def test_learnable_calibration_without_factors_is_minmax(dev):
+    """search_column_qparams passes no factors (gptq.py:358-366), so calib_algo='learnable' falls through to the
+    plain min/max range (quant.py:207-221): same weights, losses and qparams as the default calibrator."""
     spec, W0, W, U = _loop_case(16, 256, 128, 128, False, 5700)
-    with pytest.raises(NotImplementedError):
-        _run_loop(dev, gp, W, U, 16, 256)
+    outs = []
+    for algo in ('learnable', 'minmax'):
+        gp = make_gptq(weight=dict(bit=4, symmetric=False, granularity='per_group', group_size=128, calib_algo=algo))
+        outs.append(_run_loop(dev, gp, W, U, 16, 256))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
 
 
 @pytest.mark.parametrize('actorder', [False, True])
@@ -612,3 +617,60 @@ def test_hessian_from_fp32_activations(dev, K, T, nb, defer):
     # the bf16-rounded activations are a different matrix at this tolerance
     rounded = G.hessian_closed_form([b.bfloat16() for b in batches])
     assert float((rounded - ref64).abs().max()) / scale > 1e-4
+
+
+@pytest.mark.parametrize('gran,n_out', [('per_group', 100), ('per_channel', 37), ('per_group', 128)])
+def test_owq_layer(dev, gran, n_out):
+    """special.owq: outlier-last column order, loop and group ranges over the non-outlier columns only, outlier
+    columns written back with the loop's compensation, per_channel qparams from the permuted non-outlier weight,
+    w_qdq restoring the kept columns - against the fp32 oracle."""
+    R, K, g, nb, T = 64, 768, 128, 6, 200
+    batches = calib_batches(nb, T, K, seed=7100)
+    W0 = (torch.randn(R, K, generator=gen(7101)) * 0.02).bfloat16()
+    spec = Q.IntSpec(4, False, gran, group_size=g)
+    Ho = torch.zeros(K, K); n = 0
+    for b in batches:
+        n = G.add_batch(Ho, n, b.unsqueeze(0))
+    ref = G.gptq_layer(W0, Ho, spec, owq_n_out=n_out)
+    wcfg = dict(bit=4, symmetric=False, granularity=gran)
+    if gran == 'per_group':
+        wcfg['group_size'] = g
+    gp = make_gptq(weight=wcfg, owq=True, n_outs=[5, n_out], actorder=True)
+    assert gp.actorder is False and gp.need_perm
+    gp.set_block_linears(['other', 'fc'])
+    layer = Layer(W0.to(dev))
+    gp.subset_init({'layers': {'fc': layer}})
+    if gran == 'per_channel':
+        gp.collect_layer_qparams(layer)
+    for b in batches:
+        gp.add_batch(layer, 'fc', b.unsqueeze(0).to(dev), None)
+    gp.layer_transform(layer, 'fc')
+    nq = K - n_out
+    perm = layer.buf_perm.cpu()
+    assert int(layer.buf_n_nonout) == nq and torch.equal(torch.sort(perm[:nq]).values, perm[:nq])
+    d = torch.diag(Ho)
+    assert float(d[perm[nq:]].min()) >= float(d[perm[:nq]].max()) * (1 - 1e-5)
+    Wq = layer.weight.data.cpu()
+    tmp = Wq[:, perm]
+    if torch.equal(perm, ref['perm']):
+        if gran == 'per_group':
+            s, z = layer.buf_scales.cpu(), layer.buf_zeros.cpu()
+            assert s.shape == ref['scales'].shape
+            codes = G.codes_from(tmp[:, :nq], s, z, spec)
+            codes_o = G.codes_from(ref['tmp_perm'][:, :nq], ref['scales'], ref['zeros'], spec)
+        else:
+            s, z = layer.buf_scales.cpu().float(), layer.buf_zeros.cpu().float()
+            so, zo = ref['static_qparams']
+            assert torch.allclose(s, so, rtol=1e-6) and torch.equal(z, zo)
+            codes = Q.int_quant(spec, tmp[:, :nq], s, z, spec.qmax, spec.qmin)
+            codes_o = Q.int_quant(spec, ref['tmp_perm'][:, :nq], so, zo, spec.qmax, spec.qmin)
+        assert float((codes == codes_o).float().mean()) >= 0.999
+        keep, keep_o = tmp[:, nq:], ref['weight'][:, perm][:, nq:]
+        assert float((keep - keep_o).abs().max()) <= 1e-3 * float(keep_o.abs().max())
+    assert abs(float(gp.last_error) - ref['loss']) <= 0.01 * ref['loss']
+    if gran == 'per_channel':
+        layer.buf_qmax, layer.buf_qmin = gp.wquantizer.qmax, gp.wquantizer.qmin
+        fq = gp.w_qdq(layer, gp.wquantizer).cpu().float()
+        assert torch.equal(fq[:, perm][:, nq:], tmp[:, nq:].bfloat16().float())
+        want = Q.int_fake_quant_static(spec, tmp, s, z, spec.qmax, spec.qmin)[:, :nq].bfloat16().float()
+        assert torch.equal(fq[:, perm][:, :nq], want)

@@ -158,3 +158,39 @@ def test_actorder_and_layer_driver_roundtrip():
     deq = Q.int_quant_dequant(spec, out['tmp_perm'].reshape(-1, 128), out['scales'], out['zeros'], spec.qmax, spec.qmin)
     What = deq.reshape(R, K)[:, torch.argsort(out['perm'])]
     assert G.recon_loss(W0, What, X) < G.recon_loss(W0, Q.int_fake_quant_dynamic(spec, W0), X)
+
+
+@pytest.mark.parametrize('gran', ['per_group', 'per_channel'])
+def test_owq_keeps_outlier_columns_and_the_loss_identity(gran):
+    """OWQ (gptq.py:44-56, 66-83, 158-167, 187-188).  Column order: the n_out largest diagonal entries last, the rest in
+    their original order.  The un-quantized columns behave like columns quantized to themselves, so the loss identity
+    holds over ALL columns with the outlier columns' compensated values on the quantized side; with n_out = 0 the
+    result is plain GPTQ in the original order."""
+    R, K, g, n_out = 4, 256, 64, 64
+    spec = Q.IntSpec(4, False, gran, group_size=g)
+    H = G.hessian_closed_form(calib_batches(6, 64, K, seed=2100))
+    perm = G.owq_order(H, n_out)
+    top = torch.argsort(torch.diag(H), descending=True)[:n_out]
+    assert torch.equal(perm[K - n_out:], top)
+    assert torch.equal(perm[:K - n_out], torch.sort(perm[:K - n_out]).values) and torch.equal(torch.sort(perm).values, torch.arange(K))
+    W0 = torch.randn(R, K, generator=gen(6), dtype=torch.float64) * 0.02
+    out = G.gptq_layer(W0, H, spec, dtype=torch.float64, owq_n_out=n_out)
+    Wp = W0[:, perm]
+    Hd = (H + 0.01 * torch.mean(torch.diag(H)) * torch.eye(K, dtype=torch.float64))[perm][:, perm]
+    tmp = out['weight'][:, perm]                            # processing order again
+    nq = K - n_out
+    if gran == 'per_group':
+        assert out['scales'].shape == (R * (nq // g), 1)
+        Qd = Q.int_quant_dequant(spec, tmp[:, :nq].reshape(-1, g), out['scales'], out['zeros'], spec.qmax, spec.qmin).reshape(R, nq)
+    else:
+        s_, z_ = out['static_qparams']
+        want_s, want_z = Q.int_tensor_qparams(spec, Wp[:, :nq])[1:3]
+        assert torch.equal(s_, want_s) and torch.equal(z_, want_z)
+        Qd = Q.int_quant_dequant(spec, tmp[:, :nq], s_, z_, spec.qmax, spec.qmin)
+    full = torch.cat([Qd, tmp[:, nq:]], dim=1)
+    D = Wp - full
+    assert abs(out['loss'] - 0.5 * float(torch.trace(D @ Hd @ D.t()))) < 1e-12 + 1e-9 * out['loss']
+    assert not torch.equal(tmp[:, nq:], Wp[:, nq:])         # the kept columns did take the compensation
+    plain = G.gptq_layer(W0, H, spec, dtype=torch.float64, static_qparams=Q.int_tensor_qparams(spec, W0)[1:3])
+    zero = G.gptq_layer(W0, H, spec, dtype=torch.float64, owq_n_out=0)
+    assert torch.equal(zero['weight'], plain['weight']) and zero['loss'] == plain['loss']
