@@ -103,151 +103,279 @@ __global__ __launch_bounds__(256) void build_kernel(const float* __restrict__ H,
   A[(long long)a * K + b] = v;
 }
 
-// Diagonal block: Cholesky factor L11 and its inverse in one elimination sweep.
-// 256 threads hold the 128x128 block of A and of B (= I, turning into L11^-1) in registers, 8x8 each,
-// dealt out cyclically: thread (ty, tx) owns rows ty + 16 ii and columns tx + 16 cc.  The elimination
-// front therefore shrinks on every thread alike -- during columns 16P .. 16P+15 ("phase" P) a thread
-// updates (8-P)(9-P)/2 elements of A and (8-P)(P+1) of B per step, whichever thread it is -- where a
-// blocked layout leaves the last wave with 128 FMAs per step to the end while the first idles.
-// Step j:
-//   barrier; every thread reads the UNSCALED column j of A, row j of B and the pivot from LDS (double
-//   buffered; entries that must not take part are published as zeros, so no update needs a mask),
-//   derives 1/sqrt(a_jj) itself and applies
-//     a[i][k] -= l_ij l_kj  (i, k > j)      b[i][:] -= l_ij x_j[:]  (i > j)
-//   starting with the two register columns of A and rows of B that can hold column / row j+1, which
-//   their owners publish at once; the rest of the update then overlaps the next barrier.
-// The right-looking Cholesky update and the forward substitution L X = I share the broadcast.
+// Diagonal block: Cholesky factor L11 of a 128x128 block and its inverse, one workgroup of 8 waves.
+// A wave that is alone on its SIMD issues about one instruction per 8 cycles, and a column-by-column sweep with a
+// barrier per column executes ~150 instructions per column in every wave: 70 us per block, none of it arithmetic.
+// Here the 128 columns are 8 panels of 16, and the serial part of a panel runs in ONE wave without barriers:
+//   * waves 0-3 ("update waves") hold the lower triangle in registers, 8x8 per thread, dealt out cyclically (thread
+//     (ty, tx) owns rows ty + 16 ii and columns tx + 16 cc);
+//   * wave 4 (the "panel wave") takes the current 16-column panel from LDS with one or two rows per lane and factors
+//     it in registers: pivot and multipliers travel by v_readlane, 3 instructions per (column, later column) pair;
+//     it leaves the scaled panel in LDS;
+//   * the update waves apply a finished panel first to the next panel's columns, hand those to the panel wave, and
+//     apply it to the rest of their registers while the panel wave is already factoring (a right-looking update
+//     with look-ahead); two barriers per panel;
+//   * wave 5 inverts the 16x16 diagonal block of the previous panel meanwhile (forward substitution in registers);
+//   * afterwards all 8 waves merge the inverted diagonal blocks pairwise, 16 -> 32 -> 64 -> 128,
+//     [[A,0],[B,C]]^-1 = [[A^-1,0],[-C^-1 B A^-1, C^-1]], from LDS.
 constexpr int lds_slot(int r) { return (r & 15) * 8 + (r >> 4); }   // a thread's 8 rows (columns) are contiguous
+constexpr int LP = NB + 4;       // row pitch of the LDS matrices (16-byte aligned rows, 4-bank skew)
 
-template <int P>
-__device__ __forceinline__ void potrf_phase(float (&a)[8][8], float (&x)[8][8], float (*colbuf)[NB], float (*rowbuf)[NB],
-                                            float* pivbuf, int ty, int tx, bool& bad) {
+struct PotrfLds {
+  float L[8][16][LP];    // L[P][k][lds_slot(r)] = L(r, 16 P + k); zero above the diagonal inside the panel's own 16 rows
+  float X[NB][LP];       // L^-1, row-major
+  float Pn[16][NB];      // the panel on its way to the panel wave, same layout as L[P], unscaled
+  float T[64 * 64];      // products of the inverse merges
+};
+
+__device__ __forceinline__ float rdlane(float v, int l) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
+}
+
+// panel P: columns 16 P .. +15, rows 16 P .. 127; lane l owns row 16 P + l and (TWO) row 16 P + 64 + l
+template <bool TWO>
+__device__ __forceinline__ void potrf_panel(PotrfLds& s, int P, int lane, bool& bad) {
   #pragma clang fp contract(fast)   // a -= l*l as one FMA; nothing here needs op-by-op rounding
-  constexpr int P1 = (P < 7) ? P + 1 : 7;
-  #pragma unroll 1
-  for (int jl = 0; jl < 16; ++jl) {
-    const int j = 16 * P + jl, pb = j & 1;
-    __syncthreads();
-    const float pv = pivbuf[pb];
-    const f32x4 r0 = *(const f32x4*)(colbuf[pb] + 8 * ty), r1 = *(const f32x4*)(colbuf[pb] + 8 * ty + 4);
-    const f32x4 c0 = *(const f32x4*)(colbuf[pb] + 8 * tx), c1 = *(const f32x4*)(colbuf[pb] + 8 * tx + 4);
-    const f32x4 x0 = *(const f32x4*)(rowbuf[pb] + 8 * tx), x1 = *(const f32x4*)(rowbuf[pb] + 8 * tx + 4);
-    bad = bad || !(pv > 0.0f);
-    float rinv = __builtin_amdgcn_rsqf(pv);           // 1/sqrt(pivot), one Newton step to full precision
-    rinv = rinv * (1.5f - 0.5f * pv * rinv * rinv);
-    float lr[8], lc[8], xr[8];
+  const int c0 = 16 * P;
+  const int rA = c0 + lane, rB = c0 + 64 + lane;
+  const bool okA = rA < NB, okB = TWO && rB < NB;
+  const int sA = lds_slot(okA ? rA : 0), sB = lds_slot(okB ? rB : 0);
+  float a0[16], a1[16];
+  #pragma unroll
+  for (int k = 0; k < 16; ++k) {
+    a0[k] = okA ? s.Pn[k][sA] : 0.0f;
+    a1[k] = okB ? s.Pn[k][sB] : 0.0f;
+  }
+  #pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    const float piv = rdlane(a0[j], j);
+    bad = bad || !(piv > 0.0f);
+    float rinv = __builtin_amdgcn_rsqf(piv);          // 1/sqrt(pivot), one Newton step to full precision
+    rinv = rinv * (1.5f - 0.5f * piv * rinv * rinv);
+    a0[j] *= rinv;                                    // the diagonal entry becomes sqrt(pivot); rows above it hold zeros
+    if (TWO) a1[j] *= rinv;
     #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      lr[k] = r0[k] * rinv; lr[4 + k] = r1[k] * rinv;
-      lc[k] = c0[k] * rinv; lc[4 + k] = c1[k] * rinv;
-      xr[k] = x0[k] * rinv; xr[4 + k] = x1[k] * rinv;
+    for (int c = j + 1; c < 16; ++c) {
+      const float m = rdlane(a0[j], c);               // L(16 P + c, 16 P + j)
+      a0[c] -= a0[j] * m;                             // (entries above the diagonal pick up garbage; never read, masked below)
+      if (TWO) a1[c] -= a1[j] * m;
     }
-    // ---- first: what column j+1 of A and row j+1 of B can depend on ----
-    #pragma unroll
-    for (int ii = P; ii < 8; ++ii) {
-      a[ii][P] -= lr[ii] * lc[P];
-      if (P1 != P && P1 <= ii) a[ii][P1] -= lr[ii] * lc[P1];
-    }
-    #pragma unroll
-    for (int cc = 0; cc <= P; ++cc) {
-      x[P][cc] -= lr[P] * xr[cc];
-      if (P1 != P) x[P1][cc] -= lr[P1] * xr[cc];
-    }
-    // owners keep the scaled column j of L and row j of X (the published zeros left their own entries alone)
-    if (tx == jl) {
-      #pragma unroll
-      for (int ii = P; ii < 8; ++ii) {
-        const int r = ty + 16 * ii;
-        if (r > j) a[ii][P] = lr[ii];
-        else if (r == j) a[ii][P] = pv * rinv;
-      }
-    }
-    if (ty == jl) {
-      #pragma unroll
-      for (int cc = 0; cc <= P; ++cc) x[P][cc] = xr[cc];
-    }
-    // ---- publish column j+1 / row j+1 for the next step ----
-    if (j + 1 < NB) {
-      const int jn = j + 1, tn = jn & 15;
-      const bool nextphase = (jl == 15);
-      if (tx == tn) {
-        f32x4 v0, v1;
-        #pragma unroll
-        for (int ii = 0; ii < 8; ++ii) {
-          const float v = (ty + 16 * ii > jn) ? (nextphase ? a[ii][P1] : a[ii][P]) : 0.0f;
-          if (ii < 4) v0[ii] = v; else v1[ii - 4] = v;
-        }
-        *(f32x4*)(colbuf[pb ^ 1] + 8 * ty) = v0;
-        *(f32x4*)(colbuf[pb ^ 1] + 8 * ty + 4) = v1;
-        if (ty == tn) pivbuf[pb ^ 1] = nextphase ? a[P1][P1] : a[P][P];
-      }
-      if (ty == tn) {
-        f32x4 v0, v1;
-        #pragma unroll
-        for (int cc = 0; cc < 8; ++cc) {
-          const float v = (tx + 16 * cc <= jn) ? (nextphase ? x[P1][cc] : x[P][cc]) : 0.0f;
-          if (cc < 4) v0[cc] = v; else v1[cc - 4] = v;
-        }
-        *(f32x4*)(rowbuf[pb ^ 1] + 8 * tx) = v0;
-        *(f32x4*)(rowbuf[pb ^ 1] + 8 * tx + 4) = v1;
-      }
-    }
-    // ---- the rest of the update ----
-    #pragma unroll
-    for (int ii = P + 2; ii < 8; ++ii)
-      #pragma unroll
-      for (int cc = P + 2; cc <= ii; ++cc) a[ii][cc] -= lr[ii] * lc[cc];
-    #pragma unroll
-    for (int ii = P + 2; ii < 8; ++ii)
-      #pragma unroll
-      for (int cc = 0; cc <= P; ++cc) x[ii][cc] -= lr[ii] * xr[cc];
+  }
+  #pragma unroll
+  for (int k = 0; k < 16; ++k) {
+    if (okA) s.L[P][k][sA] = (lane >= k) ? a0[k] : 0.0f;
+    if (okB) s.L[P][k][sB] = a1[k];
   }
 }
 
-__global__ __launch_bounds__(256) void potrf_diag_kernel(float* __restrict__ Ablk, int lda, int nb,
-                                                         float* __restrict__ Dinv, PrepScalars* sc) {
-  __shared__ __align__(16) float colbuf[2][NB];  // unscaled column j of A strictly below the diagonal, zero elsewhere
-  __shared__ __align__(16) float rowbuf[2][NB];  // unscaled row j of B up to the diagonal, zero elsewhere
-  __shared__ float pivbuf[2];                    // a_jj
-  const int tid = threadIdx.x;
-  const int ty = tid >> 4, tx = tid & 15;
-  float a[8][8], x[8][8];
+// X_QQ = L_QQ^-1 for the 16x16 diagonal block Q: lane c (mod 16) carries column c of the inverse
+__device__ __forceinline__ void potrf_diag_inv(PotrfLds& s, int Q, int lane) {
+  #pragma clang fp contract(fast)
+  const int c0 = 16 * Q, l16 = lane & 15;
+  const int sl = lds_slot(c0 + l16);
+  float t[16], x[16];
   #pragma unroll
-  for (int ii = 0; ii < 8; ++ii)
+  for (int k = 0; k < 16; ++k) t[k] = s.L[Q][k][sl];          // lane j: row j of the block
+  #pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    float acc = (l16 == j) ? 1.0f : 0.0f;
     #pragma unroll
-    for (int cc = 0; cc < 8; ++cc) {
-      const int r = ty + 16 * ii, c = tx + 16 * cc;
-      a[ii][cc] = (r < nb && c <= r) ? Ablk[(long long)r * lda + c] : ((r == c) ? 1.0f : 0.0f);   // pad with identity
-      x[ii][cc] = (r == c) ? 1.0f : 0.0f;
-    }
-  // column 0 / row 0
-  if (tx == 0) {
-    #pragma unroll
-    for (int ii = 0; ii < 8; ++ii) colbuf[0][8 * ty + ii] = (ty + 16 * ii > 0) ? a[ii][0] : 0.0f;
-    if (ty == 0) pivbuf[0] = a[0][0];
+    for (int k = 0; k < j; ++k) acc -= rdlane(t[k], j) * x[k];
+    const float d = rdlane(t[j], j);
+    float r = __builtin_amdgcn_rcpf(d);
+    r = r * (2.0f - d * r);
+    x[j] = acc * r;
   }
-  if (ty == 0) {
+  if (lane < 16) {
     #pragma unroll
-    for (int cc = 0; cc < 8; ++cc) rowbuf[0][8 * tx + cc] = (tx + 16 * cc <= 0) ? x[0][cc] : 0.0f;
+    for (int j = 0; j < 16; ++j) s.X[c0 + j][c0 + lane] = (lane <= j) ? x[j] : 0.0f;
+  }
+}
+
+// a[ii][cc] -= sum_k L(row, 16 PL + k) L(col, 16 PL + k) for the register columns CC_LO .. 7 (rows ii >= cc), or for
+// the single column CC_LO (ONE).  Compile-time ranges: a run-time range costs a branch per register column and
+// panel column, and a wave here pays ~10 cycles for every instruction it issues.
+template <int PL, int CC_LO, bool ONE>
+__device__ __forceinline__ void potrf_update(const PotrfLds& s, float (&a)[8][8], int ty, int tx) {
+  #pragma clang fp contract(fast)
+  if constexpr (CC_LO < 8) {
+    #pragma unroll 2
+    for (int k = 0; k < 16; ++k) {
+      const f32x4 r0 = *(const f32x4*)(s.L[PL][k] + 8 * ty), r1 = *(const f32x4*)(s.L[PL][k] + 8 * ty + 4);
+      const float lr[8] = {r0[0], r0[1], r0[2], r0[3], r1[0], r1[1], r1[2], r1[3]};
+      if constexpr (ONE) {
+        const float lc = s.L[PL][k][8 * tx + CC_LO];
+        #pragma unroll
+        for (int ii = CC_LO; ii < 8; ++ii) a[ii][CC_LO] -= lr[ii] * lc;
+      } else {
+        const f32x4 c0 = *(const f32x4*)(s.L[PL][k] + 8 * tx), c1 = *(const f32x4*)(s.L[PL][k] + 8 * tx + 4);
+        const float lc[8] = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
+        #pragma unroll
+        for (int cc = CC_LO; cc < 8; ++cc)
+          #pragma unroll
+          for (int ii = cc; ii < 8; ++ii) a[ii][cc] -= lr[ii] * lc[cc];
+      }
+    }
+  }
+}
+
+// register column PC (columns tx + 16 PC) -> Pn, zero above the diagonal
+template <int PC>
+__device__ __forceinline__ void potrf_publish(PotrfLds& s, const float (&a)[8][8], int ty, int tx) {
+  float v[8];
+  #pragma unroll
+  for (int ii = 0; ii < 8; ++ii) v[ii] = (ty + 16 * ii >= tx + 16 * PC) ? a[ii][PC] : 0.0f;
+  *(f32x4*)(s.Pn[tx] + 8 * ty) = f32x4{v[0], v[1], v[2], v[3]};
+  *(f32x4*)(s.Pn[tx] + 8 * ty + 4) = f32x4{v[4], v[5], v[6], v[7]};
+}
+
+// panel P of the sweep, all 8 waves
+template <int P>
+__device__ __forceinline__ void potrf_phase(PotrfLds& s, float (&a)[8][8], int wave, int lane, bool upd, int ty, int tx, bool& bad) {
+  __syncthreads();                                   // Pn holds panel P; L[P - 1] is complete
+  if (wave == 4) {
+    potrf_panel<(16 * P + 64 < NB)>(s, P, lane, bad);
+  } else if (wave == 5) {
+    if constexpr (P > 0) potrf_diag_inv(s, P - 1, lane);
+  } else if (upd) {
+    if constexpr (P > 0) potrf_update<P - 1, P + 1, false>(s, a, ty, tx);     // panel P - 1 on everything behind panel P
+  }
+  __syncthreads();                                   // L[P] is complete
+  if constexpr (P < 7) {
+    if (upd) {
+      potrf_update<P, P + 1, true>(s, a, ty, tx);      // panel P on the next panel's columns, handed over at once
+      potrf_publish<P + 1>(s, a, ty, tx);
+    }
+  }
+}
+
+// One level of the inverse: the blocks of size S on the diagonal of X are inverted already, the block below each even
+// one follows as X21 = -X22 (L21 X11), two products on the fp32 matrix pipe with operands straight from LDS.
+// v_mfma_f32_32x32x2f32: lane l supplies A(row l % 32, k = l / 32) and B(k = l / 32, column l % 32); accumulator
+// register r holds row 8 (r / 4) + 4 (l / 32) + r % 4 of column l % 32.  v_mfma_f32_16x16x4f32: A(row l % 16,
+// k = l / 16), B(k = l / 16, column l % 16), register r holds row 4 (l / 16) + r of column l % 16.
+// One wave per 32x32 (16x16) output tile; both triangular operands are cut at tile granularity and read zeros above
+// their diagonals (X is cleared at the start).
+typedef __attribute__((ext_vector_type(16))) float potrf_f32x16;
+
+template <int S>
+__device__ __forceinline__ void potrf_merge(PotrfLds& s, int wave, int lane) {
+  if constexpr (S >= 32) {
+    constexpr int TS = S / 32, TPP = TS * TS, NT = (NB / (2 * S)) * TPP;
+    const int p = wave / TPP, t = wave % TPP, ti = t / TS, tj = t % TS;
+    const int o = 2 * S * p, lm = lane & 31, lk = lane >> 5;
+    const bool on = wave < NT;
+    if (on) {
+      potrf_f32x16 acc;
+      #pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+      const int rs = lds_slot(o + S + 32 * ti + lm);
+      for (int k = 32 * tj; k < S; k += 2) {             // X11(k, j) = 0 for k < j
+        const int kk = o + k + lk;
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(s.L[kk >> 4][kk & 15][rs], s.X[kk][o + 32 * tj + lm], acc, 0, 0, 0);
+      }
+      #pragma unroll
+      for (int r = 0; r < 16; ++r)
+        s.T[(p * S + 32 * ti + 8 * (r >> 2) + 4 * lk + (r & 3)) * S + 32 * tj + lm] = acc[r];
+    }
+    __syncthreads();
+    if (on) {
+      potrf_f32x16 acc;
+      #pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+      for (int k = 0; k < 32 * (ti + 1); k += 2) {       // X22(i, k) = 0 for k > i
+        const int kk = k + lk;
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(s.X[o + S + 32 * ti + lm][o + S + kk], s.T[(p * S + kk) * S + 32 * tj + lm],
+                                                   acc, 0, 0, 0);
+      }
+      #pragma unroll
+      for (int r = 0; r < 16; ++r)
+        s.X[o + S + 32 * ti + 8 * (r >> 2) + 4 * lk + (r & 3)][o + 32 * tj + lm] = -acc[r];
+    }
+    __syncthreads();
+  } else {
+    static_assert(S == 16, "block sizes 16, 32, 64");
+    const int p = wave, o = 32 * p, lm = lane & 15, lk = lane >> 4;
+    const bool on = wave < NB / 32;
+    if (on) {
+      f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+      const int rs = lds_slot(o + 16 + lm);
+      #pragma unroll
+      for (int k = 0; k < 16; k += 4) {
+        const int kk = o + k + lk;
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(s.L[kk >> 4][kk & 15][rs], s.X[kk][o + lm], acc, 0, 0, 0);
+      }
+      #pragma unroll
+      for (int r = 0; r < 4; ++r) s.T[(p * 16 + 4 * lk + r) * 16 + lm] = acc[r];
+    }
+    __syncthreads();
+    if (on) {
+      f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+      #pragma unroll
+      for (int k = 0; k < 16; k += 4) {
+        const int kk = k + lk;
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(s.X[o + 16 + lm][o + 16 + kk], s.T[(p * 16 + kk) * 16 + lm], acc, 0, 0, 0);
+      }
+      #pragma unroll
+      for (int r = 0; r < 4; ++r) s.X[o + 16 + 4 * lk + r][o + lm] = -acc[r];
+    }
+    __syncthreads();
+  }
+}
+
+__global__ __launch_bounds__(512) void potrf_diag_kernel(float* __restrict__ Ablk, int lda, int nb,
+                                                         float* __restrict__ Dinv, PrepScalars* sc) {
+  __shared__ __align__(16) PotrfLds s;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ty = (tid >> 4) & 15, tx = tid & 15;
+  const bool upd = tid < 256;
+  for (int e = tid; e < NB * LP / 4; e += 512) ((f32x4*)&s.X[0][0])[e] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  float a[8][8];
+  if (upd) {
+    #pragma unroll
+    for (int ii = 0; ii < 8; ++ii)
+      #pragma unroll
+      for (int cc = 0; cc < 8; ++cc) {
+        const int r = ty + 16 * ii, c = tx + 16 * cc;
+        a[ii][cc] = (r < nb && c <= r) ? Ablk[(long long)r * lda + c] : ((r == c) ? 1.0f : 0.0f);   // pad with identity
+      }
+    potrf_publish<0>(s, a, ty, tx);
   }
   bool bad = false;
-  potrf_phase<0>(a, x, colbuf, rowbuf, pivbuf, ty, tx, bad);
-  if (nb > 16) potrf_phase<1>(a, x, colbuf, rowbuf, pivbuf, ty, tx, bad);
-  if (nb > 32) potrf_phase<2>(a, x, colbuf, rowbuf, pivbuf, ty, tx, bad);
-  if (nb > 48) potrf_phase<3>(a, x, colbuf, rowbuf, pivbuf, ty, tx, bad);
-  if (nb > 64) potrf_phase<4>(a, x, colbuf, rowbuf, pivbuf, ty, tx, bad);
-  if (nb > 80) potrf_phase<5>(a, x, colbuf, rowbuf, pivbuf, ty, tx, bad);
-  if (nb > 96) potrf_phase<6>(a, x, colbuf, rowbuf, pivbuf, ty, tx, bad);
-  if (nb > 112) potrf_phase<7>(a, x, colbuf, rowbuf, pivbuf, ty, tx, bad);
-  if (bad && tid == 0) sc->status = 1;
-  #pragma unroll
-  for (int ii = 0; ii < 8; ++ii)
+  potrf_phase<0>(s, a, wave, lane, upd, ty, tx, bad);
+  potrf_phase<1>(s, a, wave, lane, upd, ty, tx, bad);
+  potrf_phase<2>(s, a, wave, lane, upd, ty, tx, bad);
+  potrf_phase<3>(s, a, wave, lane, upd, ty, tx, bad);
+  potrf_phase<4>(s, a, wave, lane, upd, ty, tx, bad);
+  potrf_phase<5>(s, a, wave, lane, upd, ty, tx, bad);
+  potrf_phase<6>(s, a, wave, lane, upd, ty, tx, bad);
+  potrf_phase<7>(s, a, wave, lane, upd, ty, tx, bad);
+  __syncthreads();
+  if (wave == 5) potrf_diag_inv(s, 7, lane);
+  if (wave == 4 && bad && lane == 0) sc->status = 1;
+  __syncthreads();
+  potrf_merge<16>(s, wave, lane);
+  potrf_merge<32>(s, wave, lane);
+  potrf_merge<64>(s, wave, lane);
+  for (int v = tid; v < NB * NB / 4; v += 512) {            // L^-1, row-major, zeros above the diagonal and in the padding
+    const int r = v >> 5, c4 = (v & 31) * 4;
+    f32x4 x = *(const f32x4*)(&s.X[r][c4]);
     #pragma unroll
-    for (int cc = 0; cc < 8; ++cc) {
-      const int r = ty + 16 * ii, c = tx + 16 * cc;
-      if (r < nb && c < nb) Ablk[(long long)r * lda + c] = (c <= r) ? a[ii][cc] : 0.0f;
-      Dinv[r * NB + c] = (r < nb && c <= r && c < nb) ? x[ii][cc] : 0.0f;
+    for (int e = 0; e < 4; ++e) x[e] = (r < nb && c4 + e <= r) ? x[e] : 0.0f;
+    *(f32x4*)(Dinv + r * NB + c4) = x;
+  }
+  #pragma unroll
+  for (int q = 0; q < 4; ++q) {                             // L back into the block, in the update waves' cyclic order
+    const int cc = 2 * q + (tid >> 8), c = tx + 16 * cc;
+    const f32x4 r0 = *(const f32x4*)(s.L[cc][tx] + 8 * ty), r1 = *(const f32x4*)(s.L[cc][tx] + 8 * ty + 4);
+    const float l[8] = {r0[0], r0[1], r0[2], r0[3], r1[0], r1[1], r1[2], r1[3]};
+    #pragma unroll
+    for (int ii = 0; ii < 8; ++ii) {
+      const int r = ty + 16 * ii;
+      if (r < nb && c < nb) Ablk[(long long)r * lda + c] = (c <= r) ? l[ii] : 0.0f;
     }
+  }
 }
 
 // copy the inverted diagonal blocks into place
@@ -324,7 +452,7 @@ int lcq_chol_inv_upper(float* H, int64_t K64, const int64_t* perm, float percdam
       const int b = k0 / NB, nb = (K - k0 < NB) ? (K - k0) : NB;
       float* Akk = A + (long long)k0 * K + k0;
       float* Db = Dinv + (long long)b * NB * NB;
-      potrf_diag_kernel<<<dim3(1), dim3(256), 0, st>>>(Akk, K, nb, Db, sc);
+      potrf_diag_kernel<<<dim3(1), dim3(512), 0, st>>>(Akk, K, nb, Db, sc);
       const int k1 = k0 + nb, M = K - k1;
       if (M > 0) {
         float* A21 = A + (long long)k1 * K + k0;

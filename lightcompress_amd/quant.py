@@ -405,6 +405,12 @@ class BaseQuantizer(object):
                 t = tensor
         elif self.granularity == 'per_head':
             t = tensor.reshape(self.head_num, -1)
+        elif self.granularity == 'per_block':             # quant.py:634-638: zero-padded [M/b, b, N/b, b] view
+            m, n = tensor.shape
+            b = self.block_size
+            t_padded = torch.zeros((ceil_div(m, b) * b, ceil_div(n, b) * b), dtype=tensor.dtype, device=tensor.device)
+            t_padded[:m, :n] = tensor
+            t = t_padded.view(-1, b, t_padded.size(1) // b, b)
         else:
             t = tensor
         return t
@@ -412,6 +418,11 @@ class BaseQuantizer(object):
     def restore_tensor(self, tensor, shape):
         if tensor.shape == shape:
             return tensor
+        if self.granularity == 'per_block':                # quant.py:646-650
+            try:
+                return tensor.reshape(-1, shape[-1])[:shape[0], :]
+            except RuntimeError:
+                return tensor.reshape(shape[0], -1)[:, :shape[1]]
         try:
             return tensor.reshape(shape)
         except RuntimeError:

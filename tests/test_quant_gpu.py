@@ -337,6 +337,15 @@ def test_blockwise_fp8_casts_bit_exact(dev, dtype, shape):
         assert zq is None
         assert_bit_equal(sq, osq, 'per_block scales')
         assert_bit_equal(yq.view(torch.uint8), oyq.view(torch.uint8), f'per_block codes tie={tie}')
+    # reshape_tensor / restore_tensor for per_block (quant.py:634-651): zero-padded block view and back
+    fq = FloatQuantizer('e4m3', True, 'per_block', block_size=128, use_qtorch=True)
+    blocks = fq.reshape_tensor(wd)
+    mp, np_ = -(-shape[0] // 128) * 128, -(-shape[1] // 128) * 128
+    assert blocks.shape == (mp // 128, 128, np_ // 128, 128)
+    pad = torch.zeros(mp, np_, dtype=w.dtype)
+    pad[:shape[0], :shape[1]] = w
+    assert torch.equal(blocks.cpu(), pad.view(-1, 128, np_ // 128, 128))
+    assert torch.equal(fq.restore_tensor(blocks, wd.shape).cpu(), w)
     y2, s2 = q_to_fp8(wd, 128)
     oy2, os2, _ = Q.float_per_block_real_quant(Q.FloatSpec('e4m3', 'per_block'), w)
     assert_bit_equal(y2.view(torch.uint8), oy2.view(torch.uint8), 'quant.py weight_cast_to_fp8')
