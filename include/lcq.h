@@ -204,6 +204,10 @@ int lcq_hessian_accum_ab(float* H, int64_t K, const void* XA, const void* XB, in
 /* x [n] fp32 -> hi = bf16(x), lo = bf16(x - hi)  ([n] bf16 each; n % 4 == 0): x == hi + lo to 2^-17 relative. */
 int lcq_split_f32_bf16(const float* x, int64_t n, void* hi, void* lo, void* stream);
 
+/* The staging copy of GPTQ.add_batch (gptq.py:283-290 consumes `inp` at once; here the tokens of several calls are
+ * kept until one folded Hessian launch): dst[0 .. bytes) = src[0 .. bytes), both 16-byte aligned, bytes % 16 == 0. */
+int lcq_stage_copy(const void* src, void* dst, int64_t bytes, void* stream);
+
 /* H[j][i] = H[i][j] for i < j. */
 int lcq_symmetrize(float* H, int64_t K, void* stream);
 

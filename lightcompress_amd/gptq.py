@@ -17,7 +17,7 @@ Differences a caller can observe
   * Linears of a subset that receive the very same input tensor on every call (q/k/v, gate/up) share one Hessian
     and one Cholesky chain (``special.auto_share``, default on; detected per call, with a fallback to separate
     Hessians at the first call that differs; results are bit-identical either way);
-  * ``special.hessian_defer`` (default 'auto': 8 for K <= 8192, else 4) add_batch calls are copied to a staging buffer and
+  * ``special.hessian_defer`` (default 'auto': 16 for K <= 4096, 8 for K <= 8192, else 4) add_batch calls are copied to a staging buffer and
     folded into one launch, so ``layers_cache[name]['H']`` lags behind ``nsamples`` until
     ``hessian(name)``, ``hessian_sorting`` or ``process_hessian_and_weights`` settles it
     (``hessian_defer: 1`` updates H on every call);
@@ -247,16 +247,23 @@ class GPTQ:
         if split:
             self._halves(x, stage[f:f + x.shape[0]], cache['stage_lo'][f:f + x.shape[0]])
         else:
-            stage[f:f + x.shape[0]].copy_(x)
+            dst = stage[f:f + x.shape[0]]
+            nbytes = x.numel() * x.element_size()
+            if nbytes % 16 == 0 and x.data_ptr() % 16 == 0 and dst.data_ptr() % 16 == 0:
+                L.check(L.lib().lcq_stage_copy(L.ptr(x), C_ptr(dst), L.i64(nbytes), L.stream()), 'lcq_stage_copy')
+            else:
+                dst.copy_(x)
         cache['stage_fill'] = f + x.shape[0]
         cache['stage_batches'] += tmp
         cache['last_stage'] = (x.shape[0], tmp)
 
     def hessian_fold(self, K):
-        """add_batch calls folded into one Hessian launch for a Linear with K input features.  'auto': the launch over
-        4 calls of 2048 tokens is long enough at K = 14336 (1.5 ms); narrow Linears gain another 10 % from 8."""
+        """add_batch calls folded into one Hessian launch for a Linear with K input features.  'auto': 4 calls of 2048
+        tokens at K = 14336 (1.5 ms per launch; longer launches run at a lower sustained clock and are slower per
+        token), 8 up to K = 8192, 16 up to K = 4096 (272 tiles for 512 workgroup slots: the longer the launch, the
+        smaller the share of its ramp and tail; 0.32 -> 0.35 of the matrix peak)."""
         if self.hessian_defer == 'auto':
-            return 8 if K <= 8192 else 4
+            return 16 if K <= 4096 else (8 if K <= 8192 else 4)
         return self.hessian_defer
 
     def _halves(self, x, hi=None, lo=None):

