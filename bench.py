@@ -211,15 +211,16 @@ def bench_hessian(args, out, x=None):
     tiles = sum(K // 128 - 2 * ti for ti in range(K // 256))          # 256x128 tiles that reach the upper triangle
     exe_flops = 2.0 * TL * tiles * 256 * 128
     out['roofline'] = {
-        'kernel': f'hessian_kernel<bf16> K=14336 T={TL}', 'bound': 'mfma', 'achieved': round(alg_flops / t_h / 1e12, 2),
-        'peak': 2500.0, 'unit': 'TFLOP/s', 'frac': round(alg_flops / t_h / 2.5e15, 4),
+        'kernel': f'hessian_kernel<bf16> K=14336 T={TL}', 'bound': 'mfma', 'achieved': round(exe_flops / t_h / 1e12, 2),
+        'peak': 2500.0, 'unit': 'TFLOP/s', 'frac': round(exe_flops / t_h / 2.5e15, 4),
         'traffic': traffic_bytes('hessian_kernel_K14336_T8192') if FOLD == 4 else None,
-        'launch_us': round(t_h * 1e6, 2), 'executed_tflops': round(exe_flops / t_h / 1e12, 2),
-        'frac_executed': round(exe_flops / t_h / 2.5e15, 4),
-        'note': 'achieved counts the full 2*T*K^2 product (the algorithmic figure); only the tiles on/above the diagonal '
-                'are executed: frac_executed is the matrix-pipe utilisation against the 2.4 GHz peak.  rocprofv3 counters '
-                '(profiles/) show the pipes busy for 3/4 of the cycles at a shader clock the chip holds near 1.4 GHz '
-                'under this kernel'}
+        'launch_us': round(t_h * 1e6, 2), 'flop_executed_per_launch': exe_flops,
+        'algorithmic_tflops': round(alg_flops / t_h / 1e12, 2), 'frac_algorithmic': round(alg_flops / t_h / 2.5e15, 4),
+        'note': 'achieved / frac count the flops the matrix pipes execute (the 256x128 tiles that reach the upper '
+                'triangle of the symmetric H: matrix-pipe utilisation against the 2.4 GHz peak); the algorithmic figure '
+                '2*T*K^2 of the full product X^T X per launch is in algorithmic_tflops / frac_algorithmic.  rocprofv3 '
+                'counters (profiles/) show the pipes busy for 3/4 of the cycles at a shader clock the chip holds near '
+                '1.4 GHz under this kernel'}
 
 
 # ---------------------------------------------------------------------------------------------------------------
