@@ -218,6 +218,13 @@ int lcq_symmetrize(float* H, int64_t K, void* stream);
 int lcq_gptq_prepare_weights(const void* w, int dtype, int64_t R, int64_t K, const int64_t* perm, const uint8_t* dead,
                              float* out, void* stream);
 
+/* How the large fp32 products of the Cholesky chain (torch.linalg.cholesky / cholesky_inverse, gptq.py:172-174) and of
+ * the deferred loop update (gptq.py:244) are evaluated.  1 (default): launches of more than 256 output tiles run on
+ * the bf16 matrix pipe with every fp32 operand split into three bf16 planes and six partial products per product
+ * (accuracy of an fp32 multiply-add, 16/6 of the fp32 pipe's rate); 0: everything on the fp32 matrix pipe.
+ * Process-wide; returns the previous setting. */
+int lcq_set_gemm_split(int on);
+
 /* Dead columns, act-order permutation, damping and the Cholesky chain of
  * GPTQ.process_hessian_and_weights, gptq.py:139-141, 150-153, 169-174:
  *   dead = diag(H)==0; H[dead,dead] = 1; W[:,dead] = 0; H = H[perm][:,perm];

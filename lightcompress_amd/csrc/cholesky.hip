@@ -25,6 +25,10 @@
 #include "gemm_f32.h"
 #include "lcq_internal.h"
 
+namespace lcq {
+int g_gemm_split = 1;
+}
+
 namespace {
 using namespace lcq;
 
@@ -405,6 +409,12 @@ int64_t lcq_chol_inv_upper_workspace_bytes(int64_t K) {
   return K * K * 4 + nblk * NB * NB * 4 + ((K + 255) / 256) * 256 + 256;
 }
 
+int lcq_set_gemm_split(int on) {
+  const int was = g_gemm_split;
+  g_gemm_split = on ? 1 : 0;
+  return was;
+}
+
 int lcq_gptq_prepare_weights(const void* w, int dtype, int64_t R, int64_t K, const int64_t* perm, const uint8_t* dead,
                              float* out, void* stream) {
   if (!w || !out || R <= 0 || K <= 0 || K > 0x7fffffff || (const void*)out == w) return LCQ_EINVAL;
@@ -496,8 +506,13 @@ int lcq_chol_inv_upper(float* H, int64_t K64, const int64_t* perm, float percdam
         if (na > maxN) maxN = na;
       }
       const dim3 grid((unsigned)((maxN + GT - 1) / GT), (unsigned)((maxM + GT - 1) / GT), (unsigned)np);
-      gemm_f32_batched_kernel<false><<<grid, dim3(256), 0, st>>>(A, K, A, K, T, K, b1, 1.0f, 0.0f, GEMM_K_FROM_N);
-      gemm_f32_batched_kernel<false><<<grid, dim3(256), 0, st>>>(A, K, T, K, A, K, b2, -1.0f, 0.0f, GEMM_K_TO_M);
+      if (g_gemm_split && (long long)grid.x * grid.y * grid.z > 256) {
+        gemm_s3_batched_kernel<false><<<grid, dim3(256), 0, st>>>(A, K, A, K, T, K, b1, 1.0f, 0.0f, GEMM_K_FROM_N);
+        gemm_s3_batched_kernel<false><<<grid, dim3(256), 0, st>>>(A, K, T, K, A, K, b2, -1.0f, 0.0f, GEMM_K_TO_M);
+      } else {
+        gemm_f32_batched_kernel<false><<<grid, dim3(256), 0, st>>>(A, K, A, K, T, K, b1, 1.0f, 0.0f, GEMM_K_FROM_N);
+        gemm_f32_batched_kernel<false><<<grid, dim3(256), 0, st>>>(A, K, T, K, A, K, b2, -1.0f, 0.0f, GEMM_K_TO_M);
+      }
     }
     int w = 0;
     for (int p = 0; p < npairs; ++p) {

@@ -230,6 +230,216 @@ __device__ __forceinline__ void gemm_tile(const float* A, int lda, const float* 
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The same product on the bf16 matrix pipe: every fp32 operand is split into three bf16 planes
+//   x = hi + mid + lo,  hi = bf16(x), mid = bf16(x - hi), lo = bf16(x - hi - mid)        (both differences exact)
+// which carry 24 bits of x between them, and a product a * b is accumulated (fp32, inside the MFMA) as the six
+// partial products of weight >= 2^-16:  lo*hi + hi*lo + mid*mid + mid*hi + hi*mid + hi*hi.  The dropped terms
+// (mid*lo, lo*mid, lo*lo) are below 2^-24 of the product - the rounding of an fp32 multiply - so the result is as
+// accurate as the fp32 pipe's, at 16 / 6 times its rate (v_mfma_f32_32x32x16_bf16 against v_mfma_f32_32x32x2f32).
+// Used for the launches that fill the chip (more than one 128x128 tile per CU); small launches stay on the fp32 pipe.
+// LDS: per operand three planes of [128 rows][32 k] bf16 (row pitch 80 B: the 16 lanes of a 16-byte read hit 16
+// different bank quads) or, for B given as [k][n], of [32 k][128 n] (row pitch 320 B) read through the transposing
+// ds_read_b64_tr_b16 (a 16-lane group addresses 4 k-rows x 16 columns and receives 4 k-values of one column each).
+typedef __attribute__((ext_vector_type(8))) __bf16 s3_bf16x8;
+typedef __attribute__((ext_vector_type(4))) short s3_s16x4;
+typedef __attribute__((ext_vector_type(2))) float s3_f32x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 s3_bf16x2;
+constexpr int S3_P = 40;              // bf16 per row of a [row][k] plane
+constexpr int S3_PN = 160;            // bf16 per row of a [k][n] plane
+constexpr int S3_PLANE = GT * S3_P;   // = GK * S3_PN = 5120 bf16 per plane
+static_assert(GT * S3_P == GK * S3_PN, "plane sizes");
+
+__device__ __forceinline__ uint32_t s3_pack(float a, float b) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(s3_f32x2{a, b}, s3_bf16x2));
+}
+// four fp32 -> 4 bf16 (8 bytes) per plane
+__device__ __forceinline__ void s3_split(const f32x4& v, u32x2& hi, u32x2& mid, u32x2& lo) {
+  #pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const float a = v[2 * h], b = v[2 * h + 1];
+    const uint32_t ph = s3_pack(a, b);
+    const float ra = a - u2f(ph << 16), rb = b - u2f(ph & 0xffff0000u);
+    const uint32_t pm = s3_pack(ra, rb);
+    const float sa = ra - u2f(pm << 16), sb = rb - u2f(pm & 0xffff0000u);
+    hi[h] = ph; mid[h] = pm; lo[h] = s3_pack(sa, sb);
+  }
+}
+
+template <bool B_T>
+__device__ __forceinline__ void gemm_tile_s3(const float* A, int lda, const float* B, int ldb, float* C, int ldc, int M, int N,
+                                             int Kc, float alpha, float beta, int flags, int m0, int n0, uint16_t* sA,
+                                             uint16_t* sB) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wr = wave >> 1, wc = wave & 1;
+  int kb = 0, ke = Kc;
+  if (flags & GEMM_K_FROM_N) kb = (n0 / GK) * GK;
+  if (flags & GEMM_K_TO_M) ke = min(Kc, m0 + GT);
+
+  f32x16 acc[2][2];
+  #pragma unroll
+  for (int i = 0; i < 2; ++i)
+    #pragma unroll
+    for (int j = 0; j < 2; ++j)
+      #pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  f32x4 ra[4], rb[4];
+  auto gload = [&](int k0) {
+    #pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int idx = p * 256 + tid;
+      {
+        const int r = idx >> 3, k = k0 + (idx & 7) * 4, gm = m0 + r;
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+        if (gm < M) {
+          const float* p0 = A + (long long)gm * lda + k;
+          if (k + 3 < ke && ((((uintptr_t)p0) & 15) == 0)) v = *(const f32x4*)p0;
+          else {
+            #pragma unroll
+            for (int e = 0; e < 4; ++e) if (k + e < ke) v[e] = p0[e];
+          }
+        }
+        ra[p] = v;
+      }
+      if constexpr (B_T) {
+        const int r = idx >> 3, k = k0 + (idx & 7) * 4, gn = n0 + r;
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+        if (gn < N) {
+          const float* p0 = B + (long long)gn * ldb + k;
+          if (k + 3 < ke && ((((uintptr_t)p0) & 15) == 0)) v = *(const f32x4*)p0;
+          else {
+            #pragma unroll
+            for (int e = 0; e < 4; ++e) if (k + e < ke) v[e] = p0[e];
+          }
+        }
+        rb[p] = v;
+      } else {
+        const int k = k0 + (idx >> 5), n = n0 + (idx & 31) * 4;
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+        if (k < ke) {
+          const float* p0 = B + (long long)k * ldb + n;
+          if (n + 3 < N && ((((uintptr_t)p0) & 15) == 0)) v = *(const f32x4*)p0;
+          else {
+            #pragma unroll
+            for (int e = 0; e < 4; ++e) if (n + e < N) v[e] = p0[e];
+          }
+        }
+        rb[p] = v;
+      }
+    }
+  };
+  auto lstore = [&]() {
+    #pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int idx = p * 256 + tid;
+      u32x2 h, m, l;
+      s3_split(ra[p], h, m, l);
+      const int oa = (idx >> 3) * S3_P + (idx & 7) * 4;
+      *(u32x2*)(sA + oa) = h; *(u32x2*)(sA + S3_PLANE + oa) = m; *(u32x2*)(sA + 2 * S3_PLANE + oa) = l;
+      s3_split(rb[p], h, m, l);
+      const int ob = B_T ? oa : (idx >> 5) * S3_PN + (idx & 31) * 4;
+      *(u32x2*)(sB + ob) = h; *(u32x2*)(sB + S3_PLANE + ob) = m; *(u32x2*)(sB + 2 * S3_PLANE + ob) = l;
+    }
+  };
+  const int lm = lane & 31, lk = lane >> 5;
+  const int L = lane & 15, g16 = (lane >> 4) & 1;
+  auto compute = [&]() {
+    #pragma unroll
+    for (int ks = 0; ks < GK / 16; ++ks) {
+      s3_bf16x8 fa[2][3], fb[2][3];
+      #pragma unroll
+      for (int i = 0; i < 2; ++i)
+        #pragma unroll
+        for (int pl = 0; pl < 3; ++pl)
+          fa[i][pl] = *(const s3_bf16x8*)(sA + pl * S3_PLANE + (wr * 64 + i * 32 + lm) * S3_P + ks * 16 + lk * 8);
+      #pragma unroll
+      for (int j = 0; j < 2; ++j)
+        #pragma unroll
+        for (int pl = 0; pl < 3; ++pl) {
+          if constexpr (B_T) {
+            fb[j][pl] = *(const s3_bf16x8*)(sB + pl * S3_PLANE + (wc * 64 + j * 32 + lm) * S3_P + ks * 16 + lk * 8);
+          } else {
+            const uint16_t* q = sB + pl * S3_PLANE + (ks * 16 + lk * 8 + (L >> 2)) * S3_PN + wc * 64 + j * 32 + g16 * 16 + (L & 3) * 4;
+            const s3_s16x4 b0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s3_s16x4 __attribute__((address_space(3)))*)(q));
+            const s3_s16x4 b1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s3_s16x4 __attribute__((address_space(3)))*)(q + 4 * S3_PN));
+            fb[j][pl] = __builtin_bit_cast(s3_bf16x8, __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7));
+          }
+        }
+      #pragma unroll
+      for (int i = 0; i < 2; ++i)
+        #pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          f32x16 c = acc[i][j];
+          c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][2], fb[j][0], c, 0, 0, 0);      // small terms first
+          c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][0], fb[j][2], c, 0, 0, 0);
+          c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][1], fb[j][1], c, 0, 0, 0);
+          c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][1], fb[j][0], c, 0, 0, 0);
+          c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][0], fb[j][1], c, 0, 0, 0);
+          c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][0], fb[j][0], c, 0, 0, 0);
+          acc[i][j] = c;
+        }
+    }
+  };
+  if (kb < ke) gload(kb);
+  for (int k0 = kb; k0 < ke; k0 += GK) {
+    __syncthreads();                       // previous slab fully consumed
+    lstore();
+    __syncthreads();
+    if (k0 + GK < ke) gload(k0 + GK);      // next slab in flight while this one is multiplied
+    compute();
+  }
+  // accumulator register r of lane l: row 8*(r/4) + 4*(l/32) + r%4, column l%32 (the fp32 kernel's epilogue)
+  #pragma unroll
+  for (int i = 0; i < 2; ++i)
+    #pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int gn = n0 + wc * 64 + j * 32 + lm;
+      const int gm0 = m0 + wr * 64 + i * 32 + 4 * lk;
+      float* p0 = C + (long long)gm0 * ldc + gn;
+      float old[16];
+      if (beta != 0.0f) {
+        #pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int dm = 8 * (r >> 2) + (r & 3);
+          old[r] = (gm0 + dm < M && gn < N) ? p0[(long long)dm * ldc] : 0.0f;
+        }
+      }
+      #pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int dm = 8 * (r >> 2) + (r & 3);
+        if (gm0 + dm < M && gn < N) {
+          const float v = alpha * acc[i][j][r];
+          p0[(long long)dm * ldc] = (beta != 0.0f) ? (beta * old[r] + v) : v;
+        }
+      }
+    }
+}
+
+template <bool B_T>
+__global__ __launch_bounds__(256, 2) void gemm_s3_kernel(GemmProblem g, float alpha, float beta, int flags) {
+  __shared__ __attribute__((aligned(16))) uint16_t sA[3 * S3_PLANE];
+  __shared__ __attribute__((aligned(16))) uint16_t sB[3 * S3_PLANE];
+  const int m0 = blockIdx.y * GT, n0 = blockIdx.x * GT;
+  if ((flags & GEMM_LOWER_TILES) && n0 >= m0 + GT) return;
+  gemm_tile_s3<B_T>(g.A, g.lda, g.B, g.ldb, g.C, g.ldc, g.M, g.N, g.Kc, alpha, beta, flags, m0, n0, sA, sB);
+}
+
+template <bool B_T>
+__global__ __launch_bounds__(256, 2) void gemm_s3_batched_kernel(const float* A, int lda, const float* B, int ldb, float* C,
+                                                                 int ldc, GemmBatch bt, float alpha, float beta, int flags) {
+  __shared__ __attribute__((aligned(16))) uint16_t sA[3 * S3_PLANE];
+  __shared__ __attribute__((aligned(16))) uint16_t sB[3 * S3_PLANE];
+  const int z = blockIdx.z;
+  const int m0 = blockIdx.y * GT, n0 = blockIdx.x * GT;
+  if (m0 >= bt.M[z] || n0 >= bt.N[z]) return;
+  gemm_tile_s3<B_T>(A + bt.offA[z], lda, B + bt.offB[z], ldb, C + bt.offC[z], ldc, bt.M[z], bt.N[z], bt.Kc[z], alpha, beta,
+                    flags, m0, n0, sA, sB);
+}
+
+// 1 (default): launches of more than 256 tiles run on the bf16 matrix pipe (three-way split operands); 0: fp32 pipe only
+extern int g_gemm_split;
+
 // TM = 128 or 64 rows of C per workgroup.  The short tile is for launches that would not give every CU a
 // 128-row tile (rank-128 updates and panel solves of the blocked chains): twice the workgroups, half the serial
 // MFMA work in each.
@@ -262,6 +472,8 @@ inline void launch_gemm(const GemmProblem& g, float alpha, float beta, int flags
     gemm_f32_kernel<B_T, 64, true><<<dim3(gx, (unsigned)((g.M + 63) / 64)), dim3(256), 0, st>>>(g, alpha, beta, flags);
   else if ((long long)gx * gy <= 256)
     gemm_f32_kernel<B_T, 64><<<dim3(gx, (unsigned)((g.M + 63) / 64)), dim3(256), 0, st>>>(g, alpha, beta, flags);
+  else if (g_gemm_split)
+    gemm_s3_kernel<B_T><<<dim3(gx, gy), dim3(256), 0, st>>>(g, alpha, beta, flags);
   else
     gemm_f32_kernel<B_T, GT><<<dim3(gx, gy), dim3(256), 0, st>>>(g, alpha, beta, flags);
 }

@@ -89,11 +89,11 @@ __device__ __forceinline__ ColQ open_group(const LoopArgs& a, int idx, int lane,
   float mn = __builtin_inff(), mx = -__builtin_inff();
   if (use_held) {
     #pragma unroll
-    for (int c = 0; c < 8; ++c) { mn = fminf(mn, held[c]); mx = fmaxf(mx, held[c]); }
+    for (int c = 0; c < 8; ++c) { mn = nan_min(mn, held[c]); mx = nan_max(mx, held[c]); }      // NaN-propagating like torch.amin / amax
   } else {
     for (int col = idx + lane; col < end; col += 16) {
       const float v = a.W[rbase + col];
-      mn = fminf(mn, v); mx = fmaxf(mx, v);
+      mn = nan_min(mn, v); mx = nan_max(mx, v);
     }
   }
   mn = team_reduce<16, false>(mn);

@@ -341,9 +341,19 @@ class GPTQ:
     def subset_transform(self, subset, input_feat=None, subset_kwargs=None):
         layers_dict = subset['layers']
         self._chains_ahead(layers_dict)
-        for name in layers_dict:
-            self.layer_transform(layers_dict[name], name)
-            self.free(name)
+        try:
+            for name in layers_dict:
+                self.layer_transform(layers_dict[name], name)
+                self.free(name)
+        finally:
+            # a chain started ahead may still be running on its side stream if a Linear raised or was skipped:
+            # let the current stream wait for it before its tensors can go back to the allocator
+            for leader in [k for k, v in self._shared.items() if v.get('ahead')]:
+                done = self._shared[leader].pop('done', None)
+                if done is not None:
+                    torch.cuda.current_stream().wait_event(done)
+                if not any(c.get('leader', n) == leader for n, c in self.layers_cache.items()):
+                    del self._shared[leader]
 
     def _chains_ahead(self, layers_dict):
         """Start the Cholesky chain of every Linear of the subset now, each on its own stream.  A chain at K = 4096 is
@@ -381,7 +391,9 @@ class GPTQ:
                                                    L.i64(0), L.ptr(H), L.ptr(ws), L.i64(ws_bytes), L.ptr(status),
                                                    L.stream()), 'lcq_chol_inv_upper')
                 done = side.record_event()
-            ws.record_stream(side)                       # freed below, reusable only after the chain has run
+            for t in (ws, H, status, perm):              # allocated on the main stream, used on `side`: not to be
+                if t is not None:                        # handed out again before the chain has run
+                    t.record_stream(side)
             del ws
             self._shared[leader] = dict(U=H, perm=perm, status=status, dead=dead, done=done, ahead=True)
 
