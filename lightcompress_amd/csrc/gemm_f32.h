@@ -381,12 +381,35 @@ __device__ __forceinline__ void gemm_tile_s3(const float* A, int lda, const floa
         }
     }
   };
-  if (kb < ke) gload(kb);
+  // Tiles that lie inside the matrices with 16-byte aligned rows (nearly all of a large launch) fetch a full slab
+  // with eight unconditional 16-byte loads from per-thread pointers; the general path above costs ~15 instructions
+  // per load in bounds and alignment checks, more than the matrix pipe leaves room for at this rate.
+  const bool interior = (m0 + GT <= M) && (n0 + GT <= N) && (lda % 4 == 0) && (ldb % 4 == 0) &&
+                        (((uintptr_t)A | (uintptr_t)B) % 16 == 0) && (kb % 4 == 0);
+  const float* pa[4]; const float* pb[4];
+  #pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    const int idx = p * 256 + tid;
+    pa[p] = A + (long long)(m0 + (idx >> 3)) * lda + (idx & 7) * 4;
+    pb[p] = B_T ? B + (long long)(n0 + (idx >> 3)) * ldb + (idx & 7) * 4
+                : B + (long long)(idx >> 5) * ldb + n0 + (idx & 31) * 4;
+  }
+  auto gload_fast = [&](int k0) {
+    #pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      ra[p] = *(const f32x4*)(pa[p] + k0);
+      rb[p] = *(const f32x4*)(pb[p] + (B_T ? (long long)k0 : (long long)k0 * ldb));
+    }
+  };
+  auto fetch = [&](int k0) {
+    if (interior && k0 + GK <= ke) gload_fast(k0); else gload(k0);
+  };
+  if (kb < ke) fetch(kb);
   for (int k0 = kb; k0 < ke; k0 += GK) {
     __syncthreads();                       // previous slab fully consumed
     lstore();
     __syncthreads();
-    if (k0 + GK < ke) gload(k0 + GK);      // next slab in flight while this one is multiplied
+    if (k0 + GK < ke) fetch(k0 + GK);      // next slab in flight while this one is multiplied
     compute();
   }
   // accumulator register r of lane l: row 8*(r/4) + 4*(l/32) + r%4, column l%32 (the fp32 kernel's epilogue)
