@@ -506,7 +506,7 @@ int lcq_chol_inv_upper(float* H, int64_t K64, const int64_t* perm, float percdam
         if (na > maxN) maxN = na;
       }
       const dim3 grid((unsigned)((maxN + GT - 1) / GT), (unsigned)((maxM + GT - 1) / GT), (unsigned)np);
-      if (g_gemm_split && (long long)grid.x * grid.y * grid.z > 256) {
+      if (g_gemm_split && ((long long)grid.x * grid.y * grid.z > 256 || maxN >= 256)) {      // long contractions
         gemm_s3_batched_kernel<false><<<grid, dim3(256), 0, st>>>(A, K, A, K, T, K, b1, 1.0f, 0.0f, GEMM_K_FROM_N);
         gemm_s3_batched_kernel<false><<<grid, dim3(256), 0, st>>>(A, K, T, K, A, K, b2, -1.0f, 0.0f, GEMM_K_TO_M);
       } else {

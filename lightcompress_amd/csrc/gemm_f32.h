@@ -491,7 +491,11 @@ template <bool B_T>
 inline void launch_gemm(const GemmProblem& g, float alpha, float beta, int flags, hipStream_t st) {
   if (g.M <= 0 || g.N <= 0) return;
   const unsigned gx = (unsigned)((g.N + GT - 1) / GT), gy = (unsigned)((g.M + GT - 1) / GT);
-  if ((long long)gx * gy <= 256 && g.Kc > 0 && g.Kc <= 4 * GK && !(flags & (GEMM_K_FROM_N | GEMM_K_TO_M)))
+  // the bf16 pipe also pays for launches of at most one tile per CU when the contraction is long: a tile's time is
+  // its serial chain of slabs, 2.7x shorter there
+  if (g_gemm_split && (long long)gx * gy >= 64 && (long long)gx * gy <= 256 && g.Kc >= 256)
+    gemm_s3_kernel<B_T><<<dim3(gx, gy), dim3(256), 0, st>>>(g, alpha, beta, flags);
+  else if ((long long)gx * gy <= 256 && g.Kc > 0 && g.Kc <= 4 * GK && !(flags & (GEMM_K_FROM_N | GEMM_K_TO_M)))
     gemm_f32_kernel<B_T, 64, true><<<dim3(gx, (unsigned)((g.M + 63) / 64)), dim3(256), 0, st>>>(g, alpha, beta, flags);
   else if ((long long)gx * gy <= 256)
     gemm_f32_kernel<B_T, 64><<<dim3(gx, (unsigned)((g.M + 63) / 64)), dim3(256), 0, st>>>(g, alpha, beta, flags);
