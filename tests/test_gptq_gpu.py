@@ -674,3 +674,53 @@ def test_owq_layer(dev, gran, n_out):
         assert torch.equal(fq[:, perm][:, nq:], tmp[:, nq:].bfloat16().float())
         want = Q.int_fake_quant_static(spec, tmp, s, z, spec.qmax, spec.qmin)[:, :nq].bfloat16().float()
         assert torch.equal(fq[:, perm][:, :nq], want)
+
+
+def test_split_gemm_has_fp32_accuracy(dev):
+    """The large fp32 products run on the bf16 matrix pipe with three-way split operands (lcq_set_gemm_split, default
+    on).  Against an fp64 product: the split path is as close as the fp32 pipe, for both operand layouts ([k][n] through
+    lcq_gptq_trailing, [n][k] inside the Cholesky chain), for interior and ragged tiles; and the chain's factor agrees
+    between the two settings to fp32 rounding."""
+    import ctypes
+    from lightcompress_amd import _lib as L
+    lib = L.lib()
+    lib.lcq_set_gemm_split.restype = ctypes.c_int
+    g = gen(9100)
+    R, K = 2304, 2400                                   # 18 x 17 tiles, the last column of tiles ragged
+    W0 = (torch.randn(R, K, generator=g) * 0.02).to(dev)
+    U = torch.triu(torch.randn(K, K, generator=g) * 0.05).to(dev).contiguous()
+    Err = (torch.randn(R, 384, generator=g) * torch.exp(torch.randn(384, generator=g))).to(dev).contiguous()
+    k1, k2, j1, j2 = 0, 384, 384, K
+    want = W0.double()
+    want[:, j1:j2] -= Err.double() @ U.double()[k1:k2, j1:j2]
+    errs = {}
+    try:
+        for mode in (0, 1):
+            lib.lcq_set_gemm_split(L.i32(mode))
+            W = W0.clone()
+            L.check(lib.lcq_gptq_trailing(L.ptr(W), L.ptr(Err), L.i64(384), L.ptr(U), L.i64(R), L.i64(K), L.i64(k1), L.i64(k2),
+                                          L.i64(j1), L.i64(j2), L.stream()), 'trailing')
+            assert torch.equal(W[:, :j1], W0[:, :j1])
+            errs[mode] = float((W.double() - want).abs().max() / want.abs().max())
+        assert errs[1] <= max(2 * errs[0], 2e-7) and errs[0] < 5e-6, errs
+        # the chain: same factor either way, same distance from the fp64 identity
+        Kc = 1536
+        X = torch.randn(2 * Kc, Kc, generator=g) * torch.exp(0.7 * torch.randn(Kc, generator=g))
+        H0 = (X.t() @ X / Kc).to(dev)
+        Hd = H0.double() + 0.01 * torch.diag(H0).double().mean() * torch.eye(Kc, device=dev, dtype=torch.float64)
+        ws_bytes = lib.lcq_chol_inv_upper_workspace_bytes(L.i64(Kc))
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        status = torch.zeros(1, dtype=torch.int32, device=dev)
+        Us, res = {}, {}
+        for mode in (0, 1):
+            lib.lcq_set_gemm_split(L.i32(mode))
+            H = H0.clone()
+            L.check(lib.lcq_chol_inv_upper(L.ptr(H), L.i64(Kc), None, L.f32(0.01), None, L.i64(0), L.ptr(H), L.ptr(ws),
+                                           L.i64(ws_bytes), L.ptr(status), L.stream()), 'chain')
+            assert int(status.item()) == 0
+            Us[mode] = H.double()
+            res[mode] = float((Us[mode].t() @ Us[mode] @ Hd - torch.eye(Kc, device=dev, dtype=torch.float64)).abs().max())
+        assert res[1] <= max(2 * res[0], 1e-5) and res[0] < 2e-5, res
+        assert float((Us[0] - Us[1]).abs().max() / Us[0].abs().max()) < 1e-5
+    finally:
+        lib.lcq_set_gemm_split(L.i32(1))
