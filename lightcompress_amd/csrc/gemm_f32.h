@@ -238,17 +238,18 @@ __device__ __forceinline__ void gemm_tile(const float* A, int lda, const float* 
 // (mid*lo, lo*mid, lo*lo) are below 2^-24 of the product - the rounding of an fp32 multiply - so the result is as
 // accurate as the fp32 pipe's, at 16 / 6 times its rate (v_mfma_f32_32x32x16_bf16 against v_mfma_f32_32x32x2f32).
 // Used for the launches that fill the chip (more than one 128x128 tile per CU); small launches stay on the fp32 pipe.
-// LDS: per operand three planes of [128 rows][32 k] bf16 (row pitch 80 B: the 16 lanes of a 16-byte read hit 16
-// different bank quads) or, for B given as [k][n], of [32 k][128 n] (row pitch 320 B) read through the transposing
+// LDS: per operand three planes of [128 rows][32 k] bf16 (64-byte rows, 16-byte chunks XOR-swizzled by the row) or, for B given as [k][n], of [32 k][128 n] (row pitch 320 B) read through the transposing
 // ds_read_b64_tr_b16 (a 16-lane group addresses 4 k-rows x 16 columns and receives 4 k-values of one column each).
 typedef __attribute__((ext_vector_type(8))) __bf16 s3_bf16x8;
 typedef __attribute__((ext_vector_type(4))) short s3_s16x4;
 typedef __attribute__((ext_vector_type(2))) float s3_f32x2;
 typedef __attribute__((ext_vector_type(2))) __bf16 s3_bf16x2;
-constexpr int S3_P = 40;              // bf16 per row of a [row][k] plane
+constexpr int S3_P = 32;              // bf16 per row of a [row][k] plane: 64 bytes, four 16-byte chunks, XOR-swizzled
 constexpr int S3_PN = 160;            // bf16 per row of a [k][n] plane
-constexpr int S3_PLANE = GT * S3_P;   // = GK * S3_PN = 5120 bf16 per plane
-static_assert(GT * S3_P == GK * S3_PN, "plane sizes");
+constexpr int S3_PLANE = GK * S3_PN;  // 5120 bf16 per plane (a [row][k] plane needs 4096 of them)
+// chunk q (8 k-values) of row r sits at chunk q ^ ((r >> 2) & 3): 16 consecutive rows reading the same q hit 16
+// different bank quads, and the 4 rows x 64 bytes of a store instruction's 32 lanes cover all 64 banks once
+__device__ __forceinline__ int s3_rk(int row, int q) { return row * S3_P + ((q ^ ((row >> 2) & 3)) << 3); }
 
 __device__ __forceinline__ uint32_t s3_pack(float a, float b) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(s3_f32x2{a, b}, s3_bf16x2));
@@ -335,7 +336,7 @@ __device__ __forceinline__ void gemm_tile_s3(const float* A, int lda, const floa
       const int idx = p * 256 + tid;
       u32x2 h, m, l;
       s3_split(ra[p], h, m, l);
-      const int oa = (idx >> 3) * S3_P + (idx & 7) * 4;
+      const int oa = s3_rk(idx >> 3, (idx & 7) >> 1) + (idx & 1) * 4;
       *(u32x2*)(sA + oa) = h; *(u32x2*)(sA + S3_PLANE + oa) = m; *(u32x2*)(sA + 2 * S3_PLANE + oa) = l;
       s3_split(rb[p], h, m, l);
       const int ob = B_T ? oa : (idx >> 5) * S3_PN + (idx & 31) * 4;
@@ -352,13 +353,13 @@ __device__ __forceinline__ void gemm_tile_s3(const float* A, int lda, const floa
       for (int i = 0; i < 2; ++i)
         #pragma unroll
         for (int pl = 0; pl < 3; ++pl)
-          fa[i][pl] = *(const s3_bf16x8*)(sA + pl * S3_PLANE + (wr * 64 + i * 32 + lm) * S3_P + ks * 16 + lk * 8);
+          fa[i][pl] = *(const s3_bf16x8*)(sA + pl * S3_PLANE + s3_rk(wr * 64 + i * 32 + lm, ks * 2 + lk));
       #pragma unroll
       for (int j = 0; j < 2; ++j)
         #pragma unroll
         for (int pl = 0; pl < 3; ++pl) {
           if constexpr (B_T) {
-            fb[j][pl] = *(const s3_bf16x8*)(sB + pl * S3_PLANE + (wc * 64 + j * 32 + lm) * S3_P + ks * 16 + lk * 8);
+            fb[j][pl] = *(const s3_bf16x8*)(sB + pl * S3_PLANE + s3_rk(wc * 64 + j * 32 + lm, ks * 2 + lk));
           } else {
             const uint16_t* q = sB + pl * S3_PLANE + (ks * 16 + lk * 8 + (L >> 2)) * S3_PN + wc * 64 + j * 32 + g16 * 16 + (L & 3) * 4;
             const s3_s16x4 b0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s3_s16x4 __attribute__((address_space(3)))*)(q));
