@@ -17,6 +17,8 @@ Not carried over (they raise ``NotImplementedError``): STE rounding (training on
 """
 from __future__ import annotations
 
+import math
+
 import torch
 
 from . import _lib as L
@@ -268,6 +270,10 @@ class BaseQuantizer(object):
             else:
                 next_end_bin, beta = right, next_beta
             if next_start_bin == start_bin and next_end_bin == end_bin:
+                # Neither end moved: the reference goes on lowering beta by one step per iteration until the right
+                # end does move - 1e8 steps per unit of mass, minutes for a histogram whose last bin is heavy
+                # (clamped or rectified activations).  The same iterations, taken at once.
+                beta = self._skip_idle_steps(alpha, beta, stepsize, csum[end_bin], total)
                 continue
             norm = self.get_quantization_error(histogram, min_val, max_val, next_start_bin, next_end_bin)
             if norm > norm_min:
@@ -275,6 +281,40 @@ class BaseQuantizer(object):
             norm_min = norm
             start_bin, end_bin = next_start_bin, next_end_bin
         return min_val + bin_width * start_bin, min_val + bin_width * (end_bin + 1)
+
+    @staticmethod
+    def _beta_after(beta, n, step):
+        """beta after n iterations of `beta = beta - step` in double precision, exactly: inside one binade every
+        subtraction removes the same whole number of ulps, so runs of steps collapse into one product."""
+        while n > 0:
+            nxt = beta - step                              # one literal step (it may cross into the next binade)
+            n -= 1
+            beta = nxt
+            if n == 0 or beta <= 0.0:
+                break
+            d = beta - (beta - step)                       # exact (Sterbenz): the effective step in this binade
+            lo = 2.0 ** math.floor(math.log2(beta))        # beta in [lo, 2 lo)
+            m = min(n, int((beta - lo) / d))               # steps whose results stay >= lo
+            if m > 0 and beta - (beta - step) == d and (beta - m * d) >= lo:
+                beta, n = beta - m * d, n - m              # m * d is exact: d is a few thousand ulps, m < 2**40
+        return beta
+
+    def _skip_idle_steps(self, alpha, beta, step, cs_end, total):
+        """`beta` at the start of the first iteration in which the right end of get_hist_threshold moves, given that
+        it does not move now (iteration i tests csum[end] > fp32((beta_i - step) * total), beta_i = i steps below
+        beta); stops early where the loop would (alpha >= beta)."""
+        f32 = lambda v: torch.tensor(v, dtype=torch.float32).item()
+        idle = lambda b: b > alpha and not (cs_end > f32((b - step) * total))     # monotone: once False, False below
+        if not idle(beta):
+            return beta
+        lo, hi = 0, max(1, int((beta - alpha) / step) + 2)      # idle(beta_lo) holds; beta_hi <= alpha, so it does not
+        while hi - lo > 1:
+            mid = (lo + hi) // 2
+            if idle(self._beta_after(beta, mid, step)):
+                lo = mid
+            else:
+                hi = mid
+        return self._beta_after(beta, hi, step)
 
     def get_static_hist_range(self, act_tensors):
         """quant.py:461-521 -> (min_vals, max_vals), 0-dim fp32 CPU tensors, one per module input."""

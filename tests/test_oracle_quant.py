@@ -554,3 +554,26 @@ def test_w48_known_answers():
     # bf16 weights: the 8-bit codes are held in bf16 (integers up to 127 are exact there)
     out3 = Q.w48_fake_quant(w.bfloat16(), b4, b8)
     assert out3.dtype == torch.bfloat16 and torch.equal(out3.float().reshape(4, 4)[0], w.reshape(4, 4)[0])
+
+
+def test_hist_threshold_idle_steps_are_skipped_exactly():
+    """The host class takes the idle iterations of get_hist_threshold (neither end moves, beta sinks by 1e-8) at once.
+    The closed form of n double-precision subtractions equals the literal loop bit for bit, across a binade boundary
+    too, and the thresholds of histograms with heavy edge bins equal the literal loop's of the oracle."""
+    from lightcompress_amd.quant import BaseQuantizer
+    for beta0, n in [(1.0, 1), (1.0, 12345), (0.9999999, 2000000), (0.50001, 3000), (0.500000004, 7), (0.2500001, 1000000)]:
+        b = beta0
+        for _ in range(n):
+            b = b - 1e-8
+        assert BaseQuantizer._beta_after(beta0, n, 1e-8) == b, (beta0, n)
+    q = BaseQuantizer.__new__(BaseQuantizer)
+    q.bins, q.dst_nbins = 256, 256
+    g = gen(77)
+    for edge in (2e-4, 1e-3):
+        hist = torch.rand(256, generator=g) * 1000
+        hist[255] = float(hist.sum()) * edge / (1 - edge)            # heavy last bin: ~edge / 1e-8 idle iterations
+        hist[0] = hist[255] * 0.5
+        lo, hi = torch.tensor(-3.0), torch.tensor(5.0)
+        want = Q.hist_threshold(hist.clone(), lo, hi, 256, 256)
+        got = q.get_hist_threshold(hist.clone(), lo, hi)
+        assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
