@@ -194,18 +194,22 @@ class GPTQ:
 
     @torch.no_grad()
     def add_batch(self, layer, name, inp, out=None):
+        # Called once per Linear per calibration batch (896 times for one decoder layer): the work up to the return for
+        # a Linear that follows another one, and up to the staging copy otherwise, creates no tensor views.
         cache = self.layers_cache[name]
-        key = self._input_key(inp)
-        if len(inp.shape) == 2:
-            inp = inp.unsqueeze(0)
-        tmp = inp.shape[0]
-        if len(inp.shape) == 3:
-            inp = inp.reshape((-1, inp.shape[-1]))
+        if not inp.is_cuda:
+            raise L.LcqError('liblcq operates on GPU tensors only (no CPU fallback)')
+        shape = inp.shape
+        key = (inp.data_ptr(), shape, inp.stride(), inp.dtype, inp._version)
+        nd = len(shape)
+        tmp = 1 if nd == 2 else shape[0]
+        K = shape[-1]
+        tokens = shape[0] if nd == 2 else (shape[0] * shape[1] if nd == 3 else shape[0])
         if inp.dtype not in (torch.bfloat16, torch.float16, torch.float32):
             raise NotImplementedError(f'add_batch takes bf16 / fp16 / fp32 activations; got {inp.dtype}')
-        assert inp.shape[0] % self.chunk_num == 0, \
-            f'Error: inp.shape[1] ({inp.shape[0]}) cannot be evenly divided by chunk_num.'
-        defer = self.hessian_fold(inp.shape[1])
+        assert tokens % self.chunk_num == 0, \
+            f'Error: inp.shape[1] ({tokens}) cannot be evenly divided by chunk_num.'
+        defer = self.hessian_fold(K if nd <= 3 else shape[1])
         followed = self._follow(name, cache, key, defer > 1)
         cache['calls'] += 1
         cache['nsamples'] += tmp
@@ -214,13 +218,10 @@ class GPTQ:
         cache['last_key'] = key
         cache['last_ref'] = inp                         # keeps the memory from being handed to another tensor meanwhile
         cache['last_stage'] = (0, 0)
-        x = inp.contiguous()
         cache['upper_only'] = True
         # fp32 activations (gptq.py:289 `chunk.float()` keeps them fp32): staged as two bf16 halves, x = hi + lo
-        sdtype = torch.bfloat16 if x.dtype == torch.float32 else x.dtype
-        if defer <= 1:
-            self._accumulate(cache, *self._halves(x), tmp)
-            return
+        split = inp.dtype == torch.float32
+        sdtype = torch.bfloat16 if split else inp.dtype
         # Stage a copy of the tokens and fold several calls into one launch: the window
         # H <- H*n/(n+b1) + 2/(n+b1)*S1, then H <- H*(n+b1)/(n+b1+b2) + 2/(n+b1+b2)*S2, ...
         # telescopes to H*n/N + (2/N)*(S1+S2+...), N = n + b1 + b2 + ..., so one launch over the
@@ -228,34 +229,42 @@ class GPTQ:
         # start of the next call that needs room (or when H is asked for), so the latest call can still be told
         # apart from H when a follower needs the state before it.
         stage = cache.get('stage')
-        split = x.dtype == torch.float32
-        if stage is not None and (stage.dtype != sdtype or split != (cache.get('stage_lo') is not None)
-                                  or cache['stage_fill'] + x.shape[0] > stage.shape[0]):
-            self._flush(cache)
-            if stage.dtype != sdtype or split != (cache.get('stage_lo') is not None):
-                stage = None
-        if stage is None:
-            stage = torch.empty((defer * x.shape[0], x.shape[1]), dtype=sdtype, device=x.device)
-            cache['stage'] = stage
-            cache['stage_lo'] = torch.empty_like(stage) if split else None
-            cache['stage_fill'] = 0
-            cache['stage_batches'] = 0
-        if x.shape[0] > stage.shape[0]:
-            self._accumulate(cache, *self._halves(x), tmp)
-            return
-        f = cache['stage_fill']
-        if split:
-            self._halves(x, stage[f:f + x.shape[0]], cache['stage_lo'][f:f + x.shape[0]])
-        else:
-            dst = stage[f:f + x.shape[0]]
-            nbytes = x.numel() * x.element_size()
-            if nbytes % 16 == 0 and x.data_ptr() % 16 == 0 and dst.data_ptr() % 16 == 0:
-                L.check(L.lib().lcq_stage_copy(L.ptr(x), C_ptr(dst), L.i64(nbytes), L.stream()), 'lcq_stage_copy')
-            else:
-                dst.copy_(x)
-        cache['stage_fill'] = f + x.shape[0]
-        cache['stage_batches'] += tmp
-        cache['last_stage'] = (x.shape[0], tmp)
+        if defer > 1 and nd <= 3:
+            if stage is not None and (stage.dtype != sdtype or split != (cache.get('stage_lo') is not None)
+                                      or cache['stage_fill'] + tokens > stage.shape[0]):
+                self._flush(cache)
+                if stage.dtype != sdtype or split != (cache.get('stage_lo') is not None):
+                    stage = None
+            if stage is None:
+                stage = torch.empty((defer * tokens, K), dtype=sdtype, device=inp.device)
+                cache['stage'] = stage
+                cache['stage_lo'] = torch.empty_like(stage) if split else None
+                cache['stage_fill'] = 0
+                cache['stage_batches'] = 0
+            if tokens <= stage.shape[0]:
+                f = cache['stage_fill']
+                nbytes = tokens * K * stage.element_size()
+                dst = stage.data_ptr() + f * K * stage.element_size()
+                if not split and key[0] % 16 == 0 and nbytes % 16 == 0 and dst % 16 == 0 and inp.is_contiguous():
+                    L.check(L.lib().lcq_stage_copy(ctypes.c_void_p(key[0]), ctypes.c_void_p(dst), ctypes.c_int64(nbytes),
+                                                   L.stream()),
+                            'lcq_stage_copy')
+                else:
+                    x = inp.reshape((-1, K)).contiguous()
+                    if split:
+                        self._halves(x, stage[f:f + tokens], cache['stage_lo'][f:f + tokens])
+                    else:
+                        stage[f:f + tokens].copy_(x)
+                cache['stage_fill'] = f + tokens
+                cache['stage_batches'] += tmp
+                cache['last_stage'] = (tokens, tmp)
+                return
+        x = inp
+        if nd == 2:
+            x = x.unsqueeze(0)
+        if len(x.shape) == 3:
+            x = x.reshape((-1, K))
+        self._accumulate(cache, *self._halves(x.contiguous()), tmp)
 
     def hessian_fold(self, K):
         """add_batch calls folded into one Hessian launch for a Linear with K input features.  'auto': 4 calls of 2048
@@ -390,12 +399,25 @@ class GPTQ:
                 L.check(L.lib().lcq_chol_inv_upper(L.ptr(H), L.i64(K), L.ptr(perm), L.f32(self.percdamp), L.ptr(None),
                                                    L.i64(0), L.ptr(H), L.ptr(ws), L.i64(ws_bytes), L.ptr(status),
                                                    L.stream()), 'lcq_chol_inv_upper')
+                status_host = self._post_status(status)
                 done = side.record_event()
             for t in (ws, H, status, perm):              # allocated on the main stream, used on `side`: not to be
                 if t is not None:                        # handed out again before the chain has run
                     t.record_stream(side)
             del ws
-            self._shared[leader] = dict(U=H, perm=perm, status=status, dead=dead, done=done, ahead=True)
+            self._shared[leader] = dict(U=H, perm=perm, status=status, dead=dead, done=done, ahead=True,
+                                        status_host=status_host)
+
+    @staticmethod
+    def _post_status(status):
+        """Queues, right behind the chain on the current stream, a copy of the chain's status word to pinned host
+        memory and an event after it.  The check before the weights are written back waits for that event only, so the
+        host does not wait for the column loop queued after the chain and the GPU does not run dry behind it."""
+        host = torch.empty(1, dtype=torch.int32, pin_memory=True)
+        host.copy_(status, non_blocking=True)
+        copied = torch.cuda.Event()
+        copied.record()
+        return host, copied
 
     @torch.no_grad()
     def layer_transform(self, layer, name):
@@ -448,13 +470,14 @@ class GPTQ:
                                                L.i64(0), L.ptr(H), L.ptr(ws), L.i64(ws_bytes), L.ptr(status),
                                                L.stream()), 'lcq_chol_inv_upper')
             del ws
-            shared = dict(U=H, perm=perm, status=status, dead=dead)
+            shared = dict(U=H, perm=perm, status=status, dead=dead, status_host=self._post_status(status))
             if is_shared:
                 self._shared[leader] = shared
         elif 'done' in shared:                               # started by _chains_ahead on another stream
             torch.cuda.current_stream().wait_event(shared.pop('done'))
         U = shared['U']
         self._status = shared['status']
+        self._status_host = shared['status_host']
 
         # weight.clone().float(), W[:, dead] = 0 and W[:, perm] in one pass
         W = torch.empty((R, K), dtype=torch.float32, device=w.device)
@@ -505,8 +528,11 @@ class GPTQ:
         tmp = torch.empty_like(W)
         self.weight_transform(W, H, Losses, tmp)
         self.last_error = torch.sum(Losses)              # device scalar; .item() it to log like the reference
-        if self.check_positive_definite and int(self._status.item()) != 0:
-            raise torch.linalg.LinAlgError('GPTQ: the damped Hessian is not positive-definite')
+        if self.check_positive_definite:
+            host, copied = self._status_host
+            copied.synchronize()                         # the chain and the copy behind it; the loop may still be running
+            if int(host[0]) != 0:
+                raise torch.linalg.LinAlgError('GPTQ: the damped Hessian is not positive-definite')
         if self.owq and self.n_out > 0:                  # the outlier columns stay in floating point, with the
             tmp[:, self.n_nonout:] = W[:, self.n_nonout:]      # updates of the loop (gptq.py:187-188)
             Losses[:, self.n_nonout:] = 0
