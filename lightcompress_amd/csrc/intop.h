@@ -11,7 +11,16 @@ struct IntRow {
   float lo, hi;      // qmin - z, qmax - z: clamp bounds of the code minus the zero point
   int fast;          // x * (1/s) + guard may replace x / s
   int zint;          // zero point is a small integer: rint(t) + z and q - z are exact
+  // nibble packing (zint rows): bit patterns of 1.5 * 2^23 + (qmin - z) and + (qmax - z), and the sum over the
+  // eight nibble positions of the pattern that stands for code -8
+  int clo, chi;
+  uint32_t nib0;
 };
+
+// 1.5 * 2^23: x + RINT_BIAS rounds x to the nearest integer, ties to even (the constant is even), and leaves
+// that integer in the low mantissa bits, for |x| < 2^22
+constexpr float RINT_BIAS = 12582912.0f;
+constexpr int RINT_BIAS_BITS = 0x4B400000;
 
 // FAST: round_zp and |qmin|,qmax <= 256 (every stock configuration).
 template <bool BF_, bool FAST, bool PRESCALE = false, int CD_ = -1>
@@ -20,6 +29,7 @@ struct IntOp {
   static constexpr bool HAS_PRESCALE = PRESCALE;
   static constexpr bool HAS_FUSED_DQ = FAST;
   static constexpr bool HAS_CUSTOM_EMIT = false;
+  static constexpr bool ABS_ONLY = false;
   static constexpr int CD = CD_;
   using Row = IntRow;
   float qmin, qmax, qrange, osf;
@@ -55,6 +65,8 @@ struct IntOp {
     p.zint = (z == rintf(z)) && (fabsf(z) <= 512.0f);       // caller-given zero points need not be integers
     p.sdq = scale_f32 ? s * osf : rnd<BF>(s * osf);
     p.lo = qmin - z; p.hi = qmax - z;                       // exact: small integers
+    p.clo = RINT_BIAS_BITS + (int)p.lo; p.chi = RINT_BIAS_BITS + (int)p.hi;
+    p.nib0 = (uint32_t)(RINT_BIAS_BITS - ((int)z + 8)) * 0x11111111u;
     return p;
   }
 
@@ -146,12 +158,21 @@ struct IntOp {
   template <int N>
   __device__ __forceinline__ void quotients(const float* x, float* t, const Row& p) const {
     bool ok = p.fast;
-    #pragma unroll
-    for (int i = 0; i < N; ++i) {
-      t[i] = x[i] * p.r;
-      if constexpr (BF) {
-        ok = ok && (((f2u(t[i]) & 0xffffu) - 0x7ff8u) > 0x10u);
-      } else {
+    if constexpr (BF) {
+      // distance of the low 16 bits from the midpoint window, two products per packed 16-bit instruction
+      lcq_u16x2 nearest = {0xffff, 0xffff};
+      #pragma unroll
+      for (int i = 0; i < N; i += 2) {
+        t[i] = x[i] * p.r;
+        t[i + 1] = x[i + 1] * p.r;
+        const uint32_t lows = __builtin_amdgcn_perm(f2u(t[i + 1]), f2u(t[i]), 0x05040100u);
+        nearest = __builtin_elementwise_min(nearest, __builtin_bit_cast(lcq_u16x2, lows) - lcq_u16x2{0x7ff8, 0x7ff8});
+      }
+      ok = ok && nearest.x > 0x10 && nearest.y > 0x10;
+    } else {
+      #pragma unroll
+      for (int i = 0; i < N; ++i) {
+        t[i] = x[i] * p.r;
         const float d = t[i] - rintf(t[i]);
         ok = ok && (fabsf(fabsf(d) - 0.5f) > 4.8828125e-04f);
       }
@@ -183,10 +204,27 @@ struct IntOp {
     }
   }
 
+  // Eight 4-bit codes of one bf16 chunk as a compressed-tensors word (code + 8 in nibble i), FAST rows with an
+  // integer zero point.  t + RINT_BIAS holds rint(t) in its low mantissa bits; clamped as an integer pattern (any
+  // NaN or infinity lands on a bound), shifted to its nibble and added up, the eight patterns differ from the
+  // eight nibbles by a per-row constant (arithmetic modulo 2^32 is linear, so the high bits cancel too).
+  __device__ __forceinline__ uint32_t ct4_word(const float* x, const Row& p) const {
+    float t[8];
+    quotients<8>(x, t, p);
+    uint32_t acc = 0;
+    #pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      int b = (int)f2u(t[i] + RINT_BIAS), c;
+      asm("v_med3_i32 %0, %1, %2, %3" : "=v"(c) : "v"(b), "v"(p.clo), "v"(p.chi));
+      acc = ((uint32_t)c << (4 * i)) + acc;
+    }
+    return acc - p.nib0;
+  }
+
   // fake quant without the codes (FAST only): (clamp(rint(t) + z, qmin, qmax) - z) * s equals
-  // clamp(rint(t), qmin - z, qmax - z) * s when z is a small integer (all terms exact); "+ 0" turns the
-  // -0 that rint(-0.3) leaves into the +0 that (q - z) gives.  The products are left unrounded: the
-  // caller rounds to the row type while packing.
+  // clamp(rint(t), qmin - z, qmax - z) * s when z is a small integer (all terms exact); the "+ 0" of the
+  // fused multiply-add (one rounding, that of the product) turns the -0 that rint(-0.3) leaves into the +0
+  // that (q - z) gives.  The products are left unrounded: the caller rounds to the row type while packing.
   template <int N>
   __device__ __forceinline__ void fused_dq(const float* x, float* d, const Row& p) const {
     if (__builtin_expect(!p.zint, 0)) {
@@ -197,7 +235,7 @@ struct IntOp {
     float t[N];
     quotients<N>(x, t, p);
     #pragma unroll
-    for (int i = 0; i < N; ++i) d[i] = (__builtin_amdgcn_fmed3f(rintf(t[i]), p.lo, p.hi) + 0.0f) * p.sdq;
+    for (int i = 0; i < N; ++i) d[i] = __builtin_fmaf(__builtin_amdgcn_fmed3f(rintf(t[i]), p.lo, p.hi), p.sdq, 0.0f);
   }
 
   // dequant, quant.py:709-711 (scale already multiplied by output_scale_factor)

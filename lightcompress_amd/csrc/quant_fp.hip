@@ -23,6 +23,7 @@ using namespace lcq;
 struct FpRow {
   float s, r, sm;   // divisor, its reciprocal, multiplier of the dequantization
   int fast;
+  int inrange;      // dynamic rows: every |x / s| of the row stays below hw_lim, no per-element check needed
 };
 
 template <bool BF_>
@@ -31,6 +32,7 @@ struct FpOp {
   static constexpr bool HAS_PRESCALE = false;
   static constexpr bool HAS_FUSED_DQ = false;
   static constexpr bool HAS_CUSTOM_EMIT = true;
+  static constexpr bool ABS_ONLY = true;
   static constexpr int CD = -1;
   using Row = FpRow;
   float qmax, rqmax;
@@ -41,7 +43,7 @@ struct FpOp {
   int drop, min_exp, max_exp;
   float min_normal;
   int hw;            // 1: e4m3, 2: e5m2 with subnormals -> v_cvt_pk_fp8_f32 / v_cvt_pk_bf8_f32 do the rounding
-  float hw_lim;      // first magnitude the float8 type cannot hold although the emulated grid can
+  float hw_lim;      // quotients below this stay inside the float8 range (bf16 rows: also after their rounding to bf16)
 
   __device__ __forceinline__ Row finish(float s) const {
     Row p;
@@ -51,19 +53,25 @@ struct FpOp {
     p.r = __builtin_amdgcn_rcpf(s);      // 1 ulp: inside the error the exactness guards of x * r allow for
     const float a = fabsf(s);
     p.fast = (a > 8.6736174e-19f) && (a < 1.1529215e18f);
+    p.inrange = 0;
     return p;
   }
   // get_qparams symmetric branch, quant.py:548-552 (qmax is a float tensor here)
   __device__ __forceinline__ Row make(float mn, float mx) const {
     const float cmin = BF ? 1.0013580322265625e-05f : 1e-5f;
-    float a = nan_max(fabsf(mx), fabsf(mn));
-    a = clamp_min_nan(a, cmin);
+    const float amax = nan_max(fabsf(mx), fabsf(mn));
+    const float a = clamp_min_nan(amax, cmin);
+    Row p;
     if constexpr (BF) {                                   // a * (1/qmax) unless the product is within 8 ulp of a bf16 midpoint
       float q = a * rqmax;
       if (__builtin_expect(((f2u(q) & 0xffffu) - 0x7ff8u) <= 0x10u, 0)) q = a / qmax;
-      return finish(rnd<BF>(q));
+      p = finish(rnd<BF>(q));
+    } else {
+      p = finish(a / qmax);
     }
-    return finish(a / qmax);
+    // the largest quotient of the row, with room for the reciprocal's and the product's rounding (NaN: false)
+    p.inrange = (amax * p.r) * 1.001f < hw_lim;
+    return p;
   }
   __device__ __forceinline__ Row load(const void* scales, const void*, int64_t row) const {
     const int64_t i = scalar_qp ? 0 : row;
@@ -146,16 +154,30 @@ struct FpOp {
     const int cd = code_dtype;
     float t[N];
     bool near = !p.fast, far = false;
-    #pragma unroll
-    for (int i = 0; i < N; ++i) {
-      t[i] = x[i] * p.r;
-      if constexpr (BF) {
-        near = near || (((f2u(t[i]) & 0xffffu) - 0x7ff8u) <= 0x10u);
-      } else {
+    if constexpr (BF) {
+      // distance of the low 16 bits from the midpoint window, two products per packed 16-bit instruction
+      lcq_u16x2 nearest = {0xffff, 0xffff};
+      #pragma unroll
+      for (int i = 0; i < N; i += 2) {
+        t[i] = x[i] * p.r;
+        t[i + 1] = x[i + 1] * p.r;
+        const uint32_t lows = __builtin_amdgcn_perm(f2u(t[i + 1]), f2u(t[i]), 0x05040100u);
+        nearest = __builtin_elementwise_min(nearest, __builtin_bit_cast(lcq_u16x2, lows) - lcq_u16x2{0x7ff8, 0x7ff8});
+      }
+      near = near || nearest.x <= 0x10 || nearest.y <= 0x10;
+    } else {
+      #pragma unroll
+      for (int i = 0; i < N; ++i) {
+        t[i] = x[i] * p.r;
         const uint32_t lowm = f2u(t[i]) & ((1u << drop) - 1u);
         far = far || ((lowm - (half - 8u)) <= 16u) || !(fabsf(t[i]) >= 1.0001f * min_normal);
       }
-      far = far || !(fabsf(t[i]) < hw_lim);
+    }
+    if (!p.inrange) {                                        // static scales: any magnitude may turn up
+      float m = 0.0f;
+      #pragma unroll
+      for (int i = 0; i < N; i += 2) m = nan_max(nan_max(m, fabsf(t[i])), fabsf(t[i + 1]));
+      far = far || !(m < hw_lim);
     }
     if (__builtin_expect(far, 0)) return false;              // left to the emulated grid (rare: ties of fp32 rows, inf, NaN)
     if constexpr (BF) {
@@ -273,8 +295,11 @@ FpOp<BF> make_op(int e_bits, int m_bits, float qmax, int flags, int code_dtype) 
   c.max_mag = ((uint32_t)(c.max_exp + 127) << 23) | (((1u << m_bits) - 1u) << c.drop);
   c.min_normal = __builtin_ldexpf(1.0f, c.min_exp);
   c.hw = 0; c.hw_lim = 0.0f;
-  if (c.subnormals && e_bits == 4 && m_bits == 3) { c.hw = 1; c.hw_lim = 464.0f; }       // 448 is the float8 maximum
-  if (c.subnormals && e_bits == 5 && m_bits == 2) { c.hw = 2; c.hw_lim = 61440.0f; }     // 57344
+  // 448 / 57344 are the float8 maxima; the emulated grid goes on (480 / 65536 come next), reached from the midpoints
+  // 464 / 61440 upwards.  The test is made on the quotient before a bf16 row rounds it (steps of 2 / 256 up there), so the limit
+  // of bf16 rows lies half a step lower: anything below it rounds to the bf16 number under the midpoint at most.
+  if (c.subnormals && e_bits == 4 && m_bits == 3) { c.hw = 1; c.hw_lim = BF ? 463.0f : 464.0f; }
+  if (c.subnormals && e_bits == 5 && m_bits == 2) { c.hw = 2; c.hw_lim = BF ? 61312.0f : 61440.0f; }
   return c;
 }
 

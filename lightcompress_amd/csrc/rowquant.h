@@ -17,6 +17,7 @@
 //   uint32_t pack4(q[4])                four of them in one word
 //   bool is_static, dq_f32; int code_dtype
 //   static constexpr int CD             code storage fixed at compile time, or -1 (use code_dtype)
+//   static constexpr bool ABS_ONLY      make() uses max |x| only: min is not reduced (mn == mx == max |x| then)
 //   static constexpr bool HAS_PRESCALE; if set, prescale(chunk,row,ch,nchunks) / prescale1(x,row,col,cols)
 //   multiply the input by a per-column factor (rounded to the row type) before anything else
 #pragma once
@@ -26,6 +27,7 @@
 namespace lcq {
 
 template <bool BF> struct Vec { static constexpr int N = BF ? 8 : 4; };
+typedef unsigned short lcq_u16x2 __attribute__((ext_vector_type(2)));
 
 template <bool BF> __device__ __forceinline__ float rnd(float v) {
   if constexpr (BF) return (float)(__bf16)v; else return v;
@@ -158,6 +160,12 @@ __device__ __forceinline__ void emit_chunk_generic(const Op& op, const typename 
   float v[N], q[N];
   #pragma unroll
   for (int i = 0; i < N; ++i) v[i] = v_in[i];
+  if constexpr (Op::CD == LCQ_CODE_CT4 && N == 8 && Op::HAS_FUSED_DQ) {
+    if (codes && !dq && p.zint && p.fast) {                  // nibbles straight from the quotients
+      ((uint32_t*)codes)[cidx] = op.ct4_word(v, p);
+      return;
+    }
+  }
   op.template codes<N>(v, q, p);
   if (codes) store_codes(op, codes, cidx * N, q);
   if (dq) {
@@ -216,17 +224,22 @@ __device__ __forceinline__ void chunk_minmax(const u32x4& r, float& mn, float& m
   constexpr int N = Vec<Op::BF>::N;
   float v[N];
   unpack<Op::BF>(r, v);
-  #pragma unroll
-  for (int i = 0; i < N; i += 2) {
-    mn = nan_min(nan_min(mn, v[i]), v[i + 1]);
-    mx = nan_max(nan_max(mx, v[i]), v[i + 1]);
+  if constexpr (Op::ABS_ONLY) {                              // the op wants max |x| only: mx carries it, mn is unused
+    #pragma unroll
+    for (int i = 0; i < N; i += 2) mx = nan_max(nan_max(mx, __builtin_fabsf(v[i])), __builtin_fabsf(v[i + 1]));
+  } else {
+    #pragma unroll
+    for (int i = 0; i < N; i += 2) {
+      mn = nan_min(nan_min(mn, v[i]), v[i + 1]);
+      mx = nan_max(nan_max(mx, v[i]), v[i + 1]);
+    }
   }
 }
 // range of a row from the per-lane partials
-template <int TEAM>
+template <int TEAM, bool ABS_ONLY = false>
 __device__ __forceinline__ void team_range(float& mn, float& mx) {
-  mn = team_reduce<TEAM, false>(mn);
   mx = team_reduce<TEAM, true>(mx);
+  if constexpr (ABS_ONLY) mn = mx; else mn = team_reduce<TEAM, false>(mn);
 }
 
 // ---------------------------------------------------------------------------
@@ -271,7 +284,7 @@ __global__ __launch_bounds__(256) void row_team_kernel(
       #pragma unroll
       for (int it = 0; it < ITERS; ++it)
         if (FULL || t + it * TEAM < nchunks) chunk_minmax<Op>(raw[u][it], mn, mx);
-      team_range<TEAM>(mn, mx);
+      team_range<TEAM, Op::ABS_ONLY>(mn, mx);
       p = op.make(mn, mx);
       if (row_ok && t == 0) op.store_qp(scales, zeros, row, p);
     } else {
@@ -338,15 +351,16 @@ __device__ __forceinline__ float block_reduce(float v, float* sm) {
 }
 
 // min and max of a workgroup in one round: two barriers instead of four
+template <bool ABS_ONLY = false>
 __device__ __forceinline__ void block_range(float& mn, float& mx, float* sm) {
-  mn = team_reduce<64, false>(mn);
+  if constexpr (!ABS_ONLY) mn = team_reduce<64, false>(mn);
   mx = team_reduce<64, true>(mx);
   const int w = threadIdx.x >> 6;
   __syncthreads();                                           // previous readers of sm are done
-  if ((threadIdx.x & 63) == 0) { sm[w] = mn; sm[4 + w] = mx; }
+  if ((threadIdx.x & 63) == 0) { if constexpr (!ABS_ONLY) sm[w] = mn; sm[4 + w] = mx; }
   __syncthreads();
-  mn = nan_min(nan_min(sm[0], sm[1]), nan_min(sm[2], sm[3]));
   mx = nan_max(nan_max(sm[4], sm[5]), nan_max(sm[6], sm[7]));
+  if constexpr (ABS_ONLY) mn = mx; else mn = nan_min(nan_min(sm[0], sm[1]), nan_min(sm[2], sm[3]));
 }
 
 template <class Op, int CACHE>
@@ -374,7 +388,7 @@ __global__ __launch_bounds__(256) void row_block_kernel(
       if constexpr (Op::HAS_PRESCALE) r = op.prescale(r, row, ch, nchunks);
       chunk_minmax<Op>(r, mn, mx);
     }
-    block_range(mn, mx, sm);
+    block_range<Op::ABS_ONLY>(mn, mx, sm);
     p = op.make(mn, mx);
     if (threadIdx.x == 0) op.store_qp(scales, zeros, row, p);
   } else {

@@ -166,6 +166,31 @@ def test_float_quant_bit_exact(dev, tie, dtype, fmt, gran, shape):
         assert_bit_equal(rs, ors, 'fp8 scales')
 
 
+@pytest.mark.parametrize('tie', ['away', 'even'])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('fmt,top', [('e4m3', 448.0), ('e5m2', 57344.0)])
+def test_float_quant_given_scales_around_the_float8_maximum(dev, tie, dtype, fmt, top):
+    """Given scales let quotients pass the float8 maximum, where the reference's grid goes on (480 after 448, 65536
+    after 57344) and a hardware float8 convert would saturate: every bf16 number of magnitude 0.8 .. 1.25 times the
+    maximum, divided by scales that put the quotients between bf16 numbers (a bf16 row rounds them again)."""
+    from lightcompress_amd import FloatQuantizer
+    base = torch.arange(0, 1 << 16, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).float()
+    base = base[torch.isfinite(base) & (base.abs() >= 0.8 * top) & (base.abs() <= 1.25 * top)]
+    base = base[: base.numel() // 8 * 8]
+    factors = [1.0, 1.0234375, 0.98828125, 1.0078125, 1.046875, 0.9609375]
+    x = base[None, :].repeat(len(factors), 1).to(dtype)
+    spec = Q.FloatSpec(fmt, 'per_channel', tie=tie)
+    q = FloatQuantizer(fmt, True, 'per_channel', use_qtorch=True, fp_tie=tie)
+    rows, s, z, qmax, qmin = q.get_tensor_qparams(x.to(dev))
+    orows, os_, oz, _, _ = Q.float_tensor_qparams(spec, x)
+    mine = torch.tensor(factors, dtype=dtype).reshape(-1, 1)
+    want = Q.float_quant(spec, orows, mine.clone(), oz)
+    assert float(want.abs().max()) > top                    # the case is there: codes beyond the float8 maximum
+    assert_bit_equal(q.quant(rows, mine.to(dev), z, qmax, qmin), want, 'float quant, given scales')
+    assert_bit_equal(q.quant_dequant(rows, mine.to(dev), z, qmax, qmin),
+                     Q.float_dequant(Q.float_quant(spec, orows, mine.clone(), oz), mine, oz), 'float quant_dequant, given scales')
+
+
 def _agree(a, b):
     return float((a.cpu().float() == b.float()).float().mean())
 
