@@ -26,6 +26,7 @@ the ceiling they can be held against.
 """
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -238,9 +239,11 @@ def bench_quantizers(args, out):
         n = max(3, int(total / (shape[0] * shape[1] * torch.tensor([], dtype=dtype).element_size())))
         return [(torch.randn(*shape, device=dev) * scale).to(dtype) for _ in range(n)]
 
-    def report(name, kernel, nbytes, t):
+    def report(name, kernel, rbytes, wbytes, t):
+        nbytes = rbytes + wbytes
+        mix = min((1, 2, 4, 8), key=lambda m: abs(math.log(rbytes / wbytes / m)))    # nearest probed read:write ratio
         rows_out.append({'case': name, 'kernel': kernel, 'us': round(t * 1e6, 2), 'MB': round(nbytes / 1e6, 1),
-                         'GB/s': round(nbytes / t / 1e9, 1), 'frac': round(nbytes / t / 8e12, 4)})
+                         'GB/s': round(nbytes / t / 1e9, 1), 'frac': round(nbytes / t / 8e12, 4), 'read:write': f'{mix}:1'})
         return rows_out[-1]
 
     def quant_int(xs, rows, cols, qmin, qmax, flags, dq=None, codes=None, cd=L.CODE_NONE):
@@ -277,7 +280,18 @@ def bench_quantizers(args, out):
                        'torch_copy_GB/s': round(nb_copy / t / 1e9, 1), 'lcq_div_cols_by_one_GB/s': round(nb_copy / t2 / 1e9, 1),
                        'what': 'plain streaming copies of 256 MiB fp32 tensors on this box (read + written bytes, three rotating '
                                'pairs): torch copy_ and this library x / 1 kernel; GB/s = the faster one'}
-    del src, dst
+    # the same for other mixes of reads and writes (a quantizer that packs reads four bytes for each one it writes):
+    # this library's streaming probe, 512 MiB read per launch
+    big = torch.cat([x.view(-1) for x in src[:2]])
+    room = torch.empty_like(big)
+    mixes = {}
+    for m in (0, 1, 2, 4, 8):
+        tm = timeit(lambda i: L.check(lib.lcq_stream_probe(L.ptr(big), L.ptr(room), L.i64(big.numel() * 4), L.i64(room.numel() * 4),
+                                                           L.i32(m), st), 'lcq_stream_probe'), 20, 5)
+        mixes['read only' if m == 0 else f'{m}:1'] = round(big.numel() * 4 * (1 + (1 / m if m else 0)) / tm / 1e9, 1)
+    out['hbm_stream_mix'] = {'GB/s': mixes, 'what': 'read + written bytes per second of a kernel that only streams (xor of m 16-byte '
+                             'chunks read -> one chunk written), by its ratio of bytes read to bytes written; 512 MiB read per launch'}
+    del src, dst, big, room
 
     # RTN config: fp32 [4096, 4096], INT4 asym g128: dq + uint8 codes + scales / zeros
     xs = rot((4096, 4096), f32, 0.02)
@@ -285,19 +299,19 @@ def bench_quantizers(args, out):
     cds = [torch.empty(4096, 4096, dtype=torch.uint8, device=dev) for _ in xs]
     n, g = 4096 * 4096, 128
     t = timeit(quant_int(xs, n // g, g, 0, 15, 0, dq, cds, L.CODE_U8), 60, 25)
-    r = report('RTN int4 asym g128, fp32 4096x4096 -> dq + u8 codes + scales/zeros', 'row_team_kernel<IntOp<f32>>', n * 9 + n // g * 8, t)
+    r = report('RTN int4 asym g128, fp32 4096x4096 -> dq + u8 codes + scales/zeros', 'row_team_kernel<IntOp<f32>>', n * 4, n * 5 + n // g * 8, t)
     out['roofline_quantizer'] = {'kernel': 'row_team_kernel<IntOp<f32>> 4096x4096 g128 dq+u8', 'bound': 'hbm', 'achieved': r['GB/s'],
                                  'peak': 8000.0, 'unit': 'GB/s', 'frac': r['frac'],
                                  'traffic': traffic_bytes('rtn_quant_int4_g128_4096x4096_f32'), 'launch_us': r['us']}
     t = timeit(quant_int(xs, n // g, g, 0, 15, 0, dq), 60, 25)
-    report('RTN int4 asym g128 fake quant, fp32 4096x4096', 'row_team_kernel<IntOp<f32>>', n * 8 + n // g * 8, t)
+    report('RTN int4 asym g128 fake quant, fp32 4096x4096', 'row_team_kernel<IntOp<f32>>', n * 4, n * 4 + n // g * 8, t)
     del xs, dq, cds
     # AWQ config: bf16 [11008, 4096] fake quant, int4 asym g128
     xs = rot((11008, 4096), bf, 0.02)
     dq = [torch.empty_like(x) for x in xs]
     n = 11008 * 4096
     t = timeit(quant_int(xs, n // g, g, 0, 15, 0, dq), 60, 25)
-    report('int4 asym g128 fake quant, bf16 11008x4096', 'row_team_kernel<IntOp<bf16>>', n * 4 + n // g * 4, t)
+    report('int4 asym g128 fake quant, bf16 11008x4096', 'row_team_kernel<IntOp<bf16>>', n * 2, n * 2 + n // g * 4, t)
     del xs, dq
     # FP8 + pack config: 16 experts [2048, 7168] bf16 at once, and one expert alone
     for ne in (16, 1):
@@ -306,20 +320,21 @@ def bench_quantizers(args, out):
         n = R * K
         cds = [torch.empty(R, K, dtype=torch.uint8, device=dev) for _ in xs]
         t = timeit(quant_fp(xs, R, K, None, cds, L.CODE_FP8), 30 if ne > 1 else 60, 12 if ne > 1 else 25)
-        report(f'fp8 e4m3 per-channel real quant, bf16 {ne}x[2048,7168]', 'row_block_kernel<FpOp<bf16>>', n * 3 + R * 2, t)
+        report(f'fp8 e4m3 per-channel real quant, bf16 {ne}x[2048,7168]', 'row_block_kernel<FpOp<bf16>>', n * 2, n + R * 2, t)
         pk = [torch.empty(R, K // 8, dtype=torch.int32, device=dev) for _ in xs]
         t = timeit(quant_int(xs, n // g, g, -8, 7, L.FLAG_SYM, None, pk, L.CODE_CT4), 30 if ne > 1 else 60, 12 if ne > 1 else 25)
         report(f'int4 sym g128 quantize + compressed-tensors pack, bf16 {ne}x[2048,7168]', 'row_team_kernel<IntOp<bf16, CT4>>',
-               n * 2.5 + n // g * 2, t)
+               n * 2, n * 0.5 + n // g * 2, t)
         del xs, cds, pk
     # per-token dynamic fp8 fake quant of activations [8192, 7168]
     xs = rot((8192, 7168), bf, 1.0)
     dq = [torch.empty_like(x) for x in xs]
     n = 8192 * 7168
     t = timeit(quant_fp(xs, 8192, 7168, dq), 60, 25)
-    report('fp8 e4m3 per-token fake quant, bf16 8192x7168', 'row_block_kernel<FpOp<bf16>>', n * 4 + 8192 * 2, t)
+    report('fp8 e4m3 per-token fake quant, bf16 8192x7168', 'row_block_kernel<FpOp<bf16>>', n * 2, n * 2 + 8192 * 2, t)
     for r in rows_out:
         r['frac_of_copy'] = round(r['GB/s'] / out['hbm_copy']['GB/s'], 3)
+        r['frac_of_stream_mix'] = round(r['GB/s'] / mixes[r['read:write']], 3)
     out['quantizers'] = rows_out
 
 

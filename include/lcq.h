@@ -208,6 +208,13 @@ int lcq_split_f32_bf16(const float* x, int64_t n, void* hi, void* lo, void* stre
  * kept until one folded Hessian launch): dst[0 .. bytes) = src[0 .. bytes), both 16-byte aligned, bytes % 16 == 0. */
 int lcq_stage_copy(const void* src, void* dst, int64_t bytes, void* stream);
 
+/* No counterpart in the reference: a measurement aid for the benchmark.  Streams `bytes` (a multiple of 16, both
+ * pointers 16-byte aligned) from src and writes bytes / reads_per_write to dst (the xor of every reads_per_write
+ * consecutive 16-byte chunks of a thread's share); reads_per_write in {1, 2, 4, 8}, or 0 for a read-only pass.
+ * dst_bytes is the room behind dst: less than bytes / reads_per_write (4 KiB for a read-only pass) is refused.  The
+ * rate is the ceiling of a quantizer kernel with the same mix of reads and writes. */
+int lcq_stream_probe(const void* src, void* dst, int64_t bytes, int64_t dst_bytes, int reads_per_write, void* stream);
+
 /* H[j][i] = H[i][j] for i < j. */
 int lcq_symmetrize(float* H, int64_t K, void* stream);
 

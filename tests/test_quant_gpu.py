@@ -571,3 +571,31 @@ def test_weight48_fake_quant_bit_exact(dev, dtype, b4, b8, shape):
     got = q.fake_quant_weight_dynamic(w.to(dev))
     want = Q.w48_fake_quant(w, b4, b8)
     assert_bit_equal(got, want, 'w48 fake quant')
+
+
+@pytest.mark.parametrize('m', [1, 2, 4, 8])
+def test_stream_probe_reads_everything_and_refuses_a_short_destination(dev, m):
+    """The benchmark's streaming probe: every 16-byte chunk of the source reaches the output (xor of m chunks of a
+    thread's share), and a destination smaller than bytes / m is refused on the host."""
+    from lightcompress_amd import _lib as L
+    u = 4 if m < 4 else m                                   # chunks per thread
+    nblocks = 37
+    g = torch.Generator().manual_seed(m)
+    src = torch.randint(-2 ** 31, 2 ** 31 - 1, (nblocks, u // m, m, 256, 4), generator=g, dtype=torch.int64).to(torch.int32)
+    want = src[:, :, 0]
+    for k in range(1, m):
+        want = want ^ src[:, :, k]
+    sd = src.to(dev).contiguous()
+    out = torch.zeros(want.numel(), dtype=torch.int32, device=dev)
+    nbytes = sd.numel() * 4
+    L.check(L.lib().lcq_stream_probe(L.ptr(sd), L.ptr(out), L.i64(nbytes), L.i64(out.numel() * 4), L.i32(m), L.stream()), 'probe')
+    assert torch.equal(out.cpu(), want.reshape(-1))
+    with pytest.raises(L.LcqError):
+        L.check(L.lib().lcq_stream_probe(L.ptr(sd), L.ptr(out), L.i64(nbytes), L.i64(out.numel() * 4 - 16), L.i32(m), L.stream()),
+                'probe')
+    with pytest.raises(L.LcqError):
+        L.check(L.lib().lcq_stream_probe(L.ptr(sd), L.ptr(out), L.i64(nbytes), L.i64(out.numel() * 4), L.i32(3), L.stream()), 'probe')
+    # read-only pass: nothing is written
+    out.zero_()
+    L.check(L.lib().lcq_stream_probe(L.ptr(sd), L.ptr(out), L.i64(nbytes), L.i64(out.numel() * 4), L.i32(0), L.stream()), 'probe')
+    assert int(out.abs().sum()) == 0
