@@ -117,11 +117,17 @@ __device__ __forceinline__ ColQ open_group(const LoopArgs& a, int idx, int lane,
 // a multiple of 8 columns, so groups open only between octets and the 8 columns of an octet are straight-line code.
 template <bool STATIC, bool OCT>
 __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
-  __shared__ float Us[BS * BS];                  // Hinv1 = U[i1:i2, i1:i2], zero outside the block and below the diagonal
+  constexpr int NP = OCT ? 16 : BS;              // parameter slots of a row: one per octet, or one per column
+  __shared__ float Us[BS * BS];                  // Hinv1 = U[i1:i2, i1:i2] above the diagonal, zero everywhere else
   __shared__ float Rd[BS];                       // 1 / U[i, i]
+  __shared__ float Dg[BS];                       // U[i, i]
+  __shared__ float Ps[STATIC ? 1 : ROWS_PER_WG * NP], Pz[STATIC ? 1 : ROWS_PER_WG * NP];   // scale, zero point in force
   const int tid = threadIdx.x;
   // full block and 16-byte aligned rows (the entry point checks the base pointers): vector loads and stores
   const bool vec = (a.count == BS) && (a.K % 4 == 0) && (a.i1 % 4 == 0) && a.aligned;
+  // The diagonal is zero in LDS as well: a column's own update would only turn it into its quantized value, which
+  // nothing reads.  Left alone, the register of a finished column keeps the weight as it was when the column was
+  // quantized, which is the `tmp` output, and (w - q), err and the loss are recomputed from it once, after the loop.
   if (vec) {
     // all 16 loads of the thread in flight at once: one after the other they are 16 memory latencies,
     // which used to be most of the kernel's run time
@@ -135,7 +141,7 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
     for (int j = 0; j < 16; ++j) {
       const int e = tid + 256 * j, r = e >> 5, c = (e & 31) * 4;
       #pragma unroll
-      for (int k = 0; k < 4; ++k) if (c + k < r) v[j][k] = 0.0f;
+      for (int k = 0; k < 4; ++k) if (c + k <= r) v[j][k] = 0.0f;
       *(f32x4*)(Us + e * 4) = v[j];
     }
   } else {
@@ -145,15 +151,20 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
       if (r < a.count) {
         const float* p = a.U + (long long)(a.i1 + r) * a.K + a.i1 + c;
         #pragma unroll
-        for (int k = 0; k < 4; ++k) if (c + k < a.count && c + k >= r) v[k] = p[k];
+        for (int k = 0; k < 4; ++k) if (c + k < a.count && c + k > r) v[k] = p[k];
       }
       *(f32x4*)(Us + e * 4) = v;
     }
   }
-  if (tid < BS) Rd[tid] = (tid < a.count) ? 1.0f / a.U[(long long)(a.i1 + tid) * a.K + a.i1 + tid] : 0.0f;
+  if (tid < BS) {
+    const float d = (tid < a.count) ? a.U[(long long)(a.i1 + tid) * a.K + a.i1 + tid] : 1.0f;
+    Dg[tid] = d;
+    Rd[tid] = (tid < a.count) ? 1.0f / d : 0.0f;
+  }
 
   const int lane = tid & 15;                     // physical lane inside the row's team
-  const long long row = (long long)blockIdx.x * ROWS_PER_WG + (tid >> 4);
+  const int prow = tid >> 4;                     // the team's row inside the workgroup
+  const long long row = (long long)blockIdx.x * ROWS_PER_WG + prow;
   const bool row_ok = row < a.R;
   const long long rbase = (row_ok ? row : 0) * a.K;
 
@@ -188,13 +199,12 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
 
   // Octet `to` = columns 8*to .. 8*to+7.  After every octet the registers rotate by one lane inside the team, so
   // the owner of the current octet is always lane 0 (a constant DPP source) and lane p holds the columns of
-  // team member (p + to) mod 16.
-  // Outputs rotate with them: what lane 0 produced for octet `to` sits on lane (to - n) mod 16 after n rotations,
-  // so each lane ends up with 8 consecutive columns of tmp / (w-q) / err and stores them once.  (Stores inside the
-  // loop would make every later wait on a load wait for them too.)
-  float o_w[8], o_diff[8], o_err[8];
-  #pragma unroll
-  for (int c = 0; c < 8; ++c) { o_w[c] = 0.0f; o_diff[c] = 0.0f; o_err[c] = 0.0f; }
+  // team member (p + to) mod 16.  After the last octet lane p therefore holds the finished columns of octet
+  // (p + n_oct) mod 16, eight consecutive columns, and stores them once.  (Stores inside the loop would make every
+  // later wait on a load wait for them too.)
+  // A lone wave per SIMD issues about one instruction every ten cycles whatever the instruction is, so the run time
+  // is the number of instructions per column, not the length of the dependency chain: the loop body holds the
+  // chain, the eight fused multiply-adds of the rank-1 update and nothing else.
   const bool first = lane == 0;
   int n_oct = 0;
   for (int to = 0; to < 16; ++to) {
@@ -204,34 +214,42 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
     // dependency chain; rows past `count` are zero in LDS, so the 8 columns need no bound check
     const float* ucol = Us + (8 * to) * BS + 8 * ((lane + to) & 15);
     f32x4 u0[8], u1[8];
-    float rd[8];
     #pragma unroll
     for (int c = 0; c < 8; ++c) {
       u0[c] = *(const f32x4*)(ucol + c * BS);
       u1[c] = *(const f32x4*)(ucol + c * BS + 4);
-      rd[c] = Rd[8 * to + c];
     }
-    if (!STATIC && OCT && a.i1 + 8 * to == nextb) {
-      nextb += a.g;
-      q = open_group(a, a.i1 + 8 * to, lane, row, row_ok, rbase, w, to == 0 && a.g == BS && a.count == BS);
+    const f32x4 rda = *(const f32x4*)(Rd + 8 * to), rdb = *(const f32x4*)(Rd + 8 * to + 4);
+    const float rd[8] = {rda[0], rda[1], rda[2], rda[3], rdb[0], rdb[1], rdb[2], rdb[3]};
+    if (!STATIC && OCT) {
+      if (a.i1 + 8 * to == nextb) {
+        nextb += a.g;
+        q = open_group(a, a.i1 + 8 * to, lane, row, row_ok, rbase, w, to == 0 && a.g == BS && a.count == BS);
+      }
+      if (first) { Ps[prow * NP + to] = q.s; Pz[prow * NP + to] = q.z; }
     }
     // 8 columns.  Each: quantize-dequantize like clamp(round(w / s) + z, qmin, qmax), (q - z) * s in fp32 (only
-    // lane 0's result is used), err = (w - q) / d, rank-1 update of the lane's 8 columns.  U is upper triangular,
-    // so columns left of the current one see a zero factor and need no mask (the column itself turns into its
-    // quantized value, which nothing reads).
-    // The first pass takes the quotient through the reciprocal and only notes whether any owner came within 2^-11
-    // of a rounding boundary (or beyond 1024), where product and quotient may round apart; then the wave runs the
-    // octet again from the saved registers with true divisions.  That keeps every branch out of the chain.
+    // lane 0's result is used), err = (w - q) / d, rank-1 update of the lane's 8 columns.  U is strictly upper
+    // triangular in LDS, so the column itself and the columns left of it see a zero factor and need no mask.
+    // The first pass takes the quotient through the reciprocal and only notes how close an owner's product came to
+    // a rounding boundary: within 2^-11 product and quotient may round apart, and the wave runs the octet again
+    // from the saved registers with true divisions.  (Beyond +-1024 both round outside the clamp range, which
+    // make_colq keeps within +-1024 for `fast` parameters; an infinite or NaN product makes the distance NaN.)
+    // That keeps every branch out of the chain.
     auto octet = [&](auto exact_tag) -> bool {
       constexpr bool EXACT = decltype(exact_tag)::value;
-      bool unsure = false;
+      float margin = 0.5f;                                  // smallest distance of a product from a rounding boundary
       #pragma unroll
       for (int c = 0; c < 8; ++c) {
         if (STATIC) {
           q = make_colq(ss[c], zz[c], a.qmin, a.qmax, a.nrz);               // lane 0: the parameters of this column
-        } else if (!OCT && a.i1 + 8 * to + c == nextb && 8 * to + c < a.count) {
-          nextb += a.g;
-          q = open_group(a, a.i1 + 8 * to + c, lane, row, row_ok, rbase, w, false);
+          if (!EXACT) margin = q.fast ? margin : 0.0f;
+        } else if (!OCT) {
+          if (a.i1 + 8 * to + c == nextb && 8 * to + c < a.count) {
+            nextb += a.g;
+            q = open_group(a, a.i1 + 8 * to + c, lane, row, row_ok, rbase, w, false);
+          }
+          if (first) { Ps[prow * NP + 8 * to + c] = q.s; Pz[prow * NP + 8 * to + c] = q.z; }
         }
         const float wv = w[c];
         float diff;
@@ -240,18 +258,18 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
           diff = wv - (__builtin_amdgcn_fmed3f(code, a.qmin, a.qmax) - q.z) * q.s;
         } else {
           const float t = wv * q.r, rt = rintf(t);
-          unsure |= !((fabsf(fabsf(t - rt) - 0.5f) > 4.8828125e-04f) & (fabsf(t) <= 1024.0f) & q.fast);
+          margin = nan_min(margin, fabsf(fabsf(t - rt) - 0.5f));
           diff = wv - __builtin_amdgcn_fmed3f(rt, q.lo, q.hi) * q.s;
         }
-        const float err = diff * rd[c];
-        o_w[c] = first ? wv : o_w[c];
-        o_diff[c] = first ? diff : o_diff[c];
-        o_err[c] = first ? err : o_err[c];
-        const float eb = row16_first(err);
+        const float eb = row16_first(diff * rd[c]);
         #pragma unroll
-        for (int k = 0; k < 4; ++k) { w[k] -= eb * u0[c][k]; w[4 + k] -= eb * u1[c][k]; }
+        for (int k = 0; k < 4; ++k) {
+          w[k] = __builtin_fmaf(-eb, u0[c][k], w[k]);
+          w[4 + k] = __builtin_fmaf(-eb, u1[c][k], w[4 + k]);
+        }
       }
-      return unsure & first;
+      if (EXACT) return false;
+      return first & !((margin > 4.8828125e-04f) & (STATIC || q.fast));
     };
     if (STATIC || OCT) {
       float saved[8];
@@ -269,24 +287,35 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
     #pragma unroll
     for (int c = 0; c < 8; ++c) {
       w[c] = row16_next(w[c]);
-      o_w[c] = row16_next(o_w[c]); o_diff[c] = row16_next(o_diff[c]); o_err[c] = row16_next(o_err[c]);
       if (STATIC) { ss[c] = row16_next(ss[c]); zz[c] = row16_next(zz[c]); }
     }
   }
 
-  const int oct = (lane + n_oct) & 15;                      // the octet whose outputs this lane holds now
-  if (row_ok) {
-    float loss[8];
+  // Outputs of the lane's eight finished columns.  w still holds each column as it was when it was quantized; the
+  // quantized value, with true divisions, is the one the loop used (its reciprocal form is only taken where it
+  // rounds like the division), and err = (w - q) * (1 / d) as in the loop.
+  const int oct = (lane + n_oct) & 15;                      // the octet whose columns this lane holds now
+  if (row_ok && 8 * oct < a.count) {
+    float o_err[8], loss[8];
     #pragma unroll
     for (int c = 0; c < 8; ++c) {
-      const float d = Us[(8 * oct + c) * BS + 8 * oct + c];
-      loss[c] = (o_diff[c] * o_diff[c]) / (2.0f * (d * d));
+      const int col = 8 * oct + c;
+      float s_, z_;
+      if (STATIC) { s_ = ss[c]; z_ = zz[c]; }
+      else { s_ = Ps[prow * NP + (OCT ? oct : col)]; z_ = Pz[prow * NP + (OCT ? oct : col)]; }
+      if (col >= a.count) { s_ = 1.0f; z_ = 0.0f; }
+      const float wv = w[c];
+      const float code = a.nrz ? rintf(wv / fmaxf(s_, 1e-9f) + z_) : rintf(wv / s_) + z_;
+      const float diff = wv - (__builtin_amdgcn_fmed3f(code, a.qmin, a.qmax) - z_) * s_;
+      o_err[c] = diff * Rd[col];
+      const float d = Dg[col];
+      loss[c] = (diff * diff) / (2.0f * (d * d));
     }
     if (vec) {
       float* pt = a.tmp + rbase + a.i1 + 8 * oct;
       float* pl = a.Losses + rbase + a.i1 + 8 * oct;
-      *(f32x4*)pt = f32x4{o_w[0], o_w[1], o_w[2], o_w[3]};
-      *(f32x4*)(pt + 4) = f32x4{o_w[4], o_w[5], o_w[6], o_w[7]};
+      *(f32x4*)pt = f32x4{w[0], w[1], w[2], w[3]};
+      *(f32x4*)(pt + 4) = f32x4{w[4], w[5], w[6], w[7]};
       *(f32x4*)pl = f32x4{loss[0], loss[1], loss[2], loss[3]};
       *(f32x4*)(pl + 4) = f32x4{loss[4], loss[5], loss[6], loss[7]};
     }
@@ -303,7 +332,7 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
       for (int c = 0; c < 8; ++c) {
         const int col = 8 * oct + c;
         if (col < a.count) {
-          a.tmp[rbase + a.i1 + col] = o_w[c];
+          a.tmp[rbase + a.i1 + col] = w[c];
           a.Losses[rbase + a.i1 + col] = loss[c];
         }
       }
