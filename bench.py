@@ -122,11 +122,9 @@ def bench_layer(args, out):
             if record is None and check is None:
                 gp.subset_transform(sub)               # the reference's driver of a subset (gptq.py:96-112)
             elif check is not None:                    # untimed: the same driver, keeping each Linear's summed loss
-                gp._chains_ahead(sub['layers'])
+                gp.subset_transform(sub)
                 for n in subset:
-                    gp.layer_transform(layers[n], n)
-                    gp.free(n)
-                    check[n] = gp.last_error
+                    check[n] = gp.last_errors[n]
             else:                                      # same work one Linear at a time, with events between the phases
                 for n in subset:
                     gp.initialize_qparams_and_prepare_weights(layers[n], n)

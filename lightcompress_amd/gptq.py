@@ -17,6 +17,10 @@ Differences a caller can observe
   * Linears of a subset that receive the very same input tensor on every call (q/k/v, gate/up) share one Hessian
     and one Cholesky chain (``special.auto_share``, default on; detected per call, with a fallback to separate
     Hessians at the first call that differs; results are bit-identical either way);
+  * subset_transform runs the column loops of Linears that share a chain as one loop over their stacked rows
+    (``special.fuse_loops``, default on; rows are independent, so each Linear gets the result of its own loop, up to
+    the rounding of the update GEMM where the larger row count selects the other GEMM kernel), and leaves every
+    Linear's summed loss in ``last_errors[name]``;
   * ``special.hessian_defer`` (default 'auto': 16 for K <= 4096, 8 for K <= 8192, else 4) add_batch calls are copied to a staging buffer and
     folded into one launch, so ``layers_cache[name]['H']`` lags behind ``nsamples`` until
     ``hessian(name)``, ``hessian_sorting`` or ``process_hessian_and_weights`` settles it
@@ -74,6 +78,7 @@ class GPTQ:
         self.hessian_defer = hd if hd == 'auto' else int(hd)
         # subset_transform starts the Cholesky chains of all Linears of a subset side by side (False: one by one)
         self.chain_overlap = bool(special_config.get('chain_overlap', True))
+        self.fuse_loops = bool(special_config.get('fuse_loops', True))
         # Linears of a subset that keep receiving the very same input tensor share one Hessian and one chain
         self.auto_share = bool(special_config.get('auto_share', True))
         if self.owq:                                     # gptq.py:47-50
@@ -350,9 +355,19 @@ class GPTQ:
     def subset_transform(self, subset, input_feat=None, subset_kwargs=None):
         layers_dict = subset['layers']
         self._chains_ahead(layers_dict)
+        self.last_errors = {}                            # summed loss of every Linear of the subset (device scalars)
         try:
+            done = set()
             for name in layers_dict:
+                if name in done:
+                    continue
+                mates = self._loop_mates(name, layers_dict)
+                if len(mates) > 1:
+                    self._fused_transform(mates, layers_dict)
+                    done.update(mates)
+                    continue
                 self.layer_transform(layers_dict[name], name)
+                self.last_errors[name] = self.last_error
                 self.free(name)
         finally:
             # a chain started ahead may still be running on its side stream if a Linear raised or was skipped:
@@ -363,6 +378,20 @@ class GPTQ:
                     torch.cuda.current_stream().wait_event(done)
                 if not any(c.get('leader', n) == leader for n, c in self.layers_cache.items()):
                     del self._shared[leader]
+
+    def _loop_mates(self, name, layers_dict):
+        """The Linears of the subset whose column loops can run as one: they share `name`'s Hessian (so its column
+        order and its factor U) and have weights of the same width.  [name] alone if there are none."""
+        if not self.fuse_loops or self.owq:
+            return [name]
+        cache = self.layers_cache.get(name)
+        if cache is None:
+            return [name]
+        leader = cache.get('leader', name)
+        mates = [n for n in layers_dict
+                 if n in self.layers_cache and self.layers_cache[n].get('leader', n) == leader
+                 and self.layers_cache[n].get('columns') == cache.get('columns')]
+        return mates if len(mates) > 1 and name in mates else [name]
 
     def _chains_ahead(self, layers_dict):
         """Start the Cholesky chain of every Linear of the subset now, each on its own stream.  A chain at K = 4096 is
@@ -443,8 +472,9 @@ class GPTQ:
         elif self.actorder or self.owq:
             self.hessian_sorting(name)
 
-    def process_hessian_and_weights(self, layer, name):
-        """-> (W [R,K] fp32 in processing order, Hinv: upper factor of the damped inverse)."""
+    def process_hessian_and_weights(self, layer, name, out=None):
+        """-> (W [R,K] fp32 in processing order, Hinv: upper factor of the damped inverse).  `out`: where W goes
+        (an [R, K] fp32 tensor, e.g. the rows of a larger one), else a new tensor."""
         w = layer.weight.data
         if w.dim() > 2:
             w = w.flatten(1)
@@ -480,7 +510,9 @@ class GPTQ:
         self._status_host = shared['status_host']
 
         # weight.clone().float(), W[:, dead] = 0 and W[:, perm] in one pass
-        W = torch.empty((R, K), dtype=torch.float32, device=w.device)
+        W = torch.empty((R, K), dtype=torch.float32, device=w.device) if out is None else out
+        if W.shape != (R, K) or W.dtype != torch.float32:
+            raise L.LcqError(f'process_hessian_and_weights: `out` must be fp32 [{R}, {K}]')
         dead_u8 = shared['dead'].view(torch.uint8)
         L.check(L.lib().lcq_gptq_prepare_weights(L.ptr(w), L.i32(L.dtype_code(w.dtype)), L.i64(R), L.i64(K),
                                                  L.ptr(self.perm if (self.actorder or self.owq) else None), L.ptr(dead_u8),
@@ -527,12 +559,19 @@ class GPTQ:
         Losses = torch.empty_like(W)                     # the loop writes every entry of both
         tmp = torch.empty_like(W)
         self.weight_transform(W, H, Losses, tmp)
-        self.last_error = torch.sum(Losses)              # device scalar; .item() it to log like the reference
+        self._check_status()
+        self._write_back(layer, W, Losses, tmp)
+
+    def _check_status(self):
         if self.check_positive_definite:
             host, copied = self._status_host
             copied.synchronize()                         # the chain and the copy behind it; the loop may still be running
             if int(host[0]) != 0:
                 raise torch.linalg.LinAlgError('GPTQ: the damped Hessian is not positive-definite')
+
+    def _write_back(self, layer, W, Losses, tmp):
+        """gptq.py:178-196 after the loop: summed loss, outlier columns, tmp[:, invperm], the weight and the qparams."""
+        self.last_error = torch.sum(Losses)              # device scalar; .item() it to log like the reference
         if self.owq and self.n_out > 0:                  # the outlier columns stay in floating point, with the
             tmp[:, self.n_nonout:] = W[:, self.n_nonout:]      # updates of the loop (gptq.py:187-188)
             Losses[:, self.n_nonout:] = 0
@@ -543,9 +582,48 @@ class GPTQ:
                                                      L.ptr(self.invperm), L.ptr(None), L.ptr(out), L.stream()),
                     'lcq_gptq_prepare_weights')
             tmp = out
+        if tmp._base is not None:                        # rows of a stacked matrix: the Linear gets storage of its own
+            tmp = tmp.clone()
         layer.weight.data = tmp.reshape(layer.weight.shape)
         if self.wquantizer.granularity == 'per_group' and not self.static_groups:
             self.update_model_qparams(layer)
+
+    @torch.no_grad()
+    def _fused_transform(self, names, layers_dict):
+        """Linears that share one chain (the same input, hence the same H, column order and U) go through the column
+        loop as ONE weight matrix, their rows stacked: the loop has no term across rows (gptq.py:229-244), so every
+        row gets what it would get alone, while the block kernel, which is bound by the length of its 128 sequential
+        columns and not by the number of rows, and the update GEMMs run once instead of once per Linear."""
+        parts, r0 = [], 0
+        rows = [layers_dict[n].weight.data.flatten(1).shape[0] if layers_dict[n].weight.dim() > 2
+                else layers_dict[n].weight.shape[0] for n in names]
+        K = self.layers_cache[names[0]]['columns']
+        Wall = torch.empty((sum(rows), K), dtype=torch.float32, device=self.dev)
+        U = None
+        for n, R in zip(names, rows):
+            layer = layers_dict[n]
+            self.initialize_qparams_and_prepare_weights(layer, n)
+            _, U = self.process_hessian_and_weights(layer, n, out=Wall[r0:r0 + R])
+            parts.append((n, layer, r0, R, self._scales, self._zeros))
+            r0 += R
+        if self._static:                                 # given parameters: one row block per Linear
+            self._scales = torch.cat([p[4] for p in parts])
+            self._zeros = None if parts[0][5] is None else torch.cat([p[5] for p in parts])
+        else:
+            self._scales = torch.empty((r0, self._G), device=self.dev)
+            self._zeros = None if self.wquantizer.sym else torch.empty((r0, self._G), device=self.dev)
+        Losses, tmp = torch.empty_like(Wall), torch.empty_like(Wall)
+        self.weight_transform(Wall, U, Losses, tmp)
+        self._check_status()
+        scales, zeros = self._scales, self._zeros
+        if not hasattr(self, 'last_errors'):
+            self.last_errors = {}
+        for n, layer, a, R, _, _ in parts:
+            self._scales = scales[a:a + R]
+            self._zeros = None if zeros is None else zeros[a:a + R]
+            self._write_back(layer, Wall[a:a + R], Losses[a:a + R], tmp[a:a + R])
+            self.last_errors[n] = self.last_error
+            self.free(n)
 
     @torch.no_grad()
     def weight_transform(self, W, Hinv, Losses, tmp):

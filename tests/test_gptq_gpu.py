@@ -563,6 +563,52 @@ def test_identical_inputs_share_one_hessian_automatically(dev):
             assert torch.equal(a, b), n
 
 
+@pytest.mark.parametrize('actorder,static_groups', [(True, False), (False, False), (True, True)])
+def test_stacked_column_loop_matches_per_linear_loops(dev, actorder, static_groups):
+    """Linears that share a chain run through the column loop stacked into one matrix (special.fuse_loops, default on).
+    Rows are independent, so each Linear gets what its own loop gives: the same weights, scales, zero points and summed
+    loss (to the rounding of the update GEMM, whose kernel may change with the row count; bit for bit at this size)."""
+    K = 1024
+    Ws = {'q': (torch.randn(256, K, generator=gen(11)) * 0.02).bfloat16(), 'k': (torch.randn(64, K, generator=gen(12)) * 0.02).bfloat16(),
+          'v': (torch.randn(72, K, generator=gen(13)) * 0.02).bfloat16()}
+    xs = [b.to(dev) for b in calib_batches(6, 256, K, seed=8700)]
+    runs = []
+    for fuse in (True, False):
+        gp = make_gptq(actorder=actorder, static_groups=static_groups, fuse_loops=fuse)
+        layers = {n: Layer(w.to(dev)) for n, w in Ws.items()}
+        gp.subset_init({'layers': layers})
+        if static_groups:
+            for lay in layers.values():
+                gp.collect_layer_qparams(lay)
+        for x in xs:
+            for n in Ws:
+                gp.add_batch(layers[n], n, x.data, None)
+        assert {gp.layers_cache[n].get('leader', n) for n in Ws} == {'q'}
+        gp.subset_transform({'layers': layers})
+        torch.cuda.synchronize()
+        assert gp._shared == {} and gp.layers_cache == {}
+        for n in Ws:                                      # every Linear owns its storage (no views of the stacked matrix)
+            assert layers[n].weight.data.untyped_storage().nbytes() == Ws[n].numel() * 4
+        errs = {n: float(gp.last_errors[n]) for n in Ws} if fuse else None
+        runs.append(({n: (layers[n].weight.data.cpu(), layers[n].buf_scales.cpu(), layers[n].buf_zeros.cpu()) for n in Ws}, errs))
+    (fused, errs), (alone, _) = runs
+    for n in Ws:
+        assert fused[n][0].shape == Ws[n].shape
+        for a, b in zip(fused[n], alone[n]):
+            assert torch.equal(a, b), n
+    # the per-Linear losses of the stacked run are those of separate runs
+    for n in Ws:
+        gp = make_gptq(actorder=actorder, static_groups=static_groups, fuse_loops=False)
+        lay = Layer(Ws[n].to(dev))
+        gp.subset_init({'layers': {n: lay}})
+        if static_groups:
+            gp.collect_layer_qparams(lay)
+        for x in xs:
+            gp.add_batch(lay, n, x.data, None)
+        gp.layer_transform(lay, n)
+        assert abs(float(gp.last_error) - errs[n]) <= 1e-6 * abs(errs[n]), n
+
+
 @pytest.mark.parametrize('split_at', [1, 4, 5, 8])
 def test_sharing_falls_back_when_an_input_differs(dev, split_at):
     """The moment one call brings a different tensor the follower continues with its own Hessian - a copy of the
