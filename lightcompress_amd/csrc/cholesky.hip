@@ -72,7 +72,13 @@ __global__ __launch_bounds__(256) void apply_dead_kernel(float* __restrict__ W, 
 
 // W[r, j] = dead[c] ? 0 : float(w[r, c]),  c = perm ? perm[j] : j   -- the weight clone, fp32 cast, dead-column
 // zeroing and act-order gather of process_hessian_and_weights (gptq.py:133-141, 150-151) in one pass.  A workgroup
-// takes 4 rows; reads are gathers inside a row (it stays in cache), writes are coalesced.
+// takes 4 rows; without a permutation reads and writes are both coalesced.
+template <int DT>
+__device__ __forceinline__ float load_w(const void* w, long long i) {
+  if (DT == LCQ_F32) return ((const float*)w)[i];
+  if (DT == LCQ_BF16) return u2f((uint32_t)((const uint16_t*)w)[i] << 16);
+  return (float)((const _Float16*)w)[i];
+}
 template <int DT>
 __global__ __launch_bounds__(256) void prepare_w_kernel(const void* __restrict__ w, long long R, int K,
                                                         const long long* __restrict__ perm,
@@ -80,12 +86,39 @@ __global__ __launch_bounds__(256) void prepare_w_kernel(const void* __restrict__
   for (long long row = (long long)blockIdx.x * 4; row < R && row < (long long)blockIdx.x * 4 + 4; ++row) {
     for (int j = threadIdx.x; j < K; j += 256) {
       const long long c = perm ? perm[j] : j;
-      float v;
-      if (DT == LCQ_F32) v = ((const float*)w)[row * K + c];
-      else if (DT == LCQ_BF16) v = u2f((uint32_t)((const uint16_t*)w)[row * K + c] << 16);
-      else v = (float)((const _Float16*)w)[row * K + c];
+      float v = load_w<DT>(w, row * K + c);
       if (dead && dead[c]) v = 0.0f;
       out[row * K + j] = v;
+    }
+  }
+}
+// The same with a permutation: a gather inside every row.  From memory that is one 64-byte sector per element; here
+// the workgroup's rows (`rows` of them, as many as fit 64 KB) come in as they lie, 16 bytes per lane, and the gather
+// reads LDS.  The permutation is read once per workgroup and column.
+template <int DT>
+__global__ __launch_bounds__(256) void prepare_w_gather_kernel(const void* __restrict__ w, long long R, int K, int rows,
+                                                               const long long* __restrict__ perm,
+                                                               const uint8_t* __restrict__ dead, float* __restrict__ out) {
+  extern __shared__ __align__(16) unsigned char staged[];
+  constexpr int ES = DT == LCQ_F32 ? 4 : 2;
+  const long long row0 = (long long)blockIdx.x * rows;
+  const int n = (int)((R - row0 < rows) ? (R - row0) : rows);
+  const long long nbytes = (long long)n * K * ES;
+  const unsigned char* src = (const unsigned char*)w + row0 * K * ES;
+  if ((((uintptr_t)src) & 15) == 0) {
+    const long long n16 = nbytes >> 4;
+    for (long long i = threadIdx.x; i < n16; i += 256) ((u32x4*)staged)[i] = ((const u32x4*)src)[i];
+    for (long long i = (n16 << 4) + threadIdx.x; i < nbytes; i += 256) staged[i] = src[i];
+  } else {
+    for (long long i = threadIdx.x; i < nbytes; i += 256) staged[i] = src[i];
+  }
+  __syncthreads();
+  for (int j = threadIdx.x; j < K; j += 256) {
+    const long long c = perm[j];
+    const bool dz = dead && dead[c];
+    for (int r = 0; r < n; ++r) {
+      const float v = load_w<DT>(staged, (long long)r * K + c);
+      out[(row0 + r) * K + j] = dz ? 0.0f : v;
     }
   }
 }
@@ -422,7 +455,18 @@ int lcq_gptq_prepare_weights(const void* w, int dtype, int64_t R, int64_t K, con
   if (grid > 0x7fffffff) return LCQ_EINVAL;
   hipStream_t st = (hipStream_t)stream;
   const long long* p = (const long long*)perm;
-  if (dtype == LCQ_F32) prepare_w_kernel<LCQ_F32><<<dim3((unsigned)grid), dim3(256), 0, st>>>(w, R, (int)K, p, dead, out);
+  const int es = dtype == LCQ_F32 ? 4 : 2;
+  if (p && K * es <= 65536 && (dtype == LCQ_F32 || dtype == LCQ_BF16 || dtype == LCQ_F16)) {   // gather through LDS
+    int rows = (int)(65536 / (K * es));
+    if (rows > 8) rows = 8;
+    const int64_t g = (R + rows - 1) / rows;
+    if (g > 0x7fffffff) return LCQ_EINVAL;
+    const size_t lds = (size_t)rows * K * es;
+    if (dtype == LCQ_F32) prepare_w_gather_kernel<LCQ_F32><<<dim3((unsigned)g), dim3(256), lds, st>>>(w, R, (int)K, rows, p, dead, out);
+    else if (dtype == LCQ_BF16) prepare_w_gather_kernel<LCQ_BF16><<<dim3((unsigned)g), dim3(256), lds, st>>>(w, R, (int)K, rows, p, dead, out);
+    else prepare_w_gather_kernel<LCQ_F16><<<dim3((unsigned)g), dim3(256), lds, st>>>(w, R, (int)K, rows, p, dead, out);
+  }
+  else if (dtype == LCQ_F32) prepare_w_kernel<LCQ_F32><<<dim3((unsigned)grid), dim3(256), 0, st>>>(w, R, (int)K, p, dead, out);
   else if (dtype == LCQ_BF16) prepare_w_kernel<LCQ_BF16><<<dim3((unsigned)grid), dim3(256), 0, st>>>(w, R, (int)K, p, dead, out);
   else if (dtype == LCQ_F16) prepare_w_kernel<LCQ_F16><<<dim3((unsigned)grid), dim3(256), 0, st>>>(w, R, (int)K, p, dead, out);
   else return LCQ_EDTYPE;
