@@ -236,7 +236,8 @@ int lcq_set_gemm_split(int on);
  * GPTQ.process_hessian_and_weights, gptq.py:139-141, 150-153, 169-174:
  *   dead = diag(H)==0; H[dead,dead] = 1; W[:,dead] = 0; H = H[perm][:,perm];
  *   H += percdamp*mean(diag H)*I; U = chol(cholesky_inverse(chol(H)), upper)
- *  H [K,K] fp32, valid on and above the diagonal (its diagonal is rewritten for dead columns)
+ *  H [K,K] fp32, valid on and above the diagonal (its diagonal is rewritten for dead columns, and with a
+ *  permutation its lower triangle is filled in from the upper one)
  *  perm [K] int64 or NULL (identity); W [R,K] fp32 in ORIGINAL column order or NULL
  *  U [K,K] fp32 out: upper triangular, zeros below the diagonal; U may alias H
  *  status [1] int32 device word or NULL: 1 if a non-positive pivot was met (H not positive definite) */

@@ -140,6 +140,31 @@ __global__ __launch_bounds__(256) void build_kernel(const float* __restrict__ H,
   A[(long long)a * K + b] = v;
 }
 
+// The same from a fully symmetric H and with a permutation: row a of A draws on row perm[K-1-a] of H only, which
+// comes in as it lies (16 bytes per lane) and is gathered from LDS.  (Picking H[min][max] from memory, as build_kernel
+// does, walks down a column of H for half of the entries: one 64-byte sector per element.)
+__global__ __launch_bounds__(256) void build_gather_kernel(const float* __restrict__ H, int K, const long long* __restrict__ perm,
+                                                           const PrepScalars* __restrict__ sc, float* __restrict__ A) {
+  extern __shared__ __align__(16) float hrow[];
+  const int a = blockIdx.x;
+  const float* src = H + perm[K - 1 - a] * (long long)K;
+  if ((((uintptr_t)src) & 15) == 0 && (K & 3) == 0) {
+    for (int i = threadIdx.x; i < (K >> 2); i += 256) ((f32x4*)hrow)[i] = ((const f32x4*)src)[i];
+  } else {
+    for (int i = threadIdx.x; i < K; i += 256) hrow[i] = src[i];
+  }
+  __syncthreads();
+  const float damp = sc->damp;
+  for (int b = threadIdx.x; b < K; b += 256) {
+    float v = 0.0f;
+    if (b <= a) {
+      v = hrow[perm[K - 1 - b]];
+      if (a == b) v += damp;
+    }
+    A[(long long)a * K + b] = v;
+  }
+}
+
 // Diagonal block: Cholesky factor L11 of a 128x128 block and its inverse, one workgroup of 8 waves.
 // A wave that is alone on its SIMD issues about one instruction per 8 cycles, and a column-by-column sweep with a
 // barrier per column executes ~150 instructions per column in every wave: 70 us per block, none of it arithmetic.
@@ -493,7 +518,12 @@ int lcq_chol_inv_upper(float* H, int64_t K64, const int64_t* perm, float percdam
     if (g > 65536) g = 65536;
     apply_dead_kernel<<<dim3((unsigned)g), dim3(256), 0, st>>>(W, R, K, dead);
   }
-  build_kernel<<<dim3((unsigned)((K + 255) / 256), (unsigned)K), dim3(256), 0, st>>>(H, K, (const long long*)perm, sc, A);
+  if (perm && K <= 16384) {                       // a row of H fits the 64 KB of LDS a workgroup may ask for
+    if (lcq_symmetrize(H, K, stream) != LCQ_OK) return LCQ_ELAUNCH;
+    build_gather_kernel<<<dim3((unsigned)K), dim3(256), (size_t)K * 4, st>>>(H, K, (const long long*)perm, sc, A);
+  } else {
+    build_kernel<<<dim3((unsigned)((K + 255) / 256), (unsigned)K), dim3(256), 0, st>>>(H, K, (const long long*)perm, sc, A);
+  }
 
   // Blocked right-looking Cholesky with two block sizes: 128-column panels are factored one by
   // one, but their trailing update is applied only inside the current 512-column super-panel;
