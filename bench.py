@@ -129,7 +129,7 @@ def bench_layer(args, out):
                 for n in subset:
                     gp.initialize_qparams_and_prepare_weights(layers[n], n)
                     a = ev(); a.record()
-                    W, U = gp.process_hessian_and_weights(layers[n], n)
+                    W, U = gp.process_hessian_and_weights(layers[n], n, for_loop=True)
                     b_ = ev(); b_.record()
                     gp.update_layer_with_transformed_weights(layers[n], W, U, n)
                     c = ev(); c.record()

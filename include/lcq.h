@@ -245,6 +245,18 @@ int64_t lcq_chol_inv_upper_workspace_bytes(int64_t K);
 int lcq_chol_inv_upper(float* H, int64_t K, const int64_t* perm, float percdamp, float* W, int64_t R, float* U,
                        void* workspace, int64_t workspace_bytes, int* status, void* stream);
 
+/* The same chain without the triangular inverse, for the column loop alone (K % 128 == 0, blocks of 128 columns).
+ * With H_d = M M^T (M upper triangular) the reference's factor is U = M^-1; P [K,K] out is block upper triangular:
+ *   P[b, b] = U[b, b] = (M[b, b])^-1        the 128 x 128 diagonal blocks of U, exactly what gptq.py:205 takes as Hinv1
+ *   P[p, b] = M[p, b] U[b, b],  p < b        in place of U[p, b]
+ * From E U = W0 - Q (E the loop's errors Err1, Q the quantized weights, W0 the weights before the loop) the weights
+ * the loop finds at block b are  W0[:, b] + sum_{p<b} (W0 - Q)[:, p] P[p, b]:  lcq_gptq_block / lcq_gptq_trailing give
+ * the reference's results on P when a block hands (Q - W0) to the deferred update (the W0 argument of
+ * lcq_gptq_block).  Valid while every group of the quantizer lies inside one block (group_size divides 128, or
+ * given parameters); saves the K^3/3 flop of the inverse.  Same workspace, arguments and status as above. */
+int lcq_chol_block_factor(float* H, int64_t K, const int64_t* perm, float percdamp, float* W, int64_t R, float* P,
+                          void* workspace, int64_t workspace_bytes, int* status, void* stream);
+
 /* One lazy-batch block of GPTQ.weight_transform, gptq.py:203-243 (columns i1 .. i1+count, count <= 128):
  * per-group scale/zero refresh (search_column_qparams, :358-366), quantize-dequantize,
  * tmp[:, i] = w, Losses[:, i], in-block error feedback; Err [R,128] receives Err1.
@@ -253,10 +265,13 @@ int lcq_chol_inv_upper(float* H, int64_t K, const int64_t* perm, float percdamp,
  *  dynamic groups (default): group_size > 0, G >= ceil(n_quant/group_size), qparams are written
  *  LCQ_FLAG_STATIC: qparams are inputs; group of column c is gidx[c] (or c/group_size, or 0 if group_size == 0)
  *  n_quant: the columns [0, n_quant) are quantized, a group's range ends there at the latest (gptq.py:218-221,
- *  `self.columns - self.n_out`); K without OWQ outlier columns */
-int lcq_gptq_block(float* W, float* tmp, float* Losses, float* Err, int64_t ldErr, const float* U, int64_t R, int64_t K,
-                   int64_t n_quant, int64_t i1, int count, int group_size, float qmin, float qmax, int flags, float* scales, float* zeros,
-                   const int32_t* gidx, int64_t G, void* stream);
+ *  `self.columns - self.n_out`); K without OWQ outlier columns
+ *  W0: NULL, or the [R,K] weights as they were before the loop when U is the block factor P of
+ *  lcq_chol_block_factor: Err then receives (quantized value - W0) instead of Err1, which is what the deferred
+ *  update needs with P. */
+int lcq_gptq_block(float* W, float* tmp, float* Losses, float* Err, int64_t ldErr, const float* U, const float* W0, int64_t R,
+                   int64_t K, int64_t n_quant, int64_t i1, int count, int group_size, float qmin, float qmax, int flags,
+                   float* scales, float* zeros, const int32_t* gidx, int64_t G, void* stream);
 
 /* Deferred update of gptq.py:244, generalised to a column window (fp32 MFMA):
  *   W[:, j1:j2] -= Err[:, :k2-k1] @ U[k1:k2, j1:j2],   k2 <= j1.

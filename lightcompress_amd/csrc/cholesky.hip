@@ -499,9 +499,11 @@ int lcq_gptq_prepare_weights(const void* w, int dtype, int64_t R, int64_t K, con
   return LCQ_OK;
 }
 
-int lcq_chol_inv_upper(float* H, int64_t K64, const int64_t* perm, float percdamp, float* W, int64_t R, float* U,
-                       void* workspace, int64_t workspace_bytes, int* status, void* stream) {
+// The chain behind lcq_chol_inv_upper (blocks_only = false) and lcq_chol_block_factor (true).
+static int chol_chain(float* H, int64_t K64, const int64_t* perm, float percdamp, float* W, int64_t R, float* U,
+                      void* workspace, int64_t workspace_bytes, int* status, void* stream, bool blocks_only) {
   if (!H || !U || !workspace || K64 <= 0 || K64 > 65536 || R < 0) return LCQ_EINVAL;
+  if (blocks_only && K64 % NB != 0) return LCQ_EINVAL;     // the blocks of the reversed matrix must be the loop's blocks
   if (workspace_bytes < lcq_chol_inv_upper_workspace_bytes(K64)) return LCQ_EWORKSPACE;
   if (((uintptr_t)workspace % 16) != 0) return LCQ_EALIGN;
   const int K = (int)K64;
@@ -551,6 +553,37 @@ int lcq_chol_inv_upper(float* H, int64_t K64, const int64_t* perm, float percdam
       launch_gemm<true>(GemmProblem{P, P, A + (long long)o1 * K + o1, K - o1, K - o1, o1 - o0, K, K, K}, -1.0f, 1.0f,
                         GEMM_LOWER_TILES, st);
     }
+  }
+
+  if (blocks_only) {
+    // No triangular inverse.  With M = J L J (H_d = M M^T, M upper triangular; J reverses the order) the inverse
+    // factor is U = M^-1, and the column loop needs of it only (a) the diagonal blocks U_bb = (M_bb)^-1, which drive
+    // the recurrence inside a block, and (b) something that carries a block's effect to the columns behind it.  From
+    // E U = W - Q (E the loop's errors, Q the quantized weights, W the weights before the loop) follows
+    //   W[:, b] as the loop finds it at block b  =  W0[:, b] + sum_{p<b} (W0 - Q)[:, p] M[p, b] U_bb,
+    // so with P[p, b] = M[p, b] U_bb above the diagonal blocks and P[b, b] = U_bb the loop runs unchanged on P if a
+    // block hands (Q - W0) instead of its errors to the deferred update.  In the reversed order that is every
+    // sub-diagonal panel of L times the inverse of its diagonal block, which the factorization has already: one
+    // batched product instead of the log2(K/128) merge levels of the inverse (K^3/3 flop).
+    for (int b0 = 0; b0 + 1 < nblk; b0 += GEMM_MAX_BATCH) {
+      const int np = (nblk - 1 - b0 < GEMM_MAX_BATCH) ? (nblk - 1 - b0) : GEMM_MAX_BATCH;
+      GemmBatch bt;
+      int maxM = 0;
+      for (int q = 0; q < np; ++q) {
+        const int b = b0 + q, k0 = b * NB, k1 = k0 + NB;
+        bt.offA[q] = (long long)k1 * K + k0; bt.offB[q] = (long long)b * NB * NB; bt.offC[q] = bt.offA[q];
+        bt.M[q] = K - k1; bt.N[q] = NB; bt.Kc[q] = NB;
+        if (K - k1 > maxM) maxM = K - k1;
+      }
+      const dim3 grid(1, (unsigned)((maxM + GT - 1) / GT), (unsigned)np);
+      gemm_f32_batched_kernel<false><<<grid, dim3(256), 0, st>>>(A, K, Dinv, NB, A, K, bt, 1.0f, 0.0f, 0);
+    }
+    place_diag_kernel<<<dim3((unsigned)nblk), dim3(256), 0, st>>>(A, K, Dinv);
+    scatter_kernel<<<dim3((unsigned)((K + 255) / 256), (unsigned)K), dim3(256), 0, st>>>(A, K, U);
+    if (status)
+      (void)hipMemcpyAsync(status, &sc->status, sizeof(int), hipMemcpyDeviceToDevice, st);
+    LCQ_CHECK_LAUNCH();
+    return LCQ_OK;
   }
 
   // triangular inverse: inverted diagonal blocks, then pairwise merges
@@ -603,6 +636,16 @@ int lcq_chol_inv_upper(float* H, int64_t K64, const int64_t* perm, float percdam
     (void)hipMemcpyAsync(status, &sc->status, sizeof(int), hipMemcpyDeviceToDevice, st);
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;
+}
+
+int lcq_chol_inv_upper(float* H, int64_t K, const int64_t* perm, float percdamp, float* W, int64_t R, float* U,
+                       void* workspace, int64_t workspace_bytes, int* status, void* stream) {
+  return chol_chain(H, K, perm, percdamp, W, R, U, workspace, workspace_bytes, status, stream, false);
+}
+
+int lcq_chol_block_factor(float* H, int64_t K, const int64_t* perm, float percdamp, float* W, int64_t R, float* P,
+                          void* workspace, int64_t workspace_bytes, int* status, void* stream) {
+  return chol_chain(H, K, perm, percdamp, W, R, P, workspace, workspace_bytes, status, stream, true);
 }
 
 }  // extern "C"

@@ -48,6 +48,7 @@ constexpr int ROWS_PER_WG = 16;
 
 struct LoopArgs {
   float* W; float* tmp; float* Losses; float* Err; const float* U;
+  const float* W0;      // the weights before the loop, or null: Err then receives q - W0 instead of the errors (see lcq_chol_block_factor)
   float* scales; float* zeros; const int* gidx;
   long long R; int K, Kq, i1, count, g, G, ldErr;      // Kq: columns that are quantized (K unless outlier columns are kept)
   float qmin, qmax;
@@ -306,8 +307,10 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
       if (col >= a.count) { s_ = 1.0f; z_ = 0.0f; }
       const float wv = w[c];
       const float code = a.nrz ? rintf(wv / fmaxf(s_, 1e-9f) + z_) : rintf(wv / s_) + z_;
-      const float diff = wv - (__builtin_amdgcn_fmed3f(code, a.qmin, a.qmax) - z_) * s_;
+      const float qdq = (__builtin_amdgcn_fmed3f(code, a.qmin, a.qmax) - z_) * s_;
+      const float diff = wv - qdq;
       o_err[c] = diff * Rd[col];
+      if (a.W0) o_err[c] = (col < a.count) ? qdq - a.W0[rbase + a.i1 + col] : 0.0f;
       const float d = Dg[col];
       loss[c] = (diff * diff) / (2.0f * (d * d));
     }
@@ -344,8 +347,8 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
 
 extern "C" {
 
-int lcq_gptq_block(float* W, float* tmp, float* Losses, float* Err, int64_t ldErr, const float* U, int64_t R, int64_t K,
-                   int64_t n_quant, int64_t i1, int count, int group_size, float qmin, float qmax, int flags, float* scales, float* zeros,
+int lcq_gptq_block(float* W, float* tmp, float* Losses, float* Err, int64_t ldErr, const float* U, const float* W0, int64_t R,
+                   int64_t K, int64_t n_quant, int64_t i1, int count, int group_size, float qmin, float qmax, int flags, float* scales, float* zeros,
                    const int32_t* gidx, int64_t G, void* stream) {
   if (!W || !tmp || !Losses || !Err || !U || !scales || ldErr < count || ldErr > 0x7fffffff) return LCQ_EINVAL;
   if (R <= 0 || K <= 0 || K > 0x7fffffff || i1 < 0 || count <= 0 || count > BS) return LCQ_EINVAL;
@@ -356,7 +359,7 @@ int lcq_gptq_block(float* W, float* tmp, float* Losses, float* Err, int64_t ldEr
   if (!is_static && (group_size <= 0 || G < (n_quant + group_size - 1) / group_size)) return LCQ_EINVAL;
   if (!sym && !zeros) return LCQ_EINVAL;
   LoopArgs a;
-  a.W = W; a.tmp = tmp; a.Losses = Losses; a.Err = Err; a.U = U;
+  a.W = W; a.tmp = tmp; a.Losses = Losses; a.Err = Err; a.U = U; a.W0 = W0;
   a.scales = scales; a.zeros = zeros; a.gidx = gidx;
   a.R = R; a.K = (int)K; a.Kq = (int)n_quant; a.i1 = (int)i1; a.count = count; a.g = group_size; a.G = (int)G;
   a.qmin = qmin; a.qmax = qmax; a.sym = sym; a.is_static = is_static; a.ldErr = (int)ldErr;

@@ -79,6 +79,8 @@ class GPTQ:
         # subset_transform starts the Cholesky chains of all Linears of a subset side by side (False: one by one)
         self.chain_overlap = bool(special_config.get('chain_overlap', True))
         self.fuse_loops = bool(special_config.get('fuse_loops', True))
+        # layer_transform / subset_transform factor H without the triangular inverse where the loop allows it
+        self.block_factor = bool(special_config.get('block_factor', True))
         # Linears of a subset that keep receiving the very same input tensor share one Hessian and one chain
         self.auto_share = bool(special_config.get('auto_share', True))
         if self.owq:                                     # gptq.py:47-50
@@ -425,9 +427,10 @@ class GPTQ:
             side = self._side_streams[i % len(self._side_streams)]
             side.wait_stream(main)
             with torch.cuda.stream(side):
-                L.check(L.lib().lcq_chol_inv_upper(L.ptr(H), L.i64(K), L.ptr(perm), L.f32(self.percdamp), L.ptr(None),
-                                                   L.i64(0), L.ptr(H), L.ptr(ws), L.i64(ws_bytes), L.ptr(status),
-                                                   L.stream()), 'lcq_chol_inv_upper')
+                direct = self._block_factor_ok(K)
+                chain = L.lib().lcq_chol_block_factor if direct else L.lib().lcq_chol_inv_upper
+                L.check(chain(L.ptr(H), L.i64(K), L.ptr(perm), L.f32(self.percdamp), L.ptr(None), L.i64(0), L.ptr(H), L.ptr(ws),
+                              L.i64(ws_bytes), L.ptr(status), L.stream()), 'Cholesky chain')
                 status_host = self._post_status(status)
                 done = side.record_event()
             for t in (ws, H, status, perm):              # allocated on the main stream, used on `side`: not to be
@@ -435,7 +438,7 @@ class GPTQ:
                     t.record_stream(side)
             del ws
             self._shared[leader] = dict(U=H, perm=perm, status=status, dead=dead, done=done, ahead=True,
-                                        status_host=status_host)
+                                        status_host=status_host, direct=direct)
 
     @staticmethod
     def _post_status(status):
@@ -451,7 +454,7 @@ class GPTQ:
     @torch.no_grad()
     def layer_transform(self, layer, name):
         self.initialize_qparams_and_prepare_weights(layer, name)
-        W, H = self.process_hessian_and_weights(layer, name)
+        W, H = self.process_hessian_and_weights(layer, name, for_loop=True)
         self.update_layer_with_transformed_weights(layer, W, H, name)
 
     def initialize_qparams_and_prepare_weights(self, layer, name):
@@ -472,9 +475,22 @@ class GPTQ:
         elif self.actorder or self.owq:
             self.hessian_sorting(name)
 
-    def process_hessian_and_weights(self, layer, name, out=None):
+    def _block_factor_ok(self, K):
+        """May the loop run on the block factor P of lcq_chol_block_factor instead of U?  Every group of the
+        quantizer has to lie inside one 128-column block (or the parameters are given), K in whole blocks."""
+        if not self.block_factor or self.owq or self.blocksize != 128 or K % 128 != 0:
+            return False
+        wq = self.wquantizer
+        if wq.granularity == 'per_group' and not self.static_groups:
+            return wq.group_size > 0 and 128 % wq.group_size == 0
+        return True
+
+    def process_hessian_and_weights(self, layer, name, out=None, for_loop=False):
         """-> (W [R,K] fp32 in processing order, Hinv: upper factor of the damped inverse).  `out`: where W goes
-        (an [R, K] fp32 tensor, e.g. the rows of a larger one), else a new tensor."""
+        (an [R, K] fp32 tensor, e.g. the rows of a larger one), else a new tensor.
+        `for_loop` (what layer_transform passes): the second result is only going to feed weight_transform, so
+        where the quantizer allows it (_block_factor_ok) it is the block factor P of lcq_chol_block_factor, which has
+        U's diagonal blocks but needs no triangular inverse; weight_transform recognises it."""
         w = layer.weight.data
         if w.dim() > 2:
             w = w.flatten(1)
@@ -496,18 +512,24 @@ class GPTQ:
             ws_bytes = L.lib().lcq_chol_inv_upper_workspace_bytes(L.i64(K))
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=self.dev)
             status = torch.zeros(1, dtype=torch.int32, device=self.dev)
-            L.check(L.lib().lcq_chol_inv_upper(L.ptr(H), L.i64(K), L.ptr(perm), L.f32(self.percdamp), L.ptr(None),
-                                               L.i64(0), L.ptr(H), L.ptr(ws), L.i64(ws_bytes), L.ptr(status),
-                                               L.stream()), 'lcq_chol_inv_upper')
+            direct = for_loop and self._block_factor_ok(K)
+            chain = L.lib().lcq_chol_block_factor if direct else L.lib().lcq_chol_inv_upper
+            L.check(chain(L.ptr(H), L.i64(K), L.ptr(perm), L.f32(self.percdamp), L.ptr(None), L.i64(0), L.ptr(H), L.ptr(ws),
+                          L.i64(ws_bytes), L.ptr(status), L.stream()), 'Cholesky chain')
             del ws
-            shared = dict(U=H, perm=perm, status=status, dead=dead, status_host=self._post_status(status))
+            shared = dict(U=H, perm=perm, status=status, dead=dead, status_host=self._post_status(status), direct=direct)
             if is_shared:
                 self._shared[leader] = shared
         elif 'done' in shared:                               # started by _chains_ahead on another stream
             torch.cuda.current_stream().wait_event(shared.pop('done'))
         U = shared['U']
+        if shared.get('direct') and not for_loop:
+            raise L.LcqError('the chain of this Hessian was started for the column loop (block factor, no inverse): '
+                             'call process_hessian_and_weights(..., for_loop=True) or set special.block_factor: False')
         self._status = shared['status']
         self._status_host = shared['status_host']
+        self._loop_factor = (U.data_ptr(), bool(shared.get('direct')))      # what weight_transform is going to be handed
+        self._loop_W0 = None
 
         # weight.clone().float(), W[:, dead] = 0 and W[:, perm] in one pass
         W = torch.empty((R, K), dtype=torch.float32, device=w.device) if out is None else out
@@ -527,6 +549,8 @@ class GPTQ:
                     _, layer.buf_scales, layer.buf_zeros, _, _ = self.wquantizer.get_tensor_qparams(
                         W[:, : self.n_nonout].contiguous())
                     self._setup_groups(layer, R, K)
+        if self._loop_factor[1] and out is None:
+            self._loop_W0 = W.clone()                    # the block factor needs the weights as they were before the loop
         return W, U
 
     def _setup_groups(self, layer, R, K):
@@ -603,7 +627,7 @@ class GPTQ:
         for n, R in zip(names, rows):
             layer = layers_dict[n]
             self.initialize_qparams_and_prepare_weights(layer, n)
-            _, U = self.process_hessian_and_weights(layer, n, out=Wall[r0:r0 + R])
+            _, U = self.process_hessian_and_weights(layer, n, out=Wall[r0:r0 + R], for_loop=True)
             parts.append((n, layer, r0, R, self._scales, self._zeros))
             r0 += R
         if self._static:                                 # given parameters: one row block per Linear
@@ -612,6 +636,8 @@ class GPTQ:
         else:
             self._scales = torch.empty((r0, self._G), device=self.dev)
             self._zeros = None if self.wquantizer.sym else torch.empty((r0, self._G), device=self.dev)
+        if self._loop_factor[1]:
+            self._loop_W0 = Wall.clone()
         Losses, tmp = torch.empty_like(Wall), torch.empty_like(Wall)
         self.weight_transform(Wall, U, Losses, tmp)
         self._check_status()
@@ -637,6 +663,14 @@ class GPTQ:
         # the block kernel; any other calibrator (mse, hqq) runs on the host side before the block that opens the
         # group, on the same columns of W the kernel would read, and the kernel takes the result as given.
         host_groups = (not self._static) and wq.calib_algo in ('mse', 'hqq', 'learnable')
+        # Hinv is U, or the block factor P that process_hessian_and_weights(for_loop=True) made instead: the block
+        # kernel then hands (quantized - original) to the deferred updates and needs the original weights
+        W0 = None
+        ptr_, direct_ = getattr(self, '_loop_factor', (None, False))
+        if direct_ and ptr_ == Hinv.data_ptr():
+            W0 = self._loop_W0
+            if W0 is None or W0.shape != W.shape:
+                raise L.LcqError('weight_transform on a block factor needs the weights before the loop (_loop_W0)')
         if self._static or host_groups:
             flags |= L.FLAG_STATIC
         g = self._g
@@ -667,7 +701,7 @@ class GPTQ:
                             self._zeros[:, idx // g] = z_.reshape(-1).float()
                 err_blk = Err[:, i1 - o0:]
                 L.check(lib.lcq_gptq_block(L.ptr(W), L.ptr(tmp), L.ptr(Losses), C_ptr(err_blk), L.i64(window), L.ptr(Hinv),
-                                           L.i64(R), L.i64(K), L.i64(n), L.i64(i1), L.i32(i2 - i1), L.i32(self._g), qmin, qmax,
+                                           L.ptr(W0), L.i64(R), L.i64(K), L.i64(n), L.i64(i1), L.i32(i2 - i1), L.i32(self._g), qmin, qmax,
                                            L.i32(flags), L.ptr(self._scales), L.ptr(self._zeros), L.ptr(self._gidx),
                                            L.i64(self._G), st), 'lcq_gptq_block')
                 if i2 < hi:
