@@ -21,6 +21,12 @@ Differences a caller can observe
     (``special.fuse_loops``, default on; rows are independent, so each Linear gets the result of its own loop, up to
     the rounding of the update GEMM where the larger row count selects the other GEMM kernel), and leaves every
     Linear's summed loss in ``last_errors[name]``;
+  * layer_transform / subset_transform factor the damped Hessian WITHOUT the triangular inverse where every group of
+    the weight quantizer lies inside one 128-column block (``special.block_factor``, default on): the loop runs on a
+    block factor that has U's diagonal blocks (gptq.py:205 `Hinv1`) and carries (quantized - original) weights
+    instead of errors to later columns; the same results up to fp32 rounding (closer to fp64 than the reference's
+    cholesky / cholesky_inverse / cholesky chain).  process_hessian_and_weights called on its own returns the
+    reference's U;
   * ``special.hessian_defer`` (default 'auto': 16 for K <= 4096, 8 for K <= 8192, else 4) add_batch calls are copied to a staging buffer and
     folded into one launch, so ``layers_cache[name]['H']`` lags behind ``nsamples`` until
     ``hessian(name)``, ``hessian_sorting`` or ``process_hessian_and_weights`` settles it
