@@ -88,7 +88,23 @@ def process_hessian_and_weights(weight: torch.Tensor, H: torch.Tensor, percdamp:
 # ---------------------------------------------------------------------------
 # lazy-batch column loop   (gptq.py:198-244)
 # ---------------------------------------------------------------------------
-def weight_transform(W, Hinv, spec, blocksize=128, static_qparams=None, static_groups=None, qparams_fn=None, n_out=0):
+def block_factor(U, blocksize=128):
+    """The block upper triangular P that stands in for U in the column loop (no counterpart in the reference, which
+    always forms U; the product's chain builds P without a triangular inverse).  With M = U^-1:
+    P[b, b] = U[b, b] (gptq.py:205 takes exactly this block as Hinv1), P[p, b] = M[p, b] U[b, b] for p < b."""
+    K = U.shape[0]
+    assert K % blocksize == 0
+    M = torch.linalg.solve_triangular(U, torch.eye(K, dtype=U.dtype), upper=True)
+    P = torch.zeros_like(U)
+    for b in range(K // blocksize):
+        sl = slice(b * blocksize, (b + 1) * blocksize)
+        P[sl, sl] = U[sl, sl]
+        P[:b * blocksize, sl] = M[:b * blocksize, sl] @ U[sl, sl]
+    return P
+
+
+def weight_transform(W, Hinv, spec, blocksize=128, static_qparams=None, static_groups=None, qparams_fn=None, n_out=0,
+                     block_factor_W0=None):
     """Runs the loop in place on W (as the reference does) and returns
     (tmp, Losses, groups) where groups is the list of per-group
     (scale [R,1], zero [R,1]|0-dim) refreshed at every group boundary.
@@ -103,6 +119,8 @@ def weight_transform(W, Hinv, spec, blocksize=128, static_qparams=None, static_g
     (gptq.py:358-366 calls it, so ``calib_algo`` reaches the loop); default: min/max calibration.
     ``n_out``: OWQ - the last n_out columns are not quantized (the loop and the group ranges stop before them) but
     still receive every block's update.
+    ``block_factor_W0``: Hinv is block_factor(U) and this is a copy of W as it was before the loop; a block then hands
+    (quantized - original) instead of Err1 to the update of the later columns, everything else is the reference's loop.
     """
     qparams_fn = qparams_fn or Q.int_tensor_qparams
     R, K = W.shape
@@ -119,6 +137,7 @@ def weight_transform(W, Hinv, spec, blocksize=128, static_qparams=None, static_g
         count = i2 - i1
         W1, Hinv1 = W[:, i1:i2].clone(), Hinv[i1:i2, i1:i2]
         tmp1, Err1, Losses1 = torch.zeros_like(W1), torch.zeros_like(W1), torch.zeros_like(W1)
+        Q1 = torch.zeros_like(W1)
         for i in range(count):
             w, d = W1[:, i], Hinv1[i, i]
             if per_group and static_groups is not None:
@@ -134,11 +153,14 @@ def weight_transform(W, Hinv, spec, blocksize=128, static_qparams=None, static_g
                 groups.append((scale.clone(), zero.clone()))
             q = Q.int_quant_dequant(spec, w.unsqueeze(1), scale, zero, qmax, qmin).squeeze(1)
             tmp1[:, i] = w
+            Q1[:, i] = q
             Losses1[:, i] = ((w - q) ** 2) / (2 * d ** 2)
             err1 = (w - q) / d
             W1[:, i:] -= err1.unsqueeze(1).matmul(Hinv1[i, i:].unsqueeze(0))
             Err1[:, i] = err1
         tmp[:, i1:i2], Losses[:, i1:i2] = tmp1, Losses1
+        if block_factor_W0 is not None:
+            Err1 = Q1 - block_factor_W0[:, i1:i2]
         W[:, i2:] -= Err1.matmul(Hinv[i1:i2, i2:])
     return tmp, Losses, groups
 

@@ -107,6 +107,40 @@ def test_column_loop_matches_textbook_recurrence_and_loss_identity(blocksize):
     assert abs(float(Losses.sum()) - 0.5 * float(torch.trace(D @ Hd @ D.t()))) < 1e-12 + 1e-9 * float(Losses.sum())
 
 
+@pytest.mark.parametrize('g,static', [(128, False), (64, False), (32, False), (128, True)])
+def test_loop_on_the_block_factor_is_the_reference_loop(g, static):
+    """The chain that skips the triangular inverse hands the loop P (P[b,b] = U[b,b], P[p,b] = U^-1[p,b] U[b,b]) and
+    every block passes (quantized - original) on instead of its errors.  In fp64 that loop gives the reference loop's
+    compensated weights, losses and group parameters whenever a group lies inside one 128-column block, including
+    groups that open in the middle of a block (whose ranges the reference reads from the partly updated W)."""
+    R, K = 6, 640
+    spec = Q.IntSpec(4, False, 'per_group', group_size=g)
+    H = G.hessian_closed_form(calib_batches(6, 96, K, seed=2100 + g))
+    W0 = torch.randn(R, K, generator=gen(6), dtype=torch.float64) * 0.02
+    W, U, _ = G.process_hessian_and_weights(W0, H, 0.01, None, dtype=torch.float64)
+    P = G.block_factor(U)
+    assert torch.equal(torch.triu(P), P)
+    for b in range(K // 128):
+        assert torch.equal(P[128 * b:128 * b + 128, 128 * b:128 * b + 128], U[128 * b:128 * b + 128, 128 * b:128 * b + 128])
+    sg = None
+    if static:                                            # parameters given per group of the original order
+        _, s_, z_, _, _ = Q.int_tensor_qparams(spec, W0.float())
+        sg = (s_.reshape(R, K // g).double(), z_.reshape(R, K // g).double(), None)
+    tmp, Losses, groups = G.weight_transform(W.clone(), U, spec, static_groups=sg)
+    tmp_p, Losses_p, groups_p = G.weight_transform(W.clone(), P, spec, static_groups=sg, block_factor_W0=W.clone())
+    assert float((tmp - tmp_p).abs().max()) < 1e-12
+    assert float((Losses - Losses_p).abs().max()) < 1e-12 * max(1.0, float(Losses.abs().max()))
+    assert len(groups) == len(groups_p) == (0 if static else K // g)
+    for (s1, z1), (s2, z2) in zip(groups, groups_p):
+        assert float((s1 - s2).abs().max()) < 1e-14 and torch.equal(z1, z2)
+    # a group wider than a block is outside what P can reproduce: the ranges of its later columns differ
+    if not static and g == 128:
+        spec2 = Q.IntSpec(4, False, 'per_group', group_size=256)
+        t1, _, _ = G.weight_transform(W.clone()[:, :512], U[:512, :512], spec2)
+        t2, _, _ = G.weight_transform(W.clone()[:, :512], G.block_factor(U[:512, :512]), spec2, block_factor_W0=W.clone()[:, :512])
+        assert float((t1 - t2).abs().max()) > 1e-9
+
+
 def test_identity_hessian_reduces_to_rtn():
     R, K = 8, 256
     spec = Q.IntSpec(4, False, 'per_group', group_size=128)
