@@ -34,6 +34,7 @@ enum : int {
   GEMM_LOWER_TILES = 1,   // only tiles with n0 <= m0 (C symmetric / lower triangular)
   GEMM_K_FROM_N = 2,      // B is lower triangular [k][n]: terms with k < n0 vanish
   GEMM_K_TO_M = 4,        // A is lower triangular [m][k]: terms with k >= m0 + GT vanish
+  GEMM_XCD_ORDER = 8,     // (set by launch_gemm) workgroups take their tile from the XCD-contiguous super-block order
 };
 
 struct GemmProblem {
@@ -440,12 +441,53 @@ __device__ __forceinline__ void gemm_tile_s3(const float* A, int lda, const floa
     }
 }
 
+// Workgroup -> tile for the big launches.  Workgroups go to the 8 XCDs round-robin (block b runs on XCD b % 8) and
+// every XCD has its own 4 MB L2, while a 128 x 128 tile reads 2 x 128 x Kc x 4 bytes of operands: in the plain
+// row-major order the tiles an XCD holds at one time share one operand and stream the other from beyond L2
+// (4.4 TB/s at 140 TFLOP/s with Kc = 512, served by the Infinity Cache: worth 2 % of the chain).  Here XCD x works through the contiguous range [x * per, (x + 1) * per)
+// of a tile order made of square super-blocks (SB x SB tiles, row-major inside and between them), so what it holds
+// at one time draws on SB + SB operand tiles instead of 1 + SB * SB.
+template <int SB>
+__device__ __forceinline__ void s3_tile_of(int gx, int gy, int& tm, int& tn) {
+  const int total = gx * gy, base = total >> 3, rem = total & 7;
+  const int lin = blockIdx.y * gx + blockIdx.x, x = lin & 7;
+  int v = x * base + min(x, rem) + (lin >> 3);            // XCD x holds base (+1 for x < rem) consecutive tiles
+  const int sr = v / (SB * gx), r0 = sr * SB, nr = min(SB, gy - r0);      // super-row: nr tile rows x gx tile columns
+  v -= r0 * gx;
+  const int sc = min(v / (nr * SB), (gx - 1) / SB), c0 = sc * SB, nc = min(SB, gx - c0);
+  v -= sc * nr * SB;
+  tm = r0 + v / nc;
+  tn = c0 + v % nc;
+}
+
 template <bool B_T>
 __global__ __launch_bounds__(256, 2) void gemm_s3_kernel(GemmProblem g, float alpha, float beta, int flags) {
   __shared__ __attribute__((aligned(16))) uint16_t sA[3 * S3_PLANE];
   __shared__ __attribute__((aligned(16))) uint16_t sB[3 * S3_PLANE];
-  const int m0 = blockIdx.y * GT, n0 = blockIdx.x * GT;
+  int tm = blockIdx.y, tn = blockIdx.x;
+  if (flags & GEMM_XCD_ORDER) s3_tile_of<8>(gridDim.x, gridDim.y, tm, tn);
+  const int m0 = tm * GT, n0 = tn * GT;
   if ((flags & GEMM_LOWER_TILES) && n0 >= m0 + GT) return;
+  gemm_tile_s3<B_T>(g.A, g.lda, g.B, g.ldb, g.C, g.ldc, g.M, g.N, g.Kc, alpha, beta, flags, m0, n0, sA, sB);
+}
+
+// The lower triangle of a square launch whose side is a whole number of 4 x 4 super-blocks (the deep trailing updates
+// of the Cholesky chain): a 1-D grid over the super-blocks on and below the diagonal only, 16 tiles each, in the
+// XCD-contiguous order described above.  (A 2-D grid launches as many workgroups again that return at once.)
+template <bool B_T>
+__global__ __launch_bounds__(256, 2) void gemm_s3_lower_kernel(GemmProblem g, float alpha, float beta, int flags, int nsb) {
+  __shared__ __attribute__((aligned(16))) uint16_t sA[3 * S3_PLANE];
+  __shared__ __attribute__((aligned(16))) uint16_t sB[3 * S3_PLANE];
+  const int total = 16 * (nsb * (nsb + 1) / 2);            // a multiple of 8: the grid
+  const int lin = blockIdx.x;
+  const int v = (lin & 7) * (total >> 3) + (lin >> 3);
+  const int sb = v >> 4, t = v & 15;
+  int sr = (int)((__builtin_sqrtf(8.0f * (float)sb + 1.0f) - 1.0f) * 0.5f);
+  while (sr * (sr + 1) / 2 > sb) --sr;
+  while ((sr + 1) * (sr + 2) / 2 <= sb) ++sr;
+  const int sc = sb - sr * (sr + 1) / 2;
+  const int m0 = (sr * 4 + (t >> 2)) * GT, n0 = (sc * 4 + (t & 3)) * GT;
+  if (n0 >= m0 + GT) return;
   gemm_tile_s3<B_T>(g.A, g.lda, g.B, g.ldb, g.C, g.ldc, g.M, g.N, g.Kc, alpha, beta, flags, m0, n0, sA, sB);
 }
 
@@ -500,8 +542,11 @@ inline void launch_gemm(const GemmProblem& g, float alpha, float beta, int flags
     gemm_f32_kernel<B_T, 64, true><<<dim3(gx, (unsigned)((g.M + 63) / 64)), dim3(256), 0, st>>>(g, alpha, beta, flags);
   else if ((long long)gx * gy <= 256)
     gemm_f32_kernel<B_T, 64><<<dim3(gx, (unsigned)((g.M + 63) / 64)), dim3(256), 0, st>>>(g, alpha, beta, flags);
-  else if (g_gemm_split)
-    gemm_s3_kernel<B_T><<<dim3(gx, gy), dim3(256), 0, st>>>(g, alpha, beta, flags);
+  else if (g_gemm_split && (flags & GEMM_LOWER_TILES) && g.M == g.N && g.M % (4 * GT) == 0) {
+    const int nsb = g.M / (4 * GT), total = 16 * (nsb * (nsb + 1) / 2);
+    gemm_s3_lower_kernel<B_T><<<dim3((unsigned)total), dim3(256), 0, st>>>(g, alpha, beta, flags, nsb);
+  } else if (g_gemm_split)
+    gemm_s3_kernel<B_T><<<dim3(gx, gy), dim3(256), 0, st>>>(g, alpha, beta, flags | GEMM_XCD_ORDER);
   else
     gemm_f32_kernel<B_T, GT><<<dim3(gx, gy), dim3(256), 0, st>>>(g, alpha, beta, flags);
 }
