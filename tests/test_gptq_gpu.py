@@ -239,6 +239,62 @@ def test_column_loop_against_oracle(dev, R, K, g, bs, sym):
     assert abs(float(Losses.sum()) - float(Loss_o.sum())) <= 1e-3 * float(Loss_o.sum())
 
 
+@pytest.mark.parametrize('R,K,g,sym,variant', [(64, 512, 128, False, 'minmax'), (40, 640, 64, True, 'minmax'), (32, 512, 32, False, 'minmax'),
+                                               (40, 512, 128, False, 'round_zp_off'), (32, 512, 128, False, 'mse'),
+                                               (32, 384, 0, False, 'per_channel')])
+def test_column_loop_on_the_block_factor(dev, R, K, g, sym, variant):
+    """weight_transform handed the block factor P (and the weights as they were before the loop) instead of U: the
+    compensated weights, group parameters and losses of the reference loop on U, for dynamic groups inside a block,
+    un-rounded zero points, a calibrator that runs on the host side at every group opening, and given parameters."""
+    spec, W0, W, U = _loop_case(R, K, g if g else 128, 128, sym, 5600 + K + g)
+    wcfg = dict(bit=4, symmetric=sym, granularity='per_group', group_size=g)
+    kw, layer, fn = {}, None, None
+    if variant == 'round_zp_off':
+        spec.round_zp = False
+        wcfg['round_zp'] = False
+    if variant == 'mse':
+        wcfg['calib_algo'] = 'mse'
+    if variant == 'per_channel':
+        spec = Q.IntSpec(4, sym, 'per_channel')
+        wcfg = dict(bit=4, symmetric=sym, granularity='per_channel')
+        _, s0, z0, _, _ = Q.int_tensor_qparams(spec, W0)
+        kw['static_qparams'] = (s0, z0)
+        layer = types.SimpleNamespace(buf_scales=s0.to(dev), buf_zeros=z0.to(dev))
+    if variant == 'mse':                                  # against this library's loop on U: the same search kernel
+        tmp_o, Loss_o, s_u, _ = _run_loop(dev, make_gptq(weight=wcfg), W, U, R, K)
+    else:
+        tmp_o, Loss_o, groups = G.weight_transform(W.clone(), U, spec, qparams_fn=fn, **kw)
+    P = G.block_factor(U.double()).float()
+    gp = make_gptq(weight=wcfg)
+    assert gp._block_factor_ok(K)
+    gp.n_nonout = gp.columns = K
+    gp._setup_groups(layer, R, K)
+    Wd, Pd = W.clone().to(dev), P.to(dev).contiguous()
+    gp._loop_factor, gp._loop_W0 = (Pd.data_ptr(), True), Wd.clone()
+    tmp, Losses = torch.zeros_like(Wd), torch.zeros_like(Wd)
+    gp.weight_transform(Wd, Pd, Losses, tmp)
+    tmp, Losses = tmp.cpu(), Losses.cpu()
+    s, z = gp._scales.cpu(), (None if sym else gp._zeros.cpu())
+    if variant == 'mse':                                  # a shrink search may tie between neighbouring steps
+        same = torch.isclose(s, s_u, rtol=1e-4).all(dim=1)
+        assert float(same.float().mean()) >= 0.8
+        assert float((tmp - tmp_o)[same].abs().max()) < 1e-4 * float(tmp_o.abs().max())
+        assert abs(float(Losses.sum()) - float(Loss_o.sum())) <= 0.02 * float(Loss_o.sum())
+    else:
+        assert float((tmp - tmp_o).abs().max()) < 1e-4 * float(tmp_o.abs().max())
+        assert abs(float(Losses.sum()) - float(Loss_o.sum())) <= 1e-3 * float(Loss_o.sum())
+    if variant not in ('per_channel', 'mse'):
+        so, zo = G.merge_groups(groups)
+        assert torch.allclose(s.reshape(-1, 1), so, rtol=1e-4)
+        codes_o = G.codes_from(tmp_o, so, zo, spec)
+        codes = G.codes_from(tmp, s.reshape(-1, 1), None if sym else z.reshape(-1, 1), spec)
+        assert float((codes == codes_o).float().mean()) >= 0.999
+    # without the weights before the loop the call is refused, and U given as U still takes the reference's path
+    gp._loop_W0 = None
+    with pytest.raises(Exception):
+        gp.weight_transform(W.clone().to(dev), Pd, torch.zeros_like(Wd), torch.zeros_like(Wd))
+
+
 def test_per_channel_static_loop(dev):
     R, K = 32, 256
     spec = Q.IntSpec(4, False, 'per_channel')
