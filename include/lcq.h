@@ -232,6 +232,14 @@ int lcq_gptq_prepare_weights(const void* w, int dtype, int64_t R, int64_t K, con
  * Process-wide; returns the previous setting. */
 int lcq_set_gemm_split(int on);
 
+/* Chains of K >= 8192: 1 (default) runs the deep trailing update behind a 512-column super-panel in two parts, the
+ * columns of the next super-panel on the caller's stream and the rest on a stream the library creates once per
+ * (device, caller's stream), beside the next super-panel's narrow launches; the two are ordered by events and joined
+ * before the call's last launches, so the caller sees one stream-ordered call.  0: everything on the caller's stream.
+ * The results agree to fp32 rounding (a part of an update may select the other GEMM kernel than the whole update
+ * would) and are reproducible from run to run either way.  Process-wide; returns the previous setting. */
+int lcq_set_chain_lookahead(int on);
+
 /* Dead columns, act-order permutation, damping and the Cholesky chain of
  * GPTQ.process_hessian_and_weights, gptq.py:139-141, 150-153, 169-174:
  *   dead = diag(H)==0; H[dead,dead] = 1; W[:,dead] = 0; H = H[perm][:,perm];

@@ -22,6 +22,7 @@
 //   (batched)      triangular inverse by pairwise merging of inverted diagonal
 //                  blocks: [[A,0],[B,C]]^-1 = [[A^-1,0],[-C^-1 B A^-1, C^-1]]
 //   scatter        U[i][j] = Linv[K-1-i][K-1-j], j >= i; zeros below the diagonal
+#include <mutex>
 #include "gemm_f32.h"
 #include "lcq_internal.h"
 
@@ -499,6 +500,28 @@ int lcq_gptq_prepare_weights(const void* w, int dtype, int64_t R, int64_t K, con
   return LCQ_OK;
 }
 
+// A second stream per (device, caller's stream) for the deep trailing updates of long chains, with the two events that
+// order it against the caller's stream.  Created on first use, kept until the process ends.
+struct SideLane { int dev; hipStream_t caller; hipStream_t side; hipEvent_t fork, join; };
+static SideLane g_lanes[16];
+static int g_nlanes = 0;
+static std::mutex g_lane_mu;
+static int g_lookahead = 1;
+static SideLane* side_lane(hipStream_t st) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+  std::lock_guard<std::mutex> lock(g_lane_mu);
+  for (int i = 0; i < g_nlanes; ++i)
+    if (g_lanes[i].dev == dev && g_lanes[i].caller == st) return &g_lanes[i];
+  if (g_nlanes == 16) return nullptr;
+  SideLane l{dev, st, nullptr, nullptr, nullptr};
+  if (hipStreamCreateWithFlags(&l.side, hipStreamNonBlocking) != hipSuccess) return nullptr;       // default priority
+  if (hipEventCreateWithFlags(&l.fork, hipEventDisableTiming) != hipSuccess ||
+      hipEventCreateWithFlags(&l.join, hipEventDisableTiming) != hipSuccess) return nullptr;
+  g_lanes[g_nlanes] = l;
+  return &g_lanes[g_nlanes++];
+}
+
 // The chain behind lcq_chol_inv_upper (blocks_only = false) and lcq_chol_block_factor (true).
 static int chol_chain(float* H, int64_t K64, const int64_t* perm, float percdamp, float* W, int64_t R, float* U,
                       void* workspace, int64_t workspace_bytes, int* status, void* stream, bool blocks_only) {
@@ -532,6 +555,12 @@ static int chol_chain(float* H, int64_t K64, const int64_t* perm, float percdamp
   // the rest of the matrix is updated once per super-panel with a 512-deep contraction, which
   // cuts the read-modify-write traffic on the trailing matrix fourfold.
   constexpr int NBO = 4 * NB;
+  // Long chains: the deep update behind a super-panel is split into the columns of the NEXT super-panel (on the
+  // caller's stream, the panels that follow need it) and everything behind those (on the side stream, beside those
+  // panels: a few narrow launches that leave the chip to it).  The next deep update touches that region again and
+  // waits for it.
+  SideLane* lane = (g_lookahead && K >= 8192) ? side_lane(st) : nullptr;
+  bool pending = false;
   for (int o0 = 0; o0 < K; o0 += NBO) {
     const int o1 = (o0 + NBO < K) ? (o0 + NBO) : K;
     for (int k0 = o0; k0 < o1; k0 += NB) {
@@ -548,12 +577,29 @@ static int chol_chain(float* H, int64_t K64, const int64_t* perm, float percdamp
                             GEMM_LOWER_TILES, st);
       }
     }
-    if (o1 < K) {                                                                                 // everything behind it
+    if (o1 < K && lane) {
+      const int o2 = (o1 + NBO < K) ? (o1 + NBO) : K;
+      const float* P = A + (long long)o1 * K + o0;
+      if (pending && hipStreamWaitEvent(st, lane->join, 0) != hipSuccess) return LCQ_ELAUNCH;
+      pending = false;
+      if (hipEventRecord(lane->fork, st) != hipSuccess) return LCQ_ELAUNCH;           // the panels of this super-panel
+      launch_gemm<true>(GemmProblem{P, P, A + (long long)o1 * K + o1, K - o1, o2 - o1, o1 - o0, K, K, K}, -1.0f, 1.0f,
+                        GEMM_LOWER_TILES, st);
+      if (o2 < K) {
+        const float* P2 = A + (long long)o2 * K + o0;
+        if (hipStreamWaitEvent(lane->side, lane->fork, 0) != hipSuccess) return LCQ_ELAUNCH;
+        launch_gemm<true>(GemmProblem{P2, P2, A + (long long)o2 * K + o2, K - o2, K - o2, o1 - o0, K, K, K}, -1.0f, 1.0f,
+                          GEMM_LOWER_TILES, lane->side);
+        if (hipEventRecord(lane->join, lane->side) != hipSuccess) return LCQ_ELAUNCH;
+        pending = true;
+      }
+    } else if (o1 < K) {                                                                          // everything behind it
       const float* P = A + (long long)o1 * K + o0;
       launch_gemm<true>(GemmProblem{P, P, A + (long long)o1 * K + o1, K - o1, K - o1, o1 - o0, K, K, K}, -1.0f, 1.0f,
                         GEMM_LOWER_TILES, st);
     }
   }
+  if (pending && hipStreamWaitEvent(st, lane->join, 0) != hipSuccess) return LCQ_ELAUNCH;
 
   if (blocks_only) {
     // No triangular inverse.  With M = J L J (H_d = M M^T, M upper triangular; J reverses the order) the inverse
@@ -636,6 +682,12 @@ static int chol_chain(float* H, int64_t K64, const int64_t* perm, float percdamp
     (void)hipMemcpyAsync(status, &sc->status, sizeof(int), hipMemcpyDeviceToDevice, st);
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;
+}
+
+int lcq_set_chain_lookahead(int on) {
+  const int was = g_lookahead;
+  g_lookahead = on ? 1 : 0;
+  return was;
 }
 
 int lcq_chol_inv_upper(float* H, int64_t K, const int64_t* perm, float percdamp, float* W, int64_t R, float* U,

@@ -146,3 +146,42 @@ def test_gptq_4096_linear_against_cpu_oracle(dev):
         return float(((D @ Hd) * D).sum())
     l, lo = recon(codes, s, z), recon(codes_o, ref['scales'], ref['zeros'])
     assert abs(l - lo) <= 0.01 * lo, (l, lo)
+
+
+@pytest.mark.parametrize('entry', ['lcq_chol_inv_upper', 'lcq_chol_block_factor'])
+def test_chain_lookahead_changes_nothing(dev, entry):
+    """Chains of K >= 8192 run the far part of every deep trailing update on a second stream beside the next
+    super-panel (lcq_set_chain_lookahead, default on).  The factor is the one-stream factor up to fp32 rounding (a part
+    of an update may take the other GEMM kernel than the whole would), it is reproducible bit for bit from run to run
+    and from stream to stream (no race between the two streams), and the caller's stream is where it is ready."""
+    from lightcompress_amd import _lib as L
+    K = 8192
+    g = torch.Generator(device=dev)
+    g.manual_seed(3)
+    X = torch.randn(2 * K, K, device=dev, generator=g) * torch.exp(0.5 * torch.randn(K, device=dev, generator=g))
+    H = (X.t() @ X) / K
+    del X
+    lib = L.lib()
+    nbytes = lib.lcq_chol_inv_upper_workspace_bytes(L.i64(K))
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    status = torch.ones(1, dtype=torch.int32, device=dev)
+    outs = []
+    side = torch.cuda.Stream(device=dev)
+    try:
+        for on, stream in ((0, None), (1, None), (1, side), (1, None)):
+            lib.lcq_set_chain_lookahead(L.i32(on))
+            Hc, U = H.clone(), torch.empty(K, K, device=dev)
+            torch.cuda.synchronize()
+            with torch.cuda.stream(stream if stream is not None else torch.cuda.current_stream()):
+                L.check(getattr(lib, entry)(L.ptr(Hc), L.i64(K), L.ptr(None), L.f32(0.01), L.ptr(None), L.i64(0), L.ptr(U),
+                                            L.ptr(ws), L.i64(nbytes), L.ptr(status), L.stream()), entry)
+                total = U.sum()                           # queued behind the call on the same stream: must see all of U
+            torch.cuda.synchronize()
+            assert int(status.item()) == 0
+            assert float(total) == float(U.sum())
+            outs.append(U)
+    finally:
+        assert lib.lcq_set_chain_lookahead(L.i32(1)) in (0, 1)
+    assert torch.equal(outs[1], outs[2]) and torch.equal(outs[1], outs[3])
+    rel = float((outs[0].double() - outs[1].double()).abs().max() / outs[0].abs().max())
+    assert rel < 1e-5, rel
