@@ -206,6 +206,10 @@ def bench_hessian(args, out, x=None):
         L.check(lib.lcq_hessian_accum(L.ptr(H), L.i64(K), L.ptr(x[b]), L.i32(L.BF16), L.i64(TL), L.i64(K), L.f32(0.5),
                                       L.f32(0.01), st), 'hessian')
     t_h = timeit(hess, 32, 16)
+    # the vendor library on the same operands, for scale: the full product X^T X as one bf16 GEMM through torch
+    # (hipBLASLt; bf16 output, no accumulation into H), same token-major layout of both operands
+    xl = [x[b * FOLD:(b + 1) * FOLD].reshape(TL, K) for b in range(nb // FOLD)]
+    t_lib = timeit(lambda i: torch.matmul(xl[i % len(xl)].t(), xl[i % len(xl)]), 8, 3)
     alg_flops = 2.0 * TL * K * K
     tiles = sum(K // 128 - 2 * ti for ti in range(K // 256))          # 256x128 tiles that reach the upper triangle
     exe_flops = 2.0 * TL * tiles * 256 * 128
@@ -215,6 +219,9 @@ def bench_hessian(args, out, x=None):
         'traffic': traffic_bytes('hessian_kernel_K14336_T8192') if FOLD == 4 else None,
         'launch_us': round(t_h * 1e6, 2), 'flop_executed_per_launch': exe_flops,
         'algorithmic_tflops': round(alg_flops / t_h / 1e12, 2), 'frac_algorithmic': round(alg_flops / t_h / 2.5e15, 4),
+        'library_gemm': {'what': 'torch.matmul(X.t(), X), bf16, the whole K x K product on the same tokens (hipBLASLt)',
+                         'us': round(t_lib * 1e6, 1), 'tflops': round(alg_flops / t_lib / 1e12, 1),
+                         'frac': round(alg_flops / t_lib / 2.5e15, 4)},
         'note': 'achieved / frac count the flops the matrix pipes execute (the 256x128 tiles that reach the upper '
                 'triangle of the symmetric H: matrix-pipe utilisation against the 2.4 GHz peak); the algorithmic figure '
                 '2*T*K^2 of the full product X^T X per launch is in algorithmic_tflops / frac_algorithmic.  rocprofv3 '
