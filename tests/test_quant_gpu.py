@@ -297,6 +297,30 @@ def test_fused_quant_pack_equals_quant_then_pack(dev, dtype, gran, shape):
     assert_bit_equal(fused, opacked, 'oracle pack')
 
 
+@pytest.mark.parametrize('scale', [1.0, 0.5, 0.015625, 4.0])
+def test_fused_quant_pack_on_rounding_ties_and_clamp_bounds(dev, scale):
+    """The one-pass bf16 quantize + pack takes its nibbles from the biased quotient (t + 1.5 * 2^23): every half-integer
+    quotient (ties go to the even code), both clamp bounds, zeros of both signs, and values just beside the ties."""
+    from lightcompress_amd import IntegerQuantizer
+    from lightcompress_amd.module_utils import VllmRealQuantLinear
+    halves = torch.arange(-19, 20, dtype=torch.float32) * 0.5            # -9.5 .. 9.5 in steps of 0.5
+    near = torch.cat([halves + 0.0625, halves - 0.0625])
+    vals = torch.cat([halves, near, torch.tensor([0.0, -0.0, 7.0, -7.0, -8.0, 6.9375])])
+    vals = vals[vals.abs() <= 7.0]                                        # the row maximum fixes the scale: 7 * scale / 7
+    row = torch.zeros(128)
+    row[:vals.numel()] = vals
+    row[-1] = 7.0
+    w = (torch.stack([row, -row, row.flip(0), row * 0.5]) * scale).bfloat16()
+    assert torch.equal(w[0].float(), row * scale)                         # every value is a bf16 number
+    q = IntegerQuantizer(4, True, 'per_group', group_size=128)
+    spec = Q.IntSpec(4, True, 'per_group', group_size=128)
+    fused, fs16 = VllmRealQuantLinear.quant_pack_fused(w.to(dev), q, {'weight': {'bit': 4}})
+    ocodes, os_, _ = Q.int_real_quant_dynamic(spec, w)
+    assert float(os_[0]) == scale and int(ocodes.min()) >= -8 and int(ocodes.max()) == 7
+    opacked, _ = pack_ref.pack_ct(ocodes, os_, 4)
+    assert_bit_equal(fused, opacked, 'packed words on ties')
+
+
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize('shape', [(64, 256), (320, 1024), (2048, 512)])
 def test_gemm_pack_bit_exact(dev, dtype, shape):
