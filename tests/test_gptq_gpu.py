@@ -885,3 +885,52 @@ def test_split_gemm_has_fp32_accuracy(dev):
         assert float((Us[0] - Us[1]).abs().max() / Us[0].abs().max()) < 1e-5
     finally:
         lib.lcq_set_gemm_split(L.i32(1))
+
+
+@pytest.mark.parametrize('sym', [False, True])
+def test_groups_view_and_ready(dev, sym):
+    """`groups` is the reference's list of per-group dicts (gptq.py:358-366, 385-395): entry i holds the [R, 1]
+    scale / zero of group i, and stacking them the way update_model_qparams does (:397-409) gives the layer's
+    buffers.  `ready` (gptq.py:473-477) is False until something fills `qparams['scale']`."""
+    R, K, g = 24, 384, 128
+    gp = make_gptq(weight=dict(bit=4, symmetric=sym, granularity='per_group', group_size=g))
+    layer = linear((torch.randn(R, K, generator=gen(77)) * 0.02).bfloat16().to(dev))
+    gp.collect_layer_qparams(layer)
+    gp.layer_init(layer, 'l')
+    for b in calib_batches(3, 96, K, seed=78):
+        gp.add_batch(layer, 'l', b.bfloat16().to(dev))
+    gp.layer_transform(layer, 'l')
+    assert gp.ready() is False
+    groups = gp.groups
+    assert len(groups) == K // g
+    for d in groups:
+        assert d['scale'].shape == (R, 1) and d['qmax'] == gp.wquantizer.qmax and d['qmin'] == gp.wquantizer.qmin
+    stacked = torch.stack([d['scale'] for d in groups], dim=1).reshape(-1, 1)
+    assert torch.equal(stacked, layer.buf_scales)
+    if sym:
+        assert all(float(d['zero']) == 0.0 for d in groups)
+    else:
+        assert torch.equal(torch.stack([d['zero'] for d in groups], dim=1).reshape(-1, 1), layer.buf_zeros)
+    gp.qparams['scale'] = layer.buf_scales
+    assert bool(gp.ready()) == bool(torch.all(layer.buf_scales != 0))
+
+
+def test_indefinite_hessian_raises_unless_the_check_is_off(dev):
+    """gptq.py:172: torch.linalg.cholesky raises on a matrix that is not positive-definite; here the chain's status
+    word is read before the weights are written back.  `check_positive_definite: False` skips the read."""
+    R, K = 16, 256
+    for check in (True, False):
+        gp = make_gptq(check_positive_definite=check, weight=dict(bit=4, symmetric=False, granularity='per_group', group_size=128))
+        W0 = (torch.randn(R, K, generator=gen(79)) * 0.02).bfloat16().to(dev)
+        layer = linear(W0.clone())
+        gp.collect_layer_qparams(layer)
+        gp.layer_init(layer, 'l')
+        gp.add_batch(layer, 'l', torch.randn(64, K, generator=gen(80)).bfloat16().to(dev))
+        H = gp.hessian('l')
+        H.neg_()                                         # negative definite: the first pivot fails
+        if check:
+            with pytest.raises(torch.linalg.LinAlgError):
+                gp.layer_transform(layer, 'l')
+            assert torch.equal(layer.weight.data, W0)    # nothing was written back
+        else:
+            gp.layer_transform(layer, 'l')
