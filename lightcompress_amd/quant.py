@@ -659,7 +659,9 @@ class IntegerQuantizer(BaseQuantizer):
         return self.restore_tensor(dq.view(rows_t.shape), shape).to(dtype)
 
     def fake_quant_act_static(self, act, args={}):
-        """quant.py:718-751."""
+        """quant.py:718-751.  `args['current_bit']` is accepted and changes nothing, as in the reference: it swaps
+        `self.bit` for the duration of the call (:725-727, :742-743), which no arithmetic reads (qmin / qmax are
+        fixed at construction and the given ones are used here)."""
         if 'int_indices' in args:
             q_act = act[:, :, args['int_indices']]
             fp_act = act[:, :, args['fp_indices']]

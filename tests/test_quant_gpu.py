@@ -623,3 +623,44 @@ def test_stream_probe_reads_everything_and_refuses_a_short_destination(dev, m):
     out.zero_()
     L.check(L.lib().lcq_stream_probe(L.ptr(sd), L.ptr(out), L.i64(nbytes), L.i64(out.numel() * 4), L.i32(0), L.stream()), 'probe')
     assert int(out.abs().sum()) == 0
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+def test_int_static_activation_fake_quant_plain_and_mixed_precision(dev, dtype):
+    """fake_quant_act_static (quant.py:718-751) with parameters calibrated beforehand: the whole tensor, and the
+    mixed-precision form in which `int_indices` columns are quantized and `fp_indices` columns pass through."""
+    act = (torch.randn(3, 40, 256, generator=gen(901)) * 2).to(dtype)
+    spec = Q.IntSpec(8, True, 'per_tensor')
+    q = _iq(8, True, 'per_tensor')
+    calib = (torch.randn(3, 40, 256, generator=gen(902)) * 2).to(dtype)
+    _, s, z, qmax, qmin = Q.int_tensor_qparams(spec, calib)
+    args = dict(scales=s.to(dev), zeros=z.to(dev) if torch.is_tensor(z) else z, qmax=qmax, qmin=qmin, current_bit=4)
+    got = q.fake_quant_act_static(act.to(dev), dict(args))
+    want = Q.int_fake_quant_static(spec, act, s, z, qmax, qmin)
+    assert_bit_equal(got, want, 'fake_quant_act_static')
+    assert q.bit == 8
+    perm = torch.randperm(256, generator=gen(903))
+    ii, fi = perm[:192].sort().values, perm[192:].sort().values
+    mixed = q.fake_quant_act_static(act.to(dev), dict(args, int_indices=ii.to(dev), fp_indices=fi.to(dev)))
+    want_q = Q.int_fake_quant_static(spec, act[:, :, ii].contiguous(), s, z, qmax, qmin)
+    assert_bit_equal(mixed[:, :, ii.to(dev)], want_q, 'quantized columns')
+    assert_bit_equal(mixed[:, :, fi.to(dev)], act[:, :, fi], 'columns kept in floating point')
+
+
+def test_mixed_precision_indices_in_the_dynamic_paths(dev):
+    """`int_indices` / `fp_indices` (quant.py:753-782 activations, :832-868 weights): the named columns are quantized
+    as a tensor of their own, the others pass through."""
+    act = (torch.randn(2, 24, 384, generator=gen(911)) * 2).bfloat16()
+    perm = torch.randperm(384, generator=gen(912))
+    ii, fi = perm[:256].sort().values, perm[256:].sort().values
+    aq = _iq(8, True, 'per_token')
+    mixed = aq.fake_quant_act_dynamic(act.to(dev), dict(int_indices=ii.to(dev), fp_indices=fi.to(dev)))
+    want = Q.int_fake_quant_dynamic(Q.IntSpec(8, True, 'per_token'), act[:, :, ii].contiguous())
+    assert_bit_equal(mixed[:, :, ii.to(dev)], want, 'quantized activation columns')
+    assert_bit_equal(mixed[:, :, fi.to(dev)], act[:, :, fi], 'activation columns kept')
+    w = weight_like(64, 384, seed=913, dtype=torch.bfloat16)
+    wq = _iq(4, False, 'per_group', group_size=128)
+    mixed = wq.fake_quant_weight_dynamic(w.to(dev), dict(int_indices=ii.to(dev), fp_indices=fi.to(dev)))
+    want = Q.int_fake_quant_dynamic(Q.IntSpec(4, False, 'per_group', group_size=128), w[:, ii].contiguous())
+    assert_bit_equal(mixed[:, ii.to(dev)], want, 'quantized weight columns')
+    assert_bit_equal(mixed[:, fi.to(dev)], w[:, fi], 'weight columns kept')
