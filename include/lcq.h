@@ -204,6 +204,20 @@ int lcq_hessian_accum_ab(float* H, int64_t K, const void* XA, const void* XB, in
 /* x [n] fp32 -> hi = bf16(x), lo = bf16(x - hi)  ([n] bf16 each; n % 4 == 0): x == hi + lo to 2^-17 relative. */
 int lcq_split_f32_bf16(const float* x, int64_t n, void* hi, void* lo, void* stream);
 
+/* The same update with the tokens cut into `slices` contiguous shares (whole 32-token slabs, dealt out evenly), share
+ * s accumulating into its own matrix H + s * slice_stride (elements; >= K*K):
+ *   H_s <- alpha*H_s + beta * XA_s^T XB_s   for every s < slices (a share without tokens only scales its matrix),
+ * so the sum over s of the H_s follows the recurrence of gptq.py:279-294 like a single H does.  For Linears whose
+ * Hessian has too few tiles to fill the chip (272 at K = 4096 against 512 workgroup slots) three shares are ~17 %
+ * faster than one.  slices in 1..64; slices == 1 is lcq_hessian_accum_ab.  Matrices start zeroed (or alpha == 0). */
+int lcq_hessian_accum_sliced(float* H, int64_t K, const void* XA, const void* XB, int dtype, int64_t T, int64_t ldx,
+                             float alpha, float beta, int slices, int64_t slice_stride, void* stream);
+
+/* H_0 <- ((H_0 + H_1) + H_2) + ... and H_s <- 0 for s >= 1, over all K*K entries: the shares of
+ * lcq_hessian_accum_sliced back into the one matrix that gptq.py keeps (layers_cache[name]['H']); accumulation may
+ * go on afterwards.  H 16-byte aligned, slice_stride % 4 == 0. */
+int lcq_hessian_gather_slices(float* H, int64_t K, int slices, int64_t slice_stride, void* stream);
+
 /* The staging copy of GPTQ.add_batch (gptq.py:283-290 consumes `inp` at once; here the tokens of several calls are
  * kept until one folded Hessian launch): dst[0 .. bytes) = src[0 .. bytes), both 16-byte aligned, bytes % 16 == 0. */
 int lcq_stage_copy(const void* src, void* dst, int64_t bytes, void* stream);

@@ -111,7 +111,7 @@ template <int TN> struct HessCfg {
 template <bool IS_BF16, bool EDGE, int TN>
 __global__ __launch_bounds__(HessCfg<TN>::NW * 64, TN == 256 ? 1 : 2)
 void hessian_kernel(float* __restrict__ H, int K, const uint16_t* __restrict__ X, const uint16_t* __restrict__ XB, int ldx,
-                    int T, float alpha, float beta, int ntr, int ntc, int total) {
+                    int T, float alpha, float beta, int ntr, int ntc, int total, int slices, long long hstride) {
   using C = HessCfg<TN>;
   constexpr int ROW_B = C::ROW_B, STAGE = C::STAGE, NSTAGE = C::NSTAGE, LA = C::LA, LB = C::LB, RB = C::RB;
   __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE];
@@ -120,7 +120,23 @@ void hessian_kernel(float* __restrict__ H, int K, const uint16_t* __restrict__ X
     const int per_xcd = (total + 7) / 8;
     const int slot = blockIdx.x >> 3, xcd = blockIdx.x & 7;
     if (slot >= per_xcd || xcd * per_xcd + slot >= total) return;
-    decode_tile<TM / TN>(xcd * per_xcd + slot, ntr, ntc, ti, tj);
+    int v = xcd * per_xcd + slot;
+    if (slices > 1) {
+      // Token slices: `total` counts every tile once per slice.  Slice s takes an even share of the 32-token slabs,
+      // [s n / S, (s + 1) n / S), and its own accumulator H + s * hstride, so a launch with too few tiles for the
+      // chip (272 at K = 4096 for 512 workgroup slots) still puts two workgroups on every CU.  A slice without
+      // tokens only scales its accumulator by alpha.
+      const int tiles = total / slices, slice = v / tiles;
+      v -= slice * tiles;
+      const long long n32 = (T + BT - 1) / BT;
+      const int t0 = (int)(slice * n32 / slices) * BT;
+      const int t1 = min((int)((slice + 1) * n32 / slices) * BT, T);
+      X += (int64_t)t0 * ldx;
+      XB += (int64_t)t0 * ldx;
+      H += slice * hstride;
+      T = max(t1 - t0, 0);
+    }
+    decode_tile<TM / TN>(v, ntr, ntc, ti, tj);
   }
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -279,6 +295,20 @@ void hessian_kernel(float* __restrict__ H, int K, const uint16_t* __restrict__ X
   }
 }
 
+// H_0 <- ((H_0 + H_1) + H_2) + ..., H_s <- 0 for s >= 1: the token slices of lcq_hessian_accum_sliced back into one matrix,
+// always in this order.
+__global__ __launch_bounds__(256) void gather_slices_kernel(f32x4* __restrict__ H, int64_t n4, int slices, int64_t stride4) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (int64_t)gridDim.x * 256) {
+    f32x4 v = H[i];
+    for (int s = 1; s < slices; ++s) {
+      const f32x4 w = H[s * stride4 + i];
+      v[0] += w[0]; v[1] += w[1]; v[2] += w[2]; v[3] += w[3];
+      H[s * stride4 + i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    H[i] = v;
+  }
+}
+
 // x (fp32) -> hi = bf16(x), lo = bf16(x - hi): x = hi + lo up to 2^-17 relative, and every product of two such
 // halves is exact in fp32, so fp32 activations go through the bf16 matrix pipe as four products (hi/lo x hi/lo).
 __global__ __launch_bounds__(256) void split_f32_kernel(const f32x4* __restrict__ x, int64_t n4, u32x2* __restrict__ hi,
@@ -335,28 +365,50 @@ extern "C" {
 
 int lcq_hessian_accum(float* H, int64_t K, const void* X, int dtype, int64_t T, int64_t ldx, float alpha, float beta,
                       void* stream) {
-  return lcq_hessian_accum_ab(H, K, X, X, dtype, T, ldx, alpha, beta, stream);
+  return lcq_hessian_accum_sliced(H, K, X, X, dtype, T, ldx, alpha, beta, 1, 0, stream);
 }
 
 int lcq_hessian_accum_ab(float* H, int64_t K, const void* X, const void* XB, int dtype, int64_t T, int64_t ldx, float alpha,
                          float beta, void* stream) {
+  return lcq_hessian_accum_sliced(H, K, X, XB, dtype, T, ldx, alpha, beta, 1, 0, stream);
+}
+
+int lcq_hessian_accum_sliced(float* H, int64_t K, const void* X, const void* XB, int dtype, int64_t T, int64_t ldx,
+                             float alpha, float beta, int slices, int64_t slice_stride, void* stream) {
   if (!H || !X || !XB || K <= 0 || T < 0) return LCQ_EINVAL;
   if (K % 8 != 0 || K > (1 << 20) || T > 0x7fffffff || ldx < K || ldx % 8 != 0 || ldx > (1 << 21)) return LCQ_EINVAL;
+  if (slices < 1 || slices > 64 || (slices > 1 && slice_stride < K * K)) return LCQ_EINVAL;
   if (((uintptr_t)X % 16) != 0 || ((uintptr_t)XB % 16) != 0 || ((uintptr_t)H % 4) != 0) return LCQ_EALIGN;
   if (T == 0) return LCQ_OK;
   constexpr int TN = 128;
   const int ntr = (int)((K + TM - 1) / TM), ntc = (int)((K + TN - 1) / TN), q = TM / TN;
   int64_t total = 0;
   for (int r = 0; r < ntr; ++r) total += (ntc - q * r > 0) ? (ntc - q * r) : 0;
+  total *= slices;
+  if (total > 0x7ffffff0) return LCQ_ESIZE;
   const int64_t grid = (total + 7) / 8 * 8;                       // 8 XCD queues of equal length
   hipStream_t st = (hipStream_t)stream;
   const bool edge = (K % TM != 0) || (T % BT != 0);
   #define LCQ_HESS(BF, E) hessian_kernel<BF, E, TN><<<dim3((unsigned)grid), dim3(HessCfg<TN>::NW * 64), 0, st>>>( \
-      H, (int)K, (const uint16_t*)X, (const uint16_t*)XB, (int)ldx, (int)T, alpha, beta, ntr, ntc, (int)total)
+      H, (int)K, (const uint16_t*)X, (const uint16_t*)XB, (int)ldx, (int)T, alpha, beta, ntr, ntc, (int)total, slices, \
+      (long long)slice_stride)
   if (dtype == LCQ_BF16) { if (edge) LCQ_HESS(true, true); else LCQ_HESS(true, false); }
   else if (dtype == LCQ_F16) { if (edge) LCQ_HESS(false, true); else LCQ_HESS(false, false); }
   else return LCQ_EDTYPE;
   #undef LCQ_HESS
+  LCQ_CHECK_LAUNCH();
+  return LCQ_OK;
+}
+
+int lcq_hessian_gather_slices(float* H, int64_t K, int slices, int64_t slice_stride, void* stream) {
+  if (!H || K <= 0 || K % 8 != 0 || slices < 1 || slices > 64 || (slices > 1 && slice_stride < K * K) || slice_stride % 4 != 0)
+    return LCQ_EINVAL;
+  if (((uintptr_t)H % 16) != 0) return LCQ_EALIGN;
+  if (slices == 1) return LCQ_OK;
+  const int64_t n4 = K * K / 4;
+  int64_t grid = (n4 + 255) / 256;
+  if (grid > 8192) grid = 8192;
+  gather_slices_kernel<<<dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream>>>((f32x4*)H, n4, slices, slice_stride / 4);
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;
 }

@@ -31,6 +31,9 @@ Differences a caller can observe
     folded into one launch, so ``layers_cache[name]['H']`` lags behind ``nsamples`` until
     ``hessian(name)``, ``hessian_sorting`` or ``process_hessian_and_weights`` settles it
     (``hessian_defer: 1`` updates H on every call);
+  * ``special.hessian_slices`` (default 'auto': 3 at K = 4096, 1 at K = 14336): a launch whose Hessian has too few
+    tiles to fill the chip cuts its tokens into that many shares, each with an accumulator of its own; the same
+    calls settle them into H (a sum in a fixed order; H differs from a single accumulator's by fp32 rounding);
   * per-group qparams of the loop live in two [R, G] tensors instead of a
     Python list of dicts; ``layer.buf_scales`` / ``buf_zeros`` get the same
     [R*G, 1] layout the reference writes;
@@ -82,6 +85,9 @@ class GPTQ:
         # add_batch calls folded into one Hessian launch (1 = one launch per call)
         hd = special_config.get('hessian_defer', 'auto')
         self.hessian_defer = hd if hd == 'auto' else int(hd)
+        # token shares of one Hessian launch, each with an accumulator of its own ('auto': by the number of tiles)
+        hs = special_config.get('hessian_slices', 'auto')
+        self.hessian_slices = hs if hs == 'auto' else int(hs)
         # subset_transform starts the Cholesky chains of all Linears of a subset side by side (False: one by one)
         self.chain_overlap = bool(special_config.get('chain_overlap', True))
         self.fuse_loops = bool(special_config.get('fuse_loops', True))
@@ -113,7 +119,11 @@ class GPTQ:
         W = layer.weight.data
         K = W.shape[1] if W.dim() == 2 else W.flatten(1).shape[1]
         self.layers_cache.setdefault(name, {})
-        self.layers_cache[name]['H'] = torch.zeros((K, K), device=self.dev)
+        slices = self.hessian_shares(K)
+        acc = torch.zeros((slices, K, K), device=self.dev)
+        self.layers_cache[name]['H'] = acc[0]
+        self.layers_cache[name]['H_shares'] = acc if slices > 1 else None
+        self.layers_cache[name]['shares_apart'] = False
         self.layers_cache[name]['nsamples'] = 0
         self.layers_cache[name]['n_in_H'] = 0
         self.layers_cache[name]['calls'] = 0
@@ -135,6 +145,7 @@ class GPTQ:
         leader = names[0]
         for n in names[1:]:
             self.layers_cache[n]['H'] = self.layers_cache[leader]['H']
+            self.layers_cache[n]['H_shares'] = None
             self.layers_cache[n]['leader'] = leader
             self.layers_cache[n]['manual_share'] = True
         self.layers_cache[leader]['leader'] = leader
@@ -172,6 +183,7 @@ class GPTQ:
                     and oc['H'].shape == cache['H'].shape:
                 cache['leader'] = other
                 cache['H'] = oc['H']
+                cache['H_shares'] = None
                 oc['leader'] = other
                 return True
         return False
@@ -191,7 +203,13 @@ class GPTQ:
                 raise L.LcqError(f'{name}: the input differs from the one of {lead.get("leader")} after a call that was '
                                  'folded into the shared Hessian directly; set special.auto_share: False')
             fill, batches = fill - t_last, batches - b_last
-        cache['H'] = lead['H'].clone()
+        if lead.get('H_shares') is not None:              # every share as it is: the same state, nothing summed early
+            cache['H_shares'] = lead['H_shares'].clone()
+            cache['H'] = cache['H_shares'][0]
+        else:
+            cache['H_shares'] = None
+            cache['H'] = lead['H'].clone()
+        cache['shares_apart'] = lead.get('shares_apart', False)
         cache['n_in_H'] = lead.get('n_in_H', 0)
         cache['upper_only'] = lead.get('upper_only', False)
         for k in ('stage', 'stage_lo', 'stage_fill', 'stage_batches', 'last_stage'):
@@ -288,6 +306,29 @@ class GPTQ:
             return 16 if K <= 4096 else (8 if K <= 8192 else 4)
         return self.hessian_defer
 
+    def hessian_shares(self, K):
+        """Token shares of one Hessian launch for K input features (lcq_hessian_accum_sliced).  A launch has one
+        workgroup per 256 x 128 tile that reaches the upper triangle and the chip has 512 workgroup slots: K = 4096
+        gives 272 tiles, one workgroup on most CUs, whose four waves cannot hide their own latencies.  Cutting the
+        tokens of the launch into three shares with an accumulator each puts 816 workgroups on the chip; the
+        accumulators are summed when H is asked for.  'auto' follows what was measured on 128 calls of 2048 tokens
+        (ms, one share -> best count): K=1024 4.4 -> 1.6 (8), 2048 4.6 -> 2.0 (5), 3072 5.0 -> 3.3 (3), 4096 5.8 -> 5.1
+        (3), 6144 11.9 -> 10.6 (2), 8192 18.6 -> 17.6 (2); one share is best at K = 5120, 7168, 11008, 14336 (every
+        share reads and writes its accumulator once per launch)."""
+        if self.hessian_slices != 'auto':
+            return max(1, self.hessian_slices)
+        ntr, ntc = (K + 255) // 256, (K + 127) // 128
+        tiles = sum(max(ntc - 2 * r, 0) for r in range(ntr))
+        if tiles <= 40:
+            return 8
+        if tiles <= 100:
+            return 5
+        if tiles <= 300:
+            return 3
+        if 512 < tiles < 1536 and tiles % 512 < 128:      # a round or two of workgroups and a small rest
+            return 2
+        return 1
+
     def _halves(self, x, hi=None, lo=None):
         """(x, None) for 16-bit activations; for fp32 the two bf16 halves hi = bf16(x), lo = bf16(x - hi)."""
         if x.dtype != torch.float32:
@@ -306,15 +347,18 @@ class GPTQ:
         beta = 2.0 / (n + batches)
         cache['n_in_H'] = n + batches
         H = cache['H']
+        shares = cache.get('H_shares')
+        sl = (L.i32(1), L.i64(0)) if shares is None else (L.i32(shares.shape[0]), L.i64(shares.stride(0)))
+        cache['shares_apart'] = shares is not None
         lib, code = L.lib(), L.i32(L.dtype_code(x.dtype))
         dims = (L.i64(x.shape[0]), L.i64(x.stride(0)))
         if x_lo is None:
-            L.check(lib.lcq_hessian_accum(L.ptr(H), L.i64(H.shape[0]), L.ptr(x), code, *dims, L.f32(alpha), L.f32(beta),
-                                          L.stream()), 'lcq_hessian_accum')
+            L.check(lib.lcq_hessian_accum_sliced(L.ptr(H), L.i64(H.shape[0]), L.ptr(x), L.ptr(x), code, *dims, L.f32(alpha),
+                                                 L.f32(beta), *sl, L.stream()), 'lcq_hessian_accum_sliced')
             return
         for a, b, al in ((x_lo, x_lo, alpha), (x, x_lo, 1.0), (x_lo, x, 1.0), (x, x, 1.0)):      # small terms first
-            L.check(lib.lcq_hessian_accum_ab(L.ptr(H), L.i64(H.shape[0]), L.ptr(a), L.ptr(b), code, *dims, L.f32(al),
-                                             L.f32(beta), L.stream()), 'lcq_hessian_accum_ab')
+            L.check(lib.lcq_hessian_accum_sliced(L.ptr(H), L.i64(H.shape[0]), L.ptr(a), L.ptr(b), code, *dims, L.f32(al),
+                                                 L.f32(beta), *sl, L.stream()), 'lcq_hessian_accum_sliced')
 
     def _flush(self, cache):
         """Fold the staged tokens into H."""
@@ -333,6 +377,11 @@ class GPTQ:
         self._flush(lead)
         lead.pop('stage', None)
         lead.pop('stage_lo', None)
+        if lead.get('shares_apart'):                      # the token shares of the launches back into the one H
+            sh = lead['H_shares']
+            L.check(L.lib().lcq_hessian_gather_slices(L.ptr(sh), L.i64(sh.shape[1]), L.i32(sh.shape[0]), L.i64(sh.stride(0)),
+                                                      L.stream()), 'lcq_hessian_gather_slices')
+            lead['shares_apart'] = False
         return cache
 
     def hessian(self, name):
@@ -506,6 +555,7 @@ class GPTQ:
         leader = cache.get('leader', name)
         H = cache['H']
         del cache['H']
+        cache.pop('H_shares', None)
 
         self._setup_groups(layer, R, K)
 

@@ -59,6 +59,39 @@ def test_hessian_within_1e5(dev, K, T, nb):
     assert torch.equal(H, H.t())
 
 
+@pytest.mark.parametrize('K,T,slices', [(512, 1000, 3), (1000, 333, 5), (256, 40, 8), (4096, 416, 3)])
+def test_hessian_token_shares_sum_to_the_single_accumulator(dev, K, T, slices):
+    """lcq_hessian_accum_sliced: the tokens of a launch in `slices` shares with an accumulator each, two launches with
+    the recurrence's alpha / beta, then lcq_hessian_gather_slices: the sum equals what one accumulator holds (up to
+    the order of fp32 additions) and the closed form in fp64; the other accumulators come back zeroed.  (256, 40, 8)
+    leaves six shares without tokens: they only scale."""
+    from lightcompress_amd import _lib as L
+    lib = L.lib()
+    xs = [(torch.randn(T, K, generator=gen(1300 + i)) * (1 + i)).bfloat16() for i in range(2)]
+    xd = [x.to(dev) for x in xs]
+    one = torch.zeros(K, K, device=dev)
+    acc = torch.zeros(slices, K, K, device=dev)
+    for i, (al, be) in enumerate(((0.0, 2.0), (0.5, 1.0))):
+        L.check(lib.lcq_hessian_accum(L.ptr(one), L.i64(K), L.ptr(xd[i]), L.i32(L.BF16), L.i64(T), L.i64(K), L.f32(al), L.f32(be),
+                                      L.stream()), 'one')
+        L.check(lib.lcq_hessian_accum_sliced(L.ptr(acc), L.i64(K), L.ptr(xd[i]), L.ptr(xd[i]), L.i32(L.BF16), L.i64(T), L.i64(K),
+                                             L.f32(al), L.f32(be), L.i32(slices), L.i64(K * K), L.stream()), 'sliced')
+    assert int((acc[1:] != 0).any(dim=2).any(dim=1).sum()) >= min(slices - 1, (T + 31) // 32 - 1)    # shares really used
+    L.check(lib.lcq_hessian_gather_slices(L.ptr(acc), L.i64(K), L.i32(slices), L.i64(K * K), L.stream()), 'gather')
+    assert not bool(acc[1:].any())
+    up = torch.triu(torch.ones(K, K, dtype=torch.bool))
+    got, want = acc[0].cpu(), one.cpu()
+    ref = 0.5 * 2.0 * xs[0].double().t() @ xs[0].double() + xs[1].double().t() @ xs[1].double()
+    scale = float(ref.abs().max())
+    assert float((got - want)[up].abs().max()) / scale < 2e-6
+    assert float((got.double() - ref)[up].abs().max()) / scale < 1e-5
+    # refused: a stride that lets the accumulators overlap, a share count out of range
+    assert lib.lcq_hessian_accum_sliced(L.ptr(acc), L.i64(K), L.ptr(xd[0]), L.ptr(xd[0]), L.i32(L.BF16), L.i64(T), L.i64(K),
+                                        L.f32(0.0), L.f32(1.0), L.i32(slices), L.i64(K * K - 8), L.stream()) != 0
+    assert lib.lcq_hessian_accum_sliced(L.ptr(acc), L.i64(K), L.ptr(xd[0]), L.ptr(xd[0]), L.i32(L.BF16), L.i64(T), L.i64(K),
+                                        L.f32(0.0), L.f32(1.0), L.i32(65), L.i64(K * K), L.stream()) != 0
+
+
 def test_hessian_batched_call_and_fp16(dev):
     K = 256
     batches = calib_batches(4, 48, K, seed=1100, dtype=torch.float16)
