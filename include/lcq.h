@@ -209,7 +209,7 @@ int lcq_split_f32_bf16(const float* x, int64_t n, void* hi, void* lo, void* stre
  *   H_s <- alpha*H_s + beta * XA_s^T XB_s   for every s < slices (a share without tokens only scales its matrix),
  * so the sum over s of the H_s follows the recurrence of gptq.py:279-294 like a single H does.  For Linears whose
  * Hessian has too few tiles to fill the chip (272 at K = 4096 against 512 workgroup slots) three shares are ~17 %
- * faster than one.  slices in 1..64; slices == 1 is lcq_hessian_accum_ab.  Matrices start zeroed (or alpha == 0). */
+ * faster than one.  slices in 1..64 (T <= 2^30 when > 1); slices == 1 is lcq_hessian_accum_ab.  Matrices start zeroed (or alpha == 0). */
 int lcq_hessian_accum_sliced(float* H, int64_t K, const void* XA, const void* XB, int dtype, int64_t T, int64_t ldx,
                              float alpha, float beta, int slices, int64_t slice_stride, void* stream);
 

@@ -378,6 +378,7 @@ int lcq_hessian_accum_sliced(float* H, int64_t K, const void* X, const void* XB,
   if (!H || !X || !XB || K <= 0 || T < 0) return LCQ_EINVAL;
   if (K % 8 != 0 || K > (1 << 20) || T > 0x7fffffff || ldx < K || ldx % 8 != 0 || ldx > (1 << 21)) return LCQ_EINVAL;
   if (slices < 1 || slices > 64 || (slices > 1 && slice_stride < K * K)) return LCQ_EINVAL;
+  if (slices > 1 && T > (1 << 30)) return LCQ_ESIZE;               // the kernel's slab arithmetic is 32-bit
   if (((uintptr_t)X % 16) != 0 || ((uintptr_t)XB % 16) != 0 || ((uintptr_t)H % 4) != 0) return LCQ_EALIGN;
   if (T == 0) return LCQ_OK;
   constexpr int TN = 128;
