@@ -300,8 +300,8 @@ class GPTQ:
     def hessian_fold(self, K):
         """add_batch calls folded into one Hessian launch for a Linear with K input features.  'auto': 4 calls of 2048
         tokens at K = 14336 (1.5 ms per launch; longer launches run at a lower sustained clock and are slower per
-        token), 8 up to K = 8192, 16 up to K = 4096 (272 tiles for 512 workgroup slots: the longer the launch, the
-        smaller the share of its ramp and tail; 0.32 -> 0.35 of the matrix peak)."""
+        token), 8 up to K = 8192, 16 up to K = 4096 (the longer the launch, the smaller the share of its ramp and tail,
+        and the more tokens each of its shares gets, see hessian_shares)."""
         if self.hessian_defer == 'auto':
             return 16 if K <= 4096 else (8 if K <= 8192 else 4)
         return self.hessian_defer
