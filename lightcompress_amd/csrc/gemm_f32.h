@@ -55,20 +55,24 @@ __device__ __forceinline__ void gemm_tile(const float* A, int lda, const float* 
                                           float* C, int ldc, int M, int N, int Kc, float alpha, float beta,
                                           int flags, int m0, int n0, float* sA, float* sB) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wr = wave >> 1, wc = wave & 1;
-  constexpr int MI = TM / 64;           // 32-row MFMA blocks per wave (waves are 2 x 2 over the TM x 128 tile)
-  constexpr int WM = TM / 2;            // rows per wave
-  constexpr int AP = TM / 32;           // float4 of the A slab per thread
+  // waves are 2 x 2 over the TM x 128 tile; the 32-row tile puts its four waves side by side, 32 columns each
+  constexpr bool FLAT = TM == 32;
+  const int wr = FLAT ? 0 : wave >> 1, wc = FLAT ? wave : wave & 1;
+  constexpr int MI = FLAT ? 1 : TM / 64;       // 32-row MFMA blocks per wave
+  constexpr int NJ = FLAT ? 1 : 2;             // 32-column MFMA blocks per wave
+  constexpr int WM = FLAT ? 32 : TM / 2;       // rows per wave
+  constexpr int WN = 32 * NJ;                  // columns per wave
+  constexpr int AP = TM / 32;                  // float4 of the A slab per thread
 
   int kb = 0, ke = Kc;
   if (flags & GEMM_K_FROM_N) kb = (n0 / GK) * GK;
   if (flags & GEMM_K_TO_M) ke = min(Kc, m0 + TM);
 
-  f32x16 acc[MI][2];
+  f32x16 acc[MI][NJ];
   #pragma unroll
   for (int i = 0; i < MI; ++i)
     #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < NJ; ++j)
       #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
@@ -149,23 +153,23 @@ __device__ __forceinline__ void gemm_tile(const float* A, int lda, const float* 
   auto compute = [&]() {
     #pragma unroll
     for (int kk = 0; kk < GK; kk += 2) {
-      float a[MI], b[2];
+      float a[MI], b[NJ];
       #pragma unroll
       for (int i = 0; i < MI; ++i) a[i] = sA[(wr * WM + i * 32 + lm) * GPA + kk + lk];
       #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        if constexpr (B_T) b[j] = sB[(wc * 64 + j * 32 + lm) * GPA + kk + lk];
-        else b[j] = sB[(kk + lk) * GPB + wc * 64 + j * 32 + lm];
+      for (int j = 0; j < NJ; ++j) {
+        if constexpr (B_T) b[j] = sB[(wc * WN + j * 32 + lm) * GPA + kk + lk];
+        else b[j] = sB[(kk + lk) * GPB + wc * WN + j * 32 + lm];
       }
       #pragma unroll
       for (int i = 0; i < MI; ++i)
         #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < NJ; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
     }
   };
   using S0 = std::integral_constant<int, 0>;
-  float oldc[DEEP ? MI : 1][2][16];                       // DEEP: the old C values, fetched with the operands
+  float oldc[DEEP ? MI : 1][NJ][16];                       // DEEP: the old C values, fetched with the operands
   if constexpr (DEEP) {
     gload(kb, S0{});
     if (kb + GK < ke) gload(kb + GK, std::integral_constant<int, 1>{});
@@ -175,8 +179,8 @@ __device__ __forceinline__ void gemm_tile(const float* A, int lda, const float* 
       #pragma unroll
       for (int i = 0; i < MI; ++i)
         #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const int gn = n0 + wc * 64 + j * 32 + lm;
+        for (int j = 0; j < NJ; ++j) {
+          const int gn = n0 + wc * WN + j * 32 + lm;
           const int gm0 = m0 + wr * WM + i * 32 + 4 * lk;
           const float* p0 = C + (long long)gm0 * ldc + gn;
           #pragma unroll
@@ -207,8 +211,8 @@ __device__ __forceinline__ void gemm_tile(const float* A, int lda, const float* 
   #pragma unroll
   for (int i = 0; i < MI; ++i)
     #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int gn = n0 + wc * 64 + j * 32 + lm;
+    for (int j = 0; j < NJ; ++j) {
+      const int gn = n0 + wc * WN + j * 32 + lm;
       const int gm0 = m0 + wr * WM + i * 32 + 4 * lk;
       float* p0 = C + (long long)gm0 * ldc + gn;
       float old[16];
@@ -506,7 +510,7 @@ __global__ __launch_bounds__(256, 2) void gemm_s3_batched_kernel(const float* A,
 // 1 (default): launches of more than 256 tiles run on the bf16 matrix pipe (three-way split operands); 0: fp32 pipe only
 extern int g_gemm_split;
 
-// TM = 128 or 64 rows of C per workgroup.  The short tile is for launches that would not give every CU a
+// TM = 128, 64 or 32 rows of C per workgroup.  The short tiles are for launches that would not give every CU a
 // 128-row tile (rank-128 updates and panel solves of the blocked chains): twice the workgroups, half the serial
 // MFMA work in each.
 template <bool B_T, int TM, bool DEEP = false>
@@ -538,6 +542,11 @@ inline void launch_gemm(const GemmProblem& g, float alpha, float beta, int flags
   // its serial chain of slabs, 2.7x shorter there
   if (g_gemm_split && (long long)gx * gy >= 64 && (long long)gx * gy <= 256 && g.Kc >= 256)
     gemm_s3_kernel<B_T><<<dim3(gx, gy), dim3(256), 0, st>>>(g, alpha, beta, flags);
+  // at most 128 of the 64-row tiles: 32-row tiles instead, twice the CUs and half the serial MFMA work in each (a
+  // 64 x 128 tile with a 128-deep contraction is 3.9 us of fp32 MFMA on its CU; K = 4096 chain 2.14 -> 1.99 ms)
+  else if ((long long)gx * ((g.M + 63) / 64) <= 128 && g.Kc > 0 && g.Kc <= 4 * GK &&
+           !(flags & (GEMM_K_FROM_N | GEMM_K_TO_M)))
+    gemm_f32_kernel<B_T, 32, true><<<dim3(gx, (unsigned)((g.M + 31) / 32)), dim3(256), 0, st>>>(g, alpha, beta, flags);
   else if ((long long)gx * gy <= 256 && g.Kc > 0 && g.Kc <= 4 * GK && !(flags & (GEMM_K_FROM_N | GEMM_K_TO_M)))
     gemm_f32_kernel<B_T, 64, true><<<dim3(gx, (unsigned)((g.M + 63) / 64)), dim3(256), 0, st>>>(g, alpha, beta, flags);
   else if ((long long)gx * gy <= 256)
