@@ -92,6 +92,31 @@ def test_hessian_token_shares_sum_to_the_single_accumulator(dev, K, T, slices):
                                         L.f32(0.0), L.f32(1.0), L.i32(65), L.i64(K * K), L.stream()) != 0
 
 
+@pytest.mark.parametrize('slices', [1, 3, 'auto'])
+def test_hessian_shares_through_add_batch_and_reads_in_between(dev, slices):
+    """`special.hessian_slices`: whatever the number of accumulators, reading H in the middle of the calibration
+    (which sums the shares and clears all but the first) and going on afterwards ends at the closed form."""
+    K, T = 512, 160
+    batches = calib_batches(7, T, K, seed=1400)
+    g = make_gptq(hessian_slices=slices, hessian_defer=3)
+    layer = Layer(torch.zeros(8, K, device=dev))
+    g.layers_cache['l'] = {}
+    g.layer_init(layer, 'l')
+    assert (g.layers_cache['l']['H_shares'] is None) == (slices == 1)
+    for i, b in enumerate(batches):
+        g.add_batch(layer, 'l', b.unsqueeze(0).to(dev), None)
+        if i in (1, 4):
+            part = g.hessian('l').cpu().double()
+            ref = G.hessian_closed_form(batches[:i + 1])
+            assert float((part - ref).abs().max() / ref.abs().max()) < 1e-5
+            sh = g.layers_cache['l']['H_shares']
+            assert sh is None or not bool(sh[1:].any())
+    H = g.hessian('l').cpu()
+    ref = G.hessian_closed_form(batches)
+    assert float((H.double() - ref).abs().max() / ref.abs().max()) < 1e-5
+    assert torch.equal(H, H.t())
+
+
 def test_hessian_batched_call_and_fp16(dev):
     K = 256
     batches = calib_batches(4, 48, K, seed=1100, dtype=torch.float16)
