@@ -11,11 +11,24 @@
  *  - every pointer is a DEVICE pointer owned by the caller (a torch tensor's
  *    data_ptr()); `stream` is a hipStream_t passed as void* (NULL = default
  *    stream); calls only enqueue work and return immediately;
- *  - no entry point allocates: scratch memory is a caller-provided workspace
- *    whose size the matching *_workspace_bytes() call returns;
+ *  - no entry point allocates device memory: scratch memory is a
+ *    caller-provided workspace whose size the matching *_workspace_bytes()
+ *    call returns;
  *  - return value: 0 ok, <0 rejected before any launch (LCQ_E*);
  *  - matrices are dense row-major;
- *  - stateless and re-entrant; calls on one stream execute in order.
+ *  - calls on one stream execute in order.  Entry points keep no state between
+ *    calls, with these exceptions, all of them stated again where they apply:
+ *      * lcq_set_gemm_split / lcq_set_chain_lookahead are process-wide
+ *        switches (atomic words, read by every later call);
+ *      * lcq_chol_inv_upper / lcq_chol_block_factor with K >= 8192 and the
+ *        look-ahead switch on create, on first use for a (device, caller's
+ *        stream) pair, one more HIP stream (default priority) and two events,
+ *        and keep them until the process ends; at most 16 such pairs exist,
+ *        later pairs run the chain on the caller's stream alone.  The pair's
+ *        events order the two streams, so ONE host thread at a time may
+ *        submit chains to a given stream (two threads on two streams are
+ *        fine);
+ *      * lcq_sq_err_mean_static uses one scratch array per GPU (below).
  */
 #ifndef LCQ_H
 #define LCQ_H
@@ -190,7 +203,7 @@ int lcq_pack_awq(const void* w, int dtype, const void* scales, const int32_t* ze
  *  H [K, K] fp32; X [T, K] tokens x in_features of LCQ_BF16 | LCQ_F16, 16-byte aligned; K % 8 == 0;
  *  ldx = elements between consecutive token rows (>= K, % 8 == 0).
  * Only the tiles that reach the upper triangle are updated: call lcq_symmetrize before reading
- * anything below the diagonal. alpha == 0 does not read H. */
+ * anything below the diagonal. alpha == 0 does not read H.  T == 0 leaves H <- alpha*H (no launch when alpha == 1). */
 int lcq_hessian_accum(float* H, int64_t K, const void* X, int dtype, int64_t T, int64_t ldx, float alpha, float beta,
                       void* stream);
 
@@ -206,7 +219,7 @@ int lcq_split_f32_bf16(const float* x, int64_t n, void* hi, void* lo, void* stre
 
 /* The same update with the tokens cut into `slices` contiguous shares (whole 32-token slabs, dealt out evenly), share
  * s accumulating into its own matrix H + s * slice_stride (elements; >= K*K):
- *   H_s <- alpha*H_s + beta * XA_s^T XB_s   for every s < slices (a share without tokens only scales its matrix),
+ *   H_s <- alpha*H_s + beta * XA_s^T XB_s   for every s < slices (a share without tokens only scales its matrix; T == 0 scales all of them),
  * so the sum over s of the H_s follows the recurrence of gptq.py:279-294 like a single H does.  For Linears whose
  * Hessian has too few tiles to fill the chip (272 at K = 4096 against 512 workgroup slots) three shares are ~17 %
  * faster than one.  slices in 1..64 (T <= 2^30 when > 1); slices == 1 is lcq_hessian_accum_ab.  Matrices start zeroed (or alpha == 0). */
@@ -218,16 +231,15 @@ int lcq_hessian_accum_sliced(float* H, int64_t K, const void* XA, const void* XB
  * go on afterwards.  H 16-byte aligned, slice_stride % 4 == 0. */
 int lcq_hessian_gather_slices(float* H, int64_t K, int slices, int64_t slice_stride, void* stream);
 
+/* *flag = 1 if a[0 .. bytes) and b[0 .. bytes) differ in any bit; *flag is left alone otherwise (the caller clears it
+ * once and may let several calls report into it).  Both 16-byte aligned, bytes % 16 == 0.  No counterpart in the
+ * reference: GPTQ.add_batch here lets Linears that are handed the same tensor (the hooks of q/k/v, gptq.py:246-251)
+ * share one Hessian, and checks with this call that the tensor still holds what the first Linear saw. */
+int lcq_compare_bytes(const void* a, const void* b, int64_t bytes, int* flag, void* stream);
+
 /* The staging copy of GPTQ.add_batch (gptq.py:283-290 consumes `inp` at once; here the tokens of several calls are
  * kept until one folded Hessian launch): dst[0 .. bytes) = src[0 .. bytes), both 16-byte aligned, bytes % 16 == 0. */
 int lcq_stage_copy(const void* src, void* dst, int64_t bytes, void* stream);
-
-/* No counterpart in the reference: a measurement aid for the benchmark.  Streams `bytes` (a multiple of 16, both
- * pointers 16-byte aligned) from src and writes bytes / reads_per_write to dst (the xor of every reads_per_write
- * consecutive 16-byte chunks of a thread's share); reads_per_write in {1, 2, 4, 8}, or 0 for a read-only pass.
- * dst_bytes is the room behind dst: less than bytes / reads_per_write (4 KiB for a read-only pass) is refused.  The
- * rate is the ceiling of a quantizer kernel with the same mix of reads and writes. */
-int lcq_stream_probe(const void* src, void* dst, int64_t bytes, int64_t dst_bytes, int reads_per_write, void* stream);
 
 /* H[j][i] = H[i][j] for i < j. */
 int lcq_symmetrize(float* H, int64_t K, void* stream);
@@ -243,7 +255,7 @@ int lcq_gptq_prepare_weights(const void* w, int dtype, int64_t R, int64_t K, con
  * the deferred loop update (gptq.py:244) are evaluated.  1 (default): launches of more than 256 output tiles run on
  * the bf16 matrix pipe with every fp32 operand split into three bf16 planes and six partial products per product
  * (accuracy of an fp32 multiply-add, 16/6 of the fp32 pipe's rate); 0: everything on the fp32 matrix pipe.
- * Process-wide; returns the previous setting. */
+ * Process-wide (an atomic word that every later call reads); returns the previous setting. */
 int lcq_set_gemm_split(int on);
 
 /* Chains of K >= 8192: 1 (default) runs the deep trailing update behind a 512-column super-panel in two parts, the
@@ -251,7 +263,10 @@ int lcq_set_gemm_split(int on);
  * (device, caller's stream), beside the next super-panel's narrow launches; the two are ordered by events and joined
  * before the call's last launches, so the caller sees one stream-ordered call.  0: everything on the caller's stream.
  * The results agree to fp32 rounding (a part of an update may select the other GEMM kernel than the whole update
- * would) and are reproducible from run to run either way.  Process-wide; returns the previous setting. */
+ * would) and are reproducible from run to run either way.  Process-wide (an atomic word that every later chain reads
+ * once); returns the previous setting.  The side stream and its two events are created on the first such chain of a
+ * (device, caller's stream) pair and kept until the process ends; 16 pairs at most, further pairs run on the caller's
+ * stream alone; one host thread at a time per caller's stream. */
 int lcq_set_chain_lookahead(int on);
 
 /* Dead columns, act-order permutation, damping and the Cholesky chain of
@@ -337,7 +352,9 @@ int lcq_sq_err_mean(const void* a, const void* b, int dtype, int64_t n, float* o
 /* lcq_sq_err_mean for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses
  * that forbid hipMalloc): same kernels, same result bit for bit, but the partial sums live in a 64 KiB array that is
  * part of the library's device image instead of a caller workspace.  No counterpart in the reference.
- * Calls no hipMalloc / hipFree or other allocating routine; the first call on a device looks the array's address up.
+ * Calls no hipMalloc / hipFree or other allocating routine; the first call on a device looks the array's address up
+ * (hipGetSymbolAddress, under a mutex), which is not a kernel launch: make one call on the device OUTSIDE any stream
+ * capture first; every later call is two kernel launches and nothing else, and may be captured.
  *  n <= LCQ_SQ_ERR_STATIC_MAX_N, else LCQ_ESIZE.
  * Every call on one GPU uses that GPU's single array: calls that overlap on one GPU (different streams) race;
  * calls on one stream, or ordered by events, are safe.  Nothing needs clearing between calls. */

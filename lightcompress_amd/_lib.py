@@ -34,10 +34,12 @@ _lib = None
 
 
 def declared_symbols() -> list[str]:
-    """Names of every function include/lcq.h declares."""
-    text = HEADER.read_text()
-    text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
-    return sorted(set(re.findall(r'\b(lcq_[a-z0-9_]+)\s*\(', text)))
+    """Names of every function the headers under include/ declare (lcq.h: the boundary; lcq_bench.h: benchmark aids)."""
+    names = set()
+    for header in sorted(HEADER.parent.glob('*.h')):
+        text = re.sub(r'/\*.*?\*/', '', header.read_text(), flags=re.S)
+        names.update(re.findall(r'\b(lcq_[a-z0-9_]+)\s*\(', text))
+    return sorted(names)
 
 
 def lib() -> C.CDLL:

@@ -27,7 +27,7 @@
 #include "lcq_internal.h"
 
 namespace lcq {
-int g_gemm_split = 1;
+std::atomic<int> g_gemm_split{1};
 }
 
 namespace {
@@ -469,9 +469,7 @@ int64_t lcq_chol_inv_upper_workspace_bytes(int64_t K) {
 }
 
 int lcq_set_gemm_split(int on) {
-  const int was = g_gemm_split;
-  g_gemm_split = on ? 1 : 0;
-  return was;
+  return g_gemm_split.exchange(on ? 1 : 0);
 }
 
 int lcq_gptq_prepare_weights(const void* w, int dtype, int64_t R, int64_t K, const int64_t* perm, const uint8_t* dead,
@@ -506,7 +504,7 @@ struct SideLane { int dev; hipStream_t caller; hipStream_t side; hipEvent_t fork
 static SideLane g_lanes[16];
 static int g_nlanes = 0;
 static std::mutex g_lane_mu;
-static int g_lookahead = 1;
+static std::atomic<int> g_lookahead{1};
 static SideLane* side_lane(hipStream_t st) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return nullptr;
@@ -559,7 +557,7 @@ static int chol_chain(float* H, int64_t K64, const int64_t* perm, float percdamp
   // caller's stream, the panels that follow need it) and everything behind those (on the side stream, beside those
   // panels: a few narrow launches that leave the chip to it).  The next deep update touches that region again and
   // waits for it.
-  SideLane* lane = (g_lookahead && K >= 8192) ? side_lane(st) : nullptr;
+  SideLane* lane = (g_lookahead.load() && K >= 8192) ? side_lane(st) : nullptr;
   bool pending = false;
   for (int o0 = 0; o0 < K; o0 += NBO) {
     const int o1 = (o0 + NBO < K) ? (o0 + NBO) : K;
@@ -659,7 +657,7 @@ static int chol_chain(float* H, int64_t K64, const int64_t* perm, float percdamp
         if (na > maxN) maxN = na;
       }
       const dim3 grid((unsigned)((maxN + GT - 1) / GT), (unsigned)((maxM + GT - 1) / GT), (unsigned)np);
-      if (g_gemm_split && ((long long)grid.x * grid.y * grid.z > 256 || maxN >= 256)) {      // long contractions
+      if (g_gemm_split.load() && ((long long)grid.x * grid.y * grid.z > 256 || maxN >= 256)) {      // long contractions
         gemm_s3_batched_kernel<false><<<grid, dim3(256), 0, st>>>(A, K, A, K, T, K, b1, 1.0f, 0.0f, GEMM_K_FROM_N);
         gemm_s3_batched_kernel<false><<<grid, dim3(256), 0, st>>>(A, K, T, K, A, K, b2, -1.0f, 0.0f, GEMM_K_TO_M);
       } else {
@@ -685,9 +683,7 @@ static int chol_chain(float* H, int64_t K64, const int64_t* perm, float percdamp
 }
 
 int lcq_set_chain_lookahead(int on) {
-  const int was = g_lookahead;
-  g_lookahead = on ? 1 : 0;
-  return was;
+  return g_lookahead.exchange(on ? 1 : 0);
 }
 
 int lcq_chol_inv_upper(float* H, int64_t K, const int64_t* perm, float percdamp, float* W, int64_t R, float* U,

@@ -17,6 +17,7 @@
 // (GEMM_LOWER_TILES).  Batched launches take per-problem offsets from
 // GemmBatch (blockIdx.z).
 #pragma once
+#include <atomic>
 #include <type_traits>
 
 #include "common.h"
@@ -508,7 +509,7 @@ __global__ __launch_bounds__(256, 2) void gemm_s3_batched_kernel(const float* A,
 }
 
 // 1 (default): launches of more than 256 tiles run on the bf16 matrix pipe (three-way split operands); 0: fp32 pipe only
-extern int g_gemm_split;
+extern std::atomic<int> g_gemm_split;
 
 // TM = 128, 64 or 32 rows of C per workgroup.  The short tiles are for launches that would not give every CU a
 // 128-row tile (rank-128 updates and panel solves of the blocked chains): twice the workgroups, half the serial
@@ -538,9 +539,10 @@ template <bool B_T>
 inline void launch_gemm(const GemmProblem& g, float alpha, float beta, int flags, hipStream_t st) {
   if (g.M <= 0 || g.N <= 0) return;
   const unsigned gx = (unsigned)((g.N + GT - 1) / GT), gy = (unsigned)((g.M + GT - 1) / GT);
+  const bool split = g_gemm_split.load(std::memory_order_relaxed) != 0;
   // the bf16 pipe also pays for launches of at most one tile per CU when the contraction is long: a tile's time is
   // its serial chain of slabs, 2.7x shorter there
-  if (g_gemm_split && (long long)gx * gy >= 64 && (long long)gx * gy <= 256 && g.Kc >= 256)
+  if (split && (long long)gx * gy >= 64 && (long long)gx * gy <= 256 && g.Kc >= 256)
     gemm_s3_kernel<B_T><<<dim3(gx, gy), dim3(256), 0, st>>>(g, alpha, beta, flags);
   // at most 128 of the 64-row tiles: 32-row tiles instead, twice the CUs and half the serial MFMA work in each (a
   // 64 x 128 tile with a 128-deep contraction is 3.9 us of fp32 MFMA on its CU; K = 4096 chain 2.14 -> 1.99 ms)
@@ -551,10 +553,10 @@ inline void launch_gemm(const GemmProblem& g, float alpha, float beta, int flags
     gemm_f32_kernel<B_T, 64, true><<<dim3(gx, (unsigned)((g.M + 63) / 64)), dim3(256), 0, st>>>(g, alpha, beta, flags);
   else if ((long long)gx * gy <= 256)
     gemm_f32_kernel<B_T, 64><<<dim3(gx, (unsigned)((g.M + 63) / 64)), dim3(256), 0, st>>>(g, alpha, beta, flags);
-  else if (g_gemm_split && (flags & GEMM_LOWER_TILES) && g.M == g.N && g.M % (4 * GT) == 0) {
+  else if (split && (flags & GEMM_LOWER_TILES) && g.M == g.N && g.M % (4 * GT) == 0) {
     const int nsb = g.M / (4 * GT), total = 16 * (nsb * (nsb + 1) / 2);
     gemm_s3_lower_kernel<B_T><<<dim3((unsigned)total), dim3(256), 0, st>>>(g, alpha, beta, flags, nsb);
-  } else if (g_gemm_split)
+  } else if (split)
     gemm_s3_kernel<B_T><<<dim3(gx, gy), dim3(256), 0, st>>>(g, alpha, beta, flags | GEMM_XCD_ORDER);
   else
     gemm_f32_kernel<B_T, GT><<<dim3(gx, gy), dim3(256), 0, st>>>(g, alpha, beta, flags);

@@ -342,6 +342,28 @@ __global__ __launch_bounds__(256) void stage_copy_kernel(const u32x4* __restrict
   }
 }
 
+// Do two byte ranges hold the same bits?  *flag = 1 if any 16-byte piece differs (never cleared here).  add_batch uses
+// it for a Linear that shares another Linear's Hessian: the tokens it was handed against the copy the other Linear
+// staged from the same memory a moment earlier.
+__global__ __launch_bounds__(256) void compare_kernel(const u32x4* __restrict__ a, const u32x4* __restrict__ b, int64_t n16,
+                                                      int* __restrict__ flag) {
+  const int64_t stride = (int64_t)gridDim.x * 1024;
+  uint32_t diff = 0;
+  for (int64_t base = (int64_t)blockIdx.x * 1024; base < n16; base += stride) {
+    u32x4 va[4], vb[4];
+    #pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int64_t i = base + k * 256 + threadIdx.x;
+      if (i < n16) { va[k] = __builtin_nontemporal_load(a + i); vb[k] = __builtin_nontemporal_load(b + i); }
+      else { va[k] = u32x4{0, 0, 0, 0}; vb[k] = va[k]; }
+    }
+    #pragma unroll
+    for (int k = 0; k < 4; ++k)
+      diff |= (va[k][0] ^ vb[k][0]) | (va[k][1] ^ vb[k][1]) | (va[k][2] ^ vb[k][2]) | (va[k][3] ^ vb[k][3]);
+  }
+  if (diff != 0) *flag = 1;                                // every writer stores the same value
+}
+
 // fill the lower triangle from the upper one: H[j][i] = H[i][j], i < j
 __global__ __launch_bounds__(256) void symmetrize_kernel(float* __restrict__ H, int K) {
   __shared__ float tile[32][33];
@@ -380,7 +402,7 @@ int lcq_hessian_accum_sliced(float* H, int64_t K, const void* X, const void* XB,
   if (slices < 1 || slices > 64 || (slices > 1 && slice_stride < K * K)) return LCQ_EINVAL;
   if (slices > 1 && T > (1 << 30)) return LCQ_ESIZE;               // the kernel's slab arithmetic is 32-bit
   if (((uintptr_t)X % 16) != 0 || ((uintptr_t)XB % 16) != 0 || ((uintptr_t)H % 4) != 0) return LCQ_EALIGN;
-  if (T == 0) return LCQ_OK;
+  if (T == 0 && alpha == 1.0f) return LCQ_OK;                      // nothing to add and nothing to scale
   constexpr int TN = 128;
   const int ntr = (int)((K + TM - 1) / TM), ntc = (int)((K + TN - 1) / TN), q = TM / TN;
   int64_t total = 0;
@@ -433,6 +455,18 @@ int lcq_stage_copy(const void* src, void* dst, int64_t bytes, void* stream) {
   int64_t grid = (n16 + 1023) / 1024;
   if (grid > 2048) grid = 2048;
   stage_copy_kernel<<<dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream>>>((const u32x4*)src, (u32x4*)dst, n16);
+  LCQ_CHECK_LAUNCH();
+  return LCQ_OK;
+}
+
+int lcq_compare_bytes(const void* a, const void* b, int64_t bytes, int* flag, void* stream) {
+  if (!a || !b || !flag || bytes < 0 || bytes % 16 != 0) return LCQ_EINVAL;
+  if ((((uintptr_t)a | (uintptr_t)b) % 16) != 0 || ((uintptr_t)flag % 4) != 0) return LCQ_EALIGN;
+  if (bytes == 0) return LCQ_OK;
+  const int64_t n16 = bytes / 16;
+  int64_t grid = (n16 + 1023) / 1024;
+  if (grid > 2048) grid = 2048;
+  compare_kernel<<<dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream>>>((const u32x4*)a, (const u32x4*)b, n16, flag);
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;
 }

@@ -75,6 +75,7 @@ extern "C" {
 int lcq_histc(const void* x, int dtype, int64_t n, int bins, float lo, float hi, void* counts, float* hist, void* stream) {
   if (!x || !counts || !hist || n < 0 || bins <= 0 || bins > HIST_MAX_BINS) return LCQ_EINVAL;
   if (!(lo <= hi) || !(__builtin_isfinite(lo) && __builtin_isfinite(hi))) return LCQ_EINVAL;   // torch: "max must be larger than min", finite range
+  if (dtype != LCQ_F32 && dtype != LCQ_BF16 && dtype != LCQ_F16) return LCQ_EDTYPE;     // before anything is launched
   if (((uintptr_t)x % 16) != 0) return LCQ_EALIGN;
   if (lo == hi) { lo -= 1.0f; hi += 1.0f; }
   hipStream_t st = (hipStream_t)stream;
@@ -86,8 +87,7 @@ int lcq_histc(const void* x, int dtype, int64_t n, int bins, float lo, float hi,
   if (grid > 2048) grid = 2048;
   if (dtype == LCQ_F32) hist_kernel<false, false><<<dim3((unsigned)grid), dim3(256), 0, st>>>(x, n, bins, lo, hi, (uint32_t*)counts);
   else if (dtype == LCQ_BF16) hist_kernel<true, false><<<dim3((unsigned)grid), dim3(256), 0, st>>>(x, n, bins, lo, hi, (uint32_t*)counts);
-  else if (dtype == LCQ_F16) hist_kernel<false, true><<<dim3((unsigned)grid), dim3(256), 0, st>>>(x, n, bins, lo, hi, (uint32_t*)counts);
-  else return LCQ_EDTYPE;
+  else hist_kernel<false, true><<<dim3((unsigned)grid), dim3(256), 0, st>>>(x, n, bins, lo, hi, (uint32_t*)counts);
   hist_to_float_kernel<<<dim3(zb), dim3(256), 0, st>>>((const uint32_t*)counts, bins, hist);
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;

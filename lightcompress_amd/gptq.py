@@ -15,8 +15,21 @@ Differences a caller can observe
   * H is kept valid on and above the diagonal only while it accumulates
     (``hessian(name)`` returns the full symmetric matrix);
   * Linears of a subset that receive the very same input tensor on every call (q/k/v, gate/up) share one Hessian
-    and one Cholesky chain (``special.auto_share``, default on; detected per call, with a fallback to separate
-    Hessians at the first call that differs; results are bit-identical either way);
+    and one Cholesky chain (``special.auto_share``, default on; detected per call by address, shape, strides and
+    type, with a fallback to separate Hessians at the first call that differs; results are bit-identical either
+    way).  The hooks hand over ``inp[0].data`` (gptq.py:246-251), an alias whose version counter always reads 0, so
+    nothing on the host can tell whether the memory was written between two hooks of one forward pass: every
+    shared call is therefore compared on the device, bit for bit, with the copy the first Linear staged
+    (``special.share_verify``, default on; lcq_compare_bytes), and a difference raises ``LcqError`` where the
+    Hessian is consumed (``hessian(name)``, the transform of the Linear) instead of giving the follower the
+    leader's Hessian.  With ``share_verify: False`` the caller vouches that no hook input is modified in place
+    between the hooks of one forward pass;
+  * ``transformers.Conv1D`` (weight stored [in, out], gptq.py:132-133, 190-191, 302) and ``nn.Conv2d`` (inputs
+    unfolded into patches, gptq.py:268-278) layers are taken like the reference takes them; their Hessians are
+    never shared;
+  * ``blocksize`` above 128 runs as passes of at most 128 columns; a group that opens in a later pass of a block
+    takes its range from the weights as they were when the block started, which is what the reference's read of
+    the block-stale ``W`` (gptq.py:216-222) amounts to;
   * subset_transform runs the column loops of Linears that share a chain as one loop over their stacked rows
     (``special.fuse_loops``, default on; rows are independent, so each Linear gets the result of its own loop, up to
     the rounding of the update GEMM where the larger row count selects the other GEMM kernel), and leaves every
@@ -95,12 +108,14 @@ class GPTQ:
         self.block_factor = bool(special_config.get('block_factor', True))
         # Linears of a subset that keep receiving the very same input tensor share one Hessian and one chain
         self.auto_share = bool(special_config.get('auto_share', True))
+        # every shared add_batch call is compared on the device with the tokens the leading Linear staged
+        self.share_verify = bool(special_config.get('share_verify', True))
         if self.owq:                                     # gptq.py:47-50
             self.n_outs = special_config['n_outs']
             self.static_groups = False
             self.actorder = False
-        if self.blocksize > 128:
-            raise NotImplementedError('blocksize above 128 is not supported by the column-loop kernel')
+        if int(self.blocksize) != self.blocksize or self.blocksize < 1:
+            raise ValueError(f'blocksize: {self.blocksize}')
         self.need_perm = (
             self.wquantizer.granularity == 'per_group'
             and not self.static_groups
@@ -113,11 +128,31 @@ class GPTQ:
         needs no call."""
         self.n_out_dict = {name: self.n_outs[i] for i, name in enumerate(names)}
 
+    @staticmethod
+    def _layer_kind(layer):
+        """'conv2d' (weight [out, in, kh, kw], inputs unfolded), 'conv1d' (transformers.Conv1D: weight [in, out]) or
+        'linear' (anything else with a [out, in] weight), as gptq.py:130-133, 262-278 tell them apart."""
+        if isinstance(layer, torch.nn.Conv2d):
+            return 'conv2d'
+        cls = type(layer)
+        if cls.__name__ == 'Conv1D' and cls.__module__.split('.')[0] == 'transformers':
+            return 'conv1d'
+        return 'linear'
+
+    def _weight_2d(self, layer):
+        """The layer's weight as the [out_features, in_features] matrix the loop works on (gptq.py:129-133)."""
+        w = layer.weight.data
+        kind = self._layer_kind(layer)
+        if kind == 'conv2d' or w.dim() > 2:
+            w = w.flatten(1)
+        elif kind == 'conv1d':
+            w = w.t()
+        return w
+
     # -- Hessian (gptq.py:253-308) ---------------------------------------------
     @torch.no_grad()
     def layer_init(self, layer, name):
-        W = layer.weight.data
-        K = W.shape[1] if W.dim() == 2 else W.flatten(1).shape[1]
+        K = self._weight_2d(layer).shape[1]
         self.layers_cache.setdefault(name, {})
         slices = self.hessian_shares(K)
         acc = torch.zeros((slices, K, K), device=self.dev)
@@ -127,10 +162,13 @@ class GPTQ:
         self.layers_cache[name]['nsamples'] = 0
         self.layers_cache[name]['n_in_H'] = 0
         self.layers_cache[name]['calls'] = 0
-        for k in ('stage', 'stage_lo', 'stage_fill', 'stage_batches', 'last_stage', 'last_key', 'last_ref', 'manual_share'):
+        for k in ('stage', 'stage_lo', 'stage_fill', 'stage_batches', 'last_stage', 'last_key', 'last_ref', 'manual_share',
+                  'share_flag'):
             self.layers_cache[name].pop(k, None)
         self.layers_cache[name]['columns'] = K
+        self.layers_cache[name]['kind'] = self._layer_kind(layer)
         self.layers_cache[name].pop('leader', None)
+        self.layers_cache[name].pop('followers', None)
 
     @torch.no_grad()
     def subset_init(self, subset):
@@ -153,53 +191,95 @@ class GPTQ:
 
     @staticmethod
     def _input_key(t):
-        """Identity of an input tensor as the hooks hand it over: same memory, same layout, same version."""
-        return (t.data_ptr(), tuple(t.shape), tuple(t.stride()), t.dtype, t._version)
+        """Identity of an input tensor as the hooks hand it over: same memory, same layout, same type.  (The version
+        counter is left out on purpose: `inp[0].data` is a fresh alias whose counter always reads 0.)"""
+        return (t.data_ptr(), tuple(t.shape), tuple(t.stride()), t.dtype)
 
-    def _follow(self, name, cache, key, separable):
+    def _same_tokens(self, lead, inp, tokens, K):
+        """Queues the comparison of a follower's tokens with the copy its leader staged from the same memory when its
+        own hook ran (lcq_compare_bytes; a difference sets the leader's `share_flag`, read where the Hessian is
+        consumed).  False if that copy is not there to compare with."""
+        if not self.share_verify:
+            return True
+        t_last = lead.get('last_stage', (0, 0))[0]
+        stage = lead.get('stage')
+        if stage is None or t_last != tokens or lead.get('stage_fill', 0) < tokens:
+            return False
+        flag = lead.get('share_flag')
+        if flag is None:
+            flag = lead['share_flag'] = torch.zeros(1, dtype=torch.int32, device=stage.device)
+        es = stage.element_size()
+        off = (lead['stage_fill'] - tokens) * K * es
+        nbytes = tokens * K * es
+        lo = lead.get('stage_lo')
+        lib, st = L.lib(), L.stream()
+        if lo is not None:                               # fp32 activations: both bf16 halves
+            hi_, lo_ = self._halves(inp.reshape((-1, K)).contiguous())
+            L.check(lib.lcq_compare_bytes(L.ptr(hi_), ctypes.c_void_p(stage.data_ptr() + off), L.i64(nbytes), L.ptr(flag), st),
+                    'lcq_compare_bytes')
+            L.check(lib.lcq_compare_bytes(L.ptr(lo_), ctypes.c_void_p(lo.data_ptr() + off), L.i64(nbytes), L.ptr(flag), st),
+                    'lcq_compare_bytes')
+            return True
+        src = inp
+        if not (inp.is_contiguous() and inp.data_ptr() % 16 == 0):
+            src = inp.reshape((-1, K)).contiguous()
+        if nbytes % 16 != 0 or (stage.data_ptr() + off) % 16 != 0 or src.data_ptr() % 16 != 0:
+            return False
+        L.check(lib.lcq_compare_bytes(ctypes.c_void_p(src.data_ptr()), ctypes.c_void_p(stage.data_ptr() + off), L.i64(nbytes),
+                                      L.ptr(flag), st), 'lcq_compare_bytes')
+        return True
+
+    def _follow(self, name, cache, key, separable, inp, tokens, K):
         """Identical inputs need one Hessian.  The hooks of q/k/v (or gate/up) receive the very same tensor on
         every forward pass (gptq.py:246-251), so a Linear whose every call so far got the tensor that an earlier
         Linear of the subset got for the same call follows that Linear: it owns no Hessian and no Cholesky chain
-        (the results are bit-identical to separate accumulation, the arithmetic being the same).  Returns True if
-        this call is covered by the Linear it follows.  The first call that differs ends the arrangement: the
-        follower takes a copy of the Hessian and of the staged tokens as they were before that call and goes on
-        alone."""
+        (the results are bit-identical to separate accumulation, the arithmetic being the same).  "The same tensor"
+        is decided by address, layout and type, and every such call is then compared on the device with the tokens
+        the leader staged (_same_tokens), because an in-place write between two hooks leaves no trace on the host.
+        Returns True if this call is covered by the Linear it follows.  The first call that differs in its key ends
+        the arrangement: the follower takes a copy of the Hessian and of the staged tokens as they were before that
+        call and goes on alone."""
         calls = cache['calls']
         lead_name = cache.get('leader', name)
         if cache.get('manual_share'):
             return lead_name != name
         if lead_name != name:                             # following: does this call match the leader's?
             lead = self.layers_cache.get(lead_name)
-            if lead is not None and lead.get('calls', 0) == calls + 1 and lead.get('last_key') == key:
+            if lead is not None and lead.get('calls', 0) == calls + 1 and lead.get('last_key') == key \
+                    and self._same_tokens(lead, inp, tokens, K):
                 return True
             self._unfollow(name, cache, lead)
             return False
-        if not (self.auto_share and separable) or calls != 0 or self.owq:
+        if not (self.auto_share and separable) or calls != 0 or self.owq or cache.get('followers'):
             return False
         for other, oc in self.layers_cache.items():       # first call: is there a Linear that just got this tensor?
             if other == name or oc.get('leader', other) != other or 'H' not in oc or oc.get('manual_share'):
                 continue
             if oc.get('calls', 0) == 1 and oc.get('last_key') == key and oc.get('last_stage', (0, 0))[0] > 0 \
-                    and oc['H'].shape == cache['H'].shape:
+                    and oc['H'].shape == cache['H'].shape and self._same_tokens(oc, inp, tokens, K):
                 cache['leader'] = other
                 cache['H'] = oc['H']
                 cache['H_shares'] = None
                 oc['leader'] = other
+                oc.setdefault('followers', []).append(name)
                 return True
         return False
 
     def _unfollow(self, name, cache, lead):
         """Give a follower its own Hessian: the state of the Linear it followed, without that Linear's latest call
-        when the follower has not seen it.  (A call that is shared is always still in the staging buffer: a full
-        buffer is folded at the start of the next call, not at the end of the one that filled it.)"""
+        when the follower has not seen it.  (That call is still in the staging buffer then: a full buffer is folded at
+        the start of the next call, not at the end of the one that filled it, and whatever folds the buffer at another
+        time first releases the followers that are a call behind, _release_laggards.)"""
         cache['leader'] = name
         if lead is None or 'H' not in lead:
             raise L.LcqError(f'{name} followed a Linear whose Hessian is gone')
+        if name in lead.get('followers', ()):
+            lead['followers'].remove(name)
         ahead = lead['calls'] - cache['calls']            # 0 or 1
         fill, batches = lead.get('stage_fill', 0), lead.get('stage_batches', 0)
         if ahead:
             t_last, b_last = lead.get('last_stage', (0, 0))
-            if t_last == 0 or fill < t_last:
+            if ahead > 1 or t_last == 0 or fill < t_last:
                 raise L.LcqError(f'{name}: the input differs from the one of {lead.get("leader")} after a call that was '
                                  'folded into the shared Hessian directly; set special.auto_share: False')
             fill, batches = fill - t_last, batches - b_last
@@ -212,6 +292,8 @@ class GPTQ:
         cache['shares_apart'] = lead.get('shares_apart', False)
         cache['n_in_H'] = lead.get('n_in_H', 0)
         cache['upper_only'] = lead.get('upper_only', False)
+        if lead.get('share_flag') is not None:            # what was compared so far concerns this Hessian too
+            cache['share_flag'] = lead['share_flag'].clone()
         for k in ('stage', 'stage_lo', 'stage_fill', 'stage_batches', 'last_stage'):
             cache.pop(k, None)
         if fill > 0:
@@ -223,6 +305,17 @@ class GPTQ:
                 cache['stage_lo'][:fill].copy_(lead['stage_lo'][:fill])
             cache['stage_fill'], cache['stage_batches'] = fill, batches
 
+    def _release_laggards(self, lead_name, lead):
+        """Followers that have not seen their leader's latest call yet (it skipped a forward pass, or H is being read
+        between the two hooks of one pass) get their own Hessian now, while that call can still be told apart from
+        the rest: it is the last one in the staging buffer."""
+        for n in list(lead.get('followers', ())):
+            c = self.layers_cache.get(n)
+            if c is None or c.get('leader') != lead_name:
+                lead['followers'].remove(n)
+            elif c['calls'] < lead['calls']:
+                self._unfollow(n, c, lead)
+
     @torch.no_grad()
     def add_batch(self, layer, name, inp, out=None):
         # Called once per Linear per calibration batch (896 times for one decoder layer): the work up to the return for
@@ -230,25 +323,31 @@ class GPTQ:
         cache = self.layers_cache[name]
         if not inp.is_cuda:
             raise L.LcqError('liblcq operates on GPU tensors only (no CPU fallback)')
+        kind = cache.get('kind', 'linear')
+        if kind == 'conv2d':                            # gptq.py:268-278: patches as tokens, [N, L, C*kh*kw]
+            inp = torch.nn.functional.unfold(inp, layer.kernel_size, dilation=layer.dilation, padding=layer.padding,
+                                             stride=layer.stride).transpose(1, 2)
         shape = inp.shape
-        key = (inp.data_ptr(), shape, inp.stride(), inp.dtype, inp._version)
+        key = (inp.data_ptr(), shape, inp.stride(), inp.dtype)
         nd = len(shape)
         tmp = 1 if nd == 2 else shape[0]
         K = shape[-1]
         tokens = shape[0] if nd == 2 else (shape[0] * shape[1] if nd == 3 else shape[0])
+        if nd > 3 or K != cache['columns']:
+            raise L.LcqError(f'add_batch: input of shape {tuple(shape)} for a layer with {cache["columns"]} input features')
         if inp.dtype not in (torch.bfloat16, torch.float16, torch.float32):
             raise NotImplementedError(f'add_batch takes bf16 / fp16 / fp32 activations; got {inp.dtype}')
         assert tokens % self.chunk_num == 0, \
             f'Error: inp.shape[1] ({tokens}) cannot be evenly divided by chunk_num.'
-        defer = self.hessian_fold(K if nd <= 3 else shape[1])
-        followed = self._follow(name, cache, key, defer > 1)
-        cache['calls'] += 1
-        cache['nsamples'] += tmp
-        if followed:
+        defer = self.hessian_fold(K)
+        if self._follow(name, cache, key, defer > 1 and kind == 'linear', inp, tokens, K):
+            cache['calls'] += 1
+            cache['nsamples'] += tmp
             return                                      # the Linear it follows accumulates
+        if cache.get('followers'):
+            self._release_laggards(name, cache)         # a follower that skipped the previous call goes its own way
         cache['last_key'] = key
         cache['last_ref'] = inp                         # keeps the memory from being handed to another tensor meanwhile
-        cache['last_stage'] = (0, 0)
         cache['upper_only'] = True
         # fp32 activations (gptq.py:289 `chunk.float()` keeps them fp32): staged as two bf16 halves, x = hi + lo
         split = inp.dtype == torch.float32
@@ -258,44 +357,45 @@ class GPTQ:
         # telescopes to H*n/N + (2/N)*(S1+S2+...), N = n + b1 + b2 + ..., so one launch over the
         # concatenated tokens gives the same H while reading and writing it once.  A full buffer is folded at the
         # start of the next call that needs room (or when H is asked for), so the latest call can still be told
-        # apart from H when a follower needs the state before it.
+        # apart from H when a follower needs the state before it.  (`calls` counts the calls whose tokens are in
+        # the buffer or in H: it moves only once this call's tokens are.)
         stage = cache.get('stage')
-        if defer > 1 and nd <= 3:
+        if defer > 1:
             if stage is not None and (stage.dtype != sdtype or split != (cache.get('stage_lo') is not None)
                                       or cache['stage_fill'] + tokens > stage.shape[0]):
                 self._flush(cache)
-                if stage.dtype != sdtype or split != (cache.get('stage_lo') is not None):
-                    stage = None
+                if stage.dtype != sdtype or split != (cache.get('stage_lo') is not None) or tokens > stage.shape[0]:
+                    stage = None                        # another type, or a call larger than the whole buffer
             if stage is None:
                 stage = torch.empty((defer * tokens, K), dtype=sdtype, device=inp.device)
                 cache['stage'] = stage
                 cache['stage_lo'] = torch.empty_like(stage) if split else None
                 cache['stage_fill'] = 0
                 cache['stage_batches'] = 0
-            if tokens <= stage.shape[0]:
-                f = cache['stage_fill']
-                nbytes = tokens * K * stage.element_size()
-                dst = stage.data_ptr() + f * K * stage.element_size()
-                if not split and key[0] % 16 == 0 and nbytes % 16 == 0 and dst % 16 == 0 and inp.is_contiguous():
-                    L.check(L.lib().lcq_stage_copy(ctypes.c_void_p(key[0]), ctypes.c_void_p(dst), ctypes.c_int64(nbytes),
-                                                   L.stream()),
-                            'lcq_stage_copy')
+            f = cache['stage_fill']
+            nbytes = tokens * K * stage.element_size()
+            dst = stage.data_ptr() + f * K * stage.element_size()
+            if not split and key[0] % 16 == 0 and nbytes % 16 == 0 and dst % 16 == 0 and inp.is_contiguous():
+                L.check(L.lib().lcq_stage_copy(ctypes.c_void_p(key[0]), ctypes.c_void_p(dst), ctypes.c_int64(nbytes),
+                                               L.stream()),
+                        'lcq_stage_copy')
+            else:
+                x = inp.reshape((-1, K)).contiguous()
+                if split:
+                    self._halves(x, stage[f:f + tokens], cache['stage_lo'][f:f + tokens])
                 else:
-                    x = inp.reshape((-1, K)).contiguous()
-                    if split:
-                        self._halves(x, stage[f:f + tokens], cache['stage_lo'][f:f + tokens])
-                    else:
-                        stage[f:f + tokens].copy_(x)
-                cache['stage_fill'] = f + tokens
-                cache['stage_batches'] += tmp
-                cache['last_stage'] = (tokens, tmp)
-                return
-        x = inp
-        if nd == 2:
-            x = x.unsqueeze(0)
-        if len(x.shape) == 3:
-            x = x.reshape((-1, K))
-        self._accumulate(cache, *self._halves(x.contiguous()), tmp)
+                    stage[f:f + tokens].copy_(x)
+            cache['stage_fill'] = f + tokens
+            cache['stage_batches'] += tmp
+            cache['last_stage'] = (tokens, tmp)
+            cache['calls'] += 1
+            cache['nsamples'] += tmp
+            return
+        # one launch per call (hessian_defer: 1): nothing is staged, and nothing is shared (see _follow)
+        cache['last_stage'] = (0, 0)
+        cache['calls'] += 1
+        cache['nsamples'] += tmp
+        self._accumulate(cache, *self._halves(inp.reshape((-1, K)).contiguous()), tmp)
 
     def hessian_fold(self, K):
         """add_batch calls folded into one Hessian launch for a Linear with K input features.  'auto': 4 calls of 2048
@@ -373,7 +473,12 @@ class GPTQ:
     def _settle(self, name):
         """H of `name` (or of the layer it aliases) with no tokens left in staging."""
         cache = self.layers_cache[name]
-        lead = self.layers_cache.get(cache.get('leader', name), cache)
+        lead_name = cache.get('leader', name)
+        lead = self.layers_cache.get(lead_name, cache)
+        if lead.get('followers'):
+            self._release_laggards(lead_name, lead)
+            if cache.get('leader', name) != lead_name:   # `name` itself was a call behind: it owns its Hessian now
+                lead = cache
         self._flush(lead)
         lead.pop('stage', None)
         lead.pop('stage_lo', None)
@@ -384,10 +489,16 @@ class GPTQ:
             lead['shares_apart'] = False
         return cache
 
+    _SHARE_MSG = ('a Linear shared the Hessian of another Linear that was handed the same tensor, but the tensor did not '
+                  'hold the same values at the two hooks (it was written in place in between); set special.auto_share: False')
+
     def hessian(self, name):
         """The full symmetric H of a layer (fills the lower triangle on demand)."""
         cache = self._settle(name)
         H = cache['H']
+        flag = self.layers_cache.get(cache.get('leader', name), cache).get('share_flag')
+        if flag is not None and int(flag.item()) != 0:
+            raise L.LcqError(self._SHARE_MSG)
         if cache.get('upper_only', False) or self.layers_cache.get(cache.get('leader', name), {}).get('upper_only'):
             L.check(L.lib().lcq_symmetrize(L.ptr(H), L.i64(H.shape[0]), L.stream()), 'lcq_symmetrize')
             cache['upper_only'] = False
@@ -478,7 +589,7 @@ class GPTQ:
             dead = torch.diag(H) == 0
             ws_bytes = L.lib().lcq_chol_inv_upper_workspace_bytes(L.i64(K))
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=self.dev)
-            status = torch.zeros(1, dtype=torch.int32, device=self.dev)
+            status = self._status_words(leader)
             side = self._side_streams[i % len(self._side_streams)]
             side.wait_stream(main)
             with torch.cuda.stream(side):
@@ -495,12 +606,21 @@ class GPTQ:
             self._shared[leader] = dict(U=H, perm=perm, status=status, dead=dead, done=done, ahead=True,
                                         status_host=status_host, direct=direct)
 
+    def _status_words(self, leader):
+        """[chain status, inputs of a shared Hessian differed] as two device words; the chain writes the first, the
+        second is what the comparisons of add_batch left (queued earlier on the current stream)."""
+        status = torch.zeros(2, dtype=torch.int32, device=self.dev)
+        flag = self.layers_cache.get(leader, {}).get('share_flag')
+        if flag is not None:
+            status[1:].copy_(flag)
+        return status
+
     @staticmethod
     def _post_status(status):
-        """Queues, right behind the chain on the current stream, a copy of the chain's status word to pinned host
+        """Queues, right behind the chain on the current stream, a copy of the chain's status words to pinned host
         memory and an event after it.  The check before the weights are written back waits for that event only, so the
         host does not wait for the column loop queued after the chain and the GPU does not run dry behind it."""
-        host = torch.empty(1, dtype=torch.int32, pin_memory=True)
+        host = torch.empty(2, dtype=torch.int32, pin_memory=True)
         host.copy_(status, non_blocking=True)
         copied = torch.cuda.Event()
         copied.record()
@@ -546,10 +666,7 @@ class GPTQ:
         `for_loop` (what layer_transform passes): the second result is only going to feed weight_transform, so
         where the quantizer allows it (_block_factor_ok) it is the block factor P of lcq_chol_block_factor, which has
         U's diagonal blocks but needs no triangular inverse; weight_transform recognises it."""
-        w = layer.weight.data
-        if w.dim() > 2:
-            w = w.flatten(1)
-        w = w.contiguous()
+        w = self._weight_2d(layer).contiguous()          # Conv2d: flatten(1); transformers.Conv1D: t() (gptq.py:129-133)
         R, K = w.shape
         cache = self._settle(name) if 'H' in self.layers_cache[name] else self.layers_cache[name]
         leader = cache.get('leader', name)
@@ -567,7 +684,7 @@ class GPTQ:
             dead = torch.diag(H) == 0                       # before the chain rewrites H
             ws_bytes = L.lib().lcq_chol_inv_upper_workspace_bytes(L.i64(K))
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=self.dev)
-            status = torch.zeros(1, dtype=torch.int32, device=self.dev)
+            status = self._status_words(leader)
             direct = for_loop and self._block_factor_ok(K)
             chain = L.lib().lcq_chol_block_factor if direct else L.lib().lcq_chol_inv_upper
             L.check(chain(L.ptr(H), L.i64(K), L.ptr(perm), L.f32(self.percdamp), L.ptr(None), L.i64(0), L.ptr(H), L.ptr(ws),
@@ -582,7 +699,7 @@ class GPTQ:
         if shared.get('direct') and not for_loop:
             raise L.LcqError('the chain of this Hessian was started for the column loop (block factor, no inverse): '
                              'call process_hessian_and_weights(..., for_loop=True) or set special.block_factor: False')
-        self._status = shared['status']
+        self._status = shared['status'][:1]
         self._status_host = shared['status_host']
         self._loop_factor = (U.data_ptr(), bool(shared.get('direct')))      # what weight_transform is going to be handed
         self._loop_W0 = None
@@ -643,11 +760,12 @@ class GPTQ:
         self._write_back(layer, W, Losses, tmp)
 
     def _check_status(self):
-        if self.check_positive_definite:
-            host, copied = self._status_host
-            copied.synchronize()                         # the chain and the copy behind it; the loop may still be running
-            if int(host[0]) != 0:
-                raise torch.linalg.LinAlgError('GPTQ: the damped Hessian is not positive-definite')
+        host, copied = self._status_host
+        copied.synchronize()                             # the chain and the copy behind it; the loop may still be running
+        if int(host[1]) != 0:
+            raise L.LcqError(self._SHARE_MSG)
+        if self.check_positive_definite and int(host[0]) != 0:
+            raise torch.linalg.LinAlgError('GPTQ: the damped Hessian is not positive-definite')
 
     def _write_back(self, layer, W, Losses, tmp):
         """gptq.py:178-196 after the loop: summed loss, outlier columns, tmp[:, invperm], the weight and the qparams."""
@@ -662,7 +780,9 @@ class GPTQ:
                                                      L.ptr(self.invperm), L.ptr(None), L.ptr(out), L.stream()),
                     'lcq_gptq_prepare_weights')
             tmp = out
-        if tmp._base is not None:                        # rows of a stacked matrix: the Linear gets storage of its own
+        if self._layer_kind(layer) == 'conv1d':          # gptq.py:190-191
+            tmp = tmp.t().contiguous()
+        elif tmp._base is not None:                      # rows of a stacked matrix: the Linear gets storage of its own
             tmp = tmp.clone()
         layer.weight.data = tmp.reshape(layer.weight.shape)
         if self.wquantizer.granularity == 'per_group' and not self.static_groups:
@@ -675,8 +795,7 @@ class GPTQ:
         row gets what it would get alone, while the block kernel, which is bound by the length of its 128 sequential
         columns and not by the number of rows, and the update GEMMs run once instead of once per Linear."""
         parts, r0 = [], 0
-        rows = [layers_dict[n].weight.data.flatten(1).shape[0] if layers_dict[n].weight.dim() > 2
-                else layers_dict[n].weight.shape[0] for n in names]
+        rows = [self._weight_2d(layers_dict[n]).shape[0] for n in names]
         K = self.layers_cache[names[0]]['columns']
         Wall = torch.empty((sum(rows), K), dtype=torch.float32, device=self.dev)
         U = None
@@ -730,39 +849,57 @@ class GPTQ:
         if self._static or host_groups:
             flags |= L.FLAG_STATIC
         g = self._g
-        # Two-level deferral: after every block only the rest of the current 1024-column window is
+        # Two-level deferral: after every pass only the rest of the current 1024-column window is
         # updated; the columns behind the window get one update per window (8x fewer passes over W).
-        window = 8 * self.blocksize
+        B = int(self.blocksize)
+        window = 8 * B if B <= 128 else B * max(1, 1024 // B)
         Err = torch.empty((R, window), device=W.device)
         lib = L.lib()
         st = L.stream()
         qmin, qmax = L.f32(wq.qmin), L.f32(wq.qmax)
         n = self.n_nonout
+        searched = not self._static and g > 0            # group ranges are searched while the loop runs
+
+        def open_groups(c0, c1):
+            """search_column_qparams (gptq.py:358-366) for the groups that open in [c0, c1), on W as it is now."""
+            for idx in range((c0 + g - 1) // g * g, c1, g):
+                _, s_, z_, _, _ = wq.get_tensor_qparams(W[:, idx:min(idx + g, n)].contiguous())
+                self._scales[:, idx // g] = s_.reshape(-1).float()
+                if not wq.sym:
+                    self._zeros[:, idx // g] = z_.reshape(-1).float()
+
         for o0 in range(0, n, window):
             o1 = min(o0 + window, n)
             # A group that opens inside the window reads its whole column range of W (gptq.py:216-222), so the
-            # per-block updates reach to the end of the last such group; the window's deep update starts there.
+            # per-pass updates reach to the end of the last such group; the window's deep update starts there.
             hi = o1
-            if not self._static and g > 0:
+            if searched:
                 last_open = (o1 - 1) // g * g
                 if last_open >= o0:
                     hi = max(o1, min(last_open + g, n))
-            for i1 in range(o0, o1, self.blocksize):
-                i2 = min(i1 + self.blocksize, o1)
-                if host_groups:
-                    for idx in range((i1 + g - 1) // g * g, i2, g):
-                        _, s_, z_, _, _ = wq.get_tensor_qparams(W[:, idx:min(idx + g, n)].contiguous())
-                        self._scales[:, idx // g] = s_.reshape(-1).float()
-                        if not wq.sym:
-                            self._zeros[:, idx // g] = z_.reshape(-1).float()
-                err_blk = Err[:, i1 - o0:]
-                L.check(lib.lcq_gptq_block(L.ptr(W), L.ptr(tmp), L.ptr(Losses), C_ptr(err_blk), L.i64(window), L.ptr(Hinv),
-                                           L.ptr(W0), L.i64(R), L.i64(K), L.i64(n), L.i64(i1), L.i32(i2 - i1), L.i32(self._g), qmin, qmax,
-                                           L.i32(flags), L.ptr(self._scales), L.ptr(self._zeros), L.ptr(self._gidx),
-                                           L.i64(self._G), st), 'lcq_gptq_block')
-                if i2 < hi:
-                    L.check(lib.lcq_gptq_trailing(L.ptr(W), C_ptr(err_blk), L.i64(window), L.ptr(Hinv), L.i64(R), L.i64(K),
-                                                  L.i64(i1), L.i64(i2), L.i64(i2), L.i64(hi), st), 'lcq_gptq_trailing')
+            for b1 in range(o0, o1, B):                  # the reference's blocks
+                b2 = min(b1 + B, o1)
+                # A block wider than 128 columns runs as several passes.  The reference reads a group's range from
+                # the global W when the group opens (gptq.py:216-222), and the global W does not see a block's own
+                # updates before the block ends (they go to the block-local copy W1, gptq.py:203, 240): the groups
+                # that open in the later passes are therefore searched now, before the first pass touches their columns.
+                if searched and b2 - b1 > 128:
+                    open_groups(b1 + 128, b2)
+                for i1 in range(b1, b2, 128):
+                    i2 = min(i1 + 128, b2)
+                    pass_flags = flags
+                    if searched and i1 > b1:
+                        pass_flags |= L.FLAG_STATIC       # every group of this pass has its parameters already
+                    elif host_groups:
+                        open_groups(i1, i2)
+                    err_blk = Err[:, i1 - o0:]
+                    L.check(lib.lcq_gptq_block(L.ptr(W), L.ptr(tmp), L.ptr(Losses), C_ptr(err_blk), L.i64(window), L.ptr(Hinv),
+                                               L.ptr(W0), L.i64(R), L.i64(K), L.i64(n), L.i64(i1), L.i32(i2 - i1), L.i32(self._g), qmin,
+                                               qmax, L.i32(pass_flags), L.ptr(self._scales), L.ptr(self._zeros), L.ptr(self._gidx),
+                                               L.i64(self._G), st), 'lcq_gptq_block')
+                    if i2 < hi:
+                        L.check(lib.lcq_gptq_trailing(L.ptr(W), C_ptr(err_blk), L.i64(window), L.ptr(Hinv), L.i64(R), L.i64(K),
+                                                      L.i64(i1), L.i64(i2), L.i64(i2), L.i64(hi), st), 'lcq_gptq_trailing')
             if hi < K:
                 L.check(lib.lcq_gptq_trailing(L.ptr(W), L.ptr(Err), L.i64(window), L.ptr(Hinv), L.i64(R), L.i64(K),
                                               L.i64(o0), L.i64(o1), L.i64(hi), L.i64(K), st), 'lcq_gptq_trailing')

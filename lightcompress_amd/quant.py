@@ -96,12 +96,12 @@ class BaseQuantizer(object):
     def get_mse_range(self, tensor, norm=2.4, bs=256):
         """quant.py:147-205 -> fp32 (min_val, max_val) [rows, 1]: the shrunken range with the smallest
         sum |quant_dequant(x) - x| ** norm per row, one kernel instead of 80 rounds of ~10 torch ops."""
-        if getattr(self, 'quant_type', 'int-quant') != 'int-quant':
-            raise NotImplementedError('get_mse_range runs for IntegerQuantizer')
         if self.granularity == 'per_tensor' or tensor.dim() != 2:
             raise NotImplementedError('get_mse_range runs on a 2-D reshaped tensor')
         assert self.mse_b_num >= 1 and tensor.shape[0] % self.mse_b_num == 0, \
             'Batch number must be divisible by tensor.shape[0],'
+        if getattr(self, 'quant_type', 'int-quant') != 'int-quant':
+            return self._mse_range_float(tensor, norm)
         t = tensor.contiguous()
         rows, cols = t.shape
         mn = torch.empty((rows, 1), dtype=torch.float32, device=t.device)
@@ -827,9 +827,9 @@ class FloatQuantizer(BaseQuantizer):
         self.qmin = torch.tensor(self.qmin)
 
     # -- use_qtorch=False: per-element steps (quant.py:1004-1026) ----------------------------------
-    def _emu(self, rows_t, scales=None, want=()):
+    def _emu(self, rows_t, scales=None, want=(), rng=None):
         """One launch of lcq_quant_fp_emu -> dict with the requested outputs out of
-        'xc', 'scales', 'q', 'q_fp8', 'dq'.  scales=None: dynamic (per-row ranges of rows_t)."""
+        'xc', 'scales', 'q', 'q_fp8', 'dq'.  scales=None: dynamic (per-row ranges of rows_t, or `rng` = (min, max))."""
         t = rows_t.contiguous()
         flags = 0
         mn = mx = s_in = None
@@ -837,7 +837,7 @@ class FloatQuantizer(BaseQuantizer):
             if self.granularity == 'per_tensor':
                 # the reference indexes maxval.shape[0] of a 0-dim range here (quant.py:1011)
                 raise IndexError('tuple index out of range')
-            mn, mx = self.get_minmax_range(t)
+            mn, mx = self.get_minmax_range(t) if rng is None else (rng[0].to(t.dtype), rng[1].to(t.dtype))
             if self.e_bits >= 5 and t.dtype != torch.float32:
                 t, mn, mx = t.float(), mn.float(), mx.float()        # maxval.to(float32), quant.py:1014-1015
             mn, mx = mn.contiguous(), mx.contiguous()
@@ -869,10 +869,43 @@ class FloatQuantizer(BaseQuantizer):
         return out
 
     def get_float_qparams(self, tensor, tensor_range, device):
-        """quant.py:1004-1026 -> (clamped tensor, elementwise scales); the range is recomputed from
-        `tensor` (it is what get_tensor_range returned for it)."""
-        o = self._emu(tensor, want=('xc', 'scales'))
+        """quant.py:1004-1026 -> (clamped tensor, elementwise scales).  `tensor_range` None: the per-row min / max of
+        `tensor` (what get_tensor_range returns for it with calib_algo minmax); otherwise the given (min, max)."""
+        o = self._emu(tensor, want=('xc', 'scales'), rng=tensor_range)
         return o['xc'].view(tensor.shape), o['scales'].view(tensor.shape)
+
+    def _mse_range_float(self, tensor, norm):
+        """get_mse_range (quant.py:147-205) for the minifloat quantizer: the shrink grid stays a host loop, every step
+        is one range -> scale launch, one quantize-dequantize launch and the reference's elementwise error
+        (|q - x| ** norm summed per row, fp32 torch ops).  `lo` / `hi` are views of the returned ranges and a row
+        that improves overwrites them, so the next steps shrink the improved range - the reference's aliasing of
+        best_min_val with min_val (quant.py:170, 196-198)."""
+        t = tensor.float().contiguous()
+        mn, mx = self.get_minmax_range(t)
+        bs = t.shape[0] // self.mse_b_num
+        for b in range(self.mse_b_num):
+            x = t[b * bs:(b + 1) * bs]
+            lo, hi = mn[b * bs:(b + 1) * bs], mx[b * bs:(b + 1) * bs]
+            best = torch.full((x.shape[0], 1), float('inf'), device=t.device)
+            for i in range(int(self.maxshrink * self.mse_grid)):
+                p = 1 - i / self.mse_grid
+                xmin, xmax = p * lo, p * hi
+                if self.use_qtorch:
+                    scales, zeros, qmax, qmin = self.get_qparams((xmin, xmax), t.device)
+                    q = self.quant_dequant(x, scales, zeros, qmax, qmin)
+                else:
+                    q = self._emu(x, want=('dq',), rng=(xmin, xmax))['dq'].view(x.shape)
+                err = q.sub_(x).abs_().pow_(norm).sum(1, keepdim=True)
+                better = err < best
+                best = torch.where(better, err, best)
+                lo.copy_(torch.where(better, xmin, lo))
+                hi.copy_(torch.where(better, xmax, hi))
+        return (mn, mx)
+
+    def get_hqq_qparams(self, tensor, args):
+        """quant.py:1028-1040: the HQQ solver returns non-zero zero points, which the minifloat quantize kernels
+        (zero point 0, as every other calibration of this class gives) do not take."""
+        raise NotImplementedError("calib_algo='hqq' with FloatQuantizer: zero points other than 0 are not on this path")
 
     def _fp_flags(self):
         return ((L.FLAG_TIE_EVEN if self.fp_tie == 'even' else 0)
@@ -931,9 +964,18 @@ class FloatQuantizer(BaseQuantizer):
 
     def get_tensor_qparams(self, tensor, args={}):
         """quant.py:1042-1058 -> (tensor_reshaped, scales, zeros, qmax, qmin)."""
-        if self.calib_algo != 'minmax':
-            raise NotImplementedError(f'calib_algo={self.calib_algo!r}: only minmax runs on liblcq')
+        if self.calib_algo == 'hqq':
+            return self.get_hqq_qparams(tensor, args)
+        if self.granularity == 'per_block':
+            raise NotImplementedError('per_block ranges are taken inside the block-wise cast (fake / real quant methods)')
         tensor = self.reshape_tensor(tensor)
+        if self.calib_algo in ('mse', 'learnable'):          # the shared dispatch of quant.py:124-132
+            tensor_range = self.get_tensor_range(tensor, args)
+            if not self.use_qtorch:
+                xc, s = self.get_float_qparams(tensor, tensor_range, tensor.device)
+                return xc, s, torch.tensor(0), None, None
+            s, z, qmax, qmin = self.get_qparams(tensor_range, tensor.device)
+            return tensor, s, z, qmax, qmin
         if not self.use_qtorch:
             xc, s = self.get_float_qparams(tensor, None, tensor.device)
             return xc, s, torch.tensor(0), None, None
@@ -984,12 +1026,23 @@ class FloatQuantizer(BaseQuantizer):
         dq, _, _ = self._launch(tensor, static=True, scales=scales, want_dq='f32')
         return dq.view(tensor.shape)
 
-    def _fake(self, t, static_scales=None):
+    def _calibrated(self, t, args):
+        """Dynamic quantization with calib_algo mse / learnable: (rows, scales, zeros, qmax, qmin) through
+        get_tensor_qparams, as quant.py:1099-1108, 1137-1155, 1194-1206 do."""
+        rargs = {k: args[k] for k in ('lowbound_factor', 'upbound_factor') if k in args} \
+            if self.calib_algo == 'learnable' else {}
+        return self.get_tensor_qparams(t, rargs)
+
+    def _fake(self, t, static_scales=None, args={}):
         if self.granularity == 'per_block':
             if static_scales is not None:
                 raise NotImplementedError('static per_block scales')
             return self._per_block(t, True)
         shape, dtype = t.shape, t.dtype
+        if static_scales is None and self.calib_algo != 'minmax':
+            rows_t, scales, zeros, qmax, qmin = self._calibrated(t, args)
+            dq = self.quant_dequant(rows_t, scales, zeros, qmax, qmin)
+            return self.restore_tensor(dq.view(rows_t.shape), shape).to(dtype)
         rows_t = self.reshape_tensor(t)
         if not self.use_qtorch:
             dq = self._emu(rows_t, static_scales, want=('dq',))['dq']
@@ -1004,7 +1057,7 @@ class FloatQuantizer(BaseQuantizer):
         return self._fake(act, args['scales'])
 
     def fake_quant_act_dynamic(self, act, args={}):
-        return self._fake(act)
+        return self._fake(act, None, args)
 
     def fake_quant_weight_static(self, weight, args):
         if 'rounding' in args:
@@ -1015,7 +1068,7 @@ class FloatQuantizer(BaseQuantizer):
 
     def fake_quant_weight_dynamic(self, weight, args={}):
         ic = 'dim' in args and 'ic' in args['dim']
-        q = self._fake(weight.T if ic else weight)
+        q = self._fake(weight.T if ic else weight, None, args)
         return q.T if ic else q
 
     def _per_block(self, weight, want_dq):
@@ -1031,7 +1084,7 @@ class FloatQuantizer(BaseQuantizer):
             return _block_dequant(y, s, torch.float32).to(weight.dtype)
         return y, s
 
-    def _real(self, weight, static_scales, output_scale_factor):
+    def _real(self, weight, static_scales, output_scale_factor, args={}):
         assert self.bit in ['e4m3', 'e5m2'], 'Only FP8 E4M3 and E5M2 support real quant'
         if self.granularity == 'per_block':
             if static_scales is not None:
@@ -1040,6 +1093,9 @@ class FloatQuantizer(BaseQuantizer):
             return y, s * output_scale_factor, None
         dtype = torch.float8_e4m3fn if self.e_bits == 4 else torch.float8_e5m2
         org_w_shape = weight.shape
+        if static_scales is None and self.calib_algo != 'minmax':
+            rows_t, static_scales, _, _, _ = self._calibrated(weight, args)      # then as with given scales
+            weight = rows_t
         rows_t = self.reshape_tensor(weight)
         if not self.use_qtorch:
             if static_scales is None:
@@ -1068,7 +1124,7 @@ class FloatQuantizer(BaseQuantizer):
     def real_quant_weight_dynamic(self, weight, args={}):
         """quant.py:1194-1220."""
         osf = args.pop('output_scale_factor', 1) if 'output_scale_factor' in args else 1
-        return self._real(weight, None, osf)
+        return self._real(weight, None, osf, args)
 
     def __repr__(self):
         return (

@@ -35,6 +35,14 @@ def add_batch(H: torch.Tensor, nsamples: int, inp: torch.Tensor, chunk_num: int 
     return nsamples
 
 
+def conv2d_patches(inp: torch.Tensor, kernel_size, dilation=1, padding=0, stride=1) -> torch.Tensor:
+    """What add_batch makes of a Conv2d input (gptq.py:268-278): nn.Unfold -> [N, C*kh*kw, L], permuted and flattened
+    to [C*kh*kw, N*L]; returned here as [N, L, C*kh*kw] so that add_batch above (which transposes) sees the same
+    matrix, with N as the batch count."""
+    cols = torch.nn.functional.unfold(inp, kernel_size, dilation=dilation, padding=padding, stride=stride)
+    return cols.transpose(1, 2).contiguous()
+
+
 def hessian_closed_form(batches, dtype=torch.float64) -> torch.Tensor:
     """(2/N) * sum_b X_b^T X_b — what the running rescale telescopes to (N = number of batches)."""
     n = sum(1 if b.dim() == 2 else b.shape[0] for b in batches)

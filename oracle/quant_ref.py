@@ -470,6 +470,60 @@ def int_mse_range(spec, tensor: torch.Tensor, norm=2.4, maxshrink=0.8, mse_grid=
     return min_val, max_val
 
 
+def float_mse_range(spec, tensor: torch.Tensor, norm=2.4, maxshrink=0.8, mse_grid=100, mse_b_num=1):
+    """get_mse_range, quant.py:147-205, for FloatQuantizer(use_qtorch=True): the same recurrence (aliasing included)
+    with the symmetric float qparams (:544-552) and float_quantize in quant_dequant (:1060-1080)."""
+    assert mse_b_num >= 1 and tensor.shape[0] % mse_b_num == 0
+    bs = tensor.shape[0] // mse_b_num
+    tensor = tensor.float()
+    min_val, max_val = minmax_range(spec, tensor)
+    for b_num in range(mse_b_num):
+        _tensor = tensor[b_num * bs:(b_num + 1) * bs, :]
+        _min_val, _max_val = min_val[b_num * bs:(b_num + 1) * bs, :], max_val[b_num * bs:(b_num + 1) * bs, :]
+        best = torch.full([_tensor.shape[0]], float('inf'))
+        best_min_val, best_max_val = _min_val, _max_val
+        for i in range(int(maxshrink * mse_grid)):
+            p = 1 - i / mse_grid
+            xmin = p * _min_val
+            xmax = p * _max_val
+            scales, zeros, _, _ = float_qparams(spec, xmin, xmax)
+            q_tensor = float_dequant(float_quant(spec, _tensor, scales, zeros), scales, zeros)
+            q_tensor -= _tensor
+            q_tensor.abs_()
+            q_tensor.pow_(norm)
+            err = torch.sum(q_tensor, 1)
+            tmp = err < best
+            if torch.any(tmp):
+                best[tmp] = err[tmp]
+                best_min_val[tmp] = xmin[tmp]
+                best_max_val[tmp] = xmax[tmp]
+        min_val[b_num * bs:(b_num + 1) * bs, :], max_val[b_num * bs:(b_num + 1) * bs, :] = best_min_val, best_max_val
+    return min_val, max_val
+
+
+def float_fake_quant_with_range(spec, w, lo, hi):
+    """fake_quant_weight_dynamic of FloatQuantizer once get_tensor_range has given (lo, hi) - calib_algo mse or
+    learnable, quant.py:1042-1058, 1141-1158."""
+    shape, dtype = w.shape, w.dtype
+    rows = reshape_rows(spec, w)
+    s, z, _, _ = float_qparams(spec, lo, hi)
+    out = float_dequant(float_quant(spec, rows, s, z), s, z)
+    return restore_rows(spec, out, shape).to(dtype)
+
+
+def learnable_range(spec, rows, lowbound_factor=None, upbound_factor=None):
+    """get_learnable_range, quant.py:207-221."""
+    lo, hi = minmax_range(spec, rows)
+    if spec.symmetric:
+        if upbound_factor is not None:
+            abs_max = torch.max(hi.abs(), lo.abs()).clamp(min=1e-5)
+            abs_max = torch.sigmoid(upbound_factor) * abs_max
+            lo, hi = -abs_max, abs_max
+    elif upbound_factor is not None and lowbound_factor is not None:
+        lo, hi = torch.sigmoid(lowbound_factor) * lo, torch.sigmoid(upbound_factor) * hi
+    return lo, hi
+
+
 # ----------------------------------------------------------------------------
 # HQQ zero-point refinement   (quant.py:94-103, 587-609, 679-687)
 # ----------------------------------------------------------------------------

@@ -1,0 +1,340 @@
+"""The path the benchmark times, at the headline configuration's own sizes.
+
+`GPTQ.subset_transform` with default settings takes shortcuts that `process_hessian_and_weights` called on its own
+does not: Linears fed the same tensor share one Hessian (add_batch detects it), the chains of a subset start side by
+side on other streams, the damped Hessian is factored WITHOUT the triangular inverse (lcq_chol_block_factor) and
+Linears that share a chain go through the column loop as one stacked matrix.  The CPU oracle cannot run 14336-wide
+layers in test time, so this file pins those shortcuts by properties that do not depend on the size and that the
+device evaluates in fp64 with plain torch ops:
+
+  * the loss identity  sum(Losses) == 1/2 tr((W0 - Q)(H_perm + damp I)(W0 - Q)^T), which holds for any quantized
+    values Q exactly when the factor is exact and the error feedback is applied exactly (gptq.py:198-244);
+  * agreement of the integer codes with the run that keeps the reference's chain (special.block_factor: False);
+  * agreement of every Linear of a stacked loop with its own un-stacked loop;
+  * the block factor itself: the upper triangular M rebuilt from it satisfies M M^T == H_perm + damp I.
+
+The other two configurations that only ran at reduced sizes against the oracle, the AWQ search (4096 / 11008,
+128 x 512 tokens) and the float8 / int4-pack expert shapes, get their full-size checks here too: slices of the
+full-size outputs bit for bit against the CPU oracle, plus properties of the whole run.
+"""
+import types
+
+import pytest
+import torch
+
+from oracle import awq_ref as A, pack_ref, quant_ref as Q
+from tests.helpers import assert_bit_equal, gen, weight_like
+from tests.test_gptq_gpu import Layer, make_gptq
+
+pytestmark = pytest.mark.gpu
+
+G128 = 128
+
+
+def _device_batches(dev, nb, T, K, seed):
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    sigma = torch.exp(torch.randn(K, device=dev, generator=g))
+    return [(torch.randn(T, K, device=dev, generator=g) * sigma).bfloat16() for _ in range(nb)]
+
+
+def _weights(dev, R, K, seed):
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    return (torch.randn(R, K, device=dev, generator=g) * 0.02).bfloat16()
+
+
+def _hessian_fp64(xs):
+    K = xs[0].shape[1]
+    H = torch.zeros(K, K, dtype=torch.float64, device=xs[0].device)
+    for x in xs:
+        xd = x.double()
+        H.addmm_(xd.t(), xd)
+    return H * (2.0 / len(xs))
+
+
+def _damped(H64, perm):
+    Hd = H64[perm][:, perm]
+    Hd.diagonal().add_(0.01 * Hd.diagonal().mean())
+    return Hd
+
+
+def _codes(tmp, s, z):
+    R, K = tmp.shape
+    t = tmp.reshape(R, K // G128, G128)
+    return torch.clamp(torch.round(t / s.reshape(R, -1, 1)) + z.reshape(R, -1, 1), 0, 15).reshape(R, K)
+
+
+def _qdq(tmp, s, z):
+    R, K = tmp.shape
+    c = _codes(tmp, s, z).reshape(R, K // G128, G128)
+    return ((c - z.reshape(R, -1, 1)) * s.reshape(R, -1, 1)).reshape(R, K)
+
+
+def _loss_identity(layer, W0, Hd, perm, loss, what):
+    """sum(Losses) of the run against 1/2 tr(D H_d D^T), D = W0 - Q in processing order, fp64 on the device."""
+    R, K = W0.shape
+    W0p = W0.float()[:, perm]
+    tmp = layer.weight.data[:, perm]
+    s, z = layer.buf_scales.reshape(R, K // G128), layer.buf_zeros.reshape(R, K // G128)
+    assert bool(torch.isfinite(tmp).all()) and bool((s > 0).all())
+    assert bool((z == torch.round(z)).all()) and float(z.min()) >= 0 and float(z.max()) <= 15
+    assert torch.equal(tmp[:, 0], W0p[:, 0])                          # the first processed column is untouched
+    D = (W0p - _qdq(tmp, s, z)).double()
+    rhs = 0.5 * float(((D @ Hd) * D).sum())
+    print(f'{what}: sum(Losses) = {loss:.6g}, 1/2 tr((W0-Q) H_d (W0-Q)^T) = {rhs:.6g}')
+    assert abs(loss - rhs) <= 1e-4 * rhs, (what, loss, rhs)
+    # error feedback pays: plain round-to-nearest of the original weights loses more under the same metric
+    t0 = W0p.reshape(R, K // G128, G128)
+    mn, mx = t0.amin(-1), t0.amax(-1)
+    s0 = (mx - mn).clamp(min=1e-5) / 15
+    z0 = (-torch.round(mn / s0)).clamp(0, 15)
+    Dr = (W0p - _qdq(W0p, s0, z0)).double()
+    assert rhs < 0.9 * 0.5 * float(((Dr @ Hd) * Dr).sum())
+    return tmp, s, z
+
+
+def _run_subset(dev, Ws, xs, **special):
+    """subset_init -> one add_batch per Linear and batch with the SAME tensor for all of them, handed over as the
+    hooks do (`inp[0].data`, gptq.py:246-251) -> subset_transform."""
+    gp = make_gptq(actorder=True, **special)
+    layers = {n: Layer(w.clone()) for n, w in Ws.items()}
+    sub = {'layers': layers}
+    gp.subset_init(sub)
+    for x in xs:
+        xb = x.unsqueeze(0)
+        for n in Ws:
+            gp.add_batch(layers[n], n, xb.data, None)
+    leaders = {n: gp.layers_cache[n].get('leader', n) for n in Ws}
+    factors = []
+    orig = gp.weight_transform
+
+    def spy(W, Hinv, Losses, tmp):                                    # which factor and how many rows the loop was given
+        factors.append((bool(gp._loop_factor[1]), W.shape[0]))
+        return orig(W, Hinv, Losses, tmp)
+    gp.weight_transform = spy
+    gp.subset_transform(sub)
+    torch.cuda.synchronize()
+    assert gp._shared == {} and gp.layers_cache == {}
+    return gp, layers, leaders, factors
+
+
+def test_down_proj_through_subset_transform(dev):
+    """K = 14336, R = 4096, act_order, 8 x 2048 tokens (two Hessian launches of four calls): the default path (block
+    factor, no triangular inverse) against the loss identity, against round-to-nearest, and against the run that
+    keeps the reference's chain."""
+    R, K, nb, T = 4096, 14336, 8, 2048
+    xs = _device_batches(dev, nb, T, K, seed=2100)
+    W0 = _weights(dev, R, K, seed=2101)
+    H64 = _hessian_fp64(xs)
+    runs = {}
+    for bf in (True, False):
+        gp, layers, _, factors = _run_subset(dev, {'down_proj': W0}, xs, block_factor=bf)
+        assert factors == [(bf, R)]
+        lay = layers['down_proj']
+        perm = lay.buf_perm
+        assert torch.equal(torch.sort(perm).values, torch.arange(K, device=dev))
+        d = H64.diagonal()[perm]
+        assert float(((d[1:] - d[:-1]) / d[:-1]).max()) < 1e-5        # descending Hessian diagonal, up to fp32 ties
+        Hd = _damped(H64, perm)
+        tmp, s, z = _loss_identity(lay, W0, Hd, perm, float(gp.last_errors['down_proj']), f'down_proj block_factor={bf}')
+        del Hd
+        runs[bf] = (perm, _codes(tmp, s, z), s, float(gp.last_errors['down_proj']))
+    assert torch.equal(runs[True][0], runs[False][0])
+    agree = float((runs[True][1] == runs[False][1]).float().mean())
+    s_close = float(torch.isclose(runs[True][2], runs[False][2], rtol=1e-3).float().mean())
+    print(f'down_proj: codes equal on {agree:.6f} of the entries, scales within 1e-3 on {s_close:.6f}, '
+          f'losses {runs[True][3]:.6g} / {runs[False][3]:.6g}')
+    assert agree >= 0.999, agree
+    assert s_close >= 0.995
+    assert abs(runs[True][3] - runs[False][3]) <= 1e-3 * runs[False][3]
+
+
+@pytest.mark.parametrize('rows', [{'gate_proj': 14336, 'up_proj': 14336}, {'q_proj': 4096, 'k_proj': 1024, 'v_proj': 1024}])
+def test_stacked_loops_at_full_size(dev, rows):
+    """gate + up (28 672 stacked rows) and q + k + v (6144) with K = 4096, 16 x 2048 tokens through the three token
+    shares of the K = 4096 Hessian launches: the Linears share one Hessian and one chain, run the column loop as one
+    matrix on the block factor, and every Linear gets what its own loop gives (same chain, fuse_loops: False) up to the
+    rounding of the update GEMMs, whose kernel depends on the row count; each also satisfies the loss identity."""
+    K, nb, T = 4096, 16, 2048
+    xs = _device_batches(dev, nb, T, K, seed=2200 + len(rows))
+    Ws = {n: _weights(dev, R, K, seed=2210 + i) for i, (n, R) in enumerate(rows.items())}
+    first = next(iter(rows))
+    gp, layers, leaders, factors = _run_subset(dev, Ws, xs)
+    assert leaders == {n: first for n in rows}
+    assert factors == [(True, sum(rows.values()))]
+    gp1, layers1, leaders1, factors1 = _run_subset(dev, Ws, xs, fuse_loops=False)
+    assert leaders1 == leaders and factors1 == [(True, R) for R in rows.values()]
+    H64 = _hessian_fp64(xs)
+    perm = layers[first].buf_perm
+    Hd = _damped(H64, perm)
+    for n, R in rows.items():
+        assert torch.equal(layers[n].buf_perm, perm) and torch.equal(layers1[n].buf_perm, perm)
+        assert layers[n].weight.data.shape == (R, K)
+        assert layers[n].weight.data.untyped_storage().nbytes() == R * K * 4      # no view of the stacked matrix
+        tmp, s, z = _loss_identity(layers[n], Ws[n], Hd, perm, float(gp.last_errors[n]), f'{n} stacked')
+        tmp1 = layers1[n].weight.data[:, perm]
+        s1, z1 = layers1[n].buf_scales.reshape(R, -1), layers1[n].buf_zeros.reshape(R, -1)
+        same_w = float((tmp == tmp1).float().mean())
+        agree = float((_codes(tmp, s, z) == _codes(tmp1, s1, z1)).float().mean())
+        l, l1 = float(gp.last_errors[n]), float(gp1.last_errors[n])
+        print(f'{n}: stacked vs alone: weights bit-equal on {same_w:.6f}, codes equal on {agree:.6f}, losses {l:.6g} / {l1:.6g}')
+        assert agree >= 0.999, (n, agree)
+        assert float(torch.isclose(s, s1, rtol=1e-3).float().mean()) >= 0.995
+        assert abs(l - l1) <= 1e-4 * l1
+
+
+def test_block_factor_at_K14336_rebuilds_the_damped_hessian(dev):
+    """lcq_chol_block_factor on the act-ordered, lognormal-scaled K = 14336 Hessian, as subset_transform calls it.  With
+    H_d = M M^T (M upper triangular, positive diagonal: unique) the factor holds P[b, b] = (M[b, b])^-1 and
+    P[p, b] = M[p, b] P[b, b] for p < b, 128-column blocks.  Rebuilding M from P in fp64 (the 112 diagonal blocks are
+    inverted by LAPACK on the host) and multiplying it out must give H_d back."""
+    from lightcompress_amd import _lib as L
+    K, nb, T, NBLK = 14336, 8, 2048, 128
+    xs = _device_batches(dev, nb, T, K, seed=2300)
+    gp = make_gptq(actorder=True)
+    layer = Layer(torch.zeros(8, K, device=dev, dtype=torch.bfloat16))
+    gp.subset_init({'layers': {'d': layer}})
+    for x in xs:
+        gp.add_batch(layer, 'd', x.unsqueeze(0).data, None)
+    H = gp.hessian('d').clone()
+    H64 = _hessian_fp64(xs)
+    del xs
+    assert float((H.double() - H64).abs().max() / H64.abs().max()) < 1e-5
+    perm = torch.argsort(torch.diag(H), descending=True)
+    lib = L.lib()
+    nbytes = lib.lcq_chol_inv_upper_workspace_bytes(L.i64(K))
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    status = torch.ones(1, dtype=torch.int32, device=dev)
+    P = torch.empty(K, K, device=dev)
+    L.check(lib.lcq_chol_block_factor(L.ptr(H), L.i64(K), L.ptr(perm), L.f32(0.01), L.ptr(None), L.i64(0), L.ptr(P), L.ptr(ws),
+                                      L.i64(nbytes), L.ptr(status), L.stream()), 'lcq_chol_block_factor')
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0
+    del ws, H
+    assert torch.equal(torch.triu(P), P) and bool(torch.isfinite(P).all())
+    nblk = K // NBLK
+    diag = torch.stack([P[b * NBLK:(b + 1) * NBLK, b * NBLK:(b + 1) * NBLK] for b in range(nblk)]).double()
+    assert bool((torch.diagonal(diag, dim1=1, dim2=2) > 0).all())
+    eye = torch.eye(NBLK, dtype=torch.float64).expand(nblk, NBLK, NBLK)
+    Mbb = torch.linalg.solve_triangular(diag.cpu(), eye, upper=True).to(dev)           # (P[b, b])^-1 = M[b, b]
+    M = torch.empty(K, K, dtype=torch.float64, device=dev)
+    for b in range(nblk):
+        sl = slice(b * NBLK, (b + 1) * NBLK)
+        M[:, sl] = P[:, sl].double() @ Mbb[b]
+        M[sl, sl] = Mbb[b]
+    del P
+    Hd = _damped(H64, perm)
+    del H64
+    scale = float(Hd.abs().max())
+    res = M @ M.t()
+    res -= Hd
+    rel = float(res.abs().max()) / scale
+    fro = float(res.norm() / Hd.norm())
+    print(f'K={K}: M rebuilt from the block factor: max|M M^T - H_d| / max|H_d| = {rel:.3e}, Frobenius {fro:.3e}')
+    assert rel < 2e-5 and fro < 2e-5, (rel, fro)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# AWQ search at 4096 / 11008 with 128 x 512 tokens
+# ---------------------------------------------------------------------------------------------------------------
+class _Fc:
+    def __init__(self, w):
+        self.weight = types.SimpleNamespace(data=w)
+
+
+def test_awq_search_at_full_size(dev):
+    from lightcompress_amd.awq import Awq
+    Hd, I = 4096, 11008
+    spec = Q.IntSpec(4, False, 'per_group', group_size=128)
+    w = {'gate': (torch.randn(I, Hd, generator=gen(31)) * 0.02).bfloat16(), 'up': (torch.randn(I, Hd, generator=gen(32)) * 0.02).bfloat16()}
+    down = (torch.randn(Hd, I, generator=gen(33)) * 0.02).bfloat16().to(dev)
+    g = torch.Generator(device=dev)
+    g.manual_seed(34)
+    x = (torch.randn(128, 512, Hd, device=dev, generator=g) * torch.exp(torch.randn(Hd, device=dev, generator=g))).bfloat16()
+    layers = {k: _Fc(v.to(dev)) for k, v in w.items()}
+    F = torch.nn.functional
+
+    def mlp(xx, gate=None, up=None):
+        gate = layers['gate'].weight.data if gate is None else gate
+        up = layers['up'].weight.data if up is None else up
+        return (F.silu(xx @ gate.t()) * (xx @ up.t())) @ down.t()
+    awq = Awq({'weight': dict(bit=4, symmetric=False, granularity='per_group', group_size=128), 'special': {}})
+    best = awq.search_scale_subset(None, layers, [x], mlp, False, {})
+    losses = awq.search_losses.cpu()
+    assert best.shape == (Hd,) and best.dtype == torch.bfloat16
+    assert bool(torch.isfinite(losses).all()) and bool((losses > 0).all())
+    for k in w:                                                     # the layer weights are the originals again
+        assert torch.equal(layers[k].weight.data.cpu(), w[k])
+    # the scale normalisation: max * min == 1 up to the bf16 rounding of the division (awq.py:100-102)
+    prod = float(best.float().max() * best.float().min())
+    assert abs(prod - 1.0) < 2 ** -6, prod
+    # grid point 0 has ratio 0, every scale is 1 and x / 1 is x: its loss is that of plain round-to-nearest weights.
+    # The weights come from the CPU oracle at full size, the forward and the loss from torch ops on the device.
+    rtn = {k: Q.int_fake_quant_dynamic(spec, v).to(dev) for k, v in w.items()}
+    org = mlp(x)
+    out = mlp(x, rtn['gate'], rtn['up'])
+    want = float((org - out).float().pow(2).mean())
+    print(f'AWQ full size: loss at ratio 0 {float(losses[0]):.8g}, plain RTN with torch ops {want:.8g}; best grid point '
+          f'{int(torch.argmin(losses))}')
+    assert abs(float(losses[0]) - want) <= 1e-5 * want
+    assert float(losses.min()) <= float(losses[0])
+    # the chosen scales give back the stored loss of their grid point when evaluated with torch ops
+    kbest = int(torch.argmin(losses))
+    wq = {k: awq._scale_quant(layers[k].weight.data, best) for k in w}
+    xs = awq.scaling_input(x, best, False)
+    again = float((org - mlp(xs, wq['gate'], wq['up'])).float().pow(2).mean())
+    assert abs(again - float(losses[kbest])) <= 1e-5 * again
+    # slices of the full-size kernel outputs against the CPU oracle, bit for bit
+    bc = best.cpu()
+    for k in w:
+        for r0 in (0, 5376, I - 256):
+            assert_bit_equal(wq[k][r0:r0 + 256], A.scale_and_fake_quant(w[k][r0:r0 + 256], bc, spec), f'{k}[{r0}:+256] W*s -> fake quant')
+    for b, t0 in ((0, 0), (77, 130), (127, 256)):
+        assert_bit_equal(xs[b, t0:t0 + 256], A.scaling_input(x[b, t0:t0 + 256].cpu(), bc), f'x[{b}, {t0}:+256] / s')
+    xm = awq.get_act_scale(x).cpu().double()
+    ref = x.double().abs().reshape(-1, Hd).mean(0).cpu()
+    assert float(((xm - ref).abs() / ref).max()) <= 2 ** -8
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# float8 / int4 + pack at the expert shapes, per-token float8 of the 8192 x 7168 activations
+# ---------------------------------------------------------------------------------------------------------------
+def test_one_full_expert_and_the_full_activation_tensor(dev):
+    from lightcompress_amd import FloatQuantizer, IntegerQuantizer
+    from lightcompress_amd.module_utils import VllmRealQuantLinear
+    fq = FloatQuantizer('e4m3', True, 'per_channel', use_qtorch=True)
+    iq = IntegerQuantizer(4, True, 'per_group', group_size=128)
+    fs, isp = Q.FloatSpec('e4m3', 'per_channel'), Q.IntSpec(4, True, 'per_group', group_size=128)
+    torch.set_num_threads(16)
+    for name, shape, seed in (('gate', (2048, 7168), 0), ('up', (2048, 7168), 1), ('down', (7168, 2048), 2)):
+        w = weight_like(*shape, seed=seed, dtype=torch.bfloat16, std=0.006, outlier_frac=0.0005, outlier_mul=30)
+        wd = w.to(dev)
+        codes, s, z = fq.real_quant_weight_dynamic(wd)
+        oc, os_, _ = Q.float_real_quant_dynamic(fs, w)
+        assert z is None and codes.dtype == torch.float8_e4m3fn and s.shape == (shape[0], 1)
+        assert_bit_equal(codes, oc, f'{name}: fp8 codes')
+        assert_bit_equal(s, os_, f'{name}: fp8 scales')
+        assert float(codes.float().abs().max()) == 448.0
+        packed, s16 = VllmRealQuantLinear.quant_pack_fused(wd, iq, {'weight': {'bit': 4}})
+        ic, is_, _ = Q.int_real_quant_dynamic(isp, w)
+        op, os16 = pack_ref.pack_ct(ic, is_, 4)
+        assert packed.shape == (shape[0], shape[1] // 8) and packed.dtype == torch.int32
+        assert_bit_equal(packed, op, f'{name}: int4 packed words')
+        assert_bit_equal(s16, os16, f'{name}: fp16 scales')
+        assert torch.equal(pack_ref.unpack_ct(packed.cpu(), 4, shape[1]), ic.to(torch.int32))
+    # activations: the whole tensor on the device, slices of the result against the oracle
+    g = torch.Generator(device=dev)
+    g.manual_seed(5)
+    act = (torch.randn(8192, 7168, device=dev, generator=g) * torch.exp(torch.randn(7168, device=dev, generator=g))).bfloat16()
+    aq = FloatQuantizer('e4m3', True, 'per_token', use_qtorch=True)
+    got = aq.fake_quant_act_dynamic(act)
+    assert got.shape == act.shape and got.dtype == torch.bfloat16 and bool(torch.isfinite(got).all())
+    aspec = Q.FloatSpec('e4m3', 'per_token')
+    for r0 in (0, 3840, 8192 - 512):
+        assert_bit_equal(got[r0:r0 + 512], Q.float_fake_quant_dynamic(aspec, act[r0:r0 + 512].cpu()), f'activation rows {r0}:+512')
+    # the whole tensor: at most 2^-4 relative error per element inside the normal range (3 mantissa bits), row maxima kept
+    rel = ((got.float() - act.float()).abs() / act.float().abs().clamp(min=1e-30))
+    big = act.float().abs() >= act.float().abs().amax(dim=1, keepdim=True) * 2 ** -8
+    assert float(rel[big].max()) <= 2 ** -4 + 2 ** -7
+    assert float((got.float().abs().amax(dim=1) / act.float().abs().amax(dim=1) - 1).abs().max()) <= 2 ** -7

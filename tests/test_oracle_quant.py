@@ -405,6 +405,44 @@ def test_mse_range_oracle_recurrence_and_optimality():
         assert err_of(row, mn[r], mx[r]) <= err_of(row, row.min(), row.max()) * (1 + 1e-6)
 
 
+def test_float_mse_range_oracle_recurrence_and_optimality():
+    """The same pins for the minifloat quantizer's mse range: a per-row Python loop written from the recurrence, with
+    the rounding done by a nearest-point search over the enumerated e4m3 grid (exponents -6 .. 8, so 480 follows 448
+    and larger quotients saturate there - a shrunken range pushes quotients past 448; random data has no ties),
+    reproduces the vectorised restatement; the range never widens and its error never exceeds plain min/max's."""
+    spec = Q.FloatSpec('e4m3', 'per_channel', tie='even')
+    w = weight_like(12, 256, seed=93, std=0.006, outlier_frac=0.01, outlier_mul=30)
+    mn, mx = Q.float_mse_range(spec, w.clone())
+    assert mn.dtype == torch.float32 and mn.shape == (12, 1)
+    pos = [m / 8 * 2.0 ** -6 for m in range(8)] + [(1 + m / 8) * 2.0 ** e for e in range(-6, 9) for m in range(8)]
+    grid = torch.tensor(sorted(set(pos) | {-v for v in pos}), dtype=torch.float64)
+    assert float(grid.max()) == 480.0
+    def err_of(row, lo, hi):
+        s = max(abs(float(lo)), abs(float(hi)), 1e-5)
+        s = torch.tensor(s, dtype=torch.float32) / 448.0
+        t = (row / s).double()
+        q = grid[(t[:, None] - grid[None, :]).abs().argmin(1)].float() * s
+        return float((q - row).abs().pow(2.4).sum())
+    for r in range(12):
+        row = w[r].float()
+        lo, hi, best = row.min(), row.max(), float('inf')
+        for i in range(80):
+            p = 1 - i / 100
+            xlo, xhi = p * lo, p * hi
+            e = err_of(row, xlo, xhi)
+            if e < best:
+                best, lo, hi = e, xlo, xhi
+        assert abs(float(lo) - float(mn[r])) <= 1e-6 * abs(float(lo)) and abs(float(hi) - float(mx[r])) <= 1e-6 * abs(float(hi))
+        assert float(mn[r]) >= float(row.min()) and float(mx[r]) <= float(row.max())
+        assert err_of(row, mn[r], mx[r]) <= err_of(row, row.min(), row.max()) * (1 + 1e-6)
+    # learnable ranges: sigmoid(factor) = 1/2 halves the symmetric range; no factors -> plain min / max
+    lo, hi = Q.learnable_range(spec, w, upbound_factor=torch.zeros(12, 1))
+    assert torch.equal(hi, 0.5 * torch.max(w.amax(1, keepdim=True).abs(), w.amin(1, keepdim=True).abs()).clamp(min=1e-5))
+    assert torch.equal(lo, -hi)
+    lo, hi = Q.learnable_range(spec, w)
+    assert torch.equal(lo, w.amin(1, keepdim=True)) and torch.equal(hi, w.amax(1, keepdim=True))
+
+
 # ---- secondary calibrators: HQQ, static activation ranges, W4-over-W8 ---------------------------------------
 def test_hqq_shrink_is_the_soft_threshold_and_fixed_points_hold():
     """Pins for hqq_optimize (quant.py:587-609) that do not restate it:

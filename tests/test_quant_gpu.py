@@ -408,6 +408,50 @@ def test_blockwise_fp8_casts_bit_exact(dev, dtype, shape):
 
 
 @pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('fmt,gran,shape,tie', [('e4m3', 'per_channel', (48, 1024), 'away'), ('e4m3', 'per_group', (16, 512), 'even'),
+                                                ('e2m1', 'per_group', (32, 256), 'away')])
+def test_float_quantizer_with_mse_and_learnable_ranges(dev, dtype, fmt, gran, shape, tie):
+    """FloatQuantizer with calib_algo 'mse' / 'learnable' (the range dispatch of quant.py:124-132 is shared by both
+    quantizer classes).  The mse search sums |d|**2.4 through another pow and another summation order than the CPU's,
+    so a step that ties with the running best within ~1e-6 may be accepted on one side only: the ranges agree on
+    >= 98 % of the rows, the others are as good within 0.1 %; given the ranges, fake and real quantization are the
+    bit-exact static path."""
+    from lightcompress_amd import FloatQuantizer
+    kw = dict(group_size=128) if gran == 'per_group' else {}
+    w = weight_like(*shape, seed=shape[1] + 3, dtype=dtype, std=0.006, outlier_frac=0.002, outlier_mul=30)
+    spec = Q.FloatSpec(fmt, gran, group_size=kw.get('group_size', 0), tie=tie)
+    q = FloatQuantizer(fmt, True, gran, use_qtorch=True, fp_tie=tie, calib_algo='mse', **kw)
+    rows = Q.reshape_rows(spec, w)
+    omn, omx = Q.float_mse_range(spec, rows.clone())
+    mn, mx = q.get_mse_range(q.reshape_tensor(w.to(dev)))
+    assert mn.dtype == torch.float32 and mn.shape == omn.shape
+    same = ((mn.cpu() - omn).abs() <= 1e-6 * omn.abs()) & ((mx.cpu() - omx).abs() <= 1e-6 * omx.abs())
+    assert float(same.float().mean()) >= 0.98, float(same.float().mean())
+    def err(lo, hi):
+        s, z, _, _ = Q.float_qparams(spec, lo, hi)
+        return (Q.float_dequant(Q.float_quant(spec, rows.float(), s, z), s, z) - rows.float()).abs().pow(2.4).sum(1)
+    assert bool((err(mn.cpu(), mx.cpu()) <= err(omn, omx) * 1.001 + 1e-30).all())
+    got = q.fake_quant_weight_dynamic(w.to(dev))
+    assert got.dtype == dtype
+    assert_bit_equal(got, Q.float_fake_quant_with_range(spec, w, mn.cpu(), mx.cpu()), 'fake quant with the mse ranges')
+    if fmt == 'e4m3':
+        codes, s, z = q.real_quant_weight_dynamic(w.to(dev))
+        os_, oz, _, _ = Q.float_qparams(spec, mn.cpu(), mx.cpu())
+        assert z is None and codes.dtype == torch.float8_e4m3fn
+        assert_bit_equal(codes, Q.restore_rows(spec, Q.float_quant(spec, rows, os_.clone(), oz), w.shape).to(torch.float8_e4m3fn), 'fp8 codes')
+        assert_bit_equal(s, os_.view(w.shape[0], -1), 'fp8 scales')
+    # learnable: the given factors scale the symmetric range, everything after is the static path
+    ql = FloatQuantizer(fmt, True, gran, use_qtorch=True, fp_tie=tie, calib_algo='learnable', **kw)
+    up = torch.randn(rows.shape[0], 1, generator=gen(7)).to(dtype) + 2
+    lo, hi = Q.learnable_range(spec, rows, upbound_factor=up)
+    got = ql.fake_quant_weight_dynamic(w.to(dev), {'upbound_factor': up.to(dev)})
+    assert_bit_equal(got, Q.float_fake_quant_with_range(spec, w, lo, hi), 'fake quant with learnable ranges')
+    assert_bit_equal(ql.fake_quant_weight_dynamic(w.to(dev)), Q.float_fake_quant_dynamic(spec, w), 'learnable without factors')
+    with pytest.raises(NotImplementedError):
+        FloatQuantizer(fmt, True, gran, use_qtorch=True, calib_algo='hqq', **kw).fake_quant_weight_dynamic(w.to(dev))
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize('bit,sym,gran,shape', [(4, False, 'per_group', (64, 1024)), (4, True, 'per_group', (32, 512)),
                                                  (8, False, 'per_channel', (48, 777)), (3, False, 'per_group', (16, 256))])
 def test_mse_calibration_against_oracle(dev, dtype, bit, sym, gran, shape):
