@@ -51,7 +51,7 @@ def lib() -> C.CDLL:
         _lib = C.CDLL(str(LIB_PATH))
         for name in declared_symbols():
             fn = getattr(_lib, name)
-            fn.restype = C.c_int64 if name.endswith('_bytes') else C.c_int
+            fn.restype = C.c_int64 if name.endswith('_workspace_bytes') else C.c_int
     return _lib
 
 
