@@ -181,13 +181,18 @@ __global__ __launch_bounds__(256) void build_gather_kernel(const float* __restri
 //   * wave 5 inverts the 16x16 diagonal block of the previous panel meanwhile (forward substitution in registers);
 //   * afterwards all 8 waves merge the inverted diagonal blocks pairwise, 16 -> 32 -> 64 -> 128,
 //     [[A,0],[B,C]]^-1 = [[A^-1,0],[-C^-1 B A^-1, C^-1]], from LDS.
-constexpr int lds_slot(int r) { return (r & 15) * 8 + (r >> 4); }   // a thread's 8 rows (columns) are contiguous
+// Row (column) r of the block lives at float `lds_slot(r)` of an LDS row.  Thread t of the 16 x 16 update grid owns rows
+// t + 16 ii, ii < 8: the first four sit at 4 t .. 4 t + 3 and the other four at 64 + 4 t .., so both 16-byte pieces of
+// a thread are contiguous with its neighbours' (no bank conflicts for 16-byte accesses), and 16 consecutive rows are 16
+// bytes apart (none for the 4-byte accesses of the panel wave and of the matrix-pipe operand reads either).
+constexpr int lds_slot(int r) { return ((r >> 4) < 4) ? 4 * (r & 15) + (r >> 4) : 64 + 4 * (r & 15) + (r >> 4) - 4; }
 constexpr int LP = NB + 4;       // row pitch of the LDS matrices (16-byte aligned rows, 4-bank skew)
 
 struct PotrfLds {
   float L[8][16][LP];    // L[P][k][lds_slot(r)] = L(r, 16 P + k); zero above the diagonal inside the panel's own 16 rows
   float X[NB][LP];       // L^-1, row-major
-  float Pn[16][NB];      // the panel on its way to the panel wave, same layout as L[P], unscaled
+  float Pn[16][LP];      // the panel on its way to the panel wave, same layout as L[P], unscaled (padded rows: the 16
+                         // rows a publishing wave writes at once fall into different banks)
   float T[64 * 64];      // products of the inverse merges
 };
 
@@ -264,14 +269,14 @@ __device__ __forceinline__ void potrf_update(const PotrfLds& s, float (&a)[8][8]
   if constexpr (CC_LO < 8) {
     #pragma unroll 2
     for (int k = 0; k < 16; ++k) {
-      const f32x4 r0 = *(const f32x4*)(s.L[PL][k] + 8 * ty), r1 = *(const f32x4*)(s.L[PL][k] + 8 * ty + 4);
+      const f32x4 r0 = *(const f32x4*)(s.L[PL][k] + 4 * ty), r1 = *(const f32x4*)(s.L[PL][k] + 64 + 4 * ty);
       const float lr[8] = {r0[0], r0[1], r0[2], r0[3], r1[0], r1[1], r1[2], r1[3]};
       if constexpr (ONE) {
-        const float lc = s.L[PL][k][8 * tx + CC_LO];
+        const float lc = s.L[PL][k][(CC_LO < 4 ? 4 * tx + CC_LO : 64 + 4 * tx + CC_LO - 4)];
         #pragma unroll
         for (int ii = CC_LO; ii < 8; ++ii) a[ii][CC_LO] -= lr[ii] * lc;
       } else {
-        const f32x4 c0 = *(const f32x4*)(s.L[PL][k] + 8 * tx), c1 = *(const f32x4*)(s.L[PL][k] + 8 * tx + 4);
+        const f32x4 c0 = *(const f32x4*)(s.L[PL][k] + 4 * tx), c1 = *(const f32x4*)(s.L[PL][k] + 64 + 4 * tx);
         const float lc[8] = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
         #pragma unroll
         for (int cc = CC_LO; cc < 8; ++cc)
@@ -288,8 +293,8 @@ __device__ __forceinline__ void potrf_publish(PotrfLds& s, const float (&a)[8][8
   float v[8];
   #pragma unroll
   for (int ii = 0; ii < 8; ++ii) v[ii] = (ty + 16 * ii >= tx + 16 * PC) ? a[ii][PC] : 0.0f;
-  *(f32x4*)(s.Pn[tx] + 8 * ty) = f32x4{v[0], v[1], v[2], v[3]};
-  *(f32x4*)(s.Pn[tx] + 8 * ty + 4) = f32x4{v[4], v[5], v[6], v[7]};
+  *(f32x4*)(s.Pn[tx] + 4 * ty) = f32x4{v[0], v[1], v[2], v[3]};
+  *(f32x4*)(s.Pn[tx] + 64 + 4 * ty) = f32x4{v[4], v[5], v[6], v[7]};
 }
 
 // panel P of the sweep, all 8 waves
@@ -428,17 +433,8 @@ __global__ __launch_bounds__(512) void potrf_diag_kernel(float* __restrict__ Abl
     for (int e = 0; e < 4; ++e) x[e] = (r < nb && c4 + e <= r) ? x[e] : 0.0f;
     *(f32x4*)(Dinv + r * NB + c4) = x;
   }
-  #pragma unroll
-  for (int q = 0; q < 4; ++q) {                             // L back into the block, in the update waves' cyclic order
-    const int cc = 2 * q + (tid >> 8), c = tx + 16 * cc;
-    const f32x4 r0 = *(const f32x4*)(s.L[cc][tx] + 8 * ty), r1 = *(const f32x4*)(s.L[cc][tx] + 8 * ty + 4);
-    const float l[8] = {r0[0], r0[1], r0[2], r0[3], r1[0], r1[1], r1[2], r1[3]};
-    #pragma unroll
-    for (int ii = 0; ii < 8; ++ii) {
-      const int r = ty + 16 * ii;
-      if (r < nb && c < nb) Ablk[(long long)r * lda + c] = (c <= r) ? l[ii] : 0.0f;
-    }
-  }
+  // (L itself is not written back: everything after this kernel works with the inverse, the solved panels and the
+  // blocks behind them; place_diag_kernel puts the inverse where the block was.)
 }
 
 // copy the inverted diagonal blocks into place
