@@ -45,6 +45,13 @@ using namespace lcq;
 
 constexpr int BS = 128;          // columns per block (lazy batch)
 constexpr int ROWS_PER_WG = 16;
+// Hinv1 in LDS: a row holds, for each of the 16 lanes of a team, the first four of the lane's eight columns at
+// float 4 t and the other four at UH + 4 t, so the two 16-byte reads of a team are each one contiguous run (no bank
+// conflicts); the second half starts 4 floats past a multiple of 64 so that a wave's 16-byte stores, which alternate
+// between the halves while the block is loaded, do not collide either.
+constexpr int UH = 68;           // offset of the second halves inside a row
+constexpr int UP = 136;          // row pitch (floats)
+__device__ __forceinline__ int us_col(int c) { return ((c & 4) ? UH : 0) + 4 * (c >> 3) + (c & 3); }
 
 struct LoopArgs {
   float* W; float* tmp; float* Losses; float* Err; const float* U;
@@ -119,7 +126,7 @@ __device__ __forceinline__ ColQ open_group(const LoopArgs& a, int idx, int lane,
 template <bool STATIC, bool OCT>
 __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
   constexpr int NP = OCT ? 16 : BS;              // parameter slots of a row: one per octet, or one per column
-  __shared__ float Us[BS * BS];                  // Hinv1 = U[i1:i2, i1:i2] above the diagonal, zero everywhere else
+  __shared__ float Us[BS * UP];                  // Hinv1 = U[i1:i2, i1:i2] above the diagonal, zero everywhere else (us_col layout)
   __shared__ float Rd[BS];                       // 1 / U[i, i]
   __shared__ float Dg[BS];                       // U[i, i]
   __shared__ float Ps[STATIC ? 1 : ROWS_PER_WG * NP], Pz[STATIC ? 1 : ROWS_PER_WG * NP];   // scale, zero point in force
@@ -143,7 +150,7 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
       const int e = tid + 256 * j, r = e >> 5, c = (e & 31) * 4;
       #pragma unroll
       for (int k = 0; k < 4; ++k) if (c + k <= r) v[j][k] = 0.0f;
-      *(f32x4*)(Us + e * 4) = v[j];
+      *(f32x4*)(Us + r * UP + us_col(c)) = v[j];
     }
   } else {
     for (int e = tid; e < BS * BS / 4; e += 256) {
@@ -154,7 +161,7 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
         #pragma unroll
         for (int k = 0; k < 4; ++k) if (c + k < a.count && c + k > r) v[k] = p[k];
       }
-      *(f32x4*)(Us + e * 4) = v;
+      *(f32x4*)(Us + r * UP + us_col(c)) = v;
     }
   }
   if (tid < BS) {
@@ -213,12 +220,12 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
     ++n_oct;
     // the octet's 8 rows of U (this lane's 8 columns of each) and reciprocal diagonals, fetched ahead of the
     // dependency chain; rows past `count` are zero in LDS, so the 8 columns need no bound check
-    const float* ucol = Us + (8 * to) * BS + 8 * ((lane + to) & 15);
+    const float* ucol = Us + (8 * to) * UP + 4 * ((lane + to) & 15);
     f32x4 u0[8], u1[8];
     #pragma unroll
     for (int c = 0; c < 8; ++c) {
-      u0[c] = *(const f32x4*)(ucol + c * BS);
-      u1[c] = *(const f32x4*)(ucol + c * BS + 4);
+      u0[c] = *(const f32x4*)(ucol + c * UP);
+      u1[c] = *(const f32x4*)(ucol + c * UP + UH);
     }
     const f32x4 rda = *(const f32x4*)(Rd + 8 * to), rdb = *(const f32x4*)(Rd + 8 * to + 4);
     const float rd[8] = {rda[0], rda[1], rda[2], rda[3], rdb[0], rdb[1], rdb[2], rdb[3]};
