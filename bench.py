@@ -47,14 +47,36 @@ CFG = {'weight': dict(bit=4, symmetric=False, granularity='per_group', group_siz
        'special': dict(actorder=True, static_groups=False, percdamp=0.01, blocksize=128, true_sequential=True)}
 
 
-def traffic_bytes(key):
+def _sha16(path):
+    import hashlib
+    try:
+        with open(os.path.join(ROOT, path), 'rb') as f:
+            return hashlib.sha256(f.read()).hexdigest()[:16]
+    except OSError:
+        return None
+
+
+def traffic_bytes(key, launch_us=None):
     """HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, kept in
-    profiles/traffic.json next to the summaries that derive them (counters cannot be read inside the timed process)."""
+    profiles/traffic.json next to the summaries that derive them (counters cannot be read inside the timed process).
+    The entry carries the launch duration of the run it was taken at and a hash of the kernel's source file:
+    -> (bytes, stale) with stale = True when the source has changed since, or when this run's launch duration
+    differs from the recorded one by more than 10 %."""
     try:
         with open(os.path.join(ROOT, 'profiles', 'traffic.json')) as f:
-            return json.load(f).get(key, {}).get('bytes')
+            e = json.load(f).get(key, {})
     except (OSError, ValueError):
-        return None
+        return None, None
+    if 'bytes' not in e:
+        return None, None
+    stale = False
+    if e.get('source') and e.get('source_sha256_16') and _sha16(e['source']) != e['source_sha256_16']:
+        stale = True
+    if launch_us and e.get('launch_us') and abs(launch_us - e['launch_us']) > 0.1 * e['launch_us']:
+        stale = True
+    if not e.get('launch_us') or not e.get('source_sha256_16'):
+        stale = True                                      # an entry without its stamp cannot be tied to this kernel
+    return e['bytes'], stale
 
 
 class Layer:
@@ -179,7 +201,14 @@ def bench_layer(args, out):
         one_layer(False)
     torch.cuda.synchronize()
     dt_separate = (time.perf_counter() - t0) / args.steps
-    out.update({'value': round(dt, 4), 'ms_per_step': round(dt * 1e3, 2), 'seconds_separate_hessians': round(dt_separate, 4),
+    out.update({'value': round(dt, 4), 'ms_per_step': round(dt * 1e3, 2),
+                'value_is': 'seconds_shared_hessians: Linears handed the identical tensor (q/k/v, gate/up) accumulate ONE Hessian '
+                            '(4 accumulations and 4 Cholesky chains per layer, every shared call verified bit for bit on the device); '
+                            'results are bit-identical to separate accumulation',
+                'seconds_shared_hessians': round(dt, 4),
+                'seconds_separate_hessians': round(dt_separate, 4),
+                'seconds_separate_hessians_is': 'like for like with the reference: 7 Hessian accumulations and 7 chains per layer '
+                                                '(special.auto_share: False); compare THIS figure with a reference run',
                 'last_error': last_error, 'breakdown_ms': phases})
     return streams['down_in']
 
@@ -213,10 +242,11 @@ def bench_hessian(args, out, x=None):
     alg_flops = 2.0 * TL * K * K
     tiles = sum(K // 128 - 2 * ti for ti in range(K // 256))          # 256x128 tiles that reach the upper triangle
     exe_flops = 2.0 * TL * tiles * 256 * 128
+    traffic, stale = traffic_bytes('hessian_kernel_K14336_T8192', t_h * 1e6) if FOLD == 4 else (None, None)
     out['roofline'] = {
         'kernel': f'hessian_kernel<bf16> K=14336 T={TL}', 'bound': 'mfma', 'achieved': round(exe_flops / t_h / 1e12, 2),
         'peak': 2500.0, 'unit': 'TFLOP/s', 'frac': round(exe_flops / t_h / 2.5e15, 4),
-        'traffic': traffic_bytes('hessian_kernel_K14336_T8192') if FOLD == 4 else None,
+        'traffic': traffic, 'traffic_stale': stale,
         'launch_us': round(t_h * 1e6, 2), 'flop_executed_per_launch': exe_flops,
         'algorithmic_tflops': round(alg_flops / t_h / 1e12, 2), 'frac_algorithmic': round(alg_flops / t_h / 2.5e15, 4),
         'library_gemm': {'what': 'torch.matmul(X.t(), X), bf16, the whole K x K product on the same tokens (hipBLASLt)',
@@ -305,9 +335,10 @@ def bench_quantizers(args, out):
     n, g = 4096 * 4096, 128
     t = timeit(quant_int(xs, n // g, g, 0, 15, 0, dq, cds, L.CODE_U8), 60, 25)
     r = report('RTN int4 asym g128, fp32 4096x4096 -> dq + u8 codes + scales/zeros', 'row_team_kernel<IntOp<f32>>', n * 4, n * 5 + n // g * 8, t)
+    traffic, stale = traffic_bytes('rtn_quant_int4_g128_4096x4096_f32', r['us'])
     out['roofline_quantizer'] = {'kernel': 'row_team_kernel<IntOp<f32>> 4096x4096 g128 dq+u8', 'bound': 'hbm', 'achieved': r['GB/s'],
                                  'peak': 8000.0, 'unit': 'GB/s', 'frac': r['frac'],
-                                 'traffic': traffic_bytes('rtn_quant_int4_g128_4096x4096_f32'), 'launch_us': r['us']}
+                                 'traffic': traffic, 'traffic_stale': stale, 'launch_us': r['us']}
     t = timeit(quant_int(xs, n // g, g, 0, 15, 0, dq), 60, 25)
     report('RTN int4 asym g128 fake quant, fp32 4096x4096', 'row_team_kernel<IntOp<f32>>', n * 4, n * 4 + n // g * 8, t)
     del xs, dq, cds

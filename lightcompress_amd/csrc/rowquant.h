@@ -498,7 +498,7 @@ int dispatch_rows(const void* x, int64_t rows, int64_t cols, void* dq, void* cod
   else if (nchunks <= 4) LCQ_TEAM(1, 4, 1);
   else if (nchunks <= 8) LCQ_TEAM(2, 4, 1);
   else if (nchunks <= 16) LCQ_TEAM(8, 2, 1);       // 8 lanes x 16 B: whole 128-byte lines per row and instruction
-  else if (nchunks <= 32) LCQ_TEAM(8, 4, 1);
+  else if (nchunks <= 32) { if constexpr (Op::BF) LCQ_TEAM(8, 4, 1); else LCQ_TEAM(8, 4, 2); }   // fp32 rows of 512 bytes: two rows per team in flight (25.6 -> 23.9 us on 4096 x 4096; four are slower again)
   else if (nchunks <= 64) LCQ_TEAM(16, 4, 1);
   else if (nchunks <= 128) LCQ_TEAM(32, 4, 1);
   else if (nchunks <= 256) LCQ_TEAM(64, 4, 1);

@@ -384,6 +384,18 @@ class BaseQuantizer(object):
             qmax_list.append(qmax)
         return scales_list, zeros_list, qmin_list, qmax_list
 
+    # -- several experts in one launch --------------------------------------------------------------
+    def real_quant_weight_dynamic_experts(self, weights, args={}):
+        """real_quant_weight_dynamic of every matrix in `weights` (equal shapes) with ONE launch over their stacked
+        rows -> list of (codes, scales, zeros) per expert, bit-identical to separate calls.  per_channel / per_group."""
+        if self.granularity not in ('per_channel', 'per_group'):
+            raise NotImplementedError('experts are stacked along the rows: per_channel / per_group only')
+        E, (R, K) = len(weights), weights[0].shape
+        codes, scales, zeros = self.real_quant_weight_dynamic(experts_as_rows(weights), dict(args))
+        cs, ss = codes.view(E, R, -1), scales.view(E, R, -1)
+        zs = None if zeros is None else zeros.view(E, R, -1)
+        return [(cs[e], ss[e], None if zs is None else zs[e]) for e in range(E)]
+
     # -- HQQ (quant.py:587-609) -----------------------------------------------------------------
     def optimize_weights_proximal(self, tensor, scales, zeros, qmax, qmin):
         """Half-quadratic zero-point refinement: every iteration is one fused pass (lcq_hqq_step) where the
@@ -468,6 +480,21 @@ class BaseQuantizer(object):
         except RuntimeError:
             deficiency = self.group_size - shape[1] % self.group_size
             return tensor.reshape(*shape[:-1], -1)[..., :-deficiency]
+
+
+def experts_as_rows(weights):
+    """The [R, K] matrices of several experts as one [E * R, K] matrix: a view when they lie one behind the other in
+    one tensor (slices of a stacked expert weight), a copy otherwise.  Row-wise granularities (per_channel, per_group)
+    do not care which expert a row belongs to, and one launch over 16 experts runs at 0.72 - 0.75 of the HBM peak where
+    a launch over one expert (29 MB) reaches 0.46 - 0.50: its ramp and tail are half of a 10 us kernel."""
+    w0 = weights[0]
+    if any(w.shape != w0.shape or w.dtype != w0.dtype or w.dim() != 2 for w in weights):
+        raise ValueError('experts_as_rows: 2-D matrices of one shape and type')
+    step = w0.numel() * w0.element_size()
+    if all(w.is_contiguous() and w.untyped_storage().data_ptr() == w0.untyped_storage().data_ptr()
+           and w.data_ptr() == w0.data_ptr() + i * step for i, w in enumerate(weights)):
+        return w0.as_strided((len(weights) * w0.shape[0], w0.shape[1]), (w0.shape[1], 1))
+    return torch.cat(list(weights), dim=0)
 
 
 def _rows_cols(t):
@@ -775,6 +802,15 @@ class IntegerQuantizer(BaseQuantizer):
         _, packed, scales, _ = self._launch(rows_t, static=False, want_codes='ct4')
         qparams_shape = 1 if self.granularity == 'per_tensor' else (weight.shape[0], -1)
         return packed.view(weight.shape[0], weight.shape[1] // 8), scales.view(qparams_shape), None
+
+    def real_quant_pack_dynamic_experts(self, weights):
+        """real_quant_pack_dynamic of every matrix in `weights` with one launch -> list of (packed, scales, None)."""
+        if self.granularity not in ('per_channel', 'per_group'):
+            raise NotImplementedError('experts are stacked along the rows: per_channel / per_group only')
+        E, (R, K) = len(weights), weights[0].shape
+        packed, scales, _ = self.real_quant_pack_dynamic(experts_as_rows(weights))
+        ps, ss = packed.view(E, R, -1), scales.view(E, R, -1)
+        return [(ps[e], ss[e], None) for e in range(E)]
 
     def __repr__(self):
         return (

@@ -709,3 +709,34 @@ def test_mixed_precision_indices_in_the_dynamic_paths(dev):
     want = Q.int_fake_quant_dynamic(Q.IntSpec(4, False, 'per_group', group_size=128), w[:, ii].contiguous())
     assert_bit_equal(mixed[:, ii.to(dev)], want, 'quantized weight columns')
     assert_bit_equal(mixed[:, fi.to(dev)], w[:, fi], 'weight columns kept')
+
+
+def test_experts_in_one_launch_equal_expert_by_expert(dev):
+    """Several experts through one launch (their rows stacked): float8 real quant, int4 real quant and int4 quantize +
+    pack give every expert what its own call gives, bit for bit; consecutive slices of one tensor are stacked as a view."""
+    from lightcompress_amd import FloatQuantizer, IntegerQuantizer
+    from lightcompress_amd.quant import experts_as_rows
+    E, R, K = 5, 96, 1024
+    stacked = weight_like(E * R, K, seed=77, dtype=torch.bfloat16, std=0.006, outlier_frac=0.001, outlier_mul=30).to(dev).view(E, R, K)
+    slices = [stacked[e] for e in range(E)]
+    apart = [s.clone() for s in slices]
+    assert experts_as_rows(slices).data_ptr() == stacked.data_ptr()           # a view
+    assert experts_as_rows(apart).data_ptr() not in [a.data_ptr() for a in apart]
+    assert torch.equal(experts_as_rows(apart), stacked.view(E * R, K))
+    fq = FloatQuantizer('e4m3', True, 'per_channel', use_qtorch=True)
+    iq = IntegerQuantizer(4, True, 'per_group', group_size=128)
+    ia = IntegerQuantizer(4, False, 'per_group', group_size=128)
+    for ws in (slices, apart):
+        for q in (fq, iq, ia):
+            many = q.real_quant_weight_dynamic_experts(ws)
+            for e in range(E):
+                one = q.real_quant_weight_dynamic(ws[e])
+                for a, b in zip(many[e], one):
+                    assert (a is None and b is None) or (a.shape == b.shape and torch.equal(a.view(torch.uint8) if a.dtype == torch.float8_e4m3fn else a,
+                                                                                       b.view(torch.uint8) if b.dtype == torch.float8_e4m3fn else b))
+        many = iq.real_quant_pack_dynamic_experts(ws)
+        for e in range(E):
+            one = iq.real_quant_pack_dynamic(ws[e])
+            assert torch.equal(many[e][0], one[0]) and torch.equal(many[e][1], one[1])
+    with pytest.raises(NotImplementedError):
+        IntegerQuantizer(4, True, 'per_tensor').real_quant_weight_dynamic_experts(slices)
