@@ -226,6 +226,19 @@ int lcq_split_f32_bf16(const float* x, int64_t n, void* hi, void* lo, void* stre
 int lcq_hessian_accum_sliced(float* H, int64_t K, const void* XA, const void* XB, int dtype, int64_t T, int64_t ldx,
                              float alpha, float beta, int slices, int64_t slice_stride, void* stream);
 
+/* lcq_hessian_accum_ab with the last round of workgroups filled.  A launch has one workgroup per 256 x 128 tile that
+ * reaches the upper triangle and the chip runs 2 x CUs of them at a time; when the tiles are several such rounds and a
+ * small rest (K = 14336: 3192 tiles = 6 rounds of 512 and 120), the rest keeps a quarter of the chip busy for the time of a
+ * whole tile.  Here every tile of the rest is cut into 2..8 token ranges that run side by side: the first updates H like
+ * any tile, the others leave their beta * XA^T XB in the workspace, and a second small launch adds them to H in a fixed
+ * order (results are reproducible; they differ from lcq_hessian_accum_ab's by the order of fp32 additions).
+ * lcq_hessian_balanced_workspace_bytes(K, T) is the workspace this takes for a launch of T tokens, 0 where no split
+ * pays (K not in whole 256-column tiles, T not in whole 32-token slabs, fewer than two rounds, or a rest that fills
+ * half a round anyway): the call then is lcq_hessian_accum_ab and takes a NULL workspace.  Workspace 16-byte aligned. */
+int64_t lcq_hessian_balanced_workspace_bytes(int64_t K, int64_t T);
+int lcq_hessian_accum_balanced(float* H, int64_t K, const void* XA, const void* XB, int dtype, int64_t T, int64_t ldx, float alpha,
+                               float beta, void* workspace, int64_t workspace_bytes, void* stream);
+
 /* H_0 <- ((H_0 + H_1) + H_2) + ... and H_s <- 0 for s >= 1, over all K*K entries: the shares of
  * lcq_hessian_accum_sliced back into the one matrix that gptq.py keeps (layers_cache[name]['H']); accumulation may
  * go on afterwards.  H 16-byte aligned, slice_stride % 4 == 0. */

@@ -107,19 +107,50 @@ template <int TN> struct HessCfg {
   static constexpr int NL = LA + LB;
 };
 
+// How the last round of workgroup slots is filled (lcq_hessian_accum_balanced).  Per XCD: tile slots [0, full_x) run as
+// whole tiles; the rem_x tiles behind them are cut into `parts` token ranges each.  parts <= 1: nothing is split.
+struct TailSplit {
+  int full_x, rem_x, parts;
+  float* scratch;        // 8 * rem_x * (parts - 1) tiles of TM x TN floats
+};
+
 // EDGE = false: K % 256 == 0 and T % 32 == 0, no bounds checks anywhere.
 template <bool IS_BF16, bool EDGE, int TN>
 __global__ __launch_bounds__(HessCfg<TN>::NW * 64, TN == 256 ? 1 : 2)
 void hessian_kernel(float* __restrict__ H, int K, const uint16_t* __restrict__ X, const uint16_t* __restrict__ XB, int ldx,
-                    int T, float alpha, float beta, int ntr, int ntc, int total, int slices, long long hstride) {
+                    int T, float alpha, float beta, int ntr, int ntc, int total, int slices, long long hstride, TailSplit ts) {
   using C = HessCfg<TN>;
   constexpr int ROW_B = C::ROW_B, STAGE = C::STAGE, NSTAGE = C::NSTAGE, LA = C::LA, LB = C::LB, RB = C::RB;
   __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE];
   int ti = 0, tj = 0;
+  int ldh = K;                                   // row pitch of the output: H, or a packed TM x TN scratch tile
+  bool to_scratch = false;
   {
     const int per_xcd = (total + 7) / 8;
-    const int slot = blockIdx.x >> 3, xcd = blockIdx.x & 7;
-    if (slot >= per_xcd || xcd * per_xcd + slot >= total) return;
+    int slot = blockIdx.x >> 3;
+    const int xcd = blockIdx.x & 7;
+    if (ts.parts > 1 && slot >= ts.full_x) {
+      // The tiles of the last, partly filled round of workgroup slots: each is cut into `parts` token ranges that run
+      // side by side.  Part 0 updates H like any tile; the others leave beta * (their X^T X) in scratch tiles, which
+      // tail_fold_kernel adds to H afterwards in a fixed order.
+      const int i = slot - ts.full_x, r = i / ts.parts, part = i - r * ts.parts;
+      slot = ts.full_x + r;
+      if (r >= ts.rem_x || xcd * per_xcd + slot >= total) return;
+      const long long n32 = T / BT;              // EDGE launches are never split
+      const int t0 = (int)(part * n32 / ts.parts) * BT, t1 = (int)((part + 1) * n32 / ts.parts) * BT;
+      X += (int64_t)t0 * ldx;
+      XB += (int64_t)t0 * ldx;
+      T = t1 - t0;
+      if (part > 0) {
+        H = ts.scratch + ((int64_t)(xcd * ts.rem_x + r) * (ts.parts - 1) + (part - 1)) * (TM * TN);
+        ldh = TN;
+        alpha = 0.0f;
+        to_scratch = true;
+      }
+    } else if (slot >= per_xcd) {
+      return;
+    }
+    if (xcd * per_xcd + slot >= total) return;
     int v = xcd * per_xcd + slot;
     if (slices > 1) {
       // Token slices: `total` counts every tile once per slice.  Slice s takes an even share of the 32-token slabs,
@@ -263,7 +294,7 @@ void hessian_kernel(float* __restrict__ H, int K, const uint16_t* __restrict__ X
   // loads overlap; alpha == 0 (first batch) never reads H.
   const int row_l = 4 * (lane >> 5), col_l = lane & 31;
   const int grow = ti * TM + wr * 128 + row_l, gcol = tj * TN + wc * 64 + col_l;
-  float* const Hb = H + (int64_t)grow * K + gcol;
+  float* const Hb = to_scratch ? H + (wr * 128 + row_l) * TN + wc * 64 + col_l : H + (int64_t)grow * K + gcol;
   const bool rmw = (alpha != 0.0f);
   #pragma unroll
   for (int ih = 0; ih < 2; ++ih) {
@@ -277,7 +308,7 @@ void hessian_kernel(float* __restrict__ H, int K, const uint16_t* __restrict__ X
           for (int r = 0; r < 16; ++r) {
             const int dr = (ih * 2 + i2) * 32 + 8 * (r >> 2) + (r & 3), dc = j * 32;
             const bool ok = !EDGE || ((grow + dr < K) && (gcol + dc < K));
-            old[i2][j][r] = ok ? Hb[(int64_t)dr * K + dc] : 0.0f;
+            old[i2][j][r] = ok ? Hb[(int64_t)dr * ldh + dc] : 0.0f;
           }
     }
     #pragma unroll
@@ -290,8 +321,32 @@ void hessian_kernel(float* __restrict__ H, int K, const uint16_t* __restrict__ X
           const bool ok = !EDGE || ((grow + dr < K) && (gcol + dc < K));
           float v = beta * acc[ih * 2 + i2][j][r];
           if (rmw) v = alpha * old[i2][j][r] + v;
-          if (ok) Hb[(int64_t)dr * K + dc] = v;
+          if (ok) Hb[(int64_t)dr * ldh + dc] = v;
         }
+  }
+}
+
+// H tile <- ((H tile + part 1) + part 2) + ... for the tiles hessian_kernel cut into token ranges: grid (8 * rem_x, 8),
+// every workgroup an eighth of a 256 x 128 tile, 16 bytes per lane and step.
+template <int TN>
+__global__ __launch_bounds__(256) void tail_fold_kernel(float* __restrict__ H, int K, int ntr, int ntc, int total, TailSplit ts) {
+  const int per_xcd = (total + 7) / 8;
+  const int xcd = blockIdx.x / ts.rem_x, r = blockIdx.x - xcd * ts.rem_x;
+  const int v = xcd * per_xcd + ts.full_x + r;
+  if (ts.full_x + r >= per_xcd || v >= total) return;
+  int ti, tj;
+  decode_tile<TM / TN>(v, ntr, ntc, ti, tj);
+  const float* sc = ts.scratch + (int64_t)blockIdx.x * (ts.parts - 1) * (TM * TN);
+  constexpr int PER_ROW = TN / 4;
+  for (int e = blockIdx.y * 256 + threadIdx.x; e < TM * PER_ROW; e += gridDim.y * 256) {
+    const int row = e / PER_ROW, c4 = (e - row * PER_ROW) * 4;
+    float* hp = H + (int64_t)(ti * TM + row) * K + tj * TN + c4;
+    f32x4 h = *(const f32x4*)hp;
+    for (int p = 0; p < ts.parts - 1; ++p) {
+      const f32x4 w = *(const f32x4*)(sc + (int64_t)p * (TM * TN) + row * TN + c4);
+      h[0] += w[0]; h[1] += w[1]; h[2] += w[2]; h[3] += w[3];
+    }
+    *(f32x4*)hp = h;
   }
 }
 
@@ -395,8 +450,65 @@ int lcq_hessian_accum_ab(float* H, int64_t K, const void* X, const void* XB, int
   return lcq_hessian_accum_sliced(H, K, X, XB, dtype, T, ldx, alpha, beta, 1, 0, stream);
 }
 
+// Workgroup slots of the device the calling thread uses: two workgroups of the Hessian kernel per CU.
+static int hessian_slots() {
+  static int slots[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 512;
+  if (slots[dev] == 0) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    slots[dev] = 2 * cus;
+  }
+  return slots[dev];
+}
+
+// The split of the last round for a launch over T tokens of K features (see TailSplit); parts == 1: no split pays.
+static TailSplit tail_split(int64_t K, int64_t T) {
+  constexpr int TN = 128;
+  TailSplit ts{0, 0, 1, nullptr};
+  if (K % TM != 0 || T % BT != 0) return ts;
+  const int ntr = (int)(K / TM), ntc = (int)(K / TN), q = TM / TN;
+  int64_t total = 0;
+  for (int r = 0; r < ntr; ++r) total += (ntc - q * r > 0) ? (ntc - q * r) : 0;
+  const int per_xcd = (int)((total + 7) / 8), slots_x = hessian_slots() / 8;
+  if (slots_x <= 0 || per_xcd < 2 * slots_x) return ts;          // fewer than two full rounds: token shares serve better
+  const int full_x = per_xcd / slots_x * slots_x, rem_x = per_xcd - full_x;
+  if (rem_x == 0 || 2 * rem_x > slots_x) return ts;               // the last round is at least half full as it is
+  int parts = slots_x / rem_x;
+  if (parts > 8) parts = 8;
+  if (T / BT < 4 * parts) return ts;                              // too few tokens to cut
+  ts.full_x = full_x; ts.rem_x = rem_x; ts.parts = parts;
+  return ts;
+}
+
+int64_t lcq_hessian_balanced_workspace_bytes(int64_t K, int64_t T) {
+  if (K <= 0 || T <= 0 || K > (1 << 20)) return 0;
+  const TailSplit ts = tail_split(K, T);
+  return ts.parts > 1 ? (int64_t)8 * ts.rem_x * (ts.parts - 1) * TM * 128 * 4 : 0;
+}
+
+static int hessian_launch(float* H, int64_t K, const void* X, const void* XB, int dtype, int64_t T, int64_t ldx,
+                          float alpha, float beta, int slices, int64_t slice_stride, TailSplit ts, void* stream);
+
+int lcq_hessian_accum_balanced(float* H, int64_t K, const void* XA, const void* XB, int dtype, int64_t T, int64_t ldx, float alpha,
+                               float beta, void* workspace, int64_t workspace_bytes, void* stream) {
+  TailSplit ts = (K > 0 && T > 0 && K <= (1 << 20)) ? tail_split(K, T) : TailSplit{0, 0, 1, nullptr};
+  if (ts.parts > 1) {
+    if (!workspace || workspace_bytes < lcq_hessian_balanced_workspace_bytes(K, T)) return LCQ_EWORKSPACE;
+    if (((uintptr_t)workspace % 16) != 0) return LCQ_EALIGN;
+    ts.scratch = (float*)workspace;
+  }
+  return hessian_launch(H, K, XA, XB, dtype, T, ldx, alpha, beta, 1, 0, ts, stream);
+}
+
 int lcq_hessian_accum_sliced(float* H, int64_t K, const void* X, const void* XB, int dtype, int64_t T, int64_t ldx,
                              float alpha, float beta, int slices, int64_t slice_stride, void* stream) {
+  return hessian_launch(H, K, X, XB, dtype, T, ldx, alpha, beta, slices, slice_stride, TailSplit{0, 0, 1, nullptr}, stream);
+}
+
+static int hessian_launch(float* H, int64_t K, const void* X, const void* XB, int dtype, int64_t T, int64_t ldx,
+                          float alpha, float beta, int slices, int64_t slice_stride, TailSplit ts, void* stream) {
   if (!H || !X || !XB || K <= 0 || T < 0) return LCQ_EINVAL;
   if (K % 8 != 0 || K > (1 << 20) || T > 0x7fffffff || ldx < K || ldx % 8 != 0 || ldx > (1 << 21)) return LCQ_EINVAL;
   if (slices < 1 || slices > 64 || (slices > 1 && slice_stride < K * K)) return LCQ_EINVAL;
@@ -409,16 +521,20 @@ int lcq_hessian_accum_sliced(float* H, int64_t K, const void* X, const void* XB,
   for (int r = 0; r < ntr; ++r) total += (ntc - q * r > 0) ? (ntc - q * r) : 0;
   total *= slices;
   if (total > 0x7ffffff0) return LCQ_ESIZE;
-  const int64_t grid = (total + 7) / 8 * 8;                       // 8 XCD queues of equal length
+  int64_t grid = (total + 7) / 8 * 8;                             // 8 XCD queues of equal length
   hipStream_t st = (hipStream_t)stream;
   const bool edge = (K % TM != 0) || (T % BT != 0);
+  if (ts.parts > 1 && (edge || slices != 1 || dtype == LCQ_F32)) ts.parts = 1;
+  if (ts.parts > 1) grid = (int64_t)8 * (ts.full_x + ts.rem_x * ts.parts);
   #define LCQ_HESS(BF, E) hessian_kernel<BF, E, TN><<<dim3((unsigned)grid), dim3(HessCfg<TN>::NW * 64), 0, st>>>( \
       H, (int)K, (const uint16_t*)X, (const uint16_t*)XB, (int)ldx, (int)T, alpha, beta, ntr, ntc, (int)total, slices, \
-      (long long)slice_stride)
+      (long long)slice_stride, ts)
   if (dtype == LCQ_BF16) { if (edge) LCQ_HESS(true, true); else LCQ_HESS(true, false); }
   else if (dtype == LCQ_F16) { if (edge) LCQ_HESS(false, true); else LCQ_HESS(false, false); }
   else return LCQ_EDTYPE;
   #undef LCQ_HESS
+  if (ts.parts > 1)
+    tail_fold_kernel<TN><<<dim3((unsigned)(8 * ts.rem_x), 8), dim3(256), 0, st>>>(H, (int)K, ntr, ntc, (int)total, ts);
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;
 }

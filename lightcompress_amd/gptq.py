@@ -163,7 +163,7 @@ class GPTQ:
         self.layers_cache[name]['n_in_H'] = 0
         self.layers_cache[name]['calls'] = 0
         for k in ('stage', 'stage_lo', 'stage_fill', 'stage_batches', 'last_stage', 'last_key', 'last_ref', 'manual_share',
-                  'share_flag'):
+                  'share_flag', 'hws', 'hws_key'):
             self.layers_cache[name].pop(k, None)
         self.layers_cache[name]['columns'] = K
         self.layers_cache[name]['kind'] = self._layer_kind(layer)
@@ -448,17 +448,35 @@ class GPTQ:
         cache['n_in_H'] = n + batches
         H = cache['H']
         shares = cache.get('H_shares')
-        sl = (L.i32(1), L.i64(0)) if shares is None else (L.i32(shares.shape[0]), L.i64(shares.stride(0)))
         cache['shares_apart'] = shares is not None
         lib, code = L.lib(), L.i32(L.dtype_code(x.dtype))
-        dims = (L.i64(x.shape[0]), L.i64(x.stride(0)))
+        K, T = H.shape[0], x.shape[0]
+        dims = (L.i64(T), L.i64(x.stride(0)))
+        if shares is None:
+            # one accumulator: the launch that fills its last round of workgroups (lcq_hessian_accum_balanced), with a
+            # scratch buffer kept per Linear; where no split pays the call is the plain update
+            key = (K, T)
+            if cache.get('hws_key') != key:
+                nbytes = lib.lcq_hessian_balanced_workspace_bytes(L.i64(K), L.i64(T))
+                cache['hws'] = torch.empty(nbytes, dtype=torch.uint8, device=H.device) if nbytes > 0 else None
+                cache['hws_key'] = key
+            ws = cache['hws']
+            tail = (L.ptr(ws), L.i64(0 if ws is None else ws.numel()), L.stream())
+
+            def launch(a, b, al):
+                L.check(lib.lcq_hessian_accum_balanced(L.ptr(H), L.i64(K), L.ptr(a), L.ptr(b), code, *dims, L.f32(al), L.f32(beta),
+                                                       *tail), 'lcq_hessian_accum_balanced')
+        else:
+            sl = (L.i32(shares.shape[0]), L.i64(shares.stride(0)), L.stream())
+
+            def launch(a, b, al):
+                L.check(lib.lcq_hessian_accum_sliced(L.ptr(H), L.i64(K), L.ptr(a), L.ptr(b), code, *dims, L.f32(al), L.f32(beta),
+                                                     *sl), 'lcq_hessian_accum_sliced')
         if x_lo is None:
-            L.check(lib.lcq_hessian_accum_sliced(L.ptr(H), L.i64(H.shape[0]), L.ptr(x), L.ptr(x), code, *dims, L.f32(alpha),
-                                                 L.f32(beta), *sl, L.stream()), 'lcq_hessian_accum_sliced')
+            launch(x, x, alpha)
             return
         for a, b, al in ((x_lo, x_lo, alpha), (x, x_lo, 1.0), (x_lo, x, 1.0), (x, x, 1.0)):      # small terms first
-            L.check(lib.lcq_hessian_accum_sliced(L.ptr(H), L.i64(H.shape[0]), L.ptr(a), L.ptr(b), code, *dims, L.f32(al),
-                                                 L.f32(beta), *sl, L.stream()), 'lcq_hessian_accum_sliced')
+            launch(a, b, al)
 
     def _flush(self, cache):
         """Fold the staged tokens into H."""

@@ -92,6 +92,52 @@ def test_hessian_token_shares_sum_to_the_single_accumulator(dev, K, T, slices):
                                         L.f32(0.0), L.f32(1.0), L.i32(65), L.i64(K * K), L.stream()) != 0
 
 
+@pytest.mark.parametrize('K,T', [(8192, 2048), (14336, 4096)])
+def test_hessian_with_the_last_round_split(dev, K, T):
+    """lcq_hessian_accum_balanced: the tiles of the last, partly filled round of workgroups are cut into token ranges
+    whose partial sums meet in a workspace.  Same H as the plain launch up to the order of fp32 additions, the closed
+    form in fp64 within 1e-5, the same bits from run to run; where no split pays the call needs no workspace."""
+    from lightcompress_amd import _lib as L
+    lib = L.lib()
+    g = torch.Generator(device=dev)
+    g.manual_seed(K + T)
+    xs = [(torch.randn(T, K, device=dev, generator=g) * torch.exp(0.5 * torch.randn(K, device=dev, generator=g))).bfloat16() for _ in range(2)]
+    nbytes = lib.lcq_hessian_balanced_workspace_bytes(L.i64(K), L.i64(T))
+    assert nbytes > 0 and nbytes % (256 * 128 * 4) == 0
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    ws.fill_(0x7f)                                              # whatever the workspace held must not matter
+    outs = []
+    for rep in range(2):
+        Hb = torch.ones(K, K, device=dev)
+        for x, (al, be) in zip(xs, ((0.0, 2.0), (0.5, 1.0))):
+            L.check(lib.lcq_hessian_accum_balanced(L.ptr(Hb), L.i64(K), L.ptr(x), L.ptr(x), L.i32(L.BF16), L.i64(T), L.i64(K), L.f32(al),
+                                                   L.f32(be), L.ptr(ws), L.i64(nbytes), L.stream()), 'balanced')
+        outs.append(Hb)
+    assert torch.equal(outs[0], outs[1])
+    Hp = torch.ones(K, K, device=dev)
+    for x, (al, be) in zip(xs, ((0.0, 2.0), (0.5, 1.0))):
+        L.check(lib.lcq_hessian_accum(L.ptr(Hp), L.i64(K), L.ptr(x), L.i32(L.BF16), L.i64(T), L.i64(K), L.f32(al), L.f32(be), L.stream()), 'plain')
+    up = torch.triu(torch.ones(K, K, dtype=torch.bool, device=dev))
+    scale = float(Hp[up].abs().max())
+    assert float((outs[0] - Hp)[up].abs().max()) / scale < 2e-6
+    assert int((outs[0] != Hp)[up].sum()) > 0                    # the split really happened: another order of additions
+    ref = xs[0].double().t() @ xs[0].double() + xs[1].double().t() @ xs[1].double()
+    assert float((outs[0].double() - ref)[up].abs().max()) / scale < 1e-5
+    del ref
+    assert lib.lcq_hessian_accum_balanced(L.ptr(Hp), L.i64(K), L.ptr(xs[0]), L.ptr(xs[0]), L.i32(L.BF16), L.i64(T), L.i64(K), L.f32(0.0),
+                                          L.f32(1.0), L.ptr(ws), L.i64(nbytes - 16), L.stream()) == -5
+    # no split: fewer than two rounds of tiles, ragged sizes
+    for K2, T2 in ((4096, 2048), (1000, 64), (8192, 2040)):
+        assert lib.lcq_hessian_balanced_workspace_bytes(L.i64(K2), L.i64(T2)) == 0
+    K2, T2 = 1000, 64
+    x = torch.randn(T2, K2, device=dev).bfloat16()
+    a, b = torch.zeros(K2, K2, device=dev), torch.zeros(K2, K2, device=dev)
+    L.check(lib.lcq_hessian_accum_balanced(L.ptr(a), L.i64(K2), L.ptr(x), L.ptr(x), L.i32(L.BF16), L.i64(T2), L.i64(K2), L.f32(0.0), L.f32(1.0),
+                                           L.ptr(None), L.i64(0), L.stream()), 'no workspace')
+    L.check(lib.lcq_hessian_accum(L.ptr(b), L.i64(K2), L.ptr(x), L.i32(L.BF16), L.i64(T2), L.i64(K2), L.f32(0.0), L.f32(1.0), L.stream()), 'plain')
+    assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize('slices', [1, 3, 'auto'])
 def test_hessian_shares_through_add_batch_and_reads_in_between(dev, slices):
     """`special.hessian_slices`: whatever the number of accumulators, reading H in the middle of the calibration
