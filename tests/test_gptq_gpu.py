@@ -1042,3 +1042,78 @@ def test_indefinite_hessian_raises_unless_the_check_is_off(dev):
             assert torch.equal(layer.weight.data, W0)    # nothing was written back
         else:
             gp.layer_transform(layer, 'l')
+
+
+@pytest.mark.parametrize('K', [768, 1536, 2304, 3072, 5120, 6144])
+def test_hessian_auto_settings_between_the_tuned_widths(dev, K):
+    """`hessian_defer: auto` / `hessian_slices: auto` are tables tuned at a handful of widths; whatever they pick at
+    the widths in between (folds of 16 / 8 calls, 1 - 8 token shares, with or without the split last round), add_batch
+    over a number of calls that leaves a partly filled staging buffer ends at the closed form."""
+    T, nb = 96, 21
+    gp = make_gptq()
+    layer = Layer(torch.zeros(8, K, device=dev))
+    gp.layers_cache['l'] = {}
+    gp.layer_init(layer, 'l')
+    g = torch.Generator(device=dev)
+    g.manual_seed(K)
+    xs = [(torch.randn(1, T, K, device=dev, generator=g) * (1 + i % 3)).bfloat16() for i in range(nb)]
+    for x in xs:
+        gp.add_batch(layer, 'l', x, None)
+    H = gp.hessian('l')
+    ref = torch.zeros(K, K, dtype=torch.float64, device=dev)
+    for x in xs:
+        xd = x[0].double()
+        ref.addmm_(xd.t(), xd)
+    ref *= 2.0 / nb
+    assert gp.layers_cache['l']['nsamples'] == nb
+    assert float((H.double() - ref).abs().max() / ref.abs().max()) < 1e-5
+    assert torch.equal(H, H.t())
+
+
+def test_switch_combinations_give_one_result(dev):
+    """The `special` switches that only rearrange work (auto_share, fuse_loops, block_factor, chain_overlap,
+    hessian_defer, hessian_slices, share_verify) in all 128 combinations on a subset of three Linears with a common
+    input: every combination reproduces the plain one (one Hessian per Linear, one launch per call, the reference's
+    chain, one loop per Linear) to >= 99.9 % of the codes and 1e-3 of the loss; combinations that differ only in
+    switches with bit-identical semantics (sharing, verification, overlap, stacking) agree bit for bit."""
+    import itertools
+    K = 512
+    Ws = {'q': (torch.randn(96, K, generator=gen(21)) * 0.02).bfloat16(), 'k': (torch.randn(32, K, generator=gen(22)) * 0.02).bfloat16(),
+          'v': (torch.randn(48, K, generator=gen(23)) * 0.02).bfloat16()}
+    xs = [b.to(dev) for b in calib_batches(7, 128, K, seed=9900)]
+    spec = Q.IntSpec(4, False, 'per_group', group_size=128)
+
+    def run(**special):
+        gp = make_gptq(actorder=True, **special)
+        layers = {n: Layer(w.to(dev)) for n, w in Ws.items()}
+        gp.subset_init({'layers': layers})
+        for x in xs:
+            for n in Ws:
+                gp.add_batch(layers[n], n, x.data, None)
+        gp.subset_transform({'layers': layers})
+        torch.cuda.synchronize()
+        return {n: (layers[n].weight.data.cpu(), layers[n].buf_scales.cpu(), layers[n].buf_zeros.cpu(), layers[n].buf_perm.cpu(),
+                    float(gp.last_errors[n])) for n in Ws}
+
+    base = run(auto_share=False, fuse_loops=False, block_factor=False, chain_overlap=False, hessian_defer=1, hessian_slices=1)
+    seen = {}
+    for share, fuse, bf, ov, defer, slices, verify in itertools.product((True, False), (True, False), (True, False), (True, False),
+                                                                        (1, 'auto'), (1, 'auto'), (True, False)):
+        got = run(auto_share=share, fuse_loops=fuse, block_factor=bf, chain_overlap=ov, hessian_defer=defer, hessian_slices=slices,
+                  share_verify=verify)
+        for n in Ws:
+            w, s_, z_, perm, loss = got[n]
+            bw, bs_, bz_, bperm, bloss = base[n]
+            assert torch.equal(perm, bperm), (n, share, fuse, bf, ov, defer, slices)
+            codes = G.codes_from(w[:, perm], s_, z_, spec)
+            bcodes = G.codes_from(bw[:, perm], bs_, bz_, spec)
+            assert float((codes == bcodes).float().mean()) >= 0.999, (n, share, fuse, bf, ov, defer, slices)
+            assert abs(loss - bloss) <= 1e-3 * bloss
+        # the arithmetic depends on the factor (bf) and on how the Hessian was summed (defer, slices) only
+        key = (bf, defer, slices)
+        if key in seen:
+            for n in Ws:
+                for a, b in zip(got[n][:4], seen[key][n][:4]):
+                    assert torch.equal(a, b), (n, share, fuse, bf, ov, defer, slices, verify)
+        else:
+            seen[key] = got
