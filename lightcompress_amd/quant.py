@@ -1072,7 +1072,7 @@ class FloatQuantizer(BaseQuantizer):
     def _fake(self, t, static_scales=None, args={}):
         if self.granularity == 'per_block':
             if static_scales is not None:
-                raise NotImplementedError('static per_block scales')
+                return self._per_block_static(t, static_scales, True)
             return self._per_block(t, True)
         shape, dtype = t.shape, t.dtype
         if static_scales is None and self.calib_algo != 'minmax':
@@ -1120,11 +1120,40 @@ class FloatQuantizer(BaseQuantizer):
             return _block_dequant(y, s, torch.float32).to(weight.dtype)
         return y, s
 
+    def _per_block_static(self, weight, scales, want_dq):
+        """per_block with GIVEN block scales (fake / real_quant_weight_static, quant.py:1113-1139, 1160-1192 on the
+        zero-padded [mb, bs, nb, bs] view of reshape_tensor :634-638 with scales [mb, 1, nb, 1]): every block becomes
+        one row of bs * bs elements with its scale, the row kernel does the rest, and the rows go back into place.
+        -> the dequantized weight in the weight's type, or float8 codes."""
+        if not self.use_qtorch or weight.dim() != 2:
+            raise NotImplementedError('static per_block scales: 2-D weights, use_qtorch=True')
+        bs = self.block_size
+        m, n = weight.shape
+        mb, nb = -(-m // bs), -(-n // bs)
+        if scales.numel() != mb * nb:
+            raise L.LcqError(f'per_block: {scales.numel()} scales for {mb} x {nb} blocks')
+        scales[scales == 0] = 1                          # quant.py:1061 mutates the caller's tensor
+        w = weight
+        if (m, n) != (mb * bs, nb * bs):
+            w = torch.zeros((mb * bs, nb * bs), dtype=weight.dtype, device=weight.device)
+            w[:m, :n] = weight
+        rows = w.view(mb, bs, nb, bs).permute(0, 2, 1, 3).reshape(mb * nb, bs * bs)
+        s_rows = scales.reshape(mb * nb, 1).clone()
+        if want_dq:
+            out, _, _ = self._launch(rows, static=True, scales=s_rows, want_dq=True)
+        else:
+            _, out, _ = self._launch(rows, static=True, scales=s_rows,
+                                     want_codes=torch.float8_e4m3fn if self.e_bits == 4 else torch.float8_e5m2)
+        out = out.view(mb, nb, bs, bs).permute(0, 2, 1, 3).reshape(mb * bs, nb * bs)[:m, :n]
+        return out.to(weight.dtype) if want_dq else out.contiguous()
+
     def _real(self, weight, static_scales, output_scale_factor, args={}):
         assert self.bit in ['e4m3', 'e5m2'], 'Only FP8 E4M3 and E5M2 support real quant'
         if self.granularity == 'per_block':
             if static_scales is not None:
-                raise NotImplementedError('static per_block scales')
+                y = self._per_block_static(weight, static_scales, False)
+                s = static_scales * output_scale_factor
+                return y, (s.view(s.shape[0], s.shape[2]) if s.dim() == 4 else s), None
             y, s = self._per_block(weight, False)
             return y, s * output_scale_factor, None
         dtype = torch.float8_e4m3fn if self.e_bits == 4 else torch.float8_e5m2

@@ -435,6 +435,23 @@ def float_per_block_real_quant(spec, w: torch.Tensor, block_size: int = 128):
     return q.to(torch.float8_e4m3fn), scales.view(scales.shape[0], scales.shape[2]), None
 
 
+def float_per_block_static(spec, w: torch.Tensor, scales: torch.Tensor, block_size: int = 128, real=False):
+    """fake_quant_weight_static / real_quant_weight_static of FloatQuantizer with per_block granularity and GIVEN
+    scales [mb, 1, nb, 1] (quant.py:1113-1139, 1160-1192): reshape_tensor's zero-padded 4-D view (:634-638), x / s
+    broadcast per block, float_quantize, (dequantize,) restore_tensor (:647-651), cast."""
+    m, n = w.shape
+    mb, nb = -(-m // block_size), -(-n // block_size)
+    t_padded = torch.zeros((mb * block_size, nb * block_size), dtype=w.dtype)
+    t_padded[:m, :n] = w
+    t = t_padded.view(-1, block_size, t_padded.size(1) // block_size, block_size)
+    zeros = torch.tensor(0.0)
+    q = float_quant(spec, t, scales, zeros)
+    if not real:
+        q = float_dequant(q, scales, zeros)
+    q = q.reshape(-1, nb * block_size)[:m, :n]
+    return q.to(torch.float8_e4m3fn if spec.e_bits == 4 else torch.float8_e5m2) if real else q.to(w.dtype)
+
+
 # ----------------------------------------------------------------------------
 # calib_algo 'mse'
 # ----------------------------------------------------------------------------

@@ -208,6 +208,12 @@ def test_stacked_loops_at_full_size(dev, rows):
     gp, layers, leaders, factors = _run_subset(dev, Ws, xs)
     assert leaders == {n: first for n in rows}
     assert factors == [(True, sum(rows.values()))]
+    # the whole default path is deterministic: a second run reproduces every output bit for bit
+    gp2, layers2, _, _ = _run_subset(dev, Ws, xs)
+    for n in rows:
+        assert torch.equal(layers2[n].weight.data, layers[n].weight.data) and torch.equal(layers2[n].buf_scales, layers[n].buf_scales)
+        assert torch.equal(layers2[n].buf_zeros, layers[n].buf_zeros) and float(gp2.last_errors[n]) == float(gp.last_errors[n])
+    del gp2, layers2
     gp1, layers1, leaders1, factors1 = _run_subset(dev, Ws, xs, fuse_loops=False)
     assert leaders1 == leaders and factors1 == [(True, R) for R in rows.values()]
     H64 = _hessian_fp64(xs)

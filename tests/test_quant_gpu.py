@@ -740,3 +740,35 @@ def test_experts_in_one_launch_equal_expert_by_expert(dev):
             assert torch.equal(many[e][0], one[0]) and torch.equal(many[e][1], one[1])
     with pytest.raises(NotImplementedError):
         IntegerQuantizer(4, True, 'per_tensor').real_quant_weight_dynamic_experts(slices)
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('shape', [(256, 384), (200, 300)])
+def test_float_per_block_with_given_scales(dev, dtype, shape):
+    """FloatQuantizer('e4m3', per_block) with static scales (the block scales of a float8 checkpoint, or those of an
+    earlier dynamic call): fake and real quantization bit for bit against the oracle, ragged shapes padded with zeros
+    like reshape_tensor does, a zero scale replaced by 1 in the caller's tensor; with the scales of its own dynamic
+    call the static path reproduces the dynamic one."""
+    from lightcompress_amd import FloatQuantizer
+    m, n = shape
+    w = weight_like(m, n, seed=m + n, dtype=dtype, std=0.02, outlier_frac=0.002, outlier_mul=20)
+    mb, nb = -(-m // 128), -(-n // 128)
+    scales = (torch.rand(mb, 1, nb, 1, generator=gen(5)) * 4e-4 + 1e-4)
+    scales[0, 0, 0, 0] = 0.0
+    spec = Q.FloatSpec('e4m3', 'per_block')
+    q = FloatQuantizer('e4m3', True, 'per_block', use_qtorch=True, block_size=128)
+    sd = scales.clone().to(dev)
+    got = q.fake_quant_weight_static(w.to(dev), {'scales': sd, 'zeros': torch.tensor(0.0), 'qmax': q.qmax, 'qmin': q.qmin})
+    so = scales.clone()
+    assert_bit_equal(got, Q.float_per_block_static(spec, w, so), 'static per_block fake quant')
+    assert float(sd[0, 0, 0, 0]) == 1.0 and float(so[0, 0, 0, 0]) == 1.0          # both mutated the caller's scales
+    codes, rs, rz = q.real_quant_weight_static(w.to(dev), {'scales': sd, 'zeros': torch.tensor(0.0), 'qmax': q.qmax, 'qmin': q.qmin})
+    assert rz is None and rs.shape == (mb, nb) and codes.dtype == torch.float8_e4m3fn and codes.shape == (m, n)
+    assert_bit_equal(codes, Q.float_per_block_static(spec, w, so, real=True), 'static per_block codes')
+    if n % 8:                                             # the dynamic block-wise cast wants 16-byte aligned rows
+        return
+    # the scales of the dynamic call, handed back: the same codes
+    dyn_codes, dyn_s, _ = q.real_quant_weight_dynamic(w.to(dev))
+    again, _, _ = q.real_quant_weight_static(w.to(dev), {'scales': dyn_s.view(mb, 1, nb, 1).clone(), 'zeros': torch.tensor(0.0),
+                                                         'qmax': q.qmax, 'qmin': q.qmin})
+    assert_bit_equal(again, dyn_codes, 'static with the dynamic scales')
