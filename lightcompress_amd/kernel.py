@@ -14,7 +14,21 @@ from . import _lib as L
 FLAG_CLAMP_RANGE, FLAG_TIE_AWAY = 1024, 2048
 
 
+def _pad_cols(x, mult=8):
+    """x with its last dimension zero-padded to a multiple of `mult` (the kernels take whole 16-byte pieces of a row;
+    zeros change no block maximum and a pad of fewer than 8 columns never opens another 128-column block)."""
+    N = x.shape[-1]
+    if N % mult == 0:
+        return x
+    out = torch.zeros((*x.shape[:-1], (N + mult - 1) // mult * mult), dtype=x.dtype, device=x.device)
+    out[..., :N] = x
+    return out
+
+
 def _block_quant(x, block_rows, flags):
+    if x.shape[-1] % 8 and block_rows != 1:
+        y, s = _block_quant(_pad_cols(x), block_rows, flags)
+        return y[..., :x.shape[-1]].contiguous(), s
     M, N = x.numel() // x.shape[-1], x.shape[-1]
     y = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device=x.device)
     if block_rows == 1:
@@ -58,6 +72,9 @@ def _block_dequant(x, s, out_dtype):
     M, N = x.shape
     if out_dtype not in (torch.float32, torch.bfloat16):
         raise NotImplementedError(f'output dtype {out_dtype}')
+    if N % 8:
+        xp = _pad_cols(x.view(torch.uint8)).view(torch.float8_e4m3fn)
+        return _block_dequant(xp, s, out_dtype)[:, :N].contiguous()
     out = torch.empty((M, N), dtype=out_dtype, device=x.device)
     sf = s.to(torch.float32).contiguous()
     L.check(L.lib().lcq_fp8_block_dequant(L.ptr(x), L.ptr(sf), L.i64(M), L.i64(N), L.ptr(out), L.i32(L.dtype_code(out_dtype)),

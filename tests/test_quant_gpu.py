@@ -765,10 +765,11 @@ def test_float_per_block_with_given_scales(dev, dtype, shape):
     codes, rs, rz = q.real_quant_weight_static(w.to(dev), {'scales': sd, 'zeros': torch.tensor(0.0), 'qmax': q.qmax, 'qmin': q.qmin})
     assert rz is None and rs.shape == (mb, nb) and codes.dtype == torch.float8_e4m3fn and codes.shape == (m, n)
     assert_bit_equal(codes, Q.float_per_block_static(spec, w, so, real=True), 'static per_block codes')
-    if n % 8:                                             # the dynamic block-wise cast wants 16-byte aligned rows
-        return
-    # the scales of the dynamic call, handed back: the same codes
+    # the scales of the dynamic call, handed back: the same codes (ragged widths go through a zero-padded copy)
     dyn_codes, dyn_s, _ = q.real_quant_weight_dynamic(w.to(dev))
     again, _, _ = q.real_quant_weight_static(w.to(dev), {'scales': dyn_s.view(mb, 1, nb, 1).clone(), 'zeros': torch.tensor(0.0),
                                                          'qmax': q.qmax, 'qmin': q.qmin})
     assert_bit_equal(again, dyn_codes, 'static with the dynamic scales')
+    oc, os_, _ = Q.float_per_block_real_quant(spec, w)
+    assert_bit_equal(dyn_codes, oc, 'dynamic per_block codes'); assert_bit_equal(dyn_s, os_, 'dynamic per_block scales')
+    assert_bit_equal(q.fake_quant_weight_dynamic(w.to(dev)), Q.float_per_block_static(spec, w, os_.view(mb, 1, nb, 1).clone()), 'dynamic per_block fake quant')
