@@ -72,6 +72,7 @@ extern "C" {
 
 #define LCQ_FLAG_CLAMP_RANGE 1024  /* lcq_fp8_block_quant: s = clamp(max|x|, 1e-5) / 448 (the FloatQuantizer path) instead of max|x| / 448 */
 #define LCQ_FLAG_TIE_AWAY 2048     /* lcq_fp8_block_quant: exact ties round away from zero instead of to even */
+#define LCQ_FLAG_ROWS16 4096       /* lcq_gptq_block: 16 rows per workgroup whatever R is (the default takes 32 from 6144 rows on; same results bit for bit) */
 #define LCQ_FLAG_ROW_QP 512       /* lcq_quant_fp_emu, STATIC only: `scales` holds one value per row */
 
 /* errors */

@@ -44,7 +44,6 @@ namespace {
 using namespace lcq;
 
 constexpr int BS = 128;          // columns per block (lazy batch)
-constexpr int ROWS_PER_WG = 16;
 // Hinv1 in LDS: a row holds, for each of the 16 lanes of a team, the first four of the lane's eight columns at
 // float 4 t and the other four at UH + 4 t, so the two 16-byte reads of a team are each one contiguous run (no bank
 // conflicts); the second half starts 4 floats past a multiple of 64 so that a wave's 16-byte stores, which alternate
@@ -123,8 +122,12 @@ __device__ __forceinline__ ColQ open_group(const LoopArgs& a, int idx, int lane,
 
 // STATIC: scales / zero points are given (per group, or per column through gidx).  OCT: every group starts on
 // a multiple of 8 columns, so groups open only between octets and the 8 columns of an octet are straight-line code.
-template <bool STATIC, bool OCT>
-__global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
+// RW rows per workgroup (16 lanes each): 16, or 32 for launches of many rows (one copy of Hinv1 in LDS then serves
+// eight waves, and two such workgroups put four waves on every SIMD instead of two).
+template <bool STATIC, bool OCT, int RW>
+__global__ __launch_bounds__(16 * RW) void gptq_block_kernel(LoopArgs a) {
+  constexpr int NT = 16 * RW;                    // threads
+  constexpr int ROWS_PER_WG = RW;
   constexpr int NP = OCT ? 16 : BS;              // parameter slots of a row: one per octet, or one per column
   __shared__ float Us[BS * UP];                  // Hinv1 = U[i1:i2, i1:i2] above the diagonal, zero everywhere else (us_col layout)
   __shared__ float Rd[BS];                       // 1 / U[i, i]
@@ -139,21 +142,22 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a) {
   if (vec) {
     // all 16 loads of the thread in flight at once: one after the other they are 16 memory latencies,
     // which used to be most of the kernel's run time
-    f32x4 v[16];
+    constexpr int NL = BS * BS / 4 / NT;
+    f32x4 v[NL];
     #pragma unroll
-    for (int j = 0; j < 16; ++j) {
-      const int e = tid + 256 * j, r = e >> 5, c = (e & 31) * 4;
+    for (int j = 0; j < NL; ++j) {
+      const int e = tid + NT * j, r = e >> 5, c = (e & 31) * 4;
       v[j] = *(const f32x4*)(a.U + (long long)(a.i1 + r) * a.K + a.i1 + c);
     }
     #pragma unroll
-    for (int j = 0; j < 16; ++j) {
-      const int e = tid + 256 * j, r = e >> 5, c = (e & 31) * 4;
+    for (int j = 0; j < NL; ++j) {
+      const int e = tid + NT * j, r = e >> 5, c = (e & 31) * 4;
       #pragma unroll
       for (int k = 0; k < 4; ++k) if (c + k <= r) v[j][k] = 0.0f;
       *(f32x4*)(Us + r * UP + us_col(c)) = v[j];
     }
   } else {
-    for (int e = tid; e < BS * BS / 4; e += 256) {
+    for (int e = tid; e < BS * BS / 4; e += NT) {
       const int r = (e * 4) / BS, c = (e * 4) % BS;
       f32x4 v = {0.f, 0.f, 0.f, 0.f};
       if (r < a.count) {
@@ -373,11 +377,22 @@ int lcq_gptq_block(float* W, float* tmp, float* Losses, float* Err, int64_t ldEr
   a.nrz = (flags & LCQ_FLAG_NO_ROUND_ZP) != 0;
   a.aligned = ((reinterpret_cast<uintptr_t>(W) | reinterpret_cast<uintptr_t>(tmp) | reinterpret_cast<uintptr_t>(Losses) |
                 reinterpret_cast<uintptr_t>(U)) & 15) == 0;
-  const unsigned grid = (unsigned)((R + ROWS_PER_WG - 1) / ROWS_PER_WG);
   const bool oct = !is_static && group_size % 8 == 0 && i1 % 8 == 0;
-  if (is_static) gptq_block_kernel<true, true><<<dim3(grid), dim3(256), 0, (hipStream_t)stream>>>(a);
-  else if (oct) gptq_block_kernel<false, true><<<dim3(grid), dim3(256), 0, (hipStream_t)stream>>>(a);
-  else gptq_block_kernel<false, false><<<dim3(grid), dim3(256), 0, (hipStream_t)stream>>>(a);
+  hipStream_t st = (hipStream_t)stream;
+  // From 6144 rows on, 32 rows per workgroup: one copy of Hinv1 in LDS (70 KB) per eight waves, so that the two
+  // workgroups a CU holds put four waves on every SIMD (R = 28672: 57 -> 48 us per block, 14336: 35 -> 29, 6144:
+  // 20 -> 19; at 4096 rows, one workgroup per CU either way, the smaller workgroup is faster, 17 against 19 us).
+  // The rows do not interact: the results are the same bit for bit.
+  if (R >= 6144 && (is_static || oct) && !(flags & LCQ_FLAG_ROWS16)) {
+    const unsigned grid = (unsigned)((R + 31) / 32);
+    if (is_static) gptq_block_kernel<true, true, 32><<<dim3(grid), dim3(512), 0, st>>>(a);
+    else gptq_block_kernel<false, true, 32><<<dim3(grid), dim3(512), 0, st>>>(a);
+  } else {
+    const unsigned grid = (unsigned)((R + 15) / 16);
+    if (is_static) gptq_block_kernel<true, true, 16><<<dim3(grid), dim3(256), 0, st>>>(a);
+    else if (oct) gptq_block_kernel<false, true, 16><<<dim3(grid), dim3(256), 0, st>>>(a);
+    else gptq_block_kernel<false, false, 16><<<dim3(grid), dim3(256), 0, st>>>(a);
+  }
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;
 }

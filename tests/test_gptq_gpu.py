@@ -1117,3 +1117,35 @@ def test_switch_combinations_give_one_result(dev):
                     assert torch.equal(a, b), (n, share, fuse, bf, ov, defer, slices, verify)
         else:
             seen[key] = got
+
+
+@pytest.mark.parametrize('R', [6144, 6151, 9000])
+@pytest.mark.parametrize('mode', ['searched', 'searched_sym', 'static', 'block_factor'])
+def test_block_kernel_workgroup_shapes_agree(dev, R, mode):
+    """lcq_gptq_block takes 32 rows per workgroup from 6144 rows on and 16 below (the kernel every small case above
+    runs against the oracle): rows do not interact, so the two shapes must agree bit for bit on every output, also
+    with a ragged last workgroup."""
+    from lightcompress_amd import _lib as L
+    lib = L.lib()
+    K, i1, g = 512, 256, 64
+    G = K // g
+    U = (torch.triu(torch.randn(K, K, generator=gen(1)) * 0.02) + torch.eye(K) * 1.5).to(dev)
+    W0 = (torch.randn(R, K, generator=gen(2)) * 0.05).to(dev)
+    outs = []
+    for extra in (L.FLAG_ROWS16, 0):
+        flags = extra | (L.FLAG_SYM if mode == 'searched_sym' else 0) | (L.FLAG_STATIC if mode == 'static' else 0)
+        W = W0.clone()
+        W[:, i1:] += 0.01                                   # what earlier blocks' updates would have left
+        tmp, Lo = torch.zeros_like(W), torch.zeros_like(W)
+        Err = torch.zeros(R, 128, device=dev)
+        sc = (torch.rand(R, G, generator=gen(3)) * 0.01 + 0.005).to(dev)
+        ze = torch.randint(0, 16, (R, G), generator=gen(4)).float().to(dev)
+        L.check(lib.lcq_gptq_block(L.ptr(W), L.ptr(tmp), L.ptr(Lo), L.ptr(Err), L.i64(128), L.ptr(U),
+                                   L.ptr(W0) if mode == 'block_factor' else None, L.i64(R), L.i64(K), L.i64(K), L.i64(i1),
+                                   L.i32(128), L.i32(g), L.f32(0.0), L.f32(15.0), L.i32(flags), L.ptr(sc), L.ptr(ze), None,
+                                   L.i64(G), L.stream()), 'lcq_gptq_block')
+        torch.cuda.synchronize()
+        outs.append((tmp, Lo, Err, sc, ze))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    assert float(outs[0][1].sum()) > 0 and bool(torch.isfinite(outs[0][2]).all())
