@@ -66,9 +66,11 @@ extern "C" {
 #define LCQ_FLAG_RANGE_BF16 128   /* lcq_qparams_int on fp32 I/O: (max-min) and the 1e-5 clamp act in bf16,
                                      the rest in fp32 — torch's promotion when 0-dim bf16 ranges meet the
                                      0-dim fp32 (qmax-qmin) of a per_tensor quantizer */
-#define LCQ_FLAG_SCALE_F32 256    /* STATIC only: `scales` / `zeros` hold fp32 even for bf16 rows and enter the
-                                     arithmetic unrounded (a 0-dim fp32 qparam next to a bf16 tensor); results
-                                     still round to the row type */
+#define LCQ_FLAG_SCALE_F32 256    /* STATIC only: `scales` / `zeros` hold fp32 even for bf16 rows (a 0-dim fp32 qparam
+                                     next to a bf16 tensor).  torch on a GPU converts a 0-dim tensor operand to the
+                                     type of the result before every operation: the parameters are rounded to the row
+                                     type where they meet the rows (x / s, + z, - z, * s), scales * output_scale_factor
+                                     is formed in fp32 first; lcq_quant_fp multiplies its fp32 codes by the fp32 scale */
 
 #define LCQ_FLAG_CLAMP_RANGE 1024  /* lcq_fp8_block_quant: s = clamp(max|x|, 1e-5) / 448 (the FloatQuantizer path) instead of max|x| / 448 */
 #define LCQ_FLAG_TIE_AWAY 2048     /* lcq_fp8_block_quant: exact ties round away from zero instead of to even */

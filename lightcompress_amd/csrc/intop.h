@@ -63,7 +63,7 @@ struct IntOp {
     const float a = fabsf(s);
     p.fast = (a > 8.6736174e-19f) && (a < 1.1529215e18f) && (fabsf(z) <= 512.0f);   // s in 2^-60 .. 2^60
     p.zint = (z == rintf(z)) && (fabsf(z) <= 512.0f);       // caller-given zero points need not be integers
-    p.sdq = scale_f32 ? s * osf : rnd<BF>(s * osf);
+    p.sdq = rnd<BF>(s * osf);
     p.lo = qmin - z; p.hi = qmax - z;                       // exact: small integers
     p.clo = RINT_BIAS_BITS + (int)p.lo; p.chi = RINT_BIAS_BITS + (int)p.hi;
     p.nib0 = (uint32_t)(RINT_BIAS_BITS - ((int)z + 8)) * 0x11111111u;
@@ -121,7 +121,15 @@ struct IntOp {
 
   __device__ __forceinline__ Row load(const void* scales, const void* zeros, int64_t row) const {
     const int64_t i = scalar_qp ? 0 : row;
-    if (scale_f32) return finish(((const float*)scales)[i], zeros ? ((const float*)zeros)[i] : 0.0f);
+    if (scale_f32) {
+      // 0-dim fp32 parameters next to a 16-bit tensor: torch on a GPU converts a 0-dim tensor operand to the type of
+      // the result before every operation, so the quotient, the sums and the product see the parameters rounded to
+      // the row type, and scales * output_scale_factor (0-dim fp32 times a number) is rounded where it meets the rows
+      const float s32 = ((const float*)scales)[i];
+      Row p = finish(rnd<BF>(s32), zeros ? rnd<BF>(((const float*)zeros)[i]) : 0.0f);
+      p.sdq = rnd<BF>(s32 * osf);
+      return p;
+    }
     const float s = load_scalar<BF>(scales, i);
     const float z = zeros ? load_scalar<BF>(zeros, i) : 0.0f;
     return finish(s, z);

@@ -75,7 +75,16 @@ struct FpOp {
   }
   __device__ __forceinline__ Row load(const void* scales, const void*, int64_t row) const {
     const int64_t i = scalar_qp ? 0 : row;
-    return finish(scale_f32 ? ((const float*)scales)[i] : load_scalar<BF>(scales, i));
+    if (scale_f32) {
+      // a 0-dim fp32 scale next to a 16-bit tensor: the quotient sees it rounded to the row type (torch on a GPU
+      // converts a 0-dim tensor operand first), the dequantization multiplies the fp32 codes by it as it is
+      float s32 = ((const float*)scales)[i];
+      if (s32 == 0.0f) s32 = 1.0f;
+      Row p = finish(rnd<BF>(s32));
+      p.sm = s32;
+      return p;
+    }
+    return finish(load_scalar<BF>(scales, i));
   }
   __device__ __forceinline__ void store_qp(void* scales, void*, int64_t row, const Row& p) const {
     store_scalar<BF>(scales, row, p.s);

@@ -103,10 +103,11 @@ __global__ __launch_bounds__(256) void dequant_kernel(const void* __restrict__ q
   const int64_t n = rows * cols;
   for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n; e += (int64_t)gridDim.x * 256) {
     const int64_t row = scalar_qp ? 0 : e / cols;
+    // fp32 parameters (0-dim next to a 16-bit tensor) are rounded to the row type where they meet the rows
     const float s = scale_f32 ? ((const float*)scales)[row] : load_scalar<BF>(scales, row);
-    const float z = !zeros ? 0.0f : (scale_f32 ? ((const float*)zeros)[row] : load_scalar<BF>(zeros, row));
+    const float z = !zeros ? 0.0f : (scale_f32 ? rnd<BF>(((const float*)zeros)[row]) : load_scalar<BF>(zeros, row));
     const float d = rnd<BF>(load_scalar<BF>(q, e) - z);
-    store_scalar<BF>(out, e, rnd<BF>(d * (scale_f32 ? s * osf : rnd<BF>(s * osf))));
+    store_scalar<BF>(out, e, rnd<BF>(d * rnd<BF>(s * osf)));
   }
 }
 

@@ -576,7 +576,9 @@ class IntegerQuantizer(BaseQuantizer):
             if scales.dim() > 0 and scales.dtype != t.dtype:
                 common = torch.promote_types(t.dtype, scales.dtype)
                 t = t.to(common)
-            # a 0-dim fp32 qparam next to a bf16 tensor enters the arithmetic unrounded
+            # a 0-dim fp32 qparam next to a bf16 tensor (per_tensor, quant.py:544-558) goes in as fp32: torch on a GPU
+            # reads a 0-dim tensor operand through a cast to the result type, which the kernel does where the
+            # parameter meets the rows, while scales * output_scale_factor is still formed in fp32
             qp_dtype = t.dtype
             if scales.dim() == 0 and scales.dtype == torch.float32 and t.dtype != torch.float32:
                 flags |= L.FLAG_SCALE_F32

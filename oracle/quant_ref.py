@@ -107,14 +107,28 @@ def int_tensor_qparams(spec, t: torch.Tensor):
 # ----------------------------------------------------------------------------
 # quant / dequant   (quant.py:698-716)
 # ----------------------------------------------------------------------------
+def as_operand(t, q):
+    """A 0-dim floating tensor `q` as an operand of an element-wise operation with the 16-bit tensor `t`, the way the
+    reference's platform treats it.  torch on a GPU reads a 0-dim *tensor* operand through a cast to the type of the
+    result, so a 0-dim fp32 scale or zero point (per_tensor: quant.py:544-558 builds them from 0-dim ranges and the
+    0-dim fp32 qmax / qmin) is rounded to bf16 / fp16 before the division, sum or product; torch on the CPU does that
+    for sums and differences only and keeps the fp32 value in products and quotients.  The reference runs on the GPU:
+    the conversion is written out here so that the CPU evaluation gives the GPU's result
+    (tests/test_torch_gpu_semantics_gpu.py evaluates the reference's expressions with torch on the GPU)."""
+    if torch.is_tensor(q) and q.dim() == 0 and q.is_floating_point() and torch.is_tensor(t) and t.dim() > 0 \
+            and t.dtype in (torch.bfloat16, torch.float16) and q.dtype != t.dtype:
+        return q.to(t.dtype)
+    return q
+
+
 def int_quant(spec, t, scales, zeros, qmax, qmin):
     if spec.round_zp:
-        return torch.clamp(torch.round(t / scales) + zeros, qmin, qmax)
-    return torch.clamp(torch.round(t / scales.clamp_min(1e-9) + zeros), qmin, qmax)
+        return torch.clamp(torch.round(t / as_operand(t, scales)) + as_operand(t, zeros), qmin, qmax)
+    return torch.clamp(torch.round(t / as_operand(t, scales.clamp_min(1e-9)) + as_operand(t, zeros)), qmin, qmax)
 
 
 def int_dequant(t, scales, zeros):
-    return (t - zeros) * scales
+    return (t - as_operand(t, zeros)) * as_operand(t, scales)
 
 
 def int_quant_dequant(spec, t, scales, zeros, qmax, qmin, output_scale_factor=1):
@@ -296,7 +310,7 @@ def float_tensor_qparams(spec, t):
 def float_quant(spec, t, scales, zeros):
     """quant.py:1060-1071 (qtorch branch): result is fp32 whatever the input dtype."""
     scales[scales == 0] = 1
-    scaled = t / scales + zeros
+    scaled = t / as_operand(t, scales) + zeros
     return float_quantize_nearest(scaled.float(), spec.e_bits, spec.m_bits, spec.tie, spec.subnormals)
 
 

@@ -1,0 +1,91 @@
+"""per_tensor quantization of 16-bit tensors: the reference's own expressions evaluated by torch ON THE GPU.
+
+quant.py:544-558 builds per_tensor scales and zero points as 0-dim fp32 tensors (0-dim ranges meet the 0-dim fp32
+qmax / qmin), and quant.py:698-716 then combines them with the bf16 / fp16 tensor.  torch treats a 0-dim tensor operand
+differently on the two platforms: on a GPU every element-wise operation reads it through a cast to the result type
+(so the scale is rounded to bf16 before `tensor / scales`), on the CPU only sums and differences do.  The reference
+runs on the GPU, so the library and the CPU oracle (oracle.quant_ref.as_operand) follow the GPU; these tests pin
+both against torch's GPU kernels."""
+import pytest
+import torch
+
+from oracle import quant_ref as Q
+from tests.helpers import assert_bit_equal, gen
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+def test_zero_dim_operands_are_rounded_to_the_result_type_on_the_gpu(dev, dtype):
+    """The platform rule itself, operation by operation."""
+    x = (torch.randn(8192, generator=gen(1)) * 3).to(dtype).to(dev)
+    s = torch.tensor(0.16041666269302368, device=dev)
+    z = torch.tensor(21.428571701049805, device=dev)
+    assert s.to(dtype).float().item() != s.item() and z.to(dtype).float().item() != z.item()
+    for name, f, q in (('div', lambda a, b: a / b, s), ('mul', lambda a, b: a * b, s),
+                       ('add', lambda a, b: a + b, z), ('sub', lambda a, b: a - b, z)):
+        got = f(x, q)
+        assert got.dtype == dtype
+        rounded_first = f(x.float(), q.to(dtype).float()).to(dtype)
+        unrounded = f(x.float(), q).to(dtype)
+        assert torch.equal(got, rounded_first), name
+        assert not torch.equal(got, unrounded), name          # the data tell the two readings apart
+        # the oracle's helper writes the same conversion out for the CPU
+        assert torch.equal(f(x.cpu(), Q.as_operand(x.cpu(), q.cpu())), got.cpu()), name
+
+
+def _reference_per_tensor_on_gpu(t, bit, sym, round_zp):
+    """get_minmax_range / get_qparams / quant / dequant of quant.py:134-145, 544-558, 698-716 for per_tensor,
+    expression by expression, on whatever device `t` lives on."""
+    dev = t.device
+    if sym:                                              # quant.py:668-676: integer tensors, but a float 0.0
+        qmin, qmax = torch.tensor(-(2 ** (bit - 1))).to(dev), torch.tensor(2 ** (bit - 1) - 1).to(dev)
+    else:
+        qmin, qmax = torch.tensor(0.0).to(dev), torch.tensor(2 ** bit - 1).to(dev)
+    min_val, max_val = t.min(), t.max()
+    if sym:
+        abs_max = torch.max(max_val.abs(), min_val.abs())
+        abs_max = abs_max.clamp(min=1e-5)
+        scales = abs_max / qmax
+        zeros = torch.tensor(0.0)
+    else:
+        scales = (max_val - min_val).clamp(min=1e-5) / (qmax - qmin)
+        zeros = (qmin - torch.round(min_val / scales)).clamp(qmin, qmax)
+        if not round_zp:
+            zeros = qmin - (min_val / scales)
+    if round_zp:
+        q = torch.clamp(torch.round(t / scales) + zeros, qmin, qmax)
+    else:
+        q = torch.clamp(torch.round(t / scales.clamp_min(1e-9) + zeros), qmin, qmax)
+    return (q - zeros) * scales, q, scales, zeros
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('bit,sym,round_zp', [(8, True, True), (8, False, True), (4, False, True), (4, True, True),
+                                              (4, False, False), (8, False, False)])
+def test_per_tensor_integer_quantizer_equals_torch_on_the_gpu(dev, dtype, bit, sym, round_zp):
+    from lightcompress_amd import IntegerQuantizer
+    for seed, shape in ((2, (64, 512)), (3, (4, 33, 96)), (4, (1000,))):
+        t = (torch.randn(*shape, generator=gen(seed)) * 2.5 + (0.7 if not sym else 0.0)).to(dtype)
+        td = t.to(dev)
+        want, wq, ws, wz = _reference_per_tensor_on_gpu(td, bit, sym, round_zp)
+        # the promotion the whole matter rests on: a 0-dim range over the 0-dim fp32 (qmax - 0.0) gives an fp32 scale
+        # (the symmetric quantizer divides by an integer tensor and stays in the tensor's type)
+        assert ws.dim() == 0 and ws.dtype == (dtype if sym else torch.float32)
+        q = IntegerQuantizer(bit, sym, 'per_tensor', round_zp=round_zp)
+        got = q.fake_quant_weight_dynamic(td) if len(shape) == 2 else q.fake_quant_act_dynamic(td)
+        assert_bit_equal(got, want.reshape(shape).to(dtype), f'library against torch on the GPU {shape}')
+        # the CPU oracle, with the conversion written out, gives the same bits; the literal CPU evaluation does not
+        spec = Q.IntSpec(bit, sym, 'per_tensor', round_zp=round_zp)
+        assert_bit_equal(Q.int_fake_quant_dynamic(spec, t), want.reshape(shape).to(dtype).cpu(), f'oracle against torch on the GPU {shape}')
+        _, s, z, qmax, qmin = q.get_tensor_qparams(td)
+        assert_bit_equal(s, ws, 'scale')
+        if not sym:
+            assert_bit_equal(z, wz, 'zero point')
+        codes = q.quant(td.reshape(1, -1) if td.dim() != 2 else td, s, z, qmax, qmin)
+        assert_bit_equal(codes.reshape(-1), wq.reshape(-1), 'codes')
+    if dtype == torch.bfloat16 and not sym:              # (the symmetric scale is bf16 already: nothing to convert)
+        t = (torch.randn(64, 512, generator=gen(2)) * 2.5).to(dtype)
+        literal_cpu = _reference_per_tensor_on_gpu(t, bit, sym, round_zp)[0]
+        on_gpu = _reference_per_tensor_on_gpu(t.to(dev), bit, sym, round_zp)[0].cpu()
+        assert not torch.equal(literal_cpu, on_gpu)                        # why the conversion has to be written out
