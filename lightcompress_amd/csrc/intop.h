@@ -62,7 +62,9 @@ struct IntOp {
     p.r = __builtin_amdgcn_rcpf(s);      // 1 ulp: inside the error the exactness guards of x * r allow for
     const float a = fabsf(s);
     p.fast = (a > 8.6736174e-19f) && (a < 1.1529215e18f) && (fabsf(z) <= 512.0f);   // s in 2^-60 .. 2^60
-    p.zint = (z == rintf(z)) && (fabsf(z) <= 512.0f);       // caller-given zero points need not be integers
+    // caller-given zero points need not be integers; a row whose scale is infinite or NaN (an infinite or NaN weight)
+    // takes the element-wise form too, which hands NaN codes on like torch.clamp does
+    p.zint = (z == rintf(z)) && (fabsf(z) <= 512.0f) && (a < __builtin_inff());
     p.sdq = rnd<BF>(s * osf);
     p.lo = qmin - z; p.hi = qmax - z;                       // exact: small integers
     p.clo = RINT_BIAS_BITS + (int)p.lo; p.chi = RINT_BIAS_BITS + (int)p.hi;
@@ -151,6 +153,7 @@ struct IntOp {
       const float t = rnd<BF>(x / clamp_min_nan(p.s, lo));
       q = rintf(rnd<BF>(t + p.z));
     }
+    if (q != q) return q;                                    // torch.clamp hands a NaN on (inf / inf of an infinite weight)
     return __builtin_amdgcn_fmed3f(q, qmin, qmax);
   }
 

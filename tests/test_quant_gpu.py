@@ -773,3 +773,20 @@ def test_float_per_block_with_given_scales(dev, dtype, shape):
     oc, os_, _ = Q.float_per_block_real_quant(spec, w)
     assert_bit_equal(dyn_codes, oc, 'dynamic per_block codes'); assert_bit_equal(dyn_s, os_, 'dynamic per_block scales')
     assert_bit_equal(q.fake_quant_weight_dynamic(w.to(dev)), Q.float_per_block_static(spec, w, os_.view(mb, 1, nb, 1).clone()), 'dynamic per_block fake quant')
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('sym', [True, False])
+def test_int_infinite_and_nan_weights_propagate_like_torch(dev, dtype, sym):
+    """An infinite weight makes its group's scale infinite: every dequantized value of the group is 0 * inf = NaN, the
+    infinite element's own code is round(inf / inf) = NaN, which torch.clamp hands on; a NaN weight turns the range
+    and with it the whole group into NaN.  Groups without such a weight are untouched."""
+    for bad in (float('inf'), float('-inf'), float('nan')):
+        w = weight_like(16, 512, seed=77, dtype=dtype)
+        w[3, 130] = bad
+        spec = Q.IntSpec(4, sym, 'per_group', group_size=128)
+        got = _iq(4, sym, 'per_group', group_size=128).fake_quant_weight_dynamic(w.to(dev)).cpu()
+        want = Q.int_fake_quant_dynamic(spec, w)
+        assert torch.equal(torch.isnan(got), torch.isnan(want)), bad
+        assert torch.equal(torch.nan_to_num(got.float(), 0.0, 1e30, -1e30), torch.nan_to_num(want.float(), 0.0, 1e30, -1e30)), bad
+        assert bool(torch.isnan(want[3, 128:256]).all()) or not sym
