@@ -74,6 +74,7 @@ extern "C" {
 
 #define LCQ_FLAG_CLAMP_RANGE 1024  /* lcq_fp8_block_quant: s = clamp(max|x|, 1e-5) / 448 (the FloatQuantizer path) instead of max|x| / 448 */
 #define LCQ_FLAG_TIE_AWAY 2048     /* lcq_fp8_block_quant: exact ties round away from zero instead of to even */
+#define LCQ_FLAG_RANGE_F16 8192    /* LCQ_FLAG_RANGE_BF16 for ranges that were fp16 */
 #define LCQ_FLAG_ROWS16 4096       /* lcq_gptq_block: 16 rows per workgroup whatever R is (the default takes 32 from 6144 rows on; same results bit for bit) */
 #define LCQ_FLAG_ROW_QP 512       /* lcq_quant_fp_emu, STATIC only: `scales` holds one value per row */
 
@@ -94,12 +95,13 @@ extern "C" {
  * (quant / dequant / quant_dequant) and so the bodies of
  * fake_quant_{weight,act}_{dynamic,static} (:718-868) and
  * real_quant_weight_{dynamic,static} (:870-952).
- *  x       [rows, cols] of `dtype` (LCQ_F32 | LCQ_BF16)
+ *  x       [rows, cols] of `dtype` (LCQ_F32 | LCQ_BF16 | LCQ_F16; fp16 rows run through the element-wise kernel,
+ *          one wave per row: correct to the bit, not tuned; no LCQ_CODE_CT4 for them)
  *  dq      same shape/type or NULL        -> (q - z) * (s * out_scale_factor)
  *  codes   [rows, cols] of code_dtype or NULL
  *  scales  [rows] (or [1] with SCALAR_QP) of `dtype`: output, input if STATIC
  *  zeros   likewise; may be NULL (zero point 0; never written when SYM)
- * bf16 rows round to bf16 after every arithmetic step like torch does. */
+ * bf16 / fp16 rows round to their type after every arithmetic step like torch does. */
 int lcq_quant_int(const void* x, int dtype, int64_t rows, int64_t cols, float qmin, float qmax, int flags,
                   float out_scale_factor, void* dq, void* codes, int code_dtype, void* scales, void* zeros,
                   void* stream);

@@ -22,6 +22,7 @@ FLAG_SYM, FLAG_NO_ROUND_ZP, FLAG_STATIC, FLAG_SCALAR_QP = 1, 2, 4, 8
 FLAG_TIE_EVEN, FLAG_NO_SUBNORMALS, FLAG_DQ_F32 = 16, 32, 64
 FLAG_RANGE_BF16, FLAG_SCALE_F32, FLAG_ROW_QP = 128, 256, 512
 FLAG_ROWS16 = 4096
+FLAG_RANGE_F16 = 8192
 
 _ERR = {-1: 'invalid argument', -2: 'misaligned pointer', -3: 'unsupported dtype', -4: 'kernel launch failed',
         -5: 'workspace too small', -6: 'input larger than the entry point\'s stated maximum'}

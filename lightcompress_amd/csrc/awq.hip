@@ -42,7 +42,7 @@ double* static_scratch() {
 
 // ---- column-wise mean of |x| over T rows ------------------------------------------------
 // grid = (column blocks of 256 * N, row splits); every thread owns one 16-byte column chunk
-template <bool BF>
+template <int BF>
 __global__ __launch_bounds__(256) void absmean_stage1(const u32x4* __restrict__ x, int64_t T, int64_t K,
                                                       float* __restrict__ part) {
   constexpr int N = Vec<BF>::N;
@@ -64,7 +64,7 @@ __global__ __launch_bounds__(256) void absmean_stage1(const u32x4* __restrict__ 
   #pragma unroll
   for (int i = 0; i < N; ++i) p[i] = acc[i];
 }
-template <bool BF>
+template <int BF>
 __global__ __launch_bounds__(256) void absmean_stage2(const float* __restrict__ part, int nparts, int64_t T, int64_t K,
                                                       void* __restrict__ out) {
   const int64_t k = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -75,7 +75,7 @@ __global__ __launch_bounds__(256) void absmean_stage2(const float* __restrict__ 
 }
 
 // ---- x / s[None, :] -----------------------------------------------------------------------
-template <bool BF>
+template <int BF>
 __global__ __launch_bounds__(256) void div_cols_kernel(const u32x4* __restrict__ x, const u32x4* __restrict__ s,
                                                        int64_t nchunks_total, int64_t nch_row, u32x4* __restrict__ out) {
   constexpr int N = Vec<BF>::N;
@@ -91,7 +91,7 @@ __global__ __launch_bounds__(256) void div_cols_kernel(const u32x4* __restrict__
 
 // ---- in-place capable w (*|/) s[col]  or  w (*|/) s[row] -------------------------------------
 // mode: 0 multiply by a column vector, 1 divide by a column vector, 2 multiply by a row vector, 3 divide by one
-template <bool BF>
+template <int BF>
 __global__ __launch_bounds__(256) void scale_kernel(const u32x4* x, const void* __restrict__ s, int64_t nchunks_total,
                                                     int64_t nch_row, int mode, u32x4* out) {
   constexpr int N = Vec<BF>::N;
@@ -117,7 +117,7 @@ __global__ __launch_bounds__(256) void scale_kernel(const u32x4* x, const void* 
 }
 
 // ---- mean of squared differences ------------------------------------------------------------
-template <bool BF>
+template <int BF>
 __global__ __launch_bounds__(256) void sqerr_stage1(const u32x4* __restrict__ a, const u32x4* __restrict__ b,
                                                     int64_t nchunks, double* __restrict__ part) {
   constexpr int N = Vec<BF>::N;
@@ -151,7 +151,7 @@ __global__ __launch_bounds__(256) void sqerr_stage2(const double* __restrict__ p
 
 // ---- mean over rows of |W| / (group max of |W|) -----------------------------------------------
 // one workgroup per slab of rows; a group of g columns is shared by g/N consecutive lanes
-template <bool BF, int TEAM>
+template <int BF, int TEAM>
 __global__ __launch_bounds__(256) void wscale_stage1(const u32x4* __restrict__ w, int64_t R, int64_t K,
                                                      float* __restrict__ part) {
   constexpr int N = Vec<BF>::N;
@@ -185,7 +185,7 @@ __global__ __launch_bounds__(256) void wscale_stage1(const u32x4* __restrict__ w
   }
 }
 
-template <bool BF>
+template <int BF>
 int absmean(const void* x, int64_t T, int64_t K, void* out, float* part, hipStream_t st) {
   constexpr int N = Vec<BF>::N;
   if (K % N != 0 || ((uintptr_t)x % 16) != 0) return LCQ_EALIGN;
@@ -198,7 +198,7 @@ int absmean(const void* x, int64_t T, int64_t K, void* out, float* part, hipStre
   return LCQ_OK;
 }
 
-template <bool BF>
+template <int BF>
 int wscale(const void* w, int64_t R, int64_t K, int g, void* out, float* part, hipStream_t st) {
   constexpr int N = Vec<BF>::N;
   if (K % N != 0 || g % N != 0 || K % g != 0 || ((uintptr_t)w % 16) != 0) return LCQ_EALIGN;
@@ -226,6 +226,7 @@ int lcq_absmean_cols(const void* x, int dtype, int64_t T, int64_t K, void* out, 
   int rc;
   if (dtype == LCQ_F32) rc = absmean<false>(x, T, K, out, (float*)workspace, st);
   else if (dtype == LCQ_BF16) rc = absmean<true>(x, T, K, out, (float*)workspace, st);
+  else if (dtype == LCQ_F16) rc = absmean<ROW_F16>(x, T, K, out, (float*)workspace, st);
   else return LCQ_EDTYPE;
   if (rc != LCQ_OK) return rc;
   LCQ_CHECK_LAUNCH();
@@ -239,6 +240,7 @@ int lcq_awq_weight_scale(const void* w, int dtype, int64_t R, int64_t K, int gro
   int rc;
   if (dtype == LCQ_F32) rc = wscale<false>(w, R, K, group_size, out, (float*)workspace, st);
   else if (dtype == LCQ_BF16) rc = wscale<true>(w, R, K, group_size, out, (float*)workspace, st);
+  else if (dtype == LCQ_F16) rc = wscale<ROW_F16>(w, R, K, group_size, out, (float*)workspace, st);
   else return LCQ_EDTYPE;
   if (rc != LCQ_OK) return rc;
   LCQ_CHECK_LAUNCH();
@@ -247,14 +249,15 @@ int lcq_awq_weight_scale(const void* w, int dtype, int64_t R, int64_t K, int gro
 
 int lcq_div_cols(const void* x, int dtype, int64_t T, int64_t K, const void* s, void* out, void* stream) {
   if (!x || !s || !out || T <= 0 || K <= 0) return LCQ_EINVAL;
-  const int n = dtype == LCQ_BF16 ? 8 : 4;
-  if (dtype != LCQ_BF16 && dtype != LCQ_F32) return LCQ_EDTYPE;
+  const int n = dtype == LCQ_F32 ? 4 : 8;
+  if (dtype != LCQ_BF16 && dtype != LCQ_F32 && dtype != LCQ_F16) return LCQ_EDTYPE;
   if (K % n != 0 || (((uintptr_t)x | (uintptr_t)s | (uintptr_t)out) % 16) != 0) return LCQ_EALIGN;
   const int64_t nch_row = K / n, total = T * nch_row;
   int64_t grid = (total + 255) / 256;
   if (grid > 65536 * 4) grid = 65536 * 4;
   hipStream_t st = (hipStream_t)stream;
   if (dtype == LCQ_BF16) div_cols_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)x, (const u32x4*)s, total, nch_row, (u32x4*)out);
+  else if (dtype == LCQ_F16) div_cols_kernel<ROW_F16><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)x, (const u32x4*)s, total, nch_row, (u32x4*)out);
   else div_cols_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)x, (const u32x4*)s, total, nch_row, (u32x4*)out);
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;
@@ -262,27 +265,29 @@ int lcq_div_cols(const void* x, int dtype, int64_t T, int64_t K, const void* s, 
 
 int lcq_scale_matrix(const void* x, int dtype, int64_t T, int64_t K, const void* s, int mode, void* out, void* stream) {
   if (!x || !s || !out || T <= 0 || K <= 0 || mode < 0 || mode > 3) return LCQ_EINVAL;
-  const int n = dtype == LCQ_BF16 ? 8 : 4;
-  if (dtype != LCQ_BF16 && dtype != LCQ_F32) return LCQ_EDTYPE;
+  const int n = dtype == LCQ_F32 ? 4 : 8;
+  if (dtype != LCQ_BF16 && dtype != LCQ_F32 && dtype != LCQ_F16) return LCQ_EDTYPE;
   if (K % n != 0 || (((uintptr_t)x | (uintptr_t)out) % 16) != 0 || (mode < 2 && ((uintptr_t)s % 16) != 0)) return LCQ_EALIGN;
   const int64_t nch_row = K / n, total = T * nch_row;
   int64_t grid = (total + 255) / 256;
   if (grid > 65536 * 4) grid = 65536 * 4;
   hipStream_t st = (hipStream_t)stream;
   if (dtype == LCQ_BF16) scale_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)x, s, total, nch_row, mode, (u32x4*)out);
+  else if (dtype == LCQ_F16) scale_kernel<ROW_F16><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)x, s, total, nch_row, mode, (u32x4*)out);
   else scale_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)x, s, total, nch_row, mode, (u32x4*)out);
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;
 }
 
 static int sq_err_mean_launch(const void* a, const void* b, int dtype, int64_t n, float* out, double* part, hipStream_t st) {
-  const int nn = dtype == LCQ_BF16 ? 8 : 4;
-  if (dtype != LCQ_BF16 && dtype != LCQ_F32) return LCQ_EDTYPE;
+  const int nn = dtype == LCQ_F32 ? 4 : 8;
+  if (dtype != LCQ_BF16 && dtype != LCQ_F32 && dtype != LCQ_F16) return LCQ_EDTYPE;
   if (n % nn != 0 || (((uintptr_t)a | (uintptr_t)b) % 16) != 0) return LCQ_EALIGN;
   const int64_t nchunks = n / nn;
   int64_t grid = (nchunks + 255) / 256;
   if (grid > SQERR_PARTS_MAX) grid = SQERR_PARTS_MAX;
   if (dtype == LCQ_BF16) sqerr_stage1<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)a, (const u32x4*)b, nchunks, part);
+  else if (dtype == LCQ_F16) sqerr_stage1<ROW_F16><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)a, (const u32x4*)b, nchunks, part);
   else sqerr_stage1<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)a, (const u32x4*)b, nchunks, part);
   sqerr_stage2<<<dim3(1), dim3(256), 0, st>>>(part, (int)grid, (double)n, out);
   LCQ_CHECK_LAUNCH();

@@ -289,7 +289,7 @@ int lcq_awq_clip_search(const void* w, const void* x, int64_t R, int64_t K, int6
   op.qmin = qmin; op.qmax = qmax; op.qrange = qmax - qmin; op.osf = 1.0f;
   op.rqmax = (float)(1.0 / (double)qmax); op.rqrange = (float)(1.0 / (double)(qmax - qmin));
   op.sym = (flags & LCQ_FLAG_SYM) != 0; op.round_zp = 1; op.is_static = 0; op.scalar_qp = 0; op.dq_f32 = 0;
-  op.range_bf16 = 0; op.scale_f32 = 0; op.colscale = nullptr; op.wrow_cols = 1; op.code_dtype = LCQ_CODE_NONE;
+  op.range_bf16 = 0; op.range_f16 = 0; op.scale_f32 = 0; op.colscale = nullptr; op.wrow_cols = 1; op.code_dtype = LCQ_CODE_NONE;
   const dim3 grid((unsigned)((R + ROWS_PER_WG - 1) / ROWS_PER_WG), (unsigned)(K / CG));
   awq_clip_kernel<<<grid, dim3(512), 0, (hipStream_t)stream>>>((const uint16_t*)w, (const uint16_t*)x, (int)R, (int)K,
                                                                (int)T, n_grid, n_steps, clip_sym, op, (uint16_t*)best_max,

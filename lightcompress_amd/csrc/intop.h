@@ -23,9 +23,9 @@ constexpr float RINT_BIAS = 12582912.0f;
 constexpr int RINT_BIAS_BITS = 0x4B400000;
 
 // FAST: round_zp and |qmin|,qmax <= 256 (every stock configuration).
-template <bool BF_, bool FAST, bool PRESCALE = false, int CD_ = -1>
+template <int BF_, bool FAST, bool PRESCALE = false, int CD_ = -1>
 struct IntOp {
-  static constexpr bool BF = BF_;
+  static constexpr int BF = BF_;          // row type: 0 fp32, 1 bf16, 2 fp16 (element-wise forms only: FAST is false)
   static constexpr bool HAS_PRESCALE = PRESCALE;
   static constexpr bool HAS_FUSED_DQ = FAST;
   static constexpr bool HAS_CUSTOM_EMIT = false;
@@ -34,7 +34,7 @@ struct IntOp {
   using Row = IntRow;
   float qmin, qmax, qrange, osf;
   float rqmax, rqrange;         // 1 / qmax, 1 / qrange (fp32-rounded)
-  int sym, round_zp, is_static, scalar_qp, dq_f32, code_dtype, range_bf16, scale_f32;
+  int sym, round_zp, is_static, scalar_qp, dq_f32, code_dtype, range_bf16, range_f16, scale_f32;
   // optional per-column factor applied first (AWQ: W * s), rows of the reshaped tensor tile a
   // weight row of wrow_cols columns
   const void* colscale;
@@ -76,18 +76,19 @@ struct IntOp {
   // the product a * rc stands for the quotient unless it lies within 8 ulp of a bf16 rounding
   // midpoint; fp32 rows need the correctly rounded quotient itself.
   __device__ __forceinline__ float div_const(float a, float c, float rc) const {
-    if constexpr (BF) {
+    if constexpr (BF == ROW_BF16) {
       float q = a * rc;
       if (__builtin_expect(((f2u(q) & 0xffffu) - 0x7ff8u) <= 0x10u, 0)) q = a / c;
       return rnd<BF>(q);
     } else {
-      return a / c;
+      return rnd<BF>(a / c);                                 // fp32: the quotient itself; fp16: the quotient, rounded
     }
   }
 
   // get_qparams, quant.py:544-558
   __device__ __forceinline__ Row make(float mn, float mx) const {
-    const float cmin = (BF || range_bf16) ? 1.0013580322265625e-05f : 1e-5f;   // clamp(min=1e-5) in the range dtype
+    // clamp(min=1e-5) in the range dtype: 1e-5 rounds to the same number in bf16 (1.3125 * 2^-17) and fp16 (168 * 2^-24)
+    const float cmin = (BF || range_bf16 || range_f16) ? 1.0013580322265625e-05f : 1e-5f;
     float s, z;
     if (sym) {
       float a = nan_max(fabsf(mx), fabsf(mn));
@@ -97,13 +98,16 @@ struct IntOp {
     } else {
       float d = rnd<BF>(mx - mn);
       if (range_bf16) d = bf16_round(d);
+      if (range_f16) d = f16_round(d);
       d = clamp_min_nan(d, cmin);
       s = div_const(d, qrange, rqrange);
       // mn / s through the reciprocal, with the same exactness guards as the per-element quotients
       float t = mn * __builtin_amdgcn_rcpf(s);
       const float as = fabsf(s);
       bool ok = (as > 8.6736174e-19f) && (as < 1.1529215e18f);
-      if constexpr (BF) {
+      if constexpr (BF == ROW_F16) {
+        ok = false;                                          // fp16 rows: always the division
+      } else if constexpr (BF == ROW_BF16) {
         ok = ok && (((f2u(t) & 0xffffu) - 0x7ff8u) > 0x10u);
       } else {
         const float fr = t - rintf(t);
@@ -149,7 +153,7 @@ struct IntOp {
       const float t = rnd<BF>(x / p.s);
       q = rnd<BF>(rintf(t) + p.z);
     } else {
-      const float lo = BF ? 1.00044417e-09f : 1e-9f;         // scales.clamp_min(1e-9)
+      const float lo = BF == ROW_F16 ? 0.0f : (BF ? 1.00044417e-09f : 1e-9f);   // scales.clamp_min(1e-9): the bound in the row type (0 in fp16)
       const float t = rnd<BF>(x / clamp_min_nan(p.s, lo));
       q = rintf(rnd<BF>(t + p.z));
     }
@@ -252,7 +256,7 @@ struct IntOp {
   // dequant, quant.py:709-711 (scale already multiplied by output_scale_factor)
   __device__ __forceinline__ float deq_raw(float q, const Row& p) const {   // before the rounding to the row type
     float d = q - p.z;                                       // exact for small integer codes
-    if constexpr (BF) { if (!FAST || !p.zint) d = bf16_round(d); }
+    if constexpr (BF != 0) { if (!FAST || !p.zint) d = rnd<BF>(d); }
     return d * p.sdq;
   }
   __device__ __forceinline__ float deq(float q, const Row& p) const { return rnd_e<BF>(deq_raw(q, p)); }
@@ -282,6 +286,7 @@ Op make_op(float qmin, float qmax, int flags, float osf, int code_dtype) {
   c.scalar_qp = (flags & LCQ_FLAG_SCALAR_QP) != 0;
   c.dq_f32 = 0;
   c.range_bf16 = (flags & LCQ_FLAG_RANGE_BF16) != 0;
+  c.range_f16 = (flags & LCQ_FLAG_RANGE_F16) != 0;
   c.scale_f32 = (flags & LCQ_FLAG_SCALE_F32) != 0;
   c.colscale = nullptr; c.wrow_cols = 1;
   c.code_dtype = code_dtype;

@@ -26,9 +26,9 @@ struct FpRow {
   int inrange;      // dynamic rows: every |x / s| of the row stays below hw_lim, no per-element check needed
 };
 
-template <bool BF_>
+template <int BF_>
 struct FpOp {
-  static constexpr bool BF = BF_;
+  static constexpr int BF = BF_;          // row type: 0 fp32, 1 bf16, 2 fp16 (element-wise forms only)
   static constexpr bool HAS_PRESCALE = false;
   static constexpr bool HAS_FUSED_DQ = false;
   static constexpr bool HAS_CUSTOM_EMIT = true;
@@ -62,12 +62,12 @@ struct FpOp {
     const float amax = nan_max(fabsf(mx), fabsf(mn));
     const float a = clamp_min_nan(amax, cmin);
     Row p;
-    if constexpr (BF) {                                   // a * (1/qmax) unless the product is within 8 ulp of a bf16 midpoint
+    if constexpr (BF == ROW_BF16) {                       // a * (1/qmax) unless the product is within 8 ulp of a bf16 midpoint
       float q = a * rqmax;
       if (__builtin_expect(((f2u(q) & 0xffffu) - 0x7ff8u) <= 0x10u, 0)) q = a / qmax;
       p = finish(rnd<BF>(q));
     } else {
-      p = finish(a / qmax);
+      p = finish(rnd<BF>(a / qmax));
     }
     // the largest quotient of the row, with room for the reciprocal's and the product's rounding (NaN: false)
     p.inrange = (amax * p.r) * 1.001f < hw_lim;
@@ -78,9 +78,13 @@ struct FpOp {
     if (scale_f32) {
       // a 0-dim fp32 scale next to a 16-bit tensor: the quotient sees it rounded to the row type (torch on a GPU
       // converts a 0-dim tensor operand first), the dequantization multiplies the fp32 codes by it as it is
-      float s32 = ((const float*)scales)[i];
-      if (s32 == 0.0f) s32 = 1.0f;
-      Row p = finish(rnd<BF>(s32));
+      // (scales[scales == 0] = 1 acts on the fp32 value; a scale that only the rounding turns into 0 divides as 0)
+      Row p = finish(((const float*)scales)[i]);
+      const float s32 = p.s;
+      p.s = rnd<BF>(s32);
+      p.r = __builtin_amdgcn_rcpf(p.s);
+      const float a = fabsf(p.s);
+      p.fast = (a > 8.6736174e-19f) && (a < 1.1529215e18f);
       p.sm = s32;
       return p;
     }
@@ -123,7 +127,9 @@ struct FpOp {
   __device__ __forceinline__ float code(float x, const Row& p) const {
     float t = x * p.r;
     bool ok;
-    if constexpr (BF) {
+    if constexpr (BF == ROW_F16) {
+      ok = false;                                          // fp16 rows: always the division
+    } else if constexpr (BF == ROW_BF16) {
       const uint32_t low = f2u(t) & 0xffffu;               // bf16 rounding midpoint nearby?
       ok = (low - 0x7ff8u) > 0x10u;
     } else {
@@ -285,7 +291,7 @@ struct FpOp {
   }
 };
 
-template <bool BF>
+template <int BF>
 FpOp<BF> make_op(int e_bits, int m_bits, float qmax, int flags, int code_dtype) {
   FpOp<BF> c;
   c.qmax = qmax; c.rqmax = (float)(1.0 / (double)qmax); c.e_bits = e_bits; c.m_bits = m_bits;
@@ -313,7 +319,7 @@ FpOp<BF> make_op(int e_bits, int m_bits, float qmax, int flags, int code_dtype) 
 }
 
 // FloatQuantizer.dequant on stored fp32 codes: out = (q - 0) * s in fp32
-template <bool BF>
+template <int BF>
 __global__ __launch_bounds__(256) void dequant_fp_kernel(const float* __restrict__ q, int64_t rows, int64_t cols,
                                                          const void* __restrict__ scales, float* __restrict__ out,
                                                          int scalar_qp) {
@@ -420,6 +426,8 @@ int lcq_quant_fp(const void* x, int dtype, int64_t rows, int64_t cols, int e_bit
     rc = dispatch_rows(x, rows, cols, dq, codes, scales, (void*)nullptr, make_op<false>(e_bits, m_bits, qmax, flags, code_dtype), false, st);
   else if (dtype == LCQ_BF16)
     rc = dispatch_rows(x, rows, cols, dq, codes, scales, (void*)nullptr, make_op<true>(e_bits, m_bits, qmax, flags, code_dtype), false, st);
+  else if (dtype == LCQ_F16)                               // fp16 rows: the element-wise kernel (correct to the bit, not tuned)
+    rc = dispatch_rows(x, rows, cols, dq, codes, scales, (void*)nullptr, make_op<ROW_F16>(e_bits, m_bits, qmax, flags, code_dtype), true, st);
   else return LCQ_EDTYPE;
   if (rc != LCQ_OK) return rc;
   LCQ_CHECK_LAUNCH();
@@ -436,6 +444,7 @@ int lcq_dequant_fp(const float* q, int64_t rows, int64_t cols, const void* scale
   hipStream_t st = (hipStream_t)stream;
   if (scale_dtype == LCQ_F32) dequant_fp_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>(q, rows, cols, scales, out, scalar_qp);
   else if (scale_dtype == LCQ_BF16) dequant_fp_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>(q, rows, cols, scales, out, scalar_qp);
+  else if (scale_dtype == LCQ_F16) dequant_fp_kernel<ROW_F16><<<dim3((unsigned)grid), dim3(256), 0, st>>>(q, rows, cols, scales, out, scalar_qp);
   else return LCQ_EDTYPE;
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;

@@ -14,6 +14,8 @@
 //   fp32 rows : every step is one IEEE fp32 op (true division, rintf).
 //   bf16 rows : every step is computed in fp32 and rounded to bf16 (RNE)
 //               before the next step, as torch does for bf16 tensors.
+//   fp16 rows : the same with fp16 roundings, through the element-wise kernel and true divisions only (one wave per
+//               row, one element per lane and step: a compatibility path, not a tuned one).
 // The per-element division x/s is evaluated as x*(1/s) with an exactness
 // guard: whenever the approximate quotient is close enough to a rounding
 // boundary that the IEEE quotient could round differently, the lane falls
@@ -23,15 +25,20 @@
 namespace {
 using namespace lcq;
 
-template <bool BF>
+template <int BF>
 int run(const void* x, int64_t rows, int64_t cols, float qmin, float qmax, int flags, float osf, void* dq,
         void* codes, int code_dtype, void* scales, void* zeros, hipStream_t st) {
   const bool big = (qmax > 256.0f) || (qmin < -256.0f);
-  const bool general = big || (flags & LCQ_FLAG_NO_ROUND_ZP);
+  const bool general = big || (flags & LCQ_FLAG_NO_ROUND_ZP) || BF == ROW_F16;     // fp16 rows: the element-wise kernel
+  if constexpr (BF == ROW_F16) {
+    if (code_dtype == LCQ_CODE_CT4) return LCQ_EDTYPE;      // nibbles come from the vectorised bf16 / fp32 kernels only
+  }
   if (general)
     return dispatch_rows(x, rows, cols, dq, codes, scales, zeros,
                          make_op<IntOp<BF, false>>(qmin, qmax, flags, osf, code_dtype), true, st);
   // the common storage formats get kernels with the store path fixed at compile time
+  if constexpr (BF == ROW_F16) return LCQ_EDTYPE;            // not reached: `general` above
+  else {
   #define LCQ_RUN(CDV) return dispatch_rows(x, rows, cols, dq, codes, scales, zeros, \
                          make_op<IntOp<BF, true, false, CDV>>(qmin, qmax, flags, osf, code_dtype), false, st)
   switch (code_dtype) {
@@ -42,10 +49,11 @@ int run(const void* x, int64_t rows, int64_t cols, float qmin, float qmax, int f
     default: LCQ_RUN(-1);
   }
   #undef LCQ_RUN
+  }
 }
 
 // get_minmax_range (row-wise), quant.py:141-143
-template <bool BF>
+template <int BF>
 __global__ __launch_bounds__(256) void minmax_rows_kernel(const void* __restrict__ x, int64_t rows, int64_t cols,
                                                           void* __restrict__ mn_out, void* __restrict__ mx_out) {
   const int lane = threadIdx.x & 63;
@@ -62,7 +70,7 @@ __global__ __launch_bounds__(256) void minmax_rows_kernel(const void* __restrict
 }
 
 // per_tensor range, quant.py:135-137: stage 1 writes one (min,max) per workgroup
-template <bool BF>
+template <int BF>
 __global__ __launch_bounds__(256) void minmax_all_stage1(const void* __restrict__ x, int64_t n, float* __restrict__ part) {
   __shared__ float sm[8];
   float mn = __builtin_inff(), mx = -__builtin_inff();
@@ -74,7 +82,7 @@ __global__ __launch_bounds__(256) void minmax_all_stage1(const void* __restrict_
   mx = block_reduce<true>(mx, sm);
   if (threadIdx.x == 0) { part[2 * blockIdx.x] = mn; part[2 * blockIdx.x + 1] = mx; }
 }
-template <bool BF>
+template <int BF>
 __global__ __launch_bounds__(256) void minmax_all_stage2(const float* __restrict__ part, int nparts,
                                                          void* __restrict__ mn_out, void* __restrict__ mx_out) {
   __shared__ float sm[8];
@@ -86,7 +94,7 @@ __global__ __launch_bounds__(256) void minmax_all_stage2(const float* __restrict
 }
 
 // get_qparams on explicit ranges, quant.py:544-558
-template <bool BF>
+template <int BF>
 __global__ void qparams_kernel(const void* __restrict__ mn, const void* __restrict__ mx, int64_t n,
                                void* __restrict__ scales, void* __restrict__ zeros, IntOp<BF, false> op) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -96,7 +104,7 @@ __global__ void qparams_kernel(const void* __restrict__ mn, const void* __restri
 }
 
 // dequant, quant.py:709-711, on stored float codes
-template <bool BF>
+template <int BF>
 __global__ __launch_bounds__(256) void dequant_kernel(const void* __restrict__ q, int64_t rows, int64_t cols,
                                                       const void* __restrict__ scales, const void* __restrict__ zeros,
                                                       void* __restrict__ out, int scalar_qp, int scale_f32, float osf) {
@@ -117,9 +125,9 @@ __global__ __launch_bounds__(256) void dequant_kernel(const void* __restrict__ q
 // cur_min / cur_max start as the row's min / max and - as in the reference, whose best_min_val / best_max_val
 // alias the range tensors - are the values the NEXT step shrinks.  All arithmetic in fp32 (tensor.float()).
 // One wave per row; the row is re-read from L1/L2 on every step.
-template <bool BF>
+template <int BF>
 __global__ __launch_bounds__(256) void mse_range_kernel(const void* __restrict__ x, int64_t rows, int64_t cols, int steps,
-                                                        int grid_n, float norm, IntOp<false, false> op,
+                                                        int grid_n, float norm, IntOp<0, false> op,
                                                         float* __restrict__ mn_out, float* __restrict__ mx_out) {
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -212,6 +220,7 @@ int lcq_quant_int(const void* x, int dtype, int64_t rows, int64_t cols, float qm
   int rc;
   if (dtype == LCQ_F32) rc = run<false>(x, rows, cols, qmin, qmax, flags, out_scale_factor, dq, codes, code_dtype, scales, zeros, st);
   else if (dtype == LCQ_BF16) rc = run<true>(x, rows, cols, qmin, qmax, flags, out_scale_factor, dq, codes, code_dtype, scales, zeros, st);
+  else if (dtype == LCQ_F16) rc = run<ROW_F16>(x, rows, cols, qmin, qmax, flags, out_scale_factor, dq, codes, code_dtype, scales, zeros, st);
   else return LCQ_EDTYPE;
   if (rc != LCQ_OK) return rc;
   LCQ_CHECK_LAUNCH();
@@ -228,6 +237,7 @@ int lcq_mse_range(const void* x, int dtype, int64_t rows, int64_t cols, float qm
   hipStream_t st = (hipStream_t)stream;
   if (dtype == LCQ_F32) mse_range_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>(x, rows, cols, steps, grid_n, norm, op, min_out, max_out);
   else if (dtype == LCQ_BF16) mse_range_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>(x, rows, cols, steps, grid_n, norm, op, min_out, max_out);
+  else if (dtype == LCQ_F16) mse_range_kernel<ROW_F16><<<dim3((unsigned)grid), dim3(256), 0, st>>>(x, rows, cols, steps, grid_n, norm, op, min_out, max_out);
   else return LCQ_EDTYPE;
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;
@@ -262,7 +272,7 @@ int lcq_awq_scale_quant(const void* w, int dtype, int64_t R, int64_t K, const vo
   const int64_t cols = group_size > 0 ? group_size : K;
   if (K % cols != 0) return LCQ_EINVAL;
   const int64_t rows = R * (K / cols);
-  const int n = dtype == LCQ_BF16 ? 8 : 4;
+  const int n = dtype == LCQ_F32 ? 4 : 8;
   if (cols % n != 0 || K % n != 0 || ((uintptr_t)colscale % 16) != 0) return LCQ_EALIGN;
   hipStream_t st = (hipStream_t)stream;
   int rc;
@@ -275,6 +285,10 @@ int lcq_awq_scale_quant(const void* w, int dtype, int64_t R, int64_t K, const vo
     auto op = make_op<IntOp<true, true, true>>(qmin, qmax, flags, 1.0f, LCQ_CODE_NONE);
     op.colscale = colscale; op.wrow_cols = (int)K; op.is_static = 0;
     rc = dispatch_rows(w, rows, cols, out, (void*)nullptr, (void*)nullptr, (void*)nullptr, op, false, st);
+  } else if (dtype == LCQ_F16) {                           // element-wise kernel
+    auto op = make_op<IntOp<ROW_F16, false, true>>(qmin, qmax, flags, 1.0f, LCQ_CODE_NONE);
+    op.colscale = colscale; op.wrow_cols = (int)K; op.is_static = 0;
+    rc = dispatch_rows(w, rows, cols, out, (void*)nullptr, (void*)nullptr, (void*)nullptr, op, true, st);
   } else return LCQ_EDTYPE;
   if (rc != LCQ_OK) return rc;
   LCQ_CHECK_LAUNCH();
@@ -289,6 +303,7 @@ int lcq_minmax_rows(const void* x, int dtype, int64_t rows, int64_t cols, void* 
   hipStream_t st = (hipStream_t)stream;
   if (dtype == LCQ_F32) minmax_rows_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>(x, rows, cols, min_out, max_out);
   else if (dtype == LCQ_BF16) minmax_rows_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>(x, rows, cols, min_out, max_out);
+  else if (dtype == LCQ_F16) minmax_rows_kernel<ROW_F16><<<dim3((unsigned)grid), dim3(256), 0, st>>>(x, rows, cols, min_out, max_out);
   else return LCQ_EDTYPE;
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;
@@ -308,6 +323,9 @@ int lcq_minmax_all(const void* x, int dtype, int64_t n, void* min_out, void* max
   } else if (dtype == LCQ_BF16) {
     minmax_all_stage1<true><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(x, n, part);
     minmax_all_stage2<true><<<dim3(1), dim3(256), 0, st>>>(part, (int)blocks, min_out, max_out);
+  } else if (dtype == LCQ_F16) {
+    minmax_all_stage1<ROW_F16><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(x, n, part);
+    minmax_all_stage2<ROW_F16><<<dim3(1), dim3(256), 0, st>>>(part, (int)blocks, min_out, max_out);
   } else return LCQ_EDTYPE;
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;
@@ -324,6 +342,9 @@ int lcq_qparams_int(const void* min_in, const void* max_in, int dtype, int64_t n
   else if (dtype == LCQ_BF16)
     qparams_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>(
         min_in, max_in, n, scales, zeros, make_op<IntOp<true, false>>(qmin, qmax, flags, 1.0f, LCQ_CODE_NONE));
+  else if (dtype == LCQ_F16)
+    qparams_kernel<ROW_F16><<<dim3((unsigned)grid), dim3(256), 0, st>>>(
+        min_in, max_in, n, scales, zeros, make_op<IntOp<ROW_F16, false>>(qmin, qmax, flags, 1.0f, LCQ_CODE_NONE));
   else return LCQ_EDTYPE;
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;
@@ -340,6 +361,7 @@ int lcq_dequant_int(const void* q, int dtype, int64_t rows, int64_t cols, const 
   hipStream_t st = (hipStream_t)stream;
   if (dtype == LCQ_F32) dequant_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>(q, rows, cols, scales, zeros, out, scalar_qp, scale_f32, out_scale_factor);
   else if (dtype == LCQ_BF16) dequant_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>(q, rows, cols, scales, zeros, out, scalar_qp, scale_f32, out_scale_factor);
+  else if (dtype == LCQ_F16) dequant_kernel<ROW_F16><<<dim3((unsigned)grid), dim3(256), 0, st>>>(q, rows, cols, scales, zeros, out, scalar_qp, scale_f32, out_scale_factor);
   else return LCQ_EDTYPE;
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;

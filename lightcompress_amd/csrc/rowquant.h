@@ -5,7 +5,7 @@
 // dequantized values.
 //
 // An Op policy supplies the arithmetic:
-//   static constexpr bool BF            rows are bf16 (else fp32)
+//   static constexpr int BF             row type: 0 fp32, 1 bf16, 2 fp16 (a bool reads as 0 / 1)
 //   struct Row                          per-row parameters
 //   Row  make(mn, mx)                   dynamic parameters from the row range
 //   Row  load(scales, zeros, row)       static parameters
@@ -26,36 +26,50 @@
 
 namespace lcq {
 
-template <bool BF> struct Vec { static constexpr int N = BF ? 8 : 4; };
+// BF: the row type.  0 = fp32, 1 = bf16, 2 = fp16 (a bool argument reads as 0 / 1).  The fast kernels exist for fp32
+// and bf16; fp16 rows go through the element-wise kernel (row_scalar_kernel) and the element-wise forms of the ops.
+constexpr int ROW_F32 = 0, ROW_BF16 = 1, ROW_F16 = 2;
+template <int BF> struct Vec { static constexpr int N = BF ? 8 : 4; };
 typedef unsigned short lcq_u16x2 __attribute__((ext_vector_type(2)));
 
-template <bool BF> __device__ __forceinline__ float rnd(float v) {
-  if constexpr (BF) return (float)(__bf16)v; else return v;
+template <int BF> __device__ __forceinline__ float rnd(float v) {
+  if constexpr (BF == ROW_F16) return (float)(_Float16)v;
+  else if constexpr (BF) return (float)(__bf16)v;
+  else return v;
 }
-// per-element rounding: hardware RNE convert (v_cvt_pk_bf16_f32)
-template <bool BF> __device__ __forceinline__ float rnd_e(float v) {
-  if constexpr (BF) return (float)(__bf16)v; else return v;
-}
+// per-element rounding: hardware RNE convert (v_cvt_pk_bf16_f32 / v_cvt_f16_f32)
+template <int BF> __device__ __forceinline__ float rnd_e(float v) { return rnd<BF>(v); }
 __device__ __forceinline__ float clamp_min_nan(float v, float lo) { return nan_max(v, lo); }
 
 // two fp32 values -> one dword of two bf16 (RNE), a single v_cvt_pk_bf16_f32
 typedef float lcq_f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 lcq_bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 lcq_f16x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t bf16_pack_rne(float a, float b) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(lcq_f32x2{a, b}, lcq_bf16x2));
 }
+__device__ __forceinline__ uint32_t f16_pack_rne(float a, float b) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(lcq_f32x2{a, b}, lcq_f16x2));
+}
+__device__ __forceinline__ float f16_lo(uint32_t w) { return (float)__builtin_bit_cast(lcq_f16x2, w).x; }
+__device__ __forceinline__ float f16_hi(uint32_t w) { return (float)__builtin_bit_cast(lcq_f16x2, w).y; }
 // round a pair to the row type in place (bf16: one convert + two unpack ops for two elements)
-template <bool BF> __device__ __forceinline__ void rnd_pair(float& a, float& b) {
-  if constexpr (BF) {
+template <int BF> __device__ __forceinline__ void rnd_pair(float& a, float& b) {
+  if constexpr (BF == ROW_F16) {
+    a = rnd<BF>(a); b = rnd<BF>(b);
+  } else if constexpr (BF) {
     const uint32_t u = bf16_pack_rne(a, b);
     a = u2f(u << 16);
     b = u2f(u & 0xffff0000u);
   }
 }
 
-template <bool BF>
+template <int BF>
 __device__ __forceinline__ void unpack(const u32x4& raw, float* v) {
-  if constexpr (BF) {
+  if constexpr (BF == ROW_F16) {
+    #pragma unroll
+    for (int i = 0; i < 4; ++i) { v[2 * i] = f16_lo(raw[i]); v[2 * i + 1] = f16_hi(raw[i]); }
+  } else if constexpr (BF) {
     #pragma unroll
     for (int i = 0; i < 4; ++i) { v[2 * i] = bf16_lo(raw[i]); v[2 * i + 1] = bf16_hi(raw[i]); }
   } else {
@@ -63,10 +77,14 @@ __device__ __forceinline__ void unpack(const u32x4& raw, float* v) {
     for (int i = 0; i < 4; ++i) v[i] = u2f(raw[i]);
   }
 }
-template <bool BF>
+// values already exact in the row type -> one 16-byte chunk
+template <int BF>
 __device__ __forceinline__ u32x4 pack(const float* v) {
   u32x4 raw;
-  if constexpr (BF) {
+  if constexpr (BF == ROW_F16) {
+    #pragma unroll
+    for (int i = 0; i < 4; ++i) raw[i] = f16_pack_rne(v[2 * i], v[2 * i + 1]);
+  } else if constexpr (BF) {
     #pragma unroll
     for (int i = 0; i < 4; ++i) raw[i] = bf16_pack(v[2 * i], v[2 * i + 1]);
   } else {
@@ -76,22 +94,28 @@ __device__ __forceinline__ u32x4 pack(const float* v) {
   return raw;
 }
 
-template <bool BF>
+template <int BF>
 __device__ __forceinline__ float load_scalar(const void* p, int64_t i) {
-  if constexpr (BF) return u2f((uint32_t)((const uint16_t*)p)[i] << 16);
+  if constexpr (BF == ROW_F16) return (float)((const _Float16*)p)[i];
+  else if constexpr (BF) return u2f((uint32_t)((const uint16_t*)p)[i] << 16);
   else return ((const float*)p)[i];
 }
-template <bool BF>
+// v is exact in the row type
+template <int BF>
 __device__ __forceinline__ void store_scalar(void* p, int64_t i, float v) {
-  if constexpr (BF) ((uint16_t*)p)[i] = (uint16_t)(f2u(v) >> 16);
+  if constexpr (BF == ROW_F16) ((_Float16*)p)[i] = (_Float16)v;
+  else if constexpr (BF) ((uint16_t*)p)[i] = (uint16_t)(f2u(v) >> 16);
   else ((float*)p)[i] = v;
 }
 
 // values NOT yet rounded to the row type -> one 16-byte chunk, rounding (RNE) while packing
-template <bool BF>
+template <int BF>
 __device__ __forceinline__ u32x4 pack_rne(const float* v) {
   u32x4 raw;
-  if constexpr (BF) {
+  if constexpr (BF == ROW_F16) {
+    #pragma unroll
+    for (int i = 0; i < 4; ++i) raw[i] = f16_pack_rne(v[2 * i], v[2 * i + 1]);
+  } else if constexpr (BF) {
     #pragma unroll
     for (int i = 0; i < 4; ++i) raw[i] = bf16_pack_rne(v[2 * i], v[2 * i + 1]);
   } else {
@@ -104,7 +128,7 @@ __device__ __forceinline__ u32x4 pack_rne(const float* v) {
 // N codes of one 16-byte input chunk -> storage
 template <class Op>
 __device__ __forceinline__ void store_codes(const Op& op, void* codes, int64_t elem0, const float* q) {
-  constexpr bool BF = Op::BF;
+  constexpr int BF = Op::BF;
   constexpr int N = Vec<BF>::N;
   const int cd = (Op::CD >= 0) ? Op::CD : op.code_dtype;       // compile-time when the op pins it
   if (cd == LCQ_CODE_I32) {
@@ -155,7 +179,7 @@ __device__ __forceinline__ void store_code1(const Op& op, void* codes, int64_t e
 template <class Op>
 __device__ __forceinline__ void emit_chunk_generic(const Op& op, const typename Op::Row& p, const float* v_in, int64_t cidx,
                                                    void* dq, void* codes) {
-  constexpr bool BF = Op::BF;
+  constexpr int BF = Op::BF;
   constexpr int N = Vec<BF>::N;
   float v[N], q[N];
   #pragma unroll
@@ -190,7 +214,7 @@ __device__ __forceinline__ void emit_chunk_generic(const Op& op, const typename 
 template <class Op>
 __device__ __forceinline__ bool emit_chunk(const Op& op, const typename Op::Row& p, const u32x4& r, int64_t cidx,
                                            void* dq, void* codes) {
-  constexpr bool BF = Op::BF;
+  constexpr int BF = Op::BF;
   constexpr int N = Vec<BF>::N;
   float v[N], q[N];
   unpack<BF>(r, v);
@@ -426,7 +450,7 @@ template <class Op>
 __global__ __launch_bounds__(256) void row_scalar_kernel(
     const void* __restrict__ x, void* __restrict__ dq, void* __restrict__ codes,
     void* __restrict__ scales, void* __restrict__ zeros, int64_t rows, int64_t cols, Op op) {
-  constexpr bool BF = Op::BF;
+  constexpr int BF = Op::BF;
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (row >= rows) return;                                   // whole wave leaves together

@@ -143,7 +143,7 @@ class BaseQuantizer(object):
         flags = self._int_flags()
         # 0-dim ranges (per_tensor) meet the 0-dim fp32 (qmax - qmin): torch promotes the result to fp32
         if max_val.dim() == 0 and not self.sym and max_val.dtype != torch.float32:
-            flags |= L.FLAG_RANGE_BF16
+            flags |= L.FLAG_RANGE_BF16 if max_val.dtype == torch.bfloat16 else L.FLAG_RANGE_F16
             min_val, max_val = min_val.float(), max_val.float()
         scales = torch.empty_like(max_val)
         zeros = torch.tensor(0.0) if self.sym else torch.empty_like(max_val)
@@ -800,6 +800,13 @@ class IntegerQuantizer(BaseQuantizer):
         the int32 codes ever reaching HBM -> (int32 [R, K/8], scales [R, -1], None)."""
         if self.bit != 4 or not self.sym or weight.dim() != 2 or weight.shape[1] % 8 != 0:
             raise NotImplementedError('fused quantize+pack: symmetric 4-bit, 2-D weight, in_features % 8 == 0')
+        if weight.dtype == torch.float16:                   # fp16 rows have no fused kernel: quantize, then pack
+            codes, scales, _ = self.real_quant_weight_dynamic(weight)
+            packed = torch.empty((weight.shape[0], weight.shape[1] // 8), dtype=torch.int32, device=weight.device)
+            cd = {torch.int32: L.CODE_I32, torch.int8: L.CODE_I8, torch.uint8: L.CODE_U8}[codes.dtype]
+            L.check(L.lib().lcq_pack_ct(L.ptr(codes.contiguous()), L.i32(cd), L.i64(weight.shape[0]), L.i64(weight.shape[1]),
+                                        L.i32(4), L.ptr(packed), L.stream()), 'lcq_pack_ct')
+            return packed, scales, None
         rows_t = self.reshape_tensor(weight)
         _, packed, scales, _ = self._launch(rows_t, static=False, want_codes='ct4')
         qparams_shape = 1 if self.granularity == 'per_tensor' else (weight.shape[0], -1)
@@ -955,7 +962,7 @@ class FloatQuantizer(BaseQuantizer):
         flags = L.FLAG_SYM
         # 0-dim ranges (per_tensor) divided by the 0-dim fp32 qmax promote to fp32
         if max_val.dim() == 0 and max_val.dtype != torch.float32:
-            flags |= L.FLAG_RANGE_BF16
+            flags |= L.FLAG_RANGE_BF16 if max_val.dtype == torch.bfloat16 else L.FLAG_RANGE_F16
             min_val, max_val = min_val.float(), max_val.float()
         scales = torch.empty_like(max_val)
         L.check(L.lib().lcq_qparams_int(L.ptr(min_val), L.ptr(max_val), L.dtype_code(max_val.dtype),

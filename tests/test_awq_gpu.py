@@ -18,7 +18,7 @@ def make_awq(**special):
     return Awq({'weight': dict(CFG['weight']), 'special': special})
 
 
-@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32, torch.float16])
 @pytest.mark.parametrize('shape', [(256, 512), (1000, 1024), (96, 4096)])
 def test_scale_quant_bit_exact(dev, dtype, shape):
     R, K = shape
@@ -34,14 +34,14 @@ def test_scale_quant_bit_exact(dev, dtype, shape):
     assert torch.equal(wd.cpu(), w)                                # the caller's tensor is left alone
 
 
-@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32, torch.float16])
 def test_scaling_input_bit_exact(dev, dtype):
     x = (torch.randn(3, 100, 1024, generator=gen(3)) * 2).to(dtype)
     s = torch.exp(torch.randn(1024, generator=gen(4)) * 0.5).to(dtype)
     assert_bit_equal(make_awq().scaling_input(x.to(dev), s.to(dev), False), A.scaling_input(x, s), 'x / s')
 
 
-@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32, torch.float16])
 def test_act_scale_weight_scale_and_loss(dev, dtype):
     x, w, down = tiny_case(dtype, seed=5, T=300, K=512, I=640)
     awq = make_awq()
@@ -51,7 +51,7 @@ def test_act_scale_weight_scale_and_loss(dev, dtype):
     assert got.dtype == dtype
     # the sum order differs from torch's: compare before the final rounding to the tensor type
     ref64 = x.double().abs().reshape(-1, 512).mean(0)
-    tol = 2 ** -8 if dtype == torch.bfloat16 else 1e-6
+    tol = {torch.bfloat16: 2 ** -8, torch.float16: 2 ** -11, torch.float32: 1e-6}[dtype]
     assert float(((got.double() - ref64).abs() / ref64).max()) <= tol
     if dtype == torch.bfloat16:                                     # after rounding to bf16 almost all entries coincide
         assert float((got.float() != want.float()).float().mean()) < 0.02
@@ -70,7 +70,7 @@ class Fc:
         self.weight = types.SimpleNamespace(data=w)
 
 
-@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
 def test_search_scale_subset_picks_the_oracle_ratio(dev, dtype):
     x, w, down = tiny_case(dtype, seed=8, T=256, K=512, I=768)
     spec = Q.IntSpec(4, False, 'per_group', group_size=128)
@@ -84,7 +84,7 @@ def test_search_scale_subset_picks_the_oracle_ratio(dev, dtype):
     losses = awq.search_losses.cpu()
     assert best.dtype == dtype and best.shape == (512,)
     rel = ((losses.double() - torch.tensor(losses_o).double()).abs() / torch.tensor(losses_o).double()).max()
-    assert float(rel) < (0.05 if dtype == torch.bfloat16 else 1e-3), float(rel)
+    assert float(rel) < {torch.bfloat16: 0.05, torch.float16: 0.01, torch.float32: 1e-3}[dtype], float(rel)
     ko = min(range(20), key=lambda i: losses_o[i])
     kg = int(torch.argmin(losses))
     # GEMM rounding differs between CPU and GPU libraries; the chosen grid point may move only between near-ties
@@ -157,7 +157,7 @@ def test_search_scale_subset_trans_version_v1(dev, dtype):
     best_o, losses_o = A.search_scale(w, x, fwd, spec, version='v1')
     best, losses = _search_on_gpu(dev, make_awq(trans_version='v1'), w, down, [x])
     rel = ((losses.double() - torch.tensor(losses_o).double()).abs() / torch.tensor(losses_o).double()).max()
-    assert float(rel) < (0.05 if dtype == torch.bfloat16 else 1e-3), float(rel)
+    assert float(rel) < {torch.bfloat16: 0.05, torch.float16: 0.01, torch.float32: 1e-3}[dtype], float(rel)
     same, near = _same_point(losses, losses_o)
     assert near
     if same:

@@ -31,7 +31,7 @@ INT_CASES = [
 ]
 
 
-@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize('bit,sym,gran,kw,shape', INT_CASES)
 def test_int_fake_and_real_quant_bit_exact(dev, dtype, bit, sym, gran, kw, shape):
     w = weight_like(*shape, seed=bit + shape[0], dtype=dtype, outlier_frac=0.002)
@@ -63,7 +63,7 @@ def test_int_fake_and_real_quant_bit_exact(dev, dtype, bit, sym, gran, kw, shape
             assert_bit_equal(rz, orz, 'real zeros')
 
 
-@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
 def test_int_static_paths_and_minmax(dev, dtype):
     w = weight_like(128, 1024, seed=21, dtype=dtype)
     spec = Q.IntSpec(4, False, 'per_group', group_size=128)
@@ -141,7 +141,7 @@ FP_CASES = [('e4m3', 'per_channel', (64, 7168)), ('e4m3', 'per_channel', (128, 2
 
 
 @pytest.mark.parametrize('tie', ['away', 'even'])
-@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize('fmt,gran,shape', FP_CASES)
 def test_float_quant_bit_exact(dev, tie, dtype, fmt, gran, shape):
     from lightcompress_amd import FloatQuantizer
@@ -274,7 +274,7 @@ def test_pack_ct_bit_exact(dev, bits, dt, shape):
     assert torch.equal(pack_ref.unpack_ct(got.cpu(), bits, shape[1]), codes.to(torch.int32))
 
 
-@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32, torch.float16])
 @pytest.mark.parametrize('gran,shape', [('per_group', (64, 1024)), ('per_group', (2048, 7168)), ('per_channel', (96, 512)),
                                         ('per_channel', (16, 7168))])
 def test_fused_quant_pack_equals_quant_then_pack(dev, dtype, gran, shape):
@@ -670,7 +670,7 @@ def test_stream_probe_reads_everything_and_refuses_a_short_destination(dev, m):
     assert int(out.abs().sum()) == 0
 
 
-@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
 def test_int_static_activation_fake_quant_plain_and_mixed_precision(dev, dtype):
     """fake_quant_act_static (quant.py:718-751) with parameters calibrated beforehand: the whole tensor, and the
     mixed-precision form in which `int_indices` columns are quantized and `fp_indices` columns pass through."""

@@ -43,7 +43,7 @@ def test_static_scratch_entry_point_rejects_what_it_cannot_hold(dev):
     too_big = (1 << 34) + 8
     assert lib.lcq_sq_err_mean_static(L.ptr(x), L.ptr(x), L.i32(L.F32), L.i64(too_big), L.ptr(out), L.stream()) == -6
     assert lib.lcq_sq_err_mean_static(L.ptr(x), L.ptr(x), L.i32(L.F32), L.i64(0), L.ptr(out), L.stream()) == -1
-    assert lib.lcq_sq_err_mean_static(L.ptr(x), L.ptr(x), L.i32(L.F16), L.i64(64), L.ptr(out), L.stream()) == -3
+    assert lib.lcq_sq_err_mean_static(L.ptr(x), L.ptr(x), L.i32(7), L.i64(64), L.ptr(out), L.stream()) == -3      # no such type code
     with pytest.raises(L.LcqError, match='stated maximum'):
         L.check(-6, 'lcq_sq_err_mean_static')
 
