@@ -33,7 +33,13 @@ template <int BF> struct Vec { static constexpr int N = BF ? 8 : 4; };
 typedef unsigned short lcq_u16x2 __attribute__((ext_vector_type(2)));
 
 template <int BF> __device__ __forceinline__ float rnd(float v) {
-  if constexpr (BF == ROW_F16) return (float)(_Float16)v;
+  if constexpr (BF == ROW_F16) {
+    // torch rounds twice: the fp32 result of the operation, then the conversion to fp16.  The empty asm keeps the
+    // compiler from folding an fp32 multiply into a mixed-precision instruction that rounds the exact product once
+    // (v_fma_mixlo_f16): the two differ when the fp32 rounding lands on an fp16 tie (x * 1.7 does, often).
+    asm("" : "+v"(v));
+    return (float)(_Float16)v;
+  }
   else if constexpr (BF) return (float)(__bf16)v;
   else return v;
 }

@@ -28,6 +28,15 @@ def ceil_div(x, y):
     return (x + y - 1) // y
 
 
+def _scaled(scales, factor):
+    """scales * output_scale_factor as torch computes it for a number: the fp32 product, rounded, then the cast to the
+    tensor's type.  (For fp16 the GPU's fused multiply-and-convert would round the exact product once; the two differ
+    when the fp32 rounding lands on an fp16 tie, which x * 1.7 often does.)"""
+    if factor == 1 or not torch.is_tensor(scales) or scales.dtype != torch.float16:
+        return scales * factor
+    return (scales.float() * factor).to(torch.float16)
+
+
 class BaseQuantizer(object):
     """Constructor surface of quant.py:48-103."""
 
@@ -758,7 +767,7 @@ class IntegerQuantizer(BaseQuantizer):
         return torch.int32
 
     def _finish_real(self, codes, scales, zeros, output_scale_factor):
-        scales = scales * output_scale_factor
+        scales = _scaled(scales, output_scale_factor)
         dtype = self._code_dtype()
         if not self.sym and self.round_zp:
             zeros = zeros.to(dtype)
@@ -1161,10 +1170,10 @@ class FloatQuantizer(BaseQuantizer):
         if self.granularity == 'per_block':
             if static_scales is not None:
                 y = self._per_block_static(weight, static_scales, False)
-                s = static_scales * output_scale_factor
+                s = _scaled(static_scales, output_scale_factor)
                 return y, (s.view(s.shape[0], s.shape[2]) if s.dim() == 4 else s), None
             y, s = self._per_block(weight, False)
-            return y, s * output_scale_factor, None
+            return y, _scaled(s, output_scale_factor), None
         dtype = torch.float8_e4m3fn if self.e_bits == 4 else torch.float8_e5m2
         org_w_shape = weight.shape
         if static_scales is None and self.calib_algo != 'minmax':
@@ -1179,7 +1188,7 @@ class FloatQuantizer(BaseQuantizer):
                 o = self._emu(rows_t, static_scales, want=('q_fp8',))
                 scales = static_scales
             codes = self.restore_tensor(o['q_fp8'].view(rows_t.shape), org_w_shape)
-            scales = scales * output_scale_factor
+            scales = _scaled(scales, output_scale_factor)
             return codes, scales.view(1 if self.granularity == 'per_tensor' else (codes.shape[0], -1)), None
         if static_scales is None:
             _, codes, scales = self._launch(rows_t, static=False, want_codes=dtype)
@@ -1187,7 +1196,7 @@ class FloatQuantizer(BaseQuantizer):
             _, codes, _ = self._launch(rows_t, static=True, scales=static_scales, want_codes=dtype)
             scales = static_scales
         codes = self.restore_tensor(codes.view(rows_t.shape), org_w_shape)
-        scales = scales * output_scale_factor
+        scales = _scaled(scales, output_scale_factor)
         qparams_shape = 1 if self.granularity == 'per_tensor' else (codes.shape[0], -1)
         return codes, scales.view(qparams_shape), None
 

@@ -790,3 +790,28 @@ def test_int_infinite_and_nan_weights_propagate_like_torch(dev, dtype, sym):
         assert torch.equal(torch.isnan(got), torch.isnan(want)), bad
         assert torch.equal(torch.nan_to_num(got.float(), 0.0, 1e30, -1e30), torch.nan_to_num(want.float(), 0.0, 1e30, -1e30)), bad
         assert bool(torch.isnan(want[3, 128:256]).all()) or not sym
+
+
+def test_fp16_output_scale_factor_rounds_twice_like_torch(dev):
+    """scales * output_scale_factor on fp16 scales: torch forms the fp32 product, rounds it, then converts to fp16.
+    A multiply fused with the conversion rounds the exact product once, and the two disagree when the fp32 rounding lands
+    on an fp16 tie: s = 845 * 2^-11 times 1.7 is 1436.5 * 2^-11 after the fp32 rounding (1.7 is 1.70000005 in fp32, the
+    exact product lies just above the tie).  Scales built to sit on such ties, for the dequantized values and for the
+    scales real_quant_weight_static returns."""
+    k = torch.arange(5, 2048, 10)                                         # k * 1.7 = n + 0.5
+    s = (k.float() * 2.0 ** -11).to(torch.float16).reshape(-1, 1)
+    # k = 845: the exact product lies above the tie 1436.5 * 2^-11, torch's two roundings end on the even neighbour below
+    assert 845 * 2.0 ** -11 * 1.7000000476837158 > 1436.5 * 2.0 ** -11
+    assert float((s * 1.7)[84]) == 1436 * 2.0 ** -11 and float(s[84]) == 845 * 2.0 ** -11
+    R = s.shape[0]
+    x = (torch.randn(R, 64, generator=gen(5)) * 3).to(torch.float16)
+    z = torch.full((R, 1), 8.0, dtype=torch.float16)
+    spec = Q.IntSpec(4, False, 'per_channel')
+    q = _iq(4, False, 'per_channel')
+    args = dict(scales=s.to(dev), zeros=z.to(dev), qmax=spec.qmax, qmin=spec.qmin, output_scale_factor=1.7)
+    assert_bit_equal(q.fake_quant_weight_static(x.to(dev), dict(args)),
+                     Q.int_fake_quant_static(spec, x, s, z, spec.qmax, spec.qmin, output_scale_factor=1.7), 'dequantized values')
+    codes, rs, rz = q.real_quant_weight_static(x.to(dev), dict(args))
+    ocodes, ors, orz = Q.int_real_quant_static(spec, x, s, z, spec.qmax, spec.qmin, output_scale_factor=1.7)
+    assert_bit_equal(codes, ocodes, 'codes')
+    assert_bit_equal(rs, ors, 'returned scales')
