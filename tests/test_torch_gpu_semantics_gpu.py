@@ -89,3 +89,30 @@ def test_per_tensor_integer_quantizer_equals_torch_on_the_gpu(dev, dtype, bit, s
         literal_cpu = _reference_per_tensor_on_gpu(t, bit, sym, round_zp)[0]
         on_gpu = _reference_per_tensor_on_gpu(t.to(dev), bit, sym, round_zp)[0].cpu()
         assert not torch.equal(literal_cpu, on_gpu)                        # why the conversion has to be written out
+
+
+def _on(spec, dev):
+    import copy
+    s = copy.copy(spec)
+    s.qmin, s.qmax = spec.qmin.to(dev), spec.qmax.to(dev)
+    return s
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16, torch.float32])
+def test_the_integer_oracle_gives_the_same_bits_on_cpu_and_gpu_tensors(dev, dtype):
+    """The oracle is plain torch: evaluated on GPU tensors it runs torch's GPU kernels, i.e. what the reference runs.
+    Every granularity, symmetric and not, round_zp on and off, fake and real quantization: the same bits as on the CPU,
+    so a comparison with the CPU evaluation is a comparison with the GPU evaluation."""
+    w = (torch.randn(96, 1024, generator=gen(11)) * 0.05).to(dtype)
+    w[torch.rand(96, 1024, generator=gen(12)) < 0.002] *= 20
+    for bit, sym, gran, kw in ((4, False, 'per_group', dict(group_size=128)), (4, True, 'per_group', dict(group_size=64)),
+                               (3, False, 'per_group', dict(group_size=32)), (8, True, 'per_channel', {}), (8, False, 'per_channel', {}),
+                               (8, True, 'per_tensor', {}), (8, False, 'per_tensor', {}), (4, False, 'per_tensor', dict(round_zp=False)),
+                               (4, False, 'per_group', dict(group_size=128, round_zp=False)), (8, True, 'per_token', {}),
+                               (6, True, 'per_head', dict(head_num=8))):
+        spec = Q.IntSpec(bit, sym, gran, **kw)
+        assert_bit_equal(Q.int_fake_quant_dynamic(_on(spec, dev), w.to(dev)).cpu(), Q.int_fake_quant_dynamic(spec, w), f'fake {gran} {kw}')
+        if kw.get('round_zp', True) and gran not in ('per_token', 'per_head'):
+            for a, b in zip(Q.int_real_quant_dynamic(_on(spec, dev), w.to(dev)), Q.int_real_quant_dynamic(spec, w)):
+                if a is not None:
+                    assert_bit_equal(a.cpu(), b, f'real {gran} {kw}')
