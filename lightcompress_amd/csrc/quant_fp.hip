@@ -339,14 +339,17 @@ __global__ __launch_bounds__(256) void dequant_fp_kernel(const float* __restrict
 //   ls = clamp(floor(log2|xc| + bias), min=1);  s = 2^(ls - m - bias);  s == 0 -> 1
 //   q = round(xc / s + 0);  dq = (q - 0) * s
 // with a rounding to the row dtype after every operation (bf16 rows), as torch evaluates it.
-// log2 / exp2 come from the device math library: the reference's values come from another
-// vendor's library, so this path can agree with any other implementation only up to the last
-// ulp of those two functions.
+// log2 and 2^x as torch's GPU kernels compute them: the device math library's log2f, and pow(2, x) for `2.0 ** x`
+// (not exp2f, which differs from it in the last place).  With these the fp32 rows agree with torch on the GPU bit for
+// bit; torch's CPU kernels use another library and differ from both in the last place of the bias of about a quarter
+// of the rows.  bf16 rows round every intermediate to 8 bits and agree with both.
+#define LCQ_EMU_LOG2(x) log2f(x)
+#define LCQ_EMU_EXP2(x) powf(2.0f, x)
 struct EmuArgs {
   const void* x; const void* mn; const void* mx; const void* s_in;
   void* xc; void* s_out; void* q; void* dq;
   int64_t rows, cols;
-  float two_e, log_top, m_bits;
+  float two_e, m_bits;
   int is_static, scalar_qp, row_qp, q_fp8, e_bits;
 };
 
@@ -363,8 +366,10 @@ __global__ __launch_bounds__(256) void fp_emu_kernel(EmuArgs a) {
     if (!a.is_static) {
       const float mn = load_scalar<BF>(a.mn, row), mx = load_scalar<BF>(a.mx, row);
       maxval = nan_max(mx, -mn);
-      bias = rnd<BF>(a.two_e - rnd<BF>(__builtin_log2f(maxval)));
-      bias = rnd<BF>(bias + a.log_top);
+      // log2(2 - 2^-m) is a 0-dim fp32 tensor in the reference: where it is added to the 16-bit rows torch rounds it
+      // to their type first (on both platforms: a sum)
+      bias = rnd<BF>(a.two_e - rnd<BF>(LCQ_EMU_LOG2(maxval)));
+      bias = rnd<BF>(bias + rnd<BF>(LCQ_EMU_LOG2(2.0f - LCQ_EMU_EXP2(-a.m_bits))));
       bias = rnd<BF>(bias - 1.0f);
     }
     #pragma unroll
@@ -375,13 +380,13 @@ __global__ __launch_bounds__(256) void fp_emu_kernel(EmuArgs a) {
         s = load_scalar<BF>(a.s_in, a.scalar_qp ? 0 : (a.row_qp ? row : e0 + i));
       } else {
         xc[i] = nan_min(nan_max(v[i], -maxval), maxval);
-        float l = rnd<BF>(__builtin_log2f(fabsf(xc[i])));
+        float l = rnd<BF>(LCQ_EMU_LOG2(fabsf(xc[i])));
         l = rnd<BF>(l + bias);
         l = __builtin_floorf(l);
         l = clamp_min_nan(l, 1.0f);
         float ex = rnd<BF>(l - a.m_bits);
         ex = rnd<BF>(ex - bias);
-        s = rnd<BF>(__builtin_exp2f(ex));
+        s = rnd<BF>(LCQ_EMU_EXP2(ex));
       }
       if (s == 0.0f) s = 1.0f;                             // scales[scales == 0] = 1, quant.py:1061
       sc[i] = s;
@@ -475,7 +480,6 @@ int lcq_quant_fp_emu(const void* x, int dtype, int64_t rows, int64_t cols, int e
   a.x = x; a.mn = min_in; a.mx = max_in; a.s_in = scales_in; a.xc = xc; a.s_out = scales_out; a.q = q; a.dq = dq;
   a.rows = rows; a.cols = cols;
   a.two_e = (float)(1 << e_bits);
-  a.log_top = log2f(2.0f - exp2f(-(float)m_bits));
   a.m_bits = (float)m_bits;
   a.is_static = is_static; a.scalar_qp = (flags & LCQ_FLAG_SCALAR_QP) != 0; a.row_qp = (flags & LCQ_FLAG_ROW_QP) != 0;
   a.q_fp8 = q_fp8; a.e_bits = e_bits;

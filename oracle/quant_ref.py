@@ -345,13 +345,15 @@ def float_real_quant_dynamic(spec, w, output_scale_factor=1):
 # ----------------------------------------------------------------------------
 def float_emu_qparams(spec, rows: torch.Tensor, lo: torch.Tensor, hi: torch.Tensor):
     """get_float_qparams, quant.py:1004-1026, one torch op per step (the two 0-dim fp32 tensors
-    the reference creates with .cuda() live on the CPU here).  Returns (clamped rows, elementwise
-    scales).  Pinned by test_oracle_quant.py: the row maximum is a fixed point, results are
+    the reference creates with .cuda() live where the rows live).  Returns (clamped rows, elementwise
+    scales).  On GPU tensors this is the reference's own evaluation (torch's GPU log2 / pow), on CPU tensors
+    the same formula through the CPU math library: bf16 rows give the same bits either way, fp32 rows differ
+    in the last place of log2 for about a quarter of the rows.  Pinned by test_oracle_quant.py: the row maximum is a fixed point, results are
     idempotent, relative step 2**-m_bits in the normal range, fixed step below it, and an fp64
     evaluation of the same formula on exactly representable inputs."""
     maxval = torch.max(hi, -lo)
-    e_bits = torch.tensor(spec.e_bits, dtype=torch.float32)
-    m_bits = torch.tensor(spec.m_bits, dtype=torch.float32)
+    e_bits = torch.tensor(spec.e_bits, dtype=torch.float32).to(rows.device)      # `.cuda()` in the reference
+    m_bits = torch.tensor(spec.m_bits, dtype=torch.float32).to(rows.device)
     if maxval.shape[0] != 1 and len(maxval.shape) != len(rows.shape):
         maxval = maxval.view([-1] + [1] * (len(rows.shape) - 1))
     if e_bits >= 5:
