@@ -647,8 +647,8 @@ def histc_device(x: torch.Tensor, bins: int, lo: float, hi: float) -> torch.Tens
     bin = (int)((v - lo) * bins / (hi - lo)) in fp32, multiply first, the top edge counted into the last bin,
     values outside [lo, hi] dropped, lo == hi widened by one to each side.  Restated from ATen's published
     SummaryOps kernel; the CPU torch.histc divides first and so differs on values next to a bin edge - the
-    test pins this function against it up to exactly those values.  PARITY UNPINNED for the order of the
-    multiply and the divide: no device torch.histc is available to check it against."""
+    CPU test pins this function against it up to exactly those values, and the GPU test
+    (tests/test_quant_gpu.py::test_histogram_kernel) against torch.histc on GPU tensors, count for count."""
     lo32, hi32 = np.float32(lo), np.float32(hi)
     if lo32 == hi32:
         lo32, hi32 = lo32 - np.float32(1), hi32 + np.float32(1)

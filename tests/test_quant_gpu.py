@@ -578,9 +578,13 @@ def test_histogram_kernel(dev, dtype):
             got = q._histc(x.to(dev), a, b)
             want = Q.histc_device(x, bins, a, b)
             assert torch.equal(got, want), (n, bins, a, b, int((got != want).sum()))
+            # torch's own GPU kernel, as the reference calls it (quant.py:473-487): pins the binning formula itself
+            on_gpu = torch.histc(x.to(dev).float(), bins=bins, min=a, max=b).cpu()
+            assert torch.equal(got, on_gpu), (n, bins, a, b, int((got != on_gpu).sum()))
     q.bins = 64
     c = torch.full((1000,), 2.5, dtype=dtype)
     assert torch.equal(q._histc(c.to(dev), 2.5, 2.5), Q.histc_device(c, 64, 2.5, 2.5))
+    assert torch.equal(q._histc(c.to(dev), 2.5, 2.5), torch.histc(c.to(dev).float(), bins=64, min=2.5, max=2.5).cpu())
     if dtype == torch.bfloat16:
         big = torch.zeros(1 << 25, dtype=dtype, device=dev)
         big[::1024] = 1.0
