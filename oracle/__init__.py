@@ -22,6 +22,13 @@ Pinning status
   belong to the third-party QPyTorch (``qtorch``, version unpinned by the
   reference's requirements/runtime.txt), whose source is not available here:
   **parity unpinned** for those three choices; they are parameters.
+* what torch computes differently on its two platforms (0-dim tensor
+  operands next to 16-bit tensors, the math library behind log2 / pow, the
+  binning of histc): the reference runs on the GPU, so the restatements
+  follow torch's GPU kernels (``quant_ref.as_operand``, ``histc_device``) and
+  the ``-m gpu`` tests compare them, and the library, with the reference's
+  expressions evaluated by torch on GPU tensors
+  (tests/test_torch_gpu_semantics_gpu.py, test_quant_gpu.py).
 * pack / gemm_pack: pinned by unpack round trips and brute force.
 * GPTQ Hessian / Cholesky chain / column loop: pinned by fp64 closed forms
   and the loss identity  sum(Losses) == 1/2 tr((W0-Q) H (W0-Q)^T).
