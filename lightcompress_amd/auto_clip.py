@@ -26,6 +26,7 @@ import torch
 
 from . import _lib as L
 from .kernel import weight_cast_to_bf16, weight_cast_to_fp8
+from .quant import _scaled
 
 
 class AutoClipper:
@@ -151,8 +152,8 @@ class AutoClipper:
         [R, T, G, gs]-sized work is in kernels."""
         R, K = wc.shape
         G = K // group_size
-        if wc.dtype not in (torch.bfloat16, torch.float32):
-            raise NotImplementedError(f'the clip search covers bf16 and fp32 weights; got {wc.dtype}')
+        if wc.dtype not in (torch.bfloat16, torch.float32, torch.float16):
+            raise NotImplementedError(f'the clip search covers bf16, fp16 and fp32 weights; got {wc.dtype}')
         if any(x.dtype != wc.dtype for x in xs):
             raise NotImplementedError('activations and weights of different types')
         mn, mx = self._rows_minmax(wc.view(R * G, group_size))
@@ -170,8 +171,8 @@ class AutoClipper:
             if i_s == 0:
                 if self.clip_version == 'v2' and not self.w_only:
                     i_s += eps
-            max_val = org_max_val * (1 - i_s / n_grid)
-            min_val = -max_val if self.clip_sym else org_min_val * (1 - i_s / n_grid)
+            max_val = _scaled(org_max_val, 1 - i_s / n_grid)       # (fp16: the fp32 product rounded, then the cast)
+            min_val = -max_val if self.clip_sym else _scaled(org_min_val, 1 - i_s / n_grid)
             q_w = self.fake_quantize_weight(wc, min_val, max_val, org_min_val, org_max_val).contiguous()
             err_mean = 0
             for i in range(len(xs)):

@@ -125,7 +125,7 @@ __global__ __launch_bounds__(512, 1) void awq_clip_kernel(const uint16_t* __rest
   }
 }
 
-template <bool BF>
+template <int BF>
 __global__ __launch_bounds__(256) void clamp_groups_kernel(const u32x4* __restrict__ w, int64_t nchunks, int cpg,
                                                            const void* __restrict__ lo, const void* __restrict__ hi,
                                                            u32x4* __restrict__ out) {
@@ -142,7 +142,7 @@ __global__ __launch_bounds__(256) void clamp_groups_kernel(const u32x4* __restri
 }
 
 // the same clamp element by element, for group sizes that do not fill 16-byte chunks
-template <bool BF>
+template <int BF>
 __global__ __launch_bounds__(256) void clamp_groups_scalar_kernel(const void* __restrict__ w, int64_t n, int gs,
                                                                   const void* __restrict__ lo, const void* __restrict__ hi,
                                                                   void* __restrict__ out) {
@@ -162,7 +162,7 @@ __global__ __launch_bounds__(256) void clamp_groups_scalar_kernel(const void* __
 // One workgroup: 64 rows x one group, looping over 64-token tiles and 128-column chunks staged in LDS as fp32; thread
 // (ty, tx) = (tid / 16, tid % 16) owns rows ty + 16 a and tokens tx + 16 b (a, b = 0..3): 8 LDS reads per 16 products.
 constexpr int GD_J = 128, GD_P = GD_J + 1, GD_M = 64;
-template <bool BF>
+template <int BF>
 __device__ __forceinline__ void gd_stage(float (*S)[GD_P], const void* __restrict__ src, int row0, int nrows, int K,
                                          int64_t col0, int nj, bool vec, int tid) {
   constexpr int N = Vec<BF>::N;
@@ -187,7 +187,7 @@ __device__ __forceinline__ void gd_stage(float (*S)[GD_P], const void* __restric
   }
 }
 
-template <bool BF>
+template <int BF>
 __global__ __launch_bounds__(256) void group_dots_kernel(const void* __restrict__ x, const void* __restrict__ w, int R, int K,
                                                          int T, int gs, int vec, void* __restrict__ out,
                                                          const void* __restrict__ org, void* __restrict__ err) {
@@ -264,13 +264,15 @@ int lcq_group_dots(const void* x, const void* w, int dtype, int64_t R, int64_t K
   if (!x || !w || R <= 0 || K <= 0 || T <= 0 || group_size <= 0 || K % group_size != 0) return LCQ_EINVAL;
   if ((org && !err) || (!org && !out)) return LCQ_EINVAL;
   if (R > 0x7fffffff || K > 0x7fffffff || T > 0x7fffffff || K / group_size > 65535) return LCQ_EINVAL;
-  if (dtype != LCQ_BF16 && dtype != LCQ_F32) return LCQ_EDTYPE;
-  const int n = dtype == LCQ_BF16 ? 8 : 4;
+  if (dtype != LCQ_BF16 && dtype != LCQ_F32 && dtype != LCQ_F16) return LCQ_EDTYPE;
+  const int n = dtype == LCQ_F32 ? 4 : 8;
   const int vec = (K % n == 0 && group_size % n == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0) ? 1 : 0;
   const dim3 grid((unsigned)((R + GD_M - 1) / GD_M), (unsigned)(K / group_size));
   hipStream_t st = (hipStream_t)stream;
   if (dtype == LCQ_BF16)
     group_dots_kernel<true><<<grid, dim3(256), 0, st>>>(x, w, (int)R, (int)K, (int)T, group_size, vec, out, org, err);
+  else if (dtype == LCQ_F16)
+    group_dots_kernel<ROW_F16><<<grid, dim3(256), 0, st>>>(x, w, (int)R, (int)K, (int)T, group_size, vec, out, org, err);
   else
     group_dots_kernel<false><<<grid, dim3(256), 0, st>>>(x, w, (int)R, (int)K, (int)T, group_size, vec, out, org, err);
   LCQ_CHECK_LAUNCH();
@@ -301,13 +303,14 @@ int lcq_awq_clip_search(const void* w, const void* x, int64_t R, int64_t K, int6
 int lcq_clamp_groups(const void* w, int dtype, int64_t R, int64_t K, int group_size, const void* lo, const void* hi,
                      void* out, void* stream) {
   if (!w || !lo || !hi || !out || R <= 0 || K <= 0 || group_size <= 0 || K % group_size != 0) return LCQ_EINVAL;
-  if (dtype != LCQ_F32 && dtype != LCQ_BF16) return LCQ_EDTYPE;
-  const int n = dtype == LCQ_BF16 ? 8 : 4;
+  if (dtype != LCQ_F32 && dtype != LCQ_BF16 && dtype != LCQ_F16) return LCQ_EDTYPE;
+  const int n = dtype == LCQ_F32 ? 4 : 8;
   hipStream_t st = (hipStream_t)stream;
   if (group_size % n != 0 || (((uintptr_t)w | (uintptr_t)out) % 16) != 0) {
     int64_t grid = (R * K + 255) / 256;
     if (grid > 262144) grid = 262144;
     if (dtype == LCQ_BF16) clamp_groups_scalar_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>(w, R * K, group_size, lo, hi, out);
+    else if (dtype == LCQ_F16) clamp_groups_scalar_kernel<ROW_F16><<<dim3((unsigned)grid), dim3(256), 0, st>>>(w, R * K, group_size, lo, hi, out);
     else clamp_groups_scalar_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>(w, R * K, group_size, lo, hi, out);
     LCQ_CHECK_LAUNCH();
     return LCQ_OK;
@@ -316,6 +319,7 @@ int lcq_clamp_groups(const void* w, int dtype, int64_t R, int64_t K, int group_s
   int64_t grid = (nchunks + 255) / 256;
   if (grid > 262144) grid = 262144;
   if (dtype == LCQ_BF16) clamp_groups_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)w, nchunks, group_size / n, lo, hi, (u32x4*)out);
+  else if (dtype == LCQ_F16) clamp_groups_kernel<ROW_F16><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)w, nchunks, group_size / n, lo, hi, (u32x4*)out);
   else clamp_groups_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>((const u32x4*)w, nchunks, group_size / n, lo, hi, (u32x4*)out);
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;
