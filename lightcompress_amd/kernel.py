@@ -26,6 +26,8 @@ def _pad_cols(x, mult=8):
 
 
 def _block_quant(x, block_rows, flags):
+    if x.dtype == torch.float16:                            # the casts compute in fp32 (kernel.py:43, 74): an exact widening
+        return _block_quant(x.float(), block_rows, flags)
     if x.shape[-1] % 8 and block_rows != 1:
         y, s = _block_quant(_pad_cols(x), block_rows, flags)
         return y[..., :x.shape[-1]].contiguous(), s
@@ -70,6 +72,8 @@ def weight_cast_to_bf16(x, s, block_size=128):
 
 def _block_dequant(x, s, out_dtype):
     M, N = x.shape
+    if out_dtype == torch.float16:                          # float(y) * s in fp32, then the cast of the store (kernel.py:106)
+        return _block_dequant(x, s, torch.float32).to(torch.float16)
     if out_dtype not in (torch.float32, torch.bfloat16):
         raise NotImplementedError(f'output dtype {out_dtype}')
     if N % 8:

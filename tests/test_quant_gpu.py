@@ -355,7 +355,7 @@ def test_full_size_rtn_properties(dev):
     assert_bit_equal(codes[1000:1256], oc, 'slice codes'); assert_bit_equal(s[1000:1256], os_, 'slice scales')
 
 
-@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32, torch.float16])
 @pytest.mark.parametrize('shape', [(256, 384), (200, 296), (2048, 7168), (129, 8)])
 def test_blockwise_fp8_casts_bit_exact(dev, dtype, shape):
     """kernel.py (Triton semantics) and the FloatQuantizer per_block route, against their oracles: codes, scales and
