@@ -353,7 +353,7 @@ struct EmuArgs {
   int is_static, scalar_qp, row_qp, q_fp8, e_bits;
 };
 
-template <bool BF>
+template <int BF>
 __global__ __launch_bounds__(256) void fp_emu_kernel(EmuArgs a) {
   constexpr int N = Vec<BF>::N;
   const int64_t cpr = a.cols / N;                          // chunks per row (host guarantees cols % N == 0)
@@ -464,8 +464,8 @@ int lcq_quant_fp_emu(const void* x, int dtype, int64_t rows, int64_t cols, int e
   const int is_static = (flags & LCQ_FLAG_STATIC) != 0;
   if (is_static ? !scales_in : (!min_in || !max_in)) return LCQ_EINVAL;
   if ((flags & (LCQ_FLAG_SCALAR_QP | LCQ_FLAG_ROW_QP)) && !is_static) return LCQ_EINVAL;
-  if (dtype != LCQ_F32 && dtype != LCQ_BF16) return LCQ_EDTYPE;
-  const int n = (dtype == LCQ_BF16) ? 8 : 4;
+  if (dtype != LCQ_F32 && dtype != LCQ_BF16 && dtype != LCQ_F16) return LCQ_EDTYPE;
+  const int n = (dtype == LCQ_F32) ? 4 : 8;
   if (cols % n != 0) return LCQ_EINVAL;
   int q_fp8 = 0;
   if (q) {
@@ -487,6 +487,7 @@ int lcq_quant_fp_emu(const void* x, int dtype, int64_t rows, int64_t cols, int e
   if (grid > 262144) grid = 262144;
   hipStream_t st = (hipStream_t)stream;
   if (dtype == LCQ_BF16) fp_emu_kernel<true><<<dim3((unsigned)grid), dim3(256), 0, st>>>(a);
+  else if (dtype == LCQ_F16) fp_emu_kernel<ROW_F16><<<dim3((unsigned)grid), dim3(256), 0, st>>>(a);
   else fp_emu_kernel<false><<<dim3((unsigned)grid), dim3(256), 0, st>>>(a);
   LCQ_CHECK_LAUNCH();
   return LCQ_OK;

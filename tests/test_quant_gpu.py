@@ -195,7 +195,7 @@ def _agree(a, b):
     return float((a.cpu().float() == b.float()).float().mean())
 
 
-@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize('fmt,gran,shape', [('e4m3', 'per_channel', (64, 2048)), ('e4m3', 'per_group', (64, 1024)),
                                             ('e5m2', 'per_channel', (32, 1024)), ('e2m1', 'per_group', (64, 512)),
                                             ('e4m3', 'per_token', (96, 7168))])
@@ -223,6 +223,8 @@ def test_float_emulation_without_qtorch(dev, dtype, fmt, gran, shape):
         on_cpu = Q.float_emu_fake_quant_dynamic(spec, w.clone())
         if dtype == torch.bfloat16:
             assert_bit_equal(got, on_cpu, f'fake quant against the oracle on CPU tensors (case {case})')
+        elif dtype == torch.float16:                       # 11-bit intermediates: the math library shows now and then
+            assert _agree(got, on_cpu) >= 0.99
         else:
             near = (got.cpu().double() - on_cpu.double()).abs() <= on_cpu.double().abs() * 4e-6 + 1e-30
             assert float(near.float().mean()) >= 0.999
