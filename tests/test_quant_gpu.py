@@ -407,7 +407,7 @@ def test_blockwise_fp8_casts_bit_exact(dev, dtype, shape):
         assert_bit_equal(ya.view(torch.uint8), oya.view(torch.uint8), 'act codes')
 
 
-@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize('fmt,gran,shape,tie', [('e4m3', 'per_channel', (48, 1024), 'away'), ('e4m3', 'per_group', (16, 512), 'even'),
                                                 ('e2m1', 'per_group', (32, 256), 'away')])
 def test_float_quantizer_with_mse_and_learnable_ranges(dev, dtype, fmt, gran, shape, tie):
@@ -452,7 +452,7 @@ def test_float_quantizer_with_mse_and_learnable_ranges(dev, dtype, fmt, gran, sh
         FloatQuantizer(fmt, True, gran, use_qtorch=True, calib_algo='hqq', **kw).fake_quant_weight_dynamic(w.to(dev))
 
 
-@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize('bit,sym,gran,shape', [(4, False, 'per_group', (64, 1024)), (4, True, 'per_group', (32, 512)),
                                                  (8, False, 'per_channel', (48, 777)), (3, False, 'per_group', (16, 256))])
 def test_mse_calibration_against_oracle(dev, dtype, bit, sym, gran, shape):
@@ -483,19 +483,20 @@ def test_mse_calibration_against_oracle(dev, dtype, bit, sym, gran, shape):
     assert_bit_equal(got, want, 'fake quant with the calibrated ranges')
 
 
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize('bit,sym,gran,kw,shape,hqq', [
     (4, False, 'per_group', dict(group_size=64), (64, 512), {}),
     (4, False, 'per_group', dict(group_size=128), (32, 1024), dict(lp_norm=1, beta=20)),
     (3, False, 'per_channel', {}, (24, 1000), dict(iters=5)),
     (4, True, 'per_channel', {}, (16, 768), {}),
 ])
-def test_hqq_calibration_against_oracle(dev, bit, sym, gran, kw, shape, hqq):
+def test_hqq_calibration_against_oracle(dev, dtype, bit, sym, gran, kw, shape, hqq):
     """calib_algo='hqq' (quant.py:587-609, 679-687).  The scales are 1/(1/s), bit for bit.  The zero points are row
     means of fp32 terms that go through powf: they agree to 1e-4 absolute (they are of the order of qmax), the
     solver stops after the same number of iterations, and fake quantization with the kernel's own (scales, zeros)
     is the bit-exact static path."""
     from lightcompress_amd import IntegerQuantizer
-    w = weight_like(*shape, seed=shape[1] + bit, dtype=torch.bfloat16)
+    w = weight_like(*shape, seed=shape[1] + bit, dtype=dtype)
     spec = Q.IntSpec(bit, sym, gran, group_size=kw.get('group_size', 0))
     q = IntegerQuantizer(bit, sym, gran, calib_algo='hqq', **kw, **hqq)
     rows = Q.reshape_rows(spec, w.float())
