@@ -584,6 +584,25 @@ def test_histogram_kernel(dev, dtype):
             # torch's own GPU kernel, as the reference calls it (quant.py:473-487): pins the binning formula itself
             on_gpu = torch.histc(x.to(dev).float(), bins=bins, min=a, max=b).cpu()
             assert torch.equal(got, on_gpu), (n, bins, a, b, int((got != on_gpu).sum()))
+    if dtype == torch.float32:
+        # Values on and one ulp to either side of every bin edge of a range that is no power of two: here the order of
+        # the multiply and the divide matters (hundreds of these values change bin with the divide first), so equality
+        # with torch.histc on the GPU pins the order.
+        import numpy as np
+        a, b = 0.3, 7.1
+        for bins in (1000, 333):
+            e = (a + np.arange(bins + 1, dtype=np.float64) * (b - a) / bins).astype(np.float32)
+            v = np.concatenate([e, np.nextafter(e, np.float32(100)), np.nextafter(e, np.float32(-100))])
+            a32, b32 = np.float32(a), np.float32(b)
+            vi = v[(v >= a32) & (v <= b32)]
+            differ = (((vi - a32) * np.float32(bins) / (b32 - a32)).astype(np.int64)
+                      != ((vi - a32) / (b32 - a32) * np.float32(bins)).astype(np.int64)).sum()
+            assert differ >= 50, differ
+            q.bins = bins
+            xe = torch.from_numpy(v)
+            got = q._histc(xe.to(dev), a, b)
+            assert torch.equal(got, torch.histc(xe.to(dev), bins=bins, min=a, max=b).cpu()), bins
+            assert torch.equal(got, Q.histc_device(xe, bins, a, b)), bins
     q.bins = 64
     c = torch.full((1000,), 2.5, dtype=dtype)
     assert torch.equal(q._histc(c.to(dev), 2.5, 2.5), Q.histc_device(c, 64, 2.5, 2.5))
