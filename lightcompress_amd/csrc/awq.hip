@@ -64,15 +64,25 @@ __global__ __launch_bounds__(256) void absmean_stage1(const u32x4* __restrict__ 
   #pragma unroll
   for (int i = 0; i < N; ++i) p[i] = acc[i];
 }
+// torch's GPU mean is sum * factor with the fp32 factor = float(outputs) / elements (not a division by the count, which
+// is what its CPU kernel does), and the product is rounded ONCE to the output type; for fp16 outputs that is one
+// rounding of the exact product (the multiply and the conversion are one instruction there), which differs from
+// rounding to fp32 first when the fp32 product falls on a tie of the fp16 grid.
 template <int BF>
-__global__ __launch_bounds__(256) void absmean_stage2(const float* __restrict__ part, int nparts, int64_t T, int64_t K,
+__global__ __launch_bounds__(256) void absmean_stage2(const float* __restrict__ part, int nparts, float factor, int64_t K,
                                                       void* __restrict__ out) {
   const int64_t k = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (k >= K) return;
   float s = 0.0f;
   for (int p = 0; p < nparts; ++p) s += part[(int64_t)p * K + k];
-  store_scalar<BF>(out, k, rnd<BF>(s / (float)T));
+  float m;
+  if constexpr (BF == ROW_F16) m = round_to_odd_f32((double)s * (double)factor);   // 24 + 24 bits: exact in fp64
+  else m = s * factor;
+  store_scalar<BF>(out, k, rnd<BF>(m));
 }
+
+// float(outputs) / elements as torch's mean over the first dimension of [T, K] evaluates it
+inline float mean_factor(int64_t T, int64_t K) { return (float)K / (float)(T * K); }
 
 // ---- x / s[None, :] -----------------------------------------------------------------------
 template <int BF>
@@ -194,7 +204,7 @@ int absmean(const void* x, int64_t T, int64_t K, void* out, float* part, hipStre
   if (splits > PARTS_MAX) splits = PARTS_MAX;
   if (splits < 1) splits = 1;
   absmean_stage1<BF><<<dim3((unsigned)((nch + 255) / 256), (unsigned)splits), dim3(256), 0, st>>>((const u32x4*)x, T, K, part);
-  absmean_stage2<BF><<<dim3((unsigned)((K + 255) / 256)), dim3(256), 0, st>>>(part, splits, T, K, out);
+  absmean_stage2<BF><<<dim3((unsigned)((K + 255) / 256)), dim3(256), 0, st>>>(part, splits, mean_factor(T, K), K, out);
   return LCQ_OK;
 }
 
@@ -210,7 +220,7 @@ int wscale(const void* w, int64_t R, int64_t K, int g, void* out, float* part, h
   else if (team == 16) LCQ_WS(16); else if (team == 32) LCQ_WS(32); else if (team == 64) LCQ_WS(64);
   else return LCQ_EINVAL;
   #undef LCQ_WS
-  absmean_stage2<BF><<<dim3((unsigned)((K + 255) / 256)), dim3(256), 0, st>>>(part, splits, R, K, out);
+  absmean_stage2<BF><<<dim3((unsigned)((K + 255) / 256)), dim3(256), 0, st>>>(part, splits, mean_factor(R, K), K, out);
   return LCQ_OK;
 }
 

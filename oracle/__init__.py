@@ -24,8 +24,9 @@ Pinning status
   **parity unpinned** for those three choices; they are parameters.
 * what torch computes differently on its two platforms (0-dim tensor
   operands next to 16-bit tensors, the math library behind log2 / pow, the
-  binning of histc): the reference runs on the GPU, so the restatements
-  follow torch's GPU kernels (``quant_ref.as_operand``, ``histc_device``) and
+  binning of histc, the mean of a reduction): the reference runs on the GPU,
+  so the restatements follow torch's GPU kernels (``quant_ref.as_operand``,
+  ``histc_device``, ``mean_rows``) and
   the ``-m gpu`` tests compare them, and the library, with the reference's
   expressions evaluated by torch on GPU tensors
   (tests/test_torch_gpu_semantics_gpu.py, test_quant_gpu.py).

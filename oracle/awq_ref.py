@@ -24,12 +24,12 @@ def weight_scale(weights, spec):
         a = rows.abs()
         mx = a.amax(dim=1, keepdim=True)
         ls = a.div_(mx).view(shape)
-        total = ls.mean(0) if total is None else total.add_(ls.mean(0))
+        total = Q.mean_rows(ls) if total is None else total.add_(Q.mean_rows(ls))
     return total.div_(len(weights))
 
 
 def act_scale(x):
-    return x.abs().view(-1, x.shape[-1]).mean(0)
+    return Q.mean_rows(x.abs().view(-1, x.shape[-1]))
 
 
 def get_scales(x, w_max, ratio, version='v2'):
@@ -94,8 +94,8 @@ def search_scale_inputs(weights: dict, inputs: list, forward, spec, n_grid=20, v
 
     def act_scale_bs(x):                                     # get_act_scale, awq.py:74-85
         if x.shape[0] == bs:
-            return x.abs().view(-1, x.shape[-1]).mean(0)
-        means = [x[k * bs:(k + 1) * bs].abs().view(-1, x.shape[-1]).mean(0) for k in range(x.shape[0] // bs)]
+            return act_scale(x)
+        means = [act_scale(x[k * bs:(k + 1) * bs]) for k in range(x.shape[0] // bs)]
         return sum(means) / len(means)
 
     def fwd_bs(x, w):                                        # inspect_module_forward, awq.py:110-126

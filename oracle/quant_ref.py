@@ -121,6 +121,24 @@ def as_operand(t, q):
     return q
 
 
+def mean_rows(t):
+    """``t.mean(0)`` of a [N, ...] tensor (K elements per slice) the way the reference's platform computes it.  torch's GPU reduction multiplies
+    the fp32 sum by the fp32 factor float(K) / (N * K) and rounds the product ONCE to the tensor's type (for fp16 the
+    multiply and the conversion are one instruction, so even the fp32 rounding in between is absent); torch's CPU
+    kernel divides the sum by N.  The two differ in the last place for about a third of the fp32 results when N is not
+    a power of two, and for 16-bit results whenever sum / N is a tie of the 16-bit grid.  On a GPU tensor this is
+    torch itself; on a CPU tensor the GPU's rule is written out (tests/test_torch_gpu_semantics_gpu.py compares the
+    two on sums that are exact in fp32)."""
+    if t.is_cuda or t.dtype not in (torch.float32, torch.float16, torch.bfloat16):
+        return t.mean(0)
+    n, k = t.shape[0], t[0].numel()
+    factor = np.float32(k) / np.float32(n * k)
+    prod = t.float().sum(0).double() * float(factor)                # 24 x 24 bits: exact in fp64
+    if t.dtype == torch.float16:
+        return torch.from_numpy(prod.numpy().astype(np.float16))    # numpy converts fp64 -> fp16 in one rounding
+    return prod.float().to(t.dtype)
+
+
 def int_quant(spec, t, scales, zeros, qmax, qmin):
     if spec.round_zp:
         return torch.clamp(torch.round(t / as_operand(t, scales)) + as_operand(t, zeros), qmin, qmax)
@@ -617,8 +635,8 @@ def static_minmax_ranges(spec, act_tensors):
     for tensors in _batch_lists(act_tensors):
         lo = torch.stack([minmax_range(spec, reshape_rows(spec, t))[0].float() for t in tensors])
         hi = torch.stack([minmax_range(spec, reshape_rows(spec, t))[1].float() for t in tensors])
-        mins.append(lo.mean(dim=0))
-        maxs.append(hi.mean(dim=0))
+        mins.append(lo.mean(dim=0))                       # (the reference has moved the ranges to the host by now:
+        maxs.append(hi.mean(dim=0))                       # this is torch's CPU mean on either platform)
     return mins, maxs
 
 
