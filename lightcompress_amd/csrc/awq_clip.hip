@@ -114,7 +114,7 @@ __global__ __launch_bounds__(512, 1) void awq_clip_kernel(const uint16_t* __rest
       }
     }
     e += __shfl_xor(e, 32);
-    const float mean = e / (float)T;
+    const float mean = e * (1.0f / (float)T);       // torch's GPU mean: the sum times an fp32 factor
     if (errs && row_ok && h == 0) errs[((int64_t)row * G + gi) * n_steps + s] = mean;
     const float eb = rnd<true>(mean);
     if (eb < best) { best = eb; bmax = max_s; bmin = min_s; }

@@ -58,7 +58,7 @@ __global__ __launch_bounds__(1024) void diag_prep_kernel(float* __restrict__ H, 
   if (threadIdx.x == 0) {
     float t = 0.0f;
     for (int i = 0; i < 16; ++i) t += part[i];
-    sc->damp = percdamp * (t / (float)K);
+    sc->damp = percdamp * (t * (1.0f / (float)K));     // torch.mean on the GPU: the sum times an fp32 factor
     sc->status = 0;
   }
 }

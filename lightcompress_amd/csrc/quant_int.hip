@@ -190,7 +190,7 @@ __global__ __launch_bounds__(256) void hqq_step_kernel(const float* __restrict__
   acc_z = team_sum<LANES>(acc_z);
   acc_e = team_sum<LANES>(acc_e);
   if (ok && lane == 0) {
-    zeros_out[row] = acc_z / (float)cols;
+    zeros_out[row] = acc_z * (1.0f / (float)cols);      // torch.mean on the GPU: the sum times an fp32 factor
     abs_err[row] = acc_e;
     if (scales_rt) scales_rt[row] = 1.0f / inv_s;
   }

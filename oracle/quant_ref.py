@@ -500,7 +500,7 @@ def int_mse_range(spec, tensor: torch.Tensor, norm=2.4, maxshrink=0.8, mse_grid=
     for b_num in range(mse_b_num):
         _tensor = tensor[b_num * bs:(b_num + 1) * bs, :]
         _min_val, _max_val = min_val[b_num * bs:(b_num + 1) * bs, :], max_val[b_num * bs:(b_num + 1) * bs, :]
-        best = torch.full([_tensor.shape[0]], float('inf'))
+        best = torch.full([_tensor.shape[0]], float('inf'), device=_tensor.device)
         best_min_val, best_max_val = _min_val, _max_val
         for i in range(int(maxshrink * mse_grid)):
             p = 1 - i / mse_grid
@@ -531,7 +531,7 @@ def float_mse_range(spec, tensor: torch.Tensor, norm=2.4, maxshrink=0.8, mse_gri
     for b_num in range(mse_b_num):
         _tensor = tensor[b_num * bs:(b_num + 1) * bs, :]
         _min_val, _max_val = min_val[b_num * bs:(b_num + 1) * bs, :], max_val[b_num * bs:(b_num + 1) * bs, :]
-        best = torch.full([_tensor.shape[0]], float('inf'))
+        best = torch.full([_tensor.shape[0]], float('inf'), device=_tensor.device)
         best_min_val, best_max_val = _min_val, _max_val
         for i in range(int(maxshrink * mse_grid)):
             p = 1 - i / mse_grid

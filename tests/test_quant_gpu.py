@@ -492,7 +492,8 @@ def test_mse_calibration_against_oracle(dev, dtype, bit, sym, gran, shape):
 ])
 def test_hqq_calibration_against_oracle(dev, dtype, bit, sym, gran, kw, shape, hqq):
     """calib_algo='hqq' (quant.py:587-609, 679-687).  The scales are 1/(1/s), bit for bit.  The zero points are row
-    means of fp32 terms that go through powf: they agree to 1e-4 absolute (they are of the order of qmax), the
+    means of fp32 terms that go through powf: they agree to 1e-5 absolute (they are of the order of qmax: a few ulp,
+    from the order of the row sums; the oracle evaluated on GPU tensors is as far away), the
     solver stops after the same number of iterations, and fake quantization with the kernel's own (scales, zeros)
     is the bit-exact static path."""
     from lightcompress_amd import IntegerQuantizer
@@ -506,7 +507,7 @@ def test_hqq_calibration_against_oracle(dev, dtype, bit, sym, gran, kw, shape, h
     t, s, z, _, _ = q.get_tensor_qparams(w.to(dev))
     assert t.dtype == torch.float32 and s.shape == os_.shape and z.shape == oz.shape
     assert_bit_equal(s, os_, 'hqq scales')
-    assert float((z.cpu() - oz).abs().max()) <= 1e-4
+    assert float((z.cpu() - oz).abs().max()) <= 1e-5
     # same stopping point: one more iteration from the oracle's result would not be accepted either way; compare
     # the iteration count through the solver's own bookkeeping
     calls = []
