@@ -43,18 +43,6 @@ template <int BF> __device__ __forceinline__ float rnd(float v) {
   else if constexpr (BF) return (float)(__bf16)v;
   else return v;
 }
-// fp64 -> fp32 rounded to odd: the nearest fp32 toward zero, its last bit set when the value was not exact.  Rounding
-// the result to a narrower type (fp16, bf16) then gives the single correct rounding of the fp64 value.
-__device__ __forceinline__ float round_to_odd_f32(double d) {
-  float f = (float)d;
-  const double fd = (double)f;
-  if (fd != d && fd - fd == 0.0) {                       // inexact and finite
-    uint32_t u = f2u(f);
-    if (__builtin_fabs(fd) > __builtin_fabs(d)) u -= 1;  // back to the truncation (sign-magnitude: one step toward zero)
-    f = u2f(u | 1u);
-  }
-  return f;
-}
 // per-element rounding: hardware RNE convert (v_cvt_pk_bf16_f32 / v_cvt_f16_f32)
 template <int BF> __device__ __forceinline__ float rnd_e(float v) { return rnd<BF>(v); }
 __device__ __forceinline__ float clamp_min_nan(float v, float lo) { return nan_max(v, lo); }
