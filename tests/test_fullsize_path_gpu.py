@@ -349,6 +349,16 @@ def test_awq_search_at_full_size(dev):
     xm = awq.get_act_scale(x).cpu().double()
     ref = x.double().abs().reshape(-1, Hd).mean(0).cpu()
     assert float(((xm - ref).abs() / ref).max()) <= 2 ** -8
+    # the whole search once more by the oracle evaluated on the device tensors (torch's GPU kernels, the same GEMM
+    # library for the MLP): the 20 losses, the grid point and every bit of the scales
+    dspec = Q.IntSpec(4, False, 'per_group', group_size=128)
+    dspec.qmin, dspec.qmax = dspec.qmin.to(dev), dspec.qmax.to(dev)
+    best_o, losses_o = A.search_scale({k: layers[k].weight.data for k in w}, x, lambda xx, ww: mlp(xx, ww['gate'], ww['up']), dspec)
+    lo = torch.tensor(losses_o).double()
+    assert float(((losses.double() - lo).abs() / lo).max()) <= 1e-5
+    assert int(lo.argmin()) == kbest
+    assert_bit_equal(best, best_o, 'best scales against the oracle on device tensors')
+    assert_bit_equal(awq.get_act_scale(x), A.act_scale(x), 'mean |x| over 65536 tokens')
 
 
 # ---------------------------------------------------------------------------------------------------------------
