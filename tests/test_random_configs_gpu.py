@@ -297,3 +297,48 @@ def test_random_awq_configs(dev, seed):
         elif not torch.allclose(best.cpu(), best_o.cpu(), rtol=1e-5):
             problems.append(f'{desc}: fp32 scales')
     assert not problems, '\n'.join(problems)
+
+
+@pytest.mark.parametrize('seed', [0])
+def test_random_pack_configs(dev, seed):
+    """The two on-disk layouts (module_utils.py:929-955, 1097-1158) on drawn shapes, types and data: AutoAWQ words, fp16
+    scales and packed zero points from asymmetric 4-bit qparams; compressed-tensors words of symmetric 4 / 8-bit codes,
+    also with a column count that does not fill the last word, and the fused quantize-and-pack."""
+    from oracle import pack_ref as P
+    from lightcompress_amd import IntegerQuantizer
+    from lightcompress_amd.module_utils import AutoawqRealQuantLinear, VllmRealQuantLinear
+    rng = random.Random(6000 + seed)
+    problems = []
+    for it in range(40):
+        dtype = rng.choice([torch.bfloat16, torch.float16, torch.float32])
+        g = rng.choice([32, 64, 128])
+        R, K = 32 * rng.choice([1, 2, 5, 9]), g * rng.choice([1, 2, 3, 8, 17])
+        gg = torch.Generator().manual_seed(rng.randrange(1 << 30))
+        w = (torch.randn(R, K, generator=gg) * rng.choice([0.02, 1.0, 50.0])).to(dtype)
+        if rng.random() < 0.3:
+            w[torch.rand(R, K, generator=gg) < 0.01] *= 30
+        desc = f'draw {it}: {dtype} g={g} ({R},{K})'
+        spec = Q.IntSpec(4, False, 'per_group', group_size=g)
+        q = IntegerQuantizer(4, False, 'per_group', group_size=g)
+        _, s, z = q.real_quant_weight_dynamic(w.to(dev))
+        _, os_, oz = Q.int_real_quant_dynamic(spec, w)
+        got = AutoawqRealQuantLinear.gemm_pack(None, w.to(dev), s, z, {'weight': dict(bit=4, group_size=g, pack_version='gemm_pack')})
+        want = P.gemm_pack(w, os_, oz, g)
+        if not all(_same(a, b) for a, b in zip(got, want)):
+            problems.append(f'{desc}: AutoAWQ layout')
+        for bit in (4, 8):
+            kc = K if rng.random() < 0.5 else max(K - rng.choice([1, 3, 5]), 1)
+            gran = 'per_channel' if kc != K else rng.choice(['per_group', 'per_channel'])
+            kw = dict(group_size=g) if gran == 'per_group' else {}
+            wc = w[:, :kc].contiguous()
+            cspec = Q.IntSpec(bit, True, gran, group_size=kw.get('group_size', 0))
+            cq = IntegerQuantizer(bit, True, gran, **kw)
+            c, sc, _ = cq.real_quant_weight_dynamic(wc.to(dev))
+            oc, osc, _ = Q.int_real_quant_dynamic(cspec, wc)
+            want = P.pack_ct(oc, osc, bit)
+            if not all(_same(a, b) for a, b in zip(VllmRealQuantLinear.pack(c, sc, {'weight': {'bit': bit}}), want)):
+                problems.append(f'{desc}: compressed-tensors w{bit} {gran} K={kc}')
+            if bit == 4 and gran == 'per_group':
+                if not all(_same(a, b) for a, b in zip(VllmRealQuantLinear.quant_pack_fused(wc.to(dev), cq, {'weight': {'bit': 4}}), want)):
+                    problems.append(f'{desc}: fused quantize and pack')
+    assert not problems, '\n'.join(problems)
