@@ -435,7 +435,7 @@ def test_auto_clip_run_skips_query_key_and_handles_float8_weights(dev):
 
 
 # ---- apply_scale / scale_fc_fc / scale_ln_fcs / update_input_feat ---------------------------------------
-@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32, torch.float16])
 def test_scale_folding_matches_the_torch_op_sequence(dev, dtype):
     """base_blockwise_quantization.py:619-723, 772-801, 899-920: each is a literal in-place torch op in the
     reference (one IEEE multiply / divide per element in the tensor's type), so the CPU op is the oracle: bit-exact."""
