@@ -246,7 +246,9 @@ def test_random_gptq_configs(dev, seed):
 def test_random_awq_configs(dev, seed):
     """search_scale_subset (awq.py:178-278) against the oracle evaluated on GPU tensors (the inspect module then runs
     through the same GPU GEMMs on both sides): the 20 losses to 2e-5 relative, the same grid point unless two tie
-    within that, and for 16-bit models the same scale bits.  fp32 models carry the summation order of mean|x| in the
+    within that, and for 16-bit models the same scale bits (on these draws: the two means are fp32 sums in another
+    order than torch's, and a sum next to a 16-bit rounding boundary can round the other way - about one scale in a
+    thousand, none here).  fp32 models carry the summation order of mean|x| in the
     last place of every scale, which moves weights across rounding boundaries: their losses are held to 5e-3 (an 8-bit
     loss is a sum of few such events)."""
     from lightcompress_amd.awq import Awq
