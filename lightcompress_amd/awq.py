@@ -31,13 +31,17 @@ from __future__ import annotations
 import torch
 
 from . import _lib as L
+from .blockwise import ScaleFolding
 from .quant import IntegerQuantizer
 
 
-class Awq:
+class Awq(ScaleFolding):
     def __init__(self, quant_config, wquantizer=None, aquantizer=None):
         self.quant_config = quant_config
         special_config = quant_config.get('special', {})
+        self.save_scale = special_config.get('save_scale', False)
+        self.act_scales = {}
+        self.do_gqa_trans = special_config.get('do_gqa_trans', False)
         self.trans = special_config.get('trans', True)
         self.trans_version = special_config.get('trans_version', 'v2')
         self.awq_bs = special_config.get('awq_bs', None)
@@ -316,3 +320,45 @@ class Awq:
         self.search_losses = losses
         best_scales = torch.stack(scale_rows)[best]
         return best_scales
+
+    # -- awq.py:299-373 ---------------------------------------------------------------------------------
+    @torch.no_grad()
+    def subset_transform(self, subset, input_feat, subset_kwargs):
+        """Search the scales of one subset, fold them into the operator in front of it and rescale the cached inputs.
+        ``subset``: {'layers': {name: Linear}, 'prev_op': [module], 'input': [name], 'inspect': module, 'do_trans':
+        bool}.  Subsets without a single LayerNorm-like or Linear operator in front are left alone, as are Linear
+        predecessors whose width fits none of the fc-fc cases unless grouped-query scaling is on (then the statistics
+        come from the input recorded one entry earlier, the predecessor's own input)."""
+        layers_dict = subset['layers']
+        prev_op = subset['prev_op']
+        input_name = subset['input'][0]
+        inspect_module = subset['inspect']
+        if not subset.get('do_trans', True):
+            return
+        config = getattr(self, 'config', None)
+        if config is not None and config['model']['type'] == 'Starcoder' and isinstance(prev_op[0], torch.nn.Linear):
+            return
+        assert len(prev_op) in (0, 1), 'Only support single prev_op. If multi prev_ops, code need to be updated.'
+        if len(prev_op) == 0 or prev_op[0] is None:
+            return
+        op = prev_op[0]
+        is_linear = isinstance(op, torch.nn.Linear) or (hasattr(op, 'out_features') and hasattr(op, 'in_features'))
+        is_norm = not is_linear and hasattr(op, 'weight') and op.weight.dim() == 1
+        if not (is_linear or is_norm):
+            return
+        layers = list(layers_dict.values())
+        is_gqa = False
+        if is_linear:
+            width = layers[0].in_features
+            if op.out_features not in (width * 3, width * 2, width):
+                if not (self.has_gqa and self.do_gqa_trans):
+                    return
+                is_gqa = True
+                keys = list(input_feat.keys())
+                input_name = keys[keys.index(input_name) - 1]
+        scale = self.search_scale_subset(op, layers_dict, input_feat[input_name], inspect_module, is_gqa, subset_kwargs)
+        self.apply_scale(scale, prev_op, layers)
+        self.update_input_feat(scale, input_feat, layers_dict, is_gqa)
+        if self.save_scale:
+            for n in layers_dict:
+                self.act_scales[f'{self.model.block_name_prefix}.{self.block_idx}.{n}'] = scale

@@ -938,6 +938,57 @@ class GPTQ:
         if not self.wquantizer.sym:
             layer.buf_zeros = self._zeros.reshape(-1, 1).clone()
 
+    @torch.no_grad()
+    def split_qparams(self, qparams):
+        """gptq.py:332-341: a buffer as collect_block_qparams registers it, [R * G, 1] with the G groups of a row next
+        to each other, -> a list of G tensors [R, 1]."""
+        group_num = math.ceil(self.columns / self.wquantizer.group_size)
+        per_row = qparams.reshape(-1, group_num)
+        return [per_row[:, gi].reshape(-1, 1) for gi in range(group_num)]
+
+    @torch.no_grad()
+    def merge_qparams(self, qparams):
+        """gptq.py:343-356: the inverse for per_group (a list of [R, 1] -> [R * G, 1]); per_head values repeated over
+        the rows of their head; anything else as it is."""
+        if isinstance(qparams, int):
+            return qparams
+        gran = self.wquantizer.granularity
+        if gran == 'per_head':
+            head_size = self.rows // self.head_num
+            return qparams.reshape(-1).repeat_interleave(head_size).reshape(-1, 1)
+        if gran == 'per_group':
+            return torch.stack(list(qparams), dim=1).reshape(-1, 1)
+        return qparams
+
+    @torch.no_grad()
+    def search_column_qparams(self, c_tensor, idx):
+        """gptq.py:358-366: qparams of the column slab that starts at column `idx` (one group), kept as the current
+        qparams and as group idx // group_size.  (weight_transform does this inside its kernel; the method serves
+        callers that drive the loop themselves.)"""
+        _, scale, zero, qmax, qmin = self.wquantizer.get_tensor_qparams(c_tensor)
+        self.qparams = {'scale': scale, 'zero': zero, 'qmax': qmax, 'qmin': qmin}
+        gi = idx // self.wquantizer.group_size
+        if getattr(self, '_scales', None) is not None and gi < self._scales.shape[1]:
+            self._scales[:, gi] = scale.reshape(-1).float()
+            if self._zeros is not None:
+                self._zeros[:, gi] = zero.reshape(-1).float()
+
+    @torch.no_grad()
+    def search_layer_qparams(self, layer):
+        """gptq.py:368-377: the registered buffers of a per_channel / per_tensor / per_head layer as the current
+        qparams."""
+        scales = self.merge_qparams(layer.buf_scales)
+        zeros = layer.buf_zeros if self.wquantizer.sym else self.merge_qparams(layer.buf_zeros)
+        self.qparams = {'scale': scales, 'zero': zeros, 'qmax': layer.buf_qmax, 'qmin': layer.buf_qmin}
+
+    @torch.no_grad()
+    def search_group_qparams(self, layer):
+        """gptq.py:379-395: the registered per-group buffers as the loop's group table (`groups`)."""
+        G = math.ceil(self.columns / self.wquantizer.group_size)
+        self._g, self._G = self.wquantizer.group_size, G
+        self._scales = layer.buf_scales.reshape(-1, G).float().contiguous()
+        self._zeros = None if self.wquantizer.sym else layer.buf_zeros.reshape(-1, G).float().contiguous()
+
     @property
     def groups(self):
         """The reference's list of per-group dicts, materialised from the [R, G] tensors."""

@@ -210,6 +210,10 @@ class BaseQuantizer(object):
                                   L.f32(hi), L.ptr(counts), L.ptr(hist), L.stream()), 'lcq_histc')
         return hist.cpu()
 
+    def get_norm(self, delta_begin, delta_end, density):
+        """quant.py:264-277: density times the integral of x^2 over [delta_begin, delta_end]."""
+        return density * ((delta_end * delta_end * delta_end - delta_begin * delta_begin * delta_begin) / 3)
+
     def get_quantization_error(self, histogram, min_val, max_val, next_start_bin, next_end_bin):
         """quant.py:279-328: L2 error of quantizing the histogram's mass with 2**bit levels spread over the source
         bins next_start_bin..next_end_bin; every source bin is a uniform density."""
@@ -218,16 +222,15 @@ class BaseQuantizer(object):
         if dst_bin_width == 0.0:
             return 0.0
         half = dst_bin_width / 2
-        cube = lambda a, b: (b * b * b - a * a * a) / 3                       # integral of x^2 over [a, b]
         begin = (torch.arange(self.bins) - next_start_bin) * bin_width      # source bin edges from the first level's start
         end = begin + bin_width
         first = torch.clamp(torch.div(begin, dst_bin_width, rounding_mode='floor'), 0, self.dst_nbins - 1)
         last = torch.clamp(torch.div(end, dst_bin_width, rounding_mode='floor'), 0, self.dst_nbins - 1)
         density = histogram / bin_width
         norm = torch.zeros(self.bins)
-        norm += density * cube(begin - (first + 0.5) * dst_bin_width, torch.ones(self.bins) * half)
-        norm += (last - first - 1) * (density * cube(torch.tensor(-half), torch.tensor(half)))
-        norm += density * cube(torch.tensor(-half), end - (last * dst_bin_width + half))
+        norm += self.get_norm(begin - (first + 0.5) * dst_bin_width, torch.ones(self.bins) * half, density)
+        norm += (last - first - 1) * self.get_norm(torch.tensor(-half), torch.tensor(half), density)
+        norm += self.get_norm(torch.tensor(-half), end - (last * dst_bin_width + half), density)
         return norm.sum().item()
 
     def _upscale_histogram(self, histogram, orig_min, orig_max, update_min, update_max):

@@ -535,3 +535,61 @@ def test_scale_folding_float8_blockwise_weights(dev):
     assert_bit_equal(f1.weight_scale_inv.data, sc1, 'fc1 block scales')
     assert_bit_equal(f2.weight.data.view(torch.uint8), w2.view(torch.uint8), 'fc2 float8 codes')
     assert_bit_equal(f2.weight_scale_inv.data, sc2, 'fc2 block scales')
+
+
+# ---- Awq.subset_transform: search, fold, rescale the cached inputs (awq.py:299-373) ---------------------------
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+def test_subset_transform_folds_the_found_scales(dev, dtype):
+    """A norm in front of two Linears, then a Linear in front of a Linear: the scales are those of the search (the
+    oracle evaluated on the device tensors, so both sides see the same GEMMs), the operator in front is divided and
+    the Linears multiplied by them with torch's own element-wise results, the cached inputs are divided; subsets the
+    reference leaves alone are left alone."""
+    from lightcompress_amd.awq import Awq
+    K, I, T = 256, 384, 96
+    g = gen(91)
+    spec = Q.IntSpec(4, False, 'per_group', group_size=128)
+    dspec = Q.IntSpec(4, False, 'per_group', group_size=128)
+    dspec.qmin, dspec.qmax = dspec.qmin.to(dev), dspec.qmax.to(dev)
+    norm = torch.nn.LayerNorm(K).to(dtype)
+    norm.weight.data = (torch.rand(K, generator=g) + 0.5).to(dtype)
+    norm.bias.data = (torch.randn(K, generator=g) * 0.1).to(dtype)
+    gate, up, down = (torch.nn.Linear(K, I, bias=False), torch.nn.Linear(K, I, bias=False), torch.nn.Linear(I, K, bias=False))
+    for m in (gate, up, down):
+        m.weight.data = torch.randn(m.weight.shape, generator=g) * 0.03
+    norm, gate, up, down = (m.to(device=dev, dtype=dtype) for m in (norm, gate, up, down))
+    x = (torch.randn(2, T, K, generator=g) * torch.exp(torch.randn(K, generator=g))).to(dtype).to(dev)
+
+    class Mlp(torch.nn.Module):
+        def forward(self, xx):
+            return down(torch.nn.functional.silu(gate(xx)) * up(xx))
+    awq = Awq({'weight': dict(bit=4, symmetric=False, granularity='per_group', group_size=128), 'special': {}})
+    w0 = {'gate': gate.weight.data.clone(), 'up': up.weight.data.clone()}
+    nw0, nb0 = norm.weight.data.clone(), norm.bias.data.clone()
+    want_scale, _ = A.search_scale(w0, x, lambda xx, ww: down(torch.nn.functional.silu(xx @ ww['gate'].t()) * (xx @ ww['up'].t())), dspec)
+    feat = {'gate': [x.clone()], 'up': [x.clone()]}
+    awq.subset_transform({'layers': {'gate': gate, 'up': up}, 'prev_op': [norm], 'input': ['gate'], 'inspect': Mlp()}, feat, {})
+    assert_bit_equal(norm.weight.data, nw0 / want_scale, 'norm weight / s')
+    assert_bit_equal(norm.bias.data, nb0 / want_scale, 'norm bias / s')
+    assert_bit_equal(gate.weight.data, w0['gate'] * want_scale.view(1, -1), 'gate * s')
+    assert_bit_equal(up.weight.data, w0['up'] * want_scale.view(1, -1), 'up * s')
+    assert_bit_equal(feat['gate'][0], x / want_scale.view(1, -1), 'cached input / s')
+    assert_bit_equal(feat['up'][0], x / want_scale.view(1, -1), 'cached input / s')
+    # a Linear of the same width in front of one Linear (v_proj -> o_proj): rows of the first divided, with its bias
+    v, o = torch.nn.Linear(K, K, bias=True), torch.nn.Linear(K, K, bias=False)
+    for m in (v, o):
+        m.weight.data = torch.randn(m.weight.shape, generator=g) * 0.03
+    v, o = v.to(device=dev, dtype=dtype), o.to(device=dev, dtype=dtype)
+    vw0, vb0, ow0 = v.weight.data.clone(), v.bias.data.clone(), o.weight.data.clone()
+    s2, _ = A.search_scale({'o': ow0}, x, lambda xx, ww: xx @ ww['o'].t(), dspec)
+    feat = {'o': [x.clone()]}
+    awq.subset_transform({'layers': {'o': o}, 'prev_op': [v], 'input': ['o'], 'inspect': o}, feat, {})
+    assert_bit_equal(v.weight.data, vw0 / s2.view(-1, 1), 'v rows / s')
+    assert_bit_equal(v.bias.data, vb0 / s2, 'v bias / s')
+    assert_bit_equal(o.weight.data, ow0 * s2.view(1, -1), 'o * s')
+    assert_bit_equal(feat['o'][0], x / s2.view(1, -1), 'cached input / s')
+    # left alone: do_trans False, no operator in front, a predecessor of another width without grouped-query scaling
+    before = o.weight.data.clone()
+    narrow = torch.nn.Linear(K, K // 4, bias=False).to(device=dev, dtype=dtype)
+    for sub in ({'do_trans': False, 'prev_op': [v]}, {'prev_op': []}, {'prev_op': [None]}, {'prev_op': [narrow]}):
+        awq.subset_transform(dict({'layers': {'o': o}, 'input': ['o'], 'inspect': o}, **sub), {'o': [x.clone()]}, {})
+        assert torch.equal(o.weight.data, before)

@@ -1023,6 +1023,50 @@ def test_groups_view_and_ready(dev, sym):
     assert bool(gp.ready()) == bool(torch.all(layer.buf_scales != 0))
 
 
+@pytest.mark.parametrize('sym', [False, True])
+def test_qparam_bookkeeping_methods_by_name(dev, sym):
+    """split_qparams / merge_qparams / search_group_qparams / search_column_qparams / search_layer_qparams /
+    update_model_qparams (gptq.py:332-409) keep the reference's names and meaning on top of the [R, G] tables."""
+    R, K, g = 24, 384, 128
+    gp = make_gptq(weight=dict(bit=4, symmetric=sym, granularity='per_group', group_size=g))
+    w = (torch.randn(R, K, generator=gen(81)) * 0.02).bfloat16()
+    layer = linear(w.to(dev))
+    gp.collect_layer_qparams(layer)
+    gp.columns = K
+    spec = Q.IntSpec(4, sym, 'per_group', group_size=g)
+    _, os_, oz, _, _ = Q.int_tensor_qparams(spec, w)                 # [R * G, 1], groups of a row side by side
+    parts = gp.split_qparams(layer.buf_scales)
+    assert len(parts) == K // g and all(p.shape == (R, 1) for p in parts)
+    for gi, p in enumerate(parts):
+        assert_bit_equal(p, os_.reshape(R, -1)[:, gi:gi + 1], f'scales of group {gi}')
+    assert torch.equal(gp.merge_qparams(parts), layer.buf_scales) and gp.merge_qparams(3) == 3
+    gp.search_group_qparams(layer)
+    groups = gp.groups
+    assert len(groups) == K // g
+    for gi, d in enumerate(groups):
+        assert torch.equal(d['scale'], parts[gi].float())
+        if not sym:
+            assert torch.equal(d['zero'], gp.split_qparams(layer.buf_zeros)[gi].float())
+    # new parameters for the middle group from other values, as the loop finds them on the compensated weights
+    w2 = (torch.randn(R, g, generator=gen(82)) * 0.05).float()
+    gp.search_column_qparams(w2.to(dev), g)
+    _, s2, z2, _, _ = Q.int_tensor_qparams(spec, w2)
+    assert_bit_equal(gp.qparams['scale'], s2, 'current scale')
+    assert torch.equal(gp.groups[1]['scale'].cpu(), s2) and torch.equal(gp.groups[0]['scale'], parts[0].float())
+    if not sym:
+        assert torch.equal(gp.groups[1]['zero'].cpu(), z2)
+    gp.update_model_qparams(layer)
+    want = os_.reshape(R, -1).float().clone()
+    want[:, 1] = s2.reshape(-1)
+    assert torch.equal(layer.buf_scales.cpu(), want.reshape(-1, 1))
+    # per_channel: the buffers become the current qparams
+    gc = make_gptq(weight=dict(bit=4, symmetric=sym, granularity='per_channel'))
+    lc = linear(w.to(dev))
+    gc.collect_layer_qparams(lc)
+    gc.search_layer_qparams(lc)
+    assert gc.qparams['scale'] is lc.buf_scales and bool(gc.ready())
+
+
 def test_indefinite_hessian_raises_unless_the_check_is_off(dev):
     """gptq.py:172: torch.linalg.cholesky raises on a matrix that is not positive-definite; here the chain's status
     word is read before the weights are written back.  `check_positive_definite: False` skips the read."""
