@@ -45,6 +45,14 @@ class _RealQuantLinear(torch.nn.Module):
         else:
             setattr(self, name, None)
 
+    def __repr__(self):
+        """The one-line description the reference prints for its deploy modules (module_utils.py:995-1008)."""
+        fields = ('in_features', 'out_features')
+        described = ('weight_shape', 'weight_dtype', 'scales_shape', 'scales_dtype', 'zeros_shape', 'zeros_dtype')
+        parts = [f'{k}={getattr(self, k, None)}' for k in fields] + [f'bias={self.bias is not None}']
+        parts += [f'{k}={getattr(self, k, None)}' for k in described]
+        return f'{type(self).__name__}(' + ', '.join(parts) + ')'
+
 
 class VllmRealQuantLinear(_RealQuantLinear):
     def __init__(self, weight, bias, scales, input_scale, need_pack, scales_name):
@@ -103,6 +111,10 @@ class VllmRealQuantLinear(_RealQuantLinear):
         assert quant_config['weight']['bit'] == 4
         packed, scales, _ = wquantizer.real_quant_pack_dynamic(weight)
         return packed, scales.to(torch.float16)
+
+
+class SglRealQuantLinear(VllmRealQuantLinear):
+    """module_utils.py:1010-1026: the same buffers and packing under SGLang's name."""
 
 
 class AutoawqRealQuantLinear(_RealQuantLinear):

@@ -52,6 +52,14 @@ def test_vllm_new_int4_symmetric(dev, dtype, need_pack):
     assert (new.in_features, new.out_features) == (K, R) and new.scales_shape == (R, K // 128)
     with pytest.raises(NotImplementedError):
         new(torch.zeros(1, K, device=dev))
+    # the SGLang module (module_utils.py:1010-1026) is the same container under its own name
+    from lightcompress_amd.module_utils import SglRealQuantLinear
+    sgl = SglRealQuantLinear.new(Lin(w.to(dev), b.to(dev)), lambda mod: q.real_quant_weight_dynamic(mod.weight.data), cfg)
+    assert type(sgl) is SglRealQuantLinear and set(sgl.state_dict()) == set(sd)
+    for k in sd:
+        assert torch.equal(sgl.state_dict()[k], sd[k])
+    assert repr(sgl).startswith(f'SglRealQuantLinear(in_features={K}, out_features={R}, bias=True, weight_shape=')
+    assert repr(new).startswith('VllmRealQuantLinear(') and 'zeros_dtype=None' in repr(new)
 
 
 def test_vllm_new_int8_static_activation_scale(dev):
