@@ -587,6 +587,25 @@ def test_subset_transform_folds_the_found_scales(dev, dtype):
     assert_bit_equal(v.bias.data, vb0 / s2, 'v bias / s')
     assert_bit_equal(o.weight.data, ow0 * s2.view(1, -1), 'o * s')
     assert_bit_equal(feat['o'][0], x / s2.view(1, -1), 'cached input / s')
+    # grouped-query attention: v_proj is narrower than o_proj; with do_gqa_trans the statistics come from v_proj's output
+    # on the input recorded one entry earlier, and the scales are repeated over the query heads of a group
+    heads, kvh, hd = 8, 2, K // 8
+    gq = Awq({'weight': dict(bit=4, symmetric=False, granularity='per_group', group_size=128), 'special': dict(do_gqa_trans=True)})
+    gq.set_model_config(types.SimpleNamespace(hidden_size=K, num_attention_heads=heads, num_key_value_heads=kvh))
+    vk, og = torch.nn.Linear(K, kvh * hd, bias=False), torch.nn.Linear(K, K, bias=False)
+    for m in (vk, og):
+        m.weight.data = torch.randn(m.weight.shape, generator=g) * 0.03
+    vk, og = vk.to(device=dev, dtype=dtype), og.to(device=dev, dtype=dtype)
+    vw0, ow0 = vk.weight.data.clone(), og.weight.data.clone()
+    attn = (torch.randn(2, T, K, generator=g)).to(dtype).to(dev)
+    s_kv, _ = A.search_scale({'o': ow0}, x, lambda xx, ww: xx @ ww['o'].t(), dspec, gqa=(lambda xx: xx @ vw0.t(), kvh, hd, heads // kvh))
+    feat = {'v': [x.clone()], 'o': [attn.clone()]}
+    gq.subset_transform({'layers': {'o': og}, 'prev_op': [vk], 'input': ['o'], 'inspect': og}, feat, {})
+    rep = A.repeat_gqa(s_kv, kvh, hd, heads // kvh)
+    assert_bit_equal(vk.weight.data, vw0 / s_kv.view(-1, 1), 'v rows / s (grouped)')
+    assert_bit_equal(og.weight.data, ow0 * rep.view(1, -1), 'o * repeated s')
+    assert_bit_equal(feat['o'][0], attn / rep.view(1, -1), 'cached attention output / repeated s')
+    assert torch.equal(feat['v'][0], x)
     # left alone: do_trans False, no operator in front, a predecessor of another width without grouped-query scaling
     before = o.weight.data.clone()
     narrow = torch.nn.Linear(K, K // 4, bias=False).to(device=dev, dtype=dtype)
