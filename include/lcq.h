@@ -348,8 +348,8 @@ int lcq_awq_scale_quant(const void* w, int dtype, int64_t R, int64_t K, const vo
 int64_t lcq_awq_workspace_bytes(int64_t K);
 
 /* Awq.get_act_scale, awq.py:74-85: out[k] = mean_t |x[t, k]| (fp32 accumulation, result in `dtype`).
- * The mean is torch's GPU mean: the fp32 sum times the fp32 factor float(K) / (T * K), rounded once to `dtype` (torch's
- * CPU kernel divides by T instead: the last place differs when T is no power of two). */
+ * The mean is torch's GPU mean: the fp32 sum times the fp32 factor float(K) / (T * K), cast to `dtype` (torch's CPU
+ * kernel divides by T instead: the last place differs when T is no power of two). */
 int lcq_absmean_cols(const void* x, int dtype, int64_t T, int64_t K, void* out, void* workspace, void* stream);
 
 /* Awq.get_weight_scale (one layer), awq.py:58-66: out[k] = mean_r ( |W[r,k]| / max|W[r, group(k)]| ), the mean as in

@@ -65,9 +65,9 @@ __global__ __launch_bounds__(256) void absmean_stage1(const u32x4* __restrict__ 
   for (int i = 0; i < N; ++i) p[i] = acc[i];
 }
 // torch's GPU mean is sum * factor with the fp32 factor = float(outputs) / elements (not a division by the count, which
-// is what its CPU kernel does), and the product is rounded ONCE to the output type; for fp16 outputs that is one
-// rounding of the exact product (the multiply and the conversion are one instruction there), which differs from
-// rounding to fp32 first when the fp32 product falls on a tie of the fp16 grid.
+// is what its CPU kernel does); the fp32 product is then cast to the output type.  (In torch's ROCm build the compiler
+// has fused that multiply with the cast to fp16 - one rounding of the exact product, which differs when sum * factor
+// is an fp16 tie; the CUDA build rounds twice, and so does this kernel, like every other fp16 product here.)
 template <int BF>
 __global__ __launch_bounds__(256) void absmean_stage2(const float* __restrict__ part, int nparts, float factor, int64_t K,
                                                       void* __restrict__ out) {
@@ -75,10 +75,7 @@ __global__ __launch_bounds__(256) void absmean_stage2(const float* __restrict__ 
   if (k >= K) return;
   float s = 0.0f;
   for (int p = 0; p < nparts; ++p) s += part[(int64_t)p * K + k];
-  float m;
-  if constexpr (BF == ROW_F16) m = round_to_odd_f32((double)s * (double)factor);   // 24 + 24 bits: exact in fp64
-  else m = s * factor;
-  store_scalar<BF>(out, k, rnd<BF>(m));
+  store_scalar<BF>(out, k, rnd<BF>(s * factor));
 }
 
 // float(outputs) / elements as torch's mean over the first dimension of [T, K] evaluates it

@@ -17,18 +17,6 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
 __device__ __forceinline__ float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
-// fp64 -> fp32 rounded to odd: the nearest fp32 toward zero, its last bit set when the value was not exact.  Rounding
-// the result to a narrower type (fp16, bf16) then gives the single correct rounding of the fp64 value.
-__device__ __forceinline__ float round_to_odd_f32(double d) {
-  float f = (float)d;
-  const double fd = (double)f;
-  if (fd != d && fd - fd == 0.0) {                       // inexact and finite
-    uint32_t u = f2u(f);
-    if (__builtin_fabs(fd) > __builtin_fabs(d)) u -= 1;  // back to the truncation (sign-magnitude: one step toward zero)
-    f = u2f(u | 1u);
-  }
-  return f;
-}
 
 // fp32 -> bf16 (round to nearest even) -> fp32, integer form. NaN stays NaN.
 __device__ __forceinline__ float bf16_round(float f) {

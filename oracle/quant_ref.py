@@ -122,21 +122,19 @@ def as_operand(t, q):
 
 
 def mean_rows(t):
-    """``t.mean(0)`` of a [N, ...] tensor (K elements per slice) the way the reference's platform computes it.  torch's GPU reduction multiplies
-    the fp32 sum by the fp32 factor float(K) / (N * K) and rounds the product ONCE to the tensor's type (for fp16 the
-    multiply and the conversion are one instruction, so even the fp32 rounding in between is absent); torch's CPU
-    kernel divides the sum by N.  The two differ in the last place for about a third of the fp32 results when N is not
-    a power of two, and for 16-bit results whenever sum / N is a tie of the 16-bit grid.  On a GPU tensor this is
-    torch itself; on a CPU tensor the GPU's rule is written out (tests/test_torch_gpu_semantics_gpu.py compares the
-    two on sums that are exact in fp32)."""
-    if t.is_cuda or t.dtype not in (torch.float32, torch.float16, torch.bfloat16):
+    """``t.mean(0)`` of a [N, ...] tensor (K elements per slice) the way the reference's platform computes it.  torch's
+    GPU reduction multiplies the fp32 sum by the fp32 factor float(K) / (N * K) and casts the fp32 product to the
+    tensor's type; torch's CPU kernel divides the sum by N.  The two differ in the last place for about a third of the
+    fp32 results when N is not a power of two.  On a GPU tensor of fp32 or bf16 this is torch itself.  For fp16 the
+    rule is written out on either device: torch's ROCm build fuses the multiply with the cast (one rounding of the
+    exact product, different where sum * factor is an fp16 tie) while its CUDA build rounds twice, which is what the
+    restatement and the library do (tests/test_torch_gpu_semantics_gpu.py compares all of them on sums that are exact
+    in fp32)."""
+    if t.dtype not in (torch.float32, torch.float16, torch.bfloat16) or (t.is_cuda and t.dtype != torch.float16):
         return t.mean(0)
     n, k = t.shape[0], t[0].numel()
-    factor = np.float32(k) / np.float32(n * k)
-    prod = t.float().sum(0).double() * float(factor)                # 24 x 24 bits: exact in fp64
-    if t.dtype == torch.float16:
-        return torch.from_numpy(prod.numpy().astype(np.float16))    # numpy converts fp64 -> fp16 in one rounding
-    return prod.float().to(t.dtype)
+    factor = float(np.float32(k) / np.float32(n * k))
+    return (t.float().sum(0) * factor).to(t.dtype)
 
 
 def int_quant(spec, t, scales, zeros, qmax, qmin):
