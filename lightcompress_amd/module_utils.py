@@ -5,11 +5,13 @@ Mirrors ``VllmRealQuantLinear`` (module_utils.py:855-955: buffers ``weight`` / `
 ``AutoawqRealQuantLinear`` (module_utils.py:1029-1158: buffers ``qweight``, ``scales``, ``qzeros``, ``bias``;
 ``new``, ``quant_pack``, ``gemm_pack``) of ModelTC/LightCompress, so that what they hold loads in vLLM / SGLang
 (compressed-tensors) and AutoAWQ.  The reference packs on the host (numpy round trip / Python loops over
-columns); here both layouts are one kernel over device memory.
+columns); here both layouts are one kernel over device memory.  ``FakeQuantLinear`` and ``EffcientFakeQuantLinear``
+(module_utils.py:679-858) are the modules that apply the ``w_qdq`` / ``a_qdq`` partials in a forward pass.
 """
 from __future__ import annotations
 
 import math
+from functools import partial
 
 import torch
 
@@ -24,6 +26,108 @@ def _bf16_weight(module):
         from .quant import weight_cast_to_bf16
         module.weight.data = weight_cast_to_bf16(module.weight.data, module.weight_scale_inv.data,
                                                  module.block_size).to(torch.bfloat16)
+
+
+def _func_name(fn):
+    return fn.func.__name__ if isinstance(fn, partial) else fn.__name__
+
+
+class _FakeQuantBase(torch.nn.Module):
+    """What the two fake-quant modules share (module_utils.py:679-710, 775-800): the layer's weight and bias as
+    buffers, the `buf_*` entries of the original layer (qparams, clip factors, act-order indices) carried over.
+    Online rotation and the block-wise float8 GEMM of float8 checkpoints belong to other paths of the reference and
+    raise here."""
+
+    def _adopt(self, weight, bias, ori_module):
+        self.register_buffer('weight', weight)
+        if bias is not None:
+            self.register_buffer('bias', bias)
+        else:
+            self.bias = None
+        for name, buf in list(ori_module.named_buffers()) + list(ori_module.named_parameters()):
+            if name.startswith('buf_'):
+                self.register_buffer(name, buf.data)
+        if getattr(self, 'buf_rotate', False):
+            raise NotImplementedError('online rotation is not part of this path')
+        self.buf_rotate = False
+        if weight.dtype == torch.float8_e4m3fn:
+            raise NotImplementedError('forward on block-wise float8 weights (the reference\'s float8 GEMM) is not part of this path')
+        self.fp8_forward = False
+
+    def _name(self, module, w_qdq, a_qdq):
+        self.in_features, self.out_features = module.in_features, module.out_features
+        self.w_qdq_name = _func_name(w_qdq)
+        self.a_qdq_name = _func_name(a_qdq) if a_qdq is not None else 'None'
+
+
+class FakeQuantLinear(_FakeQuantBase):
+    """module_utils.py:679-772: activations through `a_qdq(x, self)`, the weight through `w_qdq(self)` on the first
+    forward (kept as `tmp_weight`; again on every forward with `dynamic_quant_weight` / `dynamic_quant_tmp_weight`),
+    then the library GEMM."""
+
+    def __init__(self, weight, bias, ori_module, w_qdq, a_qdq):
+        super().__init__()
+        self._adopt(weight, bias, ori_module)
+        self.a_qdq = a_qdq
+        self.w_qdq = w_qdq
+        self.dynamic_quant_weight = False
+        self.dynamic_quant_tmp_weight = False
+
+    def forward(self, x):
+        if self.a_qdq is not None:
+            x = self.a_qdq(x, self)
+        if not hasattr(self, 'tmp_weight'):
+            self.register_buffer('tmp_weight', self.w_qdq(self), persistent=False)
+            self.tmp_bias = self.bias
+        elif self.dynamic_quant_weight:
+            self.tmp_weight = self.w_qdq(self)
+            self.tmp_bias = self.bias
+        elif self.dynamic_quant_tmp_weight:
+            self.tmp_weight = self.w_qdq(self)
+        return torch.nn.functional.linear(x, self.tmp_weight, self.tmp_bias)
+
+    @classmethod
+    @torch.no_grad()
+    def new(cls, module, w_qdq, a_qdq):
+        bias = module.bias.data if getattr(module, 'bias', None) is not None else None
+        new_module = cls(module.weight.data, bias, ori_module=module, w_qdq=w_qdq, a_qdq=a_qdq)
+        new_module._name(module, w_qdq, a_qdq)
+        return new_module
+
+    def __repr__(self):
+        return (f'FakeQuantLinear(in_features={self.in_features},out_features={self.out_features}, '
+                f'bias={self.bias is not None},weight_quant={self.w_qdq_name},act_quant={self.a_qdq_name},'
+                f'online_rotate={self.buf_rotate})')
+
+
+class EffcientFakeQuantLinear(_FakeQuantBase):
+    """module_utils.py:775-858: the weight is fake-quantized once, when the module is made."""
+
+    def __init__(self, weight, bias, ori_module, a_qdq):
+        super().__init__()
+        self._adopt(weight, bias, ori_module)
+        self.a_qdq = a_qdq
+
+    @torch.no_grad()
+    def forward(self, x):
+        if self.a_qdq is not None:
+            x = self.a_qdq(x, self)
+        return torch.nn.functional.linear(x, self.weight, self.bias)
+
+    @classmethod
+    @torch.no_grad()
+    def new(cls, module, w_qdq, a_qdq, debug_print={}):
+        weight = w_qdq(module)
+        bias = module.bias.data if module.bias is not None else None
+        new_module = cls(weight, bias, ori_module=module, a_qdq=a_qdq)
+        new_module._name(module, w_qdq, a_qdq)
+        new_module.debug_print = debug_print
+        return new_module
+
+    def __repr__(self):
+        return (f'EffcientFakeQuantLinear(in_features={self.in_features},out_features={self.out_features},'
+                f'bias={self.bias is not None},weight_quant={self.w_qdq_name},act_quant={self.a_qdq_name},'
+                f'online_rotate={self.buf_rotate},fp8_forward={self.fp8_forward},debug_print={self.debug_print})')
 
 
 class _RealQuantLinear(torch.nn.Module):

@@ -103,3 +103,44 @@ def test_rtn_float8_blockwise_weight(dev):
     assert got.dtype == torch.float8_e4m3fn
     assert_bit_equal(got.view(torch.uint8), want8.view(torch.uint8), 'float8 codes')
     assert_bit_equal(m.weight_scale_inv.data, wants, 'fresh block scales')
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16])
+def test_fake_quant_modules_apply_the_partials(dev, dtype):
+    """FakeQuantLinear / EffcientFakeQuantLinear (module_utils.py:679-858) with the partials of get_replacement_params:
+    the forward is the library GEMM of the fake-quantized activations and weight, so with the oracle's tensors moved to
+    the device the same torch GEMM gives the same bits."""
+    from lightcompress_amd.module_utils import EffcientFakeQuantLinear, FakeQuantLinear
+    from lightcompress_amd.rtn import RTN
+    cfg = {'weight': dict(bit=4, symmetric=False, granularity='per_group', group_size=128),
+           'act': dict(bit=8, symmetric=True, granularity='per_token')}
+    rtn = RTN(cfg)
+    params = rtn.get_replacement_params('fake_quant')
+    w = weight_like(192, 512, seed=31, dtype=dtype)
+    m = torch.nn.Linear(512, 192, bias=True, dtype=dtype, device=dev)
+    m.weight.data.copy_(w)
+    b = m.bias.data.clone()
+    m.register_buffer('buf_marker', torch.ones(3, device=dev))
+    x = (torch.randn(2, 24, 512, generator=gen(32)) * 2).to(dtype)
+    wq = Q.int_fake_quant_dynamic(Q.IntSpec(4, False, 'per_group', group_size=128), w).to(dev)
+    xq = Q.int_fake_quant_dynamic(Q.IntSpec(8, True, 'per_token'), x).to(dev)
+    want = torch.nn.functional.linear(xq, wq, b)
+    for cls in (FakeQuantLinear, EffcientFakeQuantLinear):
+        new = cls.new(m, **params)
+        assert torch.equal(new.buf_marker, m.buf_marker) and (new.in_features, new.out_features) == (512, 192)
+        assert_bit_equal(new(x.to(dev)), want, cls.__name__)
+        assert f'weight_quant=w_qdq,act_quant=a_qdq' in repr(new) and repr(new).startswith(cls.__name__ + '(')
+    assert_bit_equal(EffcientFakeQuantLinear.new(m, **params).weight, wq, 'quantized once at construction')
+    lazy = FakeQuantLinear.new(m, **params)
+    assert torch.equal(lazy.weight, m.weight.data) and not hasattr(lazy, 'tmp_weight')
+    lazy(x.to(dev))
+    assert_bit_equal(lazy.tmp_weight, wq, 'quantized on the first forward')
+    lazy.weight.data.mul_(2)                                     # a later change of the weight is seen only on request
+    assert_bit_equal(lazy(x.to(dev)), want, 'cached weight')
+    lazy.dynamic_quant_weight = True
+    assert not torch.equal(lazy(x.to(dev)), want)
+    m.weight.data.copy_(w)                                       # (the module's buffer is the layer's own weight tensor)
+    # weight only
+    wo = FakeQuantLinear.new(m, **rtn.get_replacement_params('fake_quant', w_only=True))
+    assert_bit_equal(wo(x.to(dev)), torch.nn.functional.linear(x.to(dev), wq, b), 'weight only')
+    assert 'act_quant=None' in repr(wo)
