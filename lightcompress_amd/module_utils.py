@@ -54,10 +54,14 @@ class _FakeQuantBase(torch.nn.Module):
             raise NotImplementedError('forward on block-wise float8 weights (the reference\'s float8 GEMM) is not part of this path')
         self.fp8_forward = False
 
+    @classmethod
+    def get_func_name(cls, any_callable):
+        return _func_name(any_callable)
+
     def _name(self, module, w_qdq, a_qdq):
         self.in_features, self.out_features = module.in_features, module.out_features
-        self.w_qdq_name = _func_name(w_qdq)
-        self.a_qdq_name = _func_name(a_qdq) if a_qdq is not None else 'None'
+        self.w_qdq_name = self.get_func_name(w_qdq)
+        self.a_qdq_name = self.get_func_name(a_qdq) if a_qdq is not None else 'None'
 
 
 class FakeQuantLinear(_FakeQuantBase):
