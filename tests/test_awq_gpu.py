@@ -148,7 +148,7 @@ def _same_point(losses, losses_o, tol=0.02):
     return kg == ko, (kg == ko or abs(losses_o[kg] - losses_o[ko]) <= tol * losses_o[ko])
 
 
-@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
 def test_search_scale_subset_trans_version_v1(dev, dtype):
     """trans_version v1 (awq.py:97-102): scales = mean|x|^r / w_max^(1-r), w_max from get_weight_scale."""
     x, w, down = tiny_case(dtype, seed=18, T=192, K=512, I=640)

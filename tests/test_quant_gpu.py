@@ -167,7 +167,7 @@ def test_float_quant_bit_exact(dev, tie, dtype, fmt, gran, shape):
 
 
 @pytest.mark.parametrize('tie', ['away', 'even'])
-@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize('fmt,top', [('e4m3', 448.0), ('e5m2', 57344.0)])
 def test_float_quant_given_scales_around_the_float8_maximum(dev, tie, dtype, fmt, top):
     """Given scales let quotients pass the float8 maximum, where the reference's grid goes on (480 after 448, 65536
@@ -649,7 +649,7 @@ def and_bit(a, b):
     return True
 
 
-@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize('b4,b8,shape', [
     (dict(symmetric=False, granularity='per_group', group_size=128), dict(symmetric=True, granularity='per_channel'), (64, 1024)),
     (dict(symmetric=True, granularity='per_group', group_size=64, scales_bit=8, scales_symmetric=False),
@@ -800,7 +800,7 @@ def test_float_per_block_with_given_scales(dev, dtype, shape):
     assert_bit_equal(q.fake_quant_weight_dynamic(w.to(dev)), Q.float_per_block_static(spec, w, os_.view(mb, 1, nb, 1).clone()), 'dynamic per_block fake quant')
 
 
-@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize('sym', [True, False])
 def test_int_infinite_and_nan_weights_propagate_like_torch(dev, dtype, sym):
     """An infinite weight makes its group's scale infinite: every dequantized value of the group is 0 * inf = NaN, the
