@@ -56,8 +56,9 @@ class ScaleFolding:
     @torch.no_grad()
     def apply_scale(self, scales, prev_op, layers):
         assert len(prev_op) == 1, 'Only support single prev_op. If multi prev_ops, code need to be updated.'
-        if isinstance(prev_op[0], torch.nn.Linear):
-            assert len(layers) == 1
+        op = prev_op[0]
+        if isinstance(op, torch.nn.Linear) or (hasattr(op, 'out_features') and hasattr(op, 'weight') and op.weight.dim() == 2):
+            assert len(layers) == 1      # (nn.Linear and the Linear-like replacement modules, as _LLMC_LINEAR_TYPES_ there)
             self.scale_fc_fc(prev_op[0], layers[0], scales)
         elif hasattr(prev_op[0], 'weight') and prev_op[0].weight.dim() == 1:          # LayerNorm / RMSNorm
             self.scale_ln_fcs(prev_op[0], layers, scales)

@@ -587,6 +587,13 @@ def test_subset_transform_folds_the_found_scales(dev, dtype):
     assert_bit_equal(v.bias.data, vb0 / s2, 'v bias / s')
     assert_bit_equal(o.weight.data, ow0 * s2.view(1, -1), 'o * s')
     assert_bit_equal(feat['o'][0], x / s2.view(1, -1), 'cached input / s')
+    # a Linear-like replacement module in front (the reference's _LLMC_LINEAR_TYPES_) is scaled like an nn.Linear
+    from lightcompress_amd.module_utils import FakeQuantLinear
+    v.weight.data.copy_(vw0); v.bias.data.copy_(vb0); o.weight.data.copy_(ow0)
+    fv = FakeQuantLinear.new(v, w_qdq=lambda m: m.weight, a_qdq=None)
+    awq.subset_transform({'layers': {'o': o}, 'prev_op': [fv], 'input': ['o'], 'inspect': o}, {'o': [x.clone()]}, {})
+    assert_bit_equal(fv.weight.data, vw0 / s2.view(-1, 1), 'replacement module rows / s')
+    assert_bit_equal(o.weight.data, ow0 * s2.view(1, -1), 'o * s behind a replacement module')
     # grouped-query attention: v_proj is narrower than o_proj; with do_gqa_trans the statistics come from v_proj's output
     # on the input recorded one entry earlier, and the scales are repeated over the query heads of a group
     heads, kvh, hd = 8, 2, K // 8
