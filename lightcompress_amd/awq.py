@@ -31,7 +31,7 @@ from __future__ import annotations
 import torch
 
 from . import _lib as L
-from .blockwise import ScaleFolding
+from .blockwise import ScaleFolding, is_linear_like
 from .quant import IntegerQuantizer
 
 
@@ -336,13 +336,13 @@ class Awq(ScaleFolding):
         if not subset.get('do_trans', True):
             return
         config = getattr(self, 'config', None)
-        if config is not None and config['model']['type'] == 'Starcoder' and isinstance(prev_op[0], torch.nn.Linear):
+        if config is not None and config['model']['type'] == 'Starcoder' and is_linear_like(prev_op[0]):
             return
         assert len(prev_op) in (0, 1), 'Only support single prev_op. If multi prev_ops, code need to be updated.'
         if len(prev_op) == 0 or prev_op[0] is None:
             return
         op = prev_op[0]
-        is_linear = isinstance(op, torch.nn.Linear) or (hasattr(op, 'out_features') and hasattr(op, 'in_features'))
+        is_linear = is_linear_like(op)
         is_norm = not is_linear and hasattr(op, 'weight') and op.weight.dim() == 1
         if not (is_linear or is_norm):
             return

@@ -18,6 +18,15 @@ from . import _lib as L
 _MUL_COLS, _DIV_COLS, _MUL_ROWS, _DIV_ROWS = 0, 1, 2, 3
 
 
+def is_linear_like(m):
+    """nn.Linear or a module that stands in for one (the reference's _LLMC_LINEAR_TYPES_ / _TRANSFORMERS_LINEAR_TYPES_):
+    in_features, out_features and a 2-D weight."""
+    if isinstance(m, torch.nn.Linear):
+        return True
+    w = getattr(m, 'weight', None)
+    return hasattr(m, 'in_features') and hasattr(m, 'out_features') and torch.is_tensor(w) and w.dim() == 2
+
+
 def _scale_(t, s, mode):
     """In place: t (* or /) s along columns (mode 0 / 1) or rows (2 / 3); t [T, K] or [K]."""
     x = t.data
@@ -57,8 +66,8 @@ class ScaleFolding:
     def apply_scale(self, scales, prev_op, layers):
         assert len(prev_op) == 1, 'Only support single prev_op. If multi prev_ops, code need to be updated.'
         op = prev_op[0]
-        if isinstance(op, torch.nn.Linear) or (hasattr(op, 'out_features') and hasattr(op, 'weight') and op.weight.dim() == 2):
-            assert len(layers) == 1      # (nn.Linear and the Linear-like replacement modules, as _LLMC_LINEAR_TYPES_ there)
+        if is_linear_like(op):
+            assert len(layers) == 1
             self.scale_fc_fc(prev_op[0], layers[0], scales)
         elif hasattr(prev_op[0], 'weight') and prev_op[0].weight.dim() == 1:          # LayerNorm / RMSNorm
             self.scale_ln_fcs(prev_op[0], layers, scales)

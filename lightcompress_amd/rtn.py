@@ -15,7 +15,7 @@ from functools import partial
 import torch
 
 from .auto_clip import AutoClipper
-from .blockwise import ScaleFolding
+from .blockwise import ScaleFolding, is_linear_like
 from .kernel import weight_cast_to_bf16, weight_cast_to_fp8
 from .quant import FloatQuantizer, IntegerQuantizer, Weight48IntegerQuantizer
 
@@ -136,7 +136,7 @@ class RTN(ScaleFolding):
         scales_list, zeros_list, qmin_list, qmax_list = self.aquantizer.get_batch_tensors_qparams(act_tensors)
         for i, (scales, zeros, qmin, qmax) in enumerate(zip(scales_list, zeros_list, qmin_list, qmax_list)):
             for layer in layers_dict.values():
-                if not isinstance(layer, torch.nn.Linear):
+                if not is_linear_like(layer):
                     continue
                 layer.register_buffer(f'buf_act_scales_{i}', scales.cuda())
                 layer.register_buffer(f'buf_act_zeros_{i}', zeros.cuda())
